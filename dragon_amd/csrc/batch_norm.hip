@@ -1,0 +1,569 @@
+// BatchNorm kernels for gfx950.
+//
+// Replaces (dragon/kernels/normalization/op_kernels.h:36-109; CPU
+// dragon/kernels/normalization/cpu/batch_norm_kernel.cc)
+//   kernels::BatchNormExpectation   ex = sum(x)/normalizer, ex2 = sum(x^2)/normalizer
+//   kernels::BatchNorm              scale = gamma*rsig, bias = beta - scale*mu,
+//                                   y = x*scale[c] + bias[c]
+//   kernels::BatchNormWGrad         dgamma = sum dy*(x-mu)*rsig, dbeta = sum dy
+//   kernels::BatchNormTrainingGrad  dx = gamma*rsig*(dy - ((x-mu)*rsig*dgamma + dbeta)/normalizer)
+//   kernels::BatchNormInferenceGrad dx = gamma*rsig*dy (+ WGrad)
+// and fuses the training-forward operator body
+// (dragon/operators/normalization/batch_norm_op.cc:49-82: Moments, two Axpby
+// running-statistics updates, InvStd, BatchNorm) into two passes over x.
+//
+// x is [N, C, S] (NCHW) or [N, S, C] (NHWC). A channel's N*S values cannot
+// stay on-chip (800 KB per channel at 64x56x56 fp32), so statistics and
+// normalisation are separate passes over x. Per-channel reductions are split
+// over many workgroups (C alone cannot fill 256 compute units) and finished by
+// a [C]-sized kernel that also carries every [C]-sized epilogue, so no
+// separate InvStd / Axpby / fused-params launches remain on the fused path.
+#include "reduce.h"
+
+namespace dragon_hip {
+namespace {
+
+struct ChannelShape {
+  uint32_t N, C, S;
+  bool nchw;
+};
+
+inline SegmentedReduce channel_segments(const ChannelShape& sh) {
+  SegmentedReduce s{sh.C, sh.C, 0, sh.S, sh.N, sh.S, sh.C * sh.S, 1};
+  s.split = pick_split(sh.C, static_cast<int64_t>(sh.N) * sh.S);
+  return s;
+}
+inline ColumnReduce channel_columns(const ChannelShape& sh) {
+  ColumnReduce c{sh.N * sh.S, sh.C, 1};
+  c.split = pick_split(ceil_div(sh.C, kWaveSize), static_cast<int64_t>(sh.N) * sh.S * kWaveSize);
+  return c;
+}
+inline size_t channel_scratch_bytes(const ChannelShape& sh, size_t acc_bytes) {
+  const uint32_t split = sh.nchw ? channel_segments(sh).split : channel_columns(sh).split;
+  return static_cast<size_t>(sh.C) * split * 2 * acc_bytes;
+}
+
+// Runs the split reduction of accumulator F (one or two inputs) over every
+// channel and hands the per-channel totals to epilogue E.
+template <typename T, int kIn, typename F, typename E>
+void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E e,
+                     typename IO<T>::Acc* part, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const unsigned fin_grid = static_cast<unsigned>(ceil_div(sh.C, kReduceThreads));
+  if (sh.nchw) {
+    const SegmentedReduce s = channel_segments(sh);
+    const dim3 grid(s.n_out * s.split);
+    const bool vec_ok = aligned16(in0) && aligned16(in1) && sh.S % kVec == 0;
+    if (vec_ok) {
+      hipLaunchKernelGGL((reduce2_segments<T, kIn, kVec, F>), grid, dim3(kReduceThreads), 0, stream,
+                         s, in0, in1, f, part);
+    } else {
+      hipLaunchKernelGGL((reduce2_segments<T, kIn, 1, F>), grid, dim3(kReduceThreads), 0, stream, s,
+                         in0, in1, f, part);
+    }
+    hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3(fin_grid), dim3(kReduceThreads), 0, stream,
+                       sh.C, s.split, true, part, e);
+  } else {
+    const ColumnReduce c = channel_columns(sh);
+    const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
+    hipLaunchKernelGGL((reduce2_columns<T, kIn, F>), grid, dim3(kReduceThreads), 0, stream, c, in0,
+                       in1, f, part);
+    hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3(fin_grid), dim3(kReduceThreads), 0, stream,
+                       sh.C, c.split, false, part, e);
+  }
+}
+
+// ---------------------------------------------------------------- accumulators
+
+template <typename T>
+struct SumSqAccum {  // a = sum x, b = sum x^2
+  using A = typename IO<T>::Acc;
+  __device__ __forceinline__ void begin(uint32_t, uint32_t) {}
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x)[V],
+                                      const A (&)[V], A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      a += x[e];
+      b += x[e] * x[e];
+    }
+  }
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, A x, A, A& a, A& b) const {
+    a += x;
+    b += x * x;
+  }
+};
+
+template <typename T>
+struct ShiftedSumSqAccum {  // a = sum (x-s), b = sum (x-s)^2, s = first value of the channel
+  using A = typename IO<T>::Acc;
+  const T* x;
+  A shift;
+  __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
+    shift = IO<T>::load1(x + first_off);
+  }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&v)[V],
+                                      const A (&)[V], A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const A d = v[e] - shift;
+      a += d;
+      b += d * d;
+    }
+  }
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, A v, A, A& a, A& b) const {
+    const A d = v - shift;
+    a += d;
+    b += d * d;
+  }
+};
+
+template <typename T>
+struct WGradAccum {  // a = sum dy*(x-mu[c]), b = sum dy
+  using A = typename IO<T>::Acc;
+  const A* mu;
+  A m;
+  __device__ __forceinline__ void begin(uint32_t c, uint32_t) { m = mu[c]; }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x)[V],
+                                      const A (&dy)[V], A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      a += dy[e] * (x[e] - m);
+      b += dy[e];
+    }
+  }
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, A x, A dy, A& a, A& b) const {
+    a += dy * (x - m);
+    b += dy;
+  }
+};
+
+// ---------------------------------------------------------------- epilogues
+
+template <typename A>
+struct ExpectationEpilogue {
+  A normalizer;
+  A* ex;
+  A* ex2;
+  __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
+    ex[c] = a / normalizer;
+    ex2[c] = b / normalizer;
+  }
+};
+
+template <typename A>
+struct WGradEpilogue {
+  const A* rsig;
+  A* dgamma;
+  A* dbeta;
+  __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
+    dgamma[c] = a * rsig[c];
+    dbeta[c] = b;
+  }
+};
+
+// round(round(y*beta) + round(x*alpha)) as math::Axpby's Scale-then-Axpy pair.
+template <typename A>
+__device__ __forceinline__ A scale_then_axpy(A y, A beta, A x, A alpha) {
+#pragma clang fp contract(off)
+  const A scaled = y * beta;
+  const A prod = x * alpha;
+  return scaled + prod;
+}
+
+// scale = gamma*rsig; bias = beta - round(scale*mu) as the reference's array expression.
+template <typename A>
+__device__ __forceinline__ void fused_params(A mu, A rsig, A gamma, A beta, A* scale, A* bias) {
+#pragma clang fp contract(off)
+  const A s = gamma * rsig;
+  const A p = s * mu;
+  *scale = s;
+  *bias = beta - p;
+}
+
+// Everything [C]-sized of the training forward in one epilogue: mean/var from
+// the shifted sums, running statistics, rsig, scale and bias.
+template <typename T>
+struct TrainingStatsEpilogue {
+  using A = typename IO<T>::Acc;
+  const T* x;
+  uint32_t chan_stride;  // S for NCHW, 1 for NHWC
+  A inv_n, momentum, one_minus_momentum, eps;
+  const A* gamma;
+  const A* beta;
+  A* running_mean;
+  A* running_var;
+  A* mu;
+  A* rsig;
+  A* scale;
+  A* bias;
+  __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
+    const A shift = IO<T>::load1(x + c * chan_stride);
+    const A d = a * inv_n;
+    const A mean = shift + d;
+    const A var = b * inv_n - d * d;
+    running_mean[c] = scale_then_axpy(running_mean[c], momentum, mean, one_minus_momentum);
+    running_var[c] = scale_then_axpy(running_var[c], momentum, var, one_minus_momentum);
+    const A rs = acc_rsqrt_exact(var + eps);
+    mu[c] = mean;
+    rsig[c] = rs;
+    fused_params(mean, rs, gamma[c], beta[c], scale + c, bias + c);
+  }
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void fused_params_kernel(const uint32_t C, const A* mu,
+                                                           const A* rsig, const A* gamma,
+                                                           const A* beta, A* scale, A* bias) {
+  const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+  if (c < C) fused_params(mu[c], rsig[c], gamma[c], beta[c], scale + c, bias + c);
+}
+
+// ---------------------------------------------------------------- maps
+
+// Channel of the first element of a packet, and whether the packet spans kVec
+// consecutive channels (NHWC) or one channel (NCHW).
+struct ChannelIndex {
+  ChannelShape sh;
+  __device__ __forceinline__ uint32_t operator()(uint32_t i) const {
+    return sh.nchw ? (i / sh.S) % sh.C : i % sh.C;
+  }
+};
+
+template <typename T, int kVec>
+struct AffineApply {  // y = x*scale[c] + bias[c]
+  using A = typename IO<T>::Acc;
+  ChannelIndex idx;
+  const A* scale;
+  const A* bias;
+  __device__ __forceinline__ void operator()(uint32_t i, A (&v)[kVec], const A (&)[kVec]) const {
+    const uint32_t c = idx(i);
+    if (idx.sh.nchw) {
+      const A s = scale[c], b = bias[c];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) v[e] = v[e] * s + b;
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) v[e] = v[e] * scale[c + e] + bias[c + e];
+    }
+  }
+};
+
+template <typename T, int kVec>
+struct TrainingGradApply {
+  using A = typename IO<T>::Acc;
+  ChannelIndex idx;
+  const A* mu;
+  const A* rsig;
+  const A* gamma;
+  const A* dgamma;
+  const A* dbeta;
+  A normalizer;
+  __device__ __forceinline__ A one(A x, A dy, uint32_t c) const {
+    const A r = rsig[c];
+    const A x_norm = (x - mu[c]) * r;
+    return gamma[c] * r * (dy - (x_norm * dgamma[c] + dbeta[c]) / normalizer);
+  }
+  __device__ __forceinline__ void operator()(uint32_t i, A (&x)[kVec], const A (&dy)[kVec]) const {
+    const uint32_t c = idx(i);
+    if (idx.sh.nchw) {
+      const A r = rsig[c], m = mu[c], g = gamma[c] * r, dg = dgamma[c], db = dbeta[c];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        x[e] = g * (dy[e] - ((x[e] - m) * r * dg + db) / normalizer);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) x[e] = one(x[e], dy[e], c + e);
+    }
+  }
+};
+
+template <typename T, int kVec>
+struct InferenceGradApply {  // dx = dy * gamma[c] * rsig[c]
+  using A = typename IO<T>::Acc;
+  ChannelIndex idx;
+  const A* rsig;
+  const A* gamma;
+  __device__ __forceinline__ void operator()(uint32_t i, A (&dy)[kVec], const A (&)[kVec]) const {
+    const uint32_t c = idx(i);
+    if (idx.sh.nchw) {
+      const A g = gamma[c] * rsig[c];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) dy[e] = dy[e] * g;
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) dy[e] = dy[e] * (gamma[c + e] * rsig[c + e]);
+    }
+  }
+};
+
+template <typename T, int kIn, template <typename, int> class F, typename... Args>
+void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hipStream_t stream,
+                  Args... args) {
+  constexpr int kVec = IO<T>::kVec;
+  const uint32_t total = sh.N * sh.C * sh.S;
+  const bool vec_ok = aligned16(in0) && aligned16(in1) && aligned16(out) &&
+      (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
+  if (vec_ok) {
+    F<T, kVec> f{ChannelIndex{sh}, args...};
+    hipLaunchKernelGGL((map_flat<T, kIn, kVec, F<T, kVec>>), dim3(map_grid(total / kVec)), dim3(256),
+                       0, stream, total, in0, in1, out, f);
+  } else {
+    F<T, 1> f{ChannelIndex{sh}, args...};
+    hipLaunchKernelGGL((map_flat<T, kIn, 1, F<T, 1>>), dim3(map_grid(total)), dim3(256), 0, stream,
+                       total, in0, in1, out, f);
+  }
+}
+
+// ---------------------------------------------------------------- launchers
+
+template <typename T>
+int launch_expectation(const ChannelShape& sh, float normalizer, const void* x, void* ex, void* ex2,
+                       void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  const T* xp = static_cast<const T*>(x);
+  reduce_channels<T, 1>(sh, xp, xp, SumSqAccum<T>{},
+                        ExpectationEpilogue<A>{A(normalizer), static_cast<A*>(ex), static_cast<A*>(ex2)},
+                        static_cast<A*>(scratch), stream);
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_batch_norm(const ChannelShape& sh, const void* x, const void* mu, const void* rsig,
+                      const void* gamma, const void* beta, void* scale, void* bias, void* y,
+                      hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  A* sp = static_cast<A*>(scale);
+  A* bp = static_cast<A*>(bias);
+  hipLaunchKernelGGL((fused_params_kernel<A>), dim3(static_cast<unsigned>(ceil_div(sh.C, 256))),
+                     dim3(256), 0, stream, sh.C, static_cast<const A*>(mu),
+                     static_cast<const A*>(rsig), static_cast<const A*>(gamma),
+                     static_cast<const A*>(beta), sp, bp);
+  const T* xp = static_cast<const T*>(x);
+  map_channels<T, 1, AffineApply>(sh, xp, xp, static_cast<T*>(y), stream,
+                                  static_cast<const A*>(sp), static_cast<const A*>(bp));
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_wgrad(const ChannelShape& sh, const void* x, const void* mu, const void* rsig,
+                 const void* dy, void* dgamma, void* dbeta, void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  reduce_channels<T, 2>(sh, static_cast<const T*>(x), static_cast<const T*>(dy),
+                        WGradAccum<T>{static_cast<const A*>(mu), A(0)},
+                        WGradEpilogue<A>{static_cast<const A*>(rsig), static_cast<A*>(dgamma),
+                                         static_cast<A*>(dbeta)},
+                        static_cast<A*>(scratch), stream);
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_training_grad(const ChannelShape& sh, float normalizer, const void* x, const void* mu,
+                         const void* rsig, const void* gamma, const void* dgamma, const void* dbeta,
+                         const void* dy, void* dx, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  map_channels<T, 2, TrainingGradApply>(
+      sh, static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(dx), stream,
+      static_cast<const A*>(mu), static_cast<const A*>(rsig), static_cast<const A*>(gamma),
+      static_cast<const A*>(dgamma), static_cast<const A*>(dbeta), A(normalizer));
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_inference_grad(const ChannelShape& sh, const void* rsig, const void* gamma,
+                          const void* dy, void* dx, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  const T* dyp = static_cast<const T*>(dy);
+  map_channels<T, 1, InferenceGradApply>(sh, dyp, dyp, static_cast<T*>(dx), stream,
+                                         static_cast<const A*>(rsig), static_cast<const A*>(gamma));
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_training_forward(const ChannelShape& sh, float momentum, float eps, const void* x,
+                            const void* gamma, const void* beta, void* running_mean,
+                            void* running_var, void* mu, void* rsig, void* params, void* y,
+                            void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  const T* xp = static_cast<const T*>(x);
+  A* pp = static_cast<A*>(params);
+  const float one_minus = 1.f - momentum;  // evaluated in float as the operator does
+  TrainingStatsEpilogue<T> e{xp,
+                             sh.nchw ? sh.S : 1u,
+                             A(1) / A(static_cast<int64_t>(sh.N) * sh.S),
+                             A(momentum),
+                             A(one_minus),
+                             A(eps),
+                             static_cast<const A*>(gamma),
+                             static_cast<const A*>(beta),
+                             static_cast<A*>(running_mean),
+                             static_cast<A*>(running_var),
+                             static_cast<A*>(mu),
+                             static_cast<A*>(rsig),
+                             pp,
+                             pp + sh.C};
+  reduce_channels<T, 1>(sh, xp, xp, ShiftedSumSqAccum<T>{xp, A(0)}, e, static_cast<A*>(scratch),
+                        stream);
+  map_channels<T, 1, AffineApply>(sh, xp, xp, static_cast<T*>(y), stream,
+                                  static_cast<const A*>(pp), static_cast<const A*>(pp + sh.C));
+  return status_of_launch();
+}
+
+int make_shape(int64_t N, int64_t C, int64_t S, int layout, ChannelShape* sh) {
+  if (N < 0 || C <= 0 || S < 0) return DRAGON_HIP_EINVAL;
+  if (layout != DRAGON_HIP_NCHW && layout != DRAGON_HIP_NHWC) return DRAGON_HIP_EINVAL;
+  if (!fits_int32(N * C * S)) return DRAGON_HIP_EINVAL;
+  sh->N = static_cast<uint32_t>(N), sh->C = static_cast<uint32_t>(C);
+  sh->S = static_cast<uint32_t>(S), sh->nchw = layout == DRAGON_HIP_NCHW;
+  return DRAGON_HIP_OK;
+}
+
+inline size_t acc_bytes(int dtype) { return dtype == DRAGON_HIP_F64 ? 8 : 4; }
+
+inline int check_scratch(const ChannelShape& sh, int dtype, const void* scratch, size_t bytes) {
+  return (scratch && bytes >= channel_scratch_bytes(sh, acc_bytes(dtype))) ? DRAGON_HIP_OK
+                                                                           : DRAGON_HIP_ESCRATCH;
+}
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" {
+
+using dragon_hip::ChannelShape;
+
+size_t dragon_hip_batch_norm_reduce_scratch_bytes(int dtype, int64_t N, int64_t C, int64_t S,
+                                                  int layout) {
+  ChannelShape sh;
+  if (dragon_hip::make_shape(N, C, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  return dragon_hip::channel_scratch_bytes(sh, dragon_hip::acc_bytes(dtype));
+}
+
+int dragon_hip_batch_norm_expectation(int dtype, int64_t N, int64_t C, int64_t S,
+                                      float normalizer, int layout, const void* x, void* ex,
+                                      void* ex2, void* scratch, size_t scratch_bytes,
+                                      void* stream) {
+  ChannelShape sh;
+  int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (!ex || !ex2) return DRAGON_HIP_EINVAL;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (N * S == 0) {
+    const int acc_tag = dtype == DRAGON_HIP_F64 ? DRAGON_HIP_F64 : DRAGON_HIP_F32;
+    const int e1 = dragon_hip_set(acc_tag, C, 0.f, ex, s);
+    return e1 != DRAGON_HIP_OK ? e1 : dragon_hip_set(acc_tag, C, 0.f, ex2, s);
+  }
+  if (!x) return DRAGON_HIP_EINVAL;
+  if ((st = dragon_hip::check_scratch(sh, dtype, scratch, scratch_bytes)) != DRAGON_HIP_OK) return st;
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_expectation, sh, normalizer, x, ex, ex2,
+                            scratch, s);
+}
+
+int dragon_hip_batch_norm(int dtype, int64_t N, int64_t C, int64_t S, int layout, const void* x,
+                          const void* mu, const void* rsig, const void* gamma,
+                          const void* beta, void* scale, void* bias, void* y, void* stream) {
+  ChannelShape sh;
+  const int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (!mu || !rsig || !gamma || !beta || !scale || !bias) return DRAGON_HIP_EINVAL;
+  if (N * S > 0 && (!x || !y)) return DRAGON_HIP_EINVAL;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  // Aliasing conventions of the reference launcher.
+  const size_t acc = dragon_hip::acc_bytes(dtype);
+  if (scale == rsig) {
+    scale = static_cast<char*>(const_cast<void*>(rsig)) + acc * C;
+    bias = static_cast<char*>(const_cast<void*>(rsig)) + acc * C * 2;
+  } else if (scale == bias) {
+    bias = static_cast<char*>(scale) + acc * C;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_batch_norm, sh, x, mu, rsig, gamma, beta,
+                            scale, bias, y, s);
+}
+
+int dragon_hip_batch_norm_wgrad(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                const void* x, const void* mu, const void* rsig, const void* dy,
+                                void* dgamma, void* dbeta, void* scratch, size_t scratch_bytes,
+                                void* stream) {
+  ChannelShape sh;
+  int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (!dgamma || !dbeta) return DRAGON_HIP_EINVAL;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  const size_t acc = dragon_hip::acc_bytes(dtype);
+  if (dgamma == dbeta) dbeta = static_cast<char*>(dgamma) + acc * C;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (N * S == 0) {
+    const int acc_tag = dtype == DRAGON_HIP_F64 ? DRAGON_HIP_F64 : DRAGON_HIP_F32;
+    const int e1 = dragon_hip_set(acc_tag, C, 0.f, dgamma, s);
+    return e1 != DRAGON_HIP_OK ? e1 : dragon_hip_set(acc_tag, C, 0.f, dbeta, s);
+  }
+  if (!x || !mu || !rsig || !dy) return DRAGON_HIP_EINVAL;
+  if ((st = dragon_hip::check_scratch(sh, dtype, scratch, scratch_bytes)) != DRAGON_HIP_OK) return st;
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_wgrad, sh, x, mu, rsig, dy, dgamma, dbeta,
+                            scratch, s);
+}
+
+int dragon_hip_batch_norm_training_grad(int dtype, int64_t N, int64_t C, int64_t S,
+                                        float normalizer, int layout, const void* x,
+                                        const void* mu, const void* rsig, const void* gamma,
+                                        const void* dgamma, const void* dbeta, const void* dy,
+                                        void* dx, void* stream) {
+  ChannelShape sh;
+  const int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!x || !mu || !rsig || !gamma || !dgamma || !dbeta || !dy || !dx) return DRAGON_HIP_EINVAL;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  if (dgamma == dbeta) {
+    dbeta = static_cast<const char*>(dgamma) + dragon_hip::acc_bytes(dtype) * C;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_training_grad, sh, normalizer, x, mu, rsig,
+                            gamma, dgamma, dbeta, dy, dx, s);
+}
+
+int dragon_hip_batch_norm_inference_grad(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                         const void* x, const void* mu, const void* rsig,
+                                         const void* gamma, const void* dy, void* dgamma,
+                                         void* dbeta, void* dx, void* scratch,
+                                         size_t scratch_bytes, void* stream) {
+  if (dgamma != nullptr) {
+    const int st = dragon_hip_batch_norm_wgrad(dtype, N, C, S, layout, x, mu, rsig, dy, dgamma,
+                                               dbeta, scratch, scratch_bytes, stream);
+    if (st != DRAGON_HIP_OK) return st;
+  }
+  ChannelShape sh;
+  const int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!rsig || !gamma || !dy || !dx) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_inference_grad, sh, rsig, gamma, dy, dx, s);
+}
+
+int dragon_hip_batch_norm_training_forward(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                           float momentum, float eps, const void* x,
+                                           const void* gamma, const void* beta,
+                                           void* running_mean, void* running_var, void* mu,
+                                           void* rsig, void* params, void* y, void* scratch,
+                                           size_t scratch_bytes, void* stream) {
+  ChannelShape sh;
+  int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_EINVAL;  // statistics of an empty batch are undefined
+  if (!x || !gamma || !beta || !running_mean || !running_var || !mu || !rsig || !params || !y) {
+    return DRAGON_HIP_EINVAL;
+  }
+  if ((st = dragon_hip::check_scratch(sh, dtype, scratch, scratch_bytes)) != DRAGON_HIP_OK) return st;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_training_forward, sh, momentum, eps, x, gamma,
+                            beta, running_mean, running_var, mu, rsig, params, y, scratch, s);
+}
+
+} // extern "C"

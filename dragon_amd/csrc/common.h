@@ -1,0 +1,279 @@
+// Shared device-side building blocks for the gfx950 norm / softmax kernels:
+// 16-byte packet I/O with conversion to the accumulator type, wave64 and
+// workgroup reductions, Chan/Welford partial-moment combination, and the
+// launch helpers every entry point uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dragon_hip.h"
+
+namespace dragon_hip {
+
+constexpr int kWaveSize = 64;  // CDNA wavefront width
+constexpr int kNumCUs = 256;   // MI355X compute units (8 XCDs x 32)
+
+// 16-bit storage types: same bit layout as dragon::float16 / dragon::bfloat16
+// (dragon/core/types.h:36-42), a bare unsigned short.
+struct f16_t {
+  uint16_t x;
+};
+struct bf16_t {
+  uint16_t x;
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
+
+// IO<T>: how a tensor element type travels through HBM.
+//   Acc    accumulator type (math::Traits<T>::accumulator_type,
+//          dragon/utils/math/types.h:69-152)
+//   kVec   elements per 16-byte packet
+//   load / store   one aligned 16-byte packet <-> kVec accumulators
+//   load1 / store1 one element (tails and unaligned tensors)
+// Rounding on store is round-to-nearest-even in hardware, which is what the
+// reference's software conversion implements (dragon/utils/conversions.h:42-106).
+template <typename T>
+struct IO;
+
+template <>
+struct IO<float> {
+  using Acc = float;
+  static constexpr int kVec = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    f32x4 t = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+  }
+  static __device__ __forceinline__ float load1(const float* p) { return *p; }
+  static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+};
+
+template <>
+struct IO<double> {
+  using Acc = double;
+  static constexpr int kVec = 2;
+  static __device__ __forceinline__ void load(const double* p, double (&v)[2]) {
+    const f64x2 t = *reinterpret_cast<const f64x2*>(p);
+    v[0] = t.x, v[1] = t.y;
+  }
+  static __device__ __forceinline__ void store(double* p, const double (&v)[2]) {
+    f64x2 t = {v[0], v[1]};
+    __builtin_nontemporal_store(t, reinterpret_cast<f64x2*>(p));
+  }
+  static __device__ __forceinline__ double load1(const double* p) { return *p; }
+  static __device__ __forceinline__ void store1(double* p, double v) { *p = v; }
+};
+
+template <>
+struct IO<f16_t> {
+  using Acc = float;
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ void load(const f16_t* p, float (&v)[8]) {
+    const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const h16x2 h = __builtin_bit_cast(h16x2, t[i]);
+      v[2 * i] = static_cast<float>(h.x);
+      v[2 * i + 1] = static_cast<float>(h.y);
+    }
+  }
+  static __device__ __forceinline__ void store(f16_t* p, const float (&v)[8]) {
+    u32x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 f = {v[2 * i], v[2 * i + 1]};
+      t[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
+    }
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+  }
+  static __device__ __forceinline__ float load1(const f16_t* p) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, p->x));
+  }
+  static __device__ __forceinline__ void store1(f16_t* p, float v) {
+    p->x = __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+  }
+};
+
+template <>
+struct IO<bf16_t> {
+  using Acc = float;
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __builtin_bit_cast(float, t[i] << 16);
+      v[2 * i + 1] = __builtin_bit_cast(float, t[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    u32x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 f = {v[2 * i], v[2 * i + 1]};
+      t[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, b16x2));
+    }
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+  }
+  static __device__ __forceinline__ float load1(const bf16_t* p) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(p->x) << 16);
+  }
+  static __device__ __forceinline__ void store1(bf16_t* p, float v) {
+    p->x = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+  }
+};
+
+// kVec consecutive accumulator-typed parameters (gamma, beta, ...), 16-byte
+// aligned at p.
+template <int kVec>
+__device__ __forceinline__ void load_params(const float* p, float (&v)[kVec]) {
+  static_assert(kVec % 4 == 0, "float parameters travel in packets of four");
+#pragma unroll
+  for (int i = 0; i < kVec / 4; ++i) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p + 4 * i);
+    v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+  }
+}
+template <int kVec>
+__device__ __forceinline__ void load_params(const double* p, double (&v)[kVec]) {
+  static_assert(kVec == 2, "double parameters travel in packets of two");
+  const f64x2 t = *reinterpret_cast<const f64x2*>(p);
+  v[0] = t.x, v[1] = t.y;
+}
+
+// ---------------------------------------------------------------------------
+// Reductions
+// ---------------------------------------------------------------------------
+struct SumOp {
+  template <typename A>
+  __device__ __forceinline__ A operator()(A a, A b) const {
+    return a + b;
+  }
+};
+struct MaxOp {
+  template <typename A>
+  __device__ __forceinline__ A operator()(A a, A b) const {
+    return a > b ? a : b;
+  }
+};
+
+// Butterfly all-reduce over the 64 lanes of a wavefront: every lane ends up
+// with the result. kWidth < 64 reduces within aligned lane groups.
+template <typename A, typename Op, int kWidth = kWaveSize>
+__device__ __forceinline__ A wave_allreduce(A v, Op op) {
+#pragma unroll
+  for (int o = kWidth / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, kWaveSize));
+  return v;
+}
+
+// All-reduce over a workgroup of kWaves wavefronts through kWaves LDS slots.
+// `slots` must not be reused by another reduction before the next barrier.
+template <int kWaves, typename A, typename Op>
+__device__ __forceinline__ A block_allreduce(A v, Op op, A* slots) {
+  v = wave_allreduce(v, op);
+  if (kWaves == 1) return v;
+  const int wave = threadIdx.x / kWaveSize;
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) slots[wave] = v;
+  __syncthreads();
+  A r = slots[0];
+#pragma unroll
+  for (int i = 1; i < kWaves; ++i) r = op(r, slots[i]);
+  return r;
+}
+
+// Partial moments of a set of values: count, mean and M2 = sum (x - mean)^2.
+// merge() is Chan's pairwise update, the parallel form of Welford's
+// recurrence; it stays accurate when |mean| >> stddev, unlike E[x^2] - E[x]^2.
+template <typename A>
+struct Moments {
+  A n, mean, m2;
+  __device__ __forceinline__ void merge(const Moments& o) {
+    const A nn = n + o.n;
+    if (nn > A(0)) {
+      const A d = o.mean - mean;
+      const A f = o.n / nn;
+      mean += d * f;
+      m2 += o.m2 + d * d * n * f;
+      n = nn;
+    }
+  }
+};
+
+template <typename A, int kWidth = kWaveSize>
+__device__ __forceinline__ Moments<A> wave_allreduce_moments(Moments<A> v) {
+#pragma unroll
+  for (int o = kWidth / 2; o > 0; o >>= 1) {
+    Moments<A> t;
+    t.n = __shfl_xor(v.n, o, kWaveSize);
+    t.mean = __shfl_xor(v.mean, o, kWaveSize);
+    t.m2 = __shfl_xor(v.m2, o, kWaveSize);
+    v.merge(t);
+  }
+  return v;
+}
+
+template <int kWaves, typename A>
+__device__ __forceinline__ Moments<A> block_allreduce_moments(Moments<A> v, A* slots /*3*kWaves*/) {
+  v = wave_allreduce_moments(v);
+  if (kWaves == 1) return v;
+  const int wave = threadIdx.x / kWaveSize;
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+    slots[3 * wave] = v.n, slots[3 * wave + 1] = v.mean, slots[3 * wave + 2] = v.m2;
+  }
+  __syncthreads();
+  Moments<A> r = {slots[0], slots[1], slots[2]};
+#pragma unroll
+  for (int i = 1; i < kWaves; ++i) {
+    Moments<A> t = {slots[3 * i], slots[3 * i + 1], slots[3 * i + 2]};
+    r.merge(t);
+  }
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// Scalar math in the accumulator type
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float acc_rsqrt_exact(float v) { return 1.0f / sqrtf(v); }
+__device__ __forceinline__ double acc_rsqrt_exact(double v) { return 1.0 / sqrt(v); }
+__device__ __forceinline__ float acc_exp(float v) { return expf(v); }
+__device__ __forceinline__ double acc_exp(double v) { return exp(v); }
+__device__ __forceinline__ float acc_log(float v) { return logf(v); }
+__device__ __forceinline__ double acc_log(double v) { return log(v); }
+template <typename A>
+__device__ __forceinline__ A acc_neg_inf();
+template <>
+__device__ __forceinline__ float acc_neg_inf<float>() { return -__builtin_inff(); }
+template <>
+__device__ __forceinline__ double acc_neg_inf<double>() { return -__builtin_inf(); }
+
+// ---------------------------------------------------------------------------
+// Host-side helpers
+// ---------------------------------------------------------------------------
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int status_of_launch() {
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DRAGON_HIP_OK : static_cast<int>(e);
+}
+
+// Runs FN<T>(args...) for the element type a dtype tag names.
+#define DRAGON_HIP_DISPATCH_DTYPE(dtype, FN, ...)                       \
+  switch (dtype) {                                                      \
+    case DRAGON_HIP_F16: return FN<dragon_hip::f16_t>(__VA_ARGS__);     \
+    case DRAGON_HIP_BF16: return FN<dragon_hip::bf16_t>(__VA_ARGS__);   \
+    case DRAGON_HIP_F32: return FN<float>(__VA_ARGS__);                 \
+    case DRAGON_HIP_F64: return FN<double>(__VA_ARGS__);                \
+    default: return DRAGON_HIP_EDTYPE;                                  \
+  }
+
+} // namespace dragon_hip

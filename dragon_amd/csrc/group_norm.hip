@@ -1,0 +1,649 @@
+// GroupNorm forward / backward and LayerNorm backward for gfx950.
+//
+// Replaces
+//   kernels::GroupNorm      dragon/kernels/normalization/op_kernels.h:111-124
+//                           (CPU cpu/group_norm_kernel.cc:11-31,88-110)
+//   kernels::GroupNormGrad  dragon/kernels/normalization/op_kernels.h:126-143
+//                           (CPU cpu/group_norm_kernel.cc:33-84,112-147)
+// and, because LayerNormGradientOp is GroupNormGradientOp with G = S = 1,
+// D = C and layout NHWC (dragon/operators/normalization/layer_norm_op.h:39-54),
+// LayerNorm backward.
+//
+// x is [N, G, D, S] (NCHW) or [N, S, G, D] (NHWC); channel c = g*D + d, group
+// statistics index ng = n*G + g.
+//   y      = (x - mu[ng]) * rsig[ng] * gamma[c] + beta[c]
+//   ds[ng] = sum gamma[c]*dy*x          db[ng] = sum gamma[c]*dy
+//   dx     = gamma[c]*dy*rsig + ((db*mu - ds)*(x - mu)*rsig^3 - db*rsig) / (D*S)
+//   dgamma[c] = sum dy*(x - mu[ng])*rsig[ng]    dbeta[c] = sum dy
+//
+// Paths
+//   rows   (G = S = 1, i.e. LayerNorm backward): one fused kernel keeps x and
+//          dy of a row in registers, so both are read once; dgamma/dbeta are
+//          accumulated per thread across the rows a workgroup visits, combined
+//          through LDS, written as one partial row per workgroup, and summed
+//          by a second small kernel (two-stage, no atomics).
+//   general  three split reductions / one flat map, any layout, any alignment.
+#include "reduce.h"
+#include "row_tile.h"
+
+namespace dragon_hip {
+namespace {
+
+struct GroupShape {
+  uint32_t N, G, D, S, C;  // C = G*D
+  bool nchw;
+};
+
+// --------------------------------------------------------------------------
+// Forward map
+// --------------------------------------------------------------------------
+template <typename T, int kVec>
+struct GroupNormApply {
+  using A = typename IO<T>::Acc;
+  GroupShape sh;
+  const A* mu;
+  const A* rsig;
+  const A* gamma;
+  const A* beta;
+  __device__ __forceinline__ void operator()(uint32_t i, A (&v)[kVec], const A (&)[kVec]) const {
+    if (sh.nchw) {
+      // A packet never straddles a row of S elements (kVec divides S or is 1).
+      const uint32_t row = i / sh.S;  // = n*C + c
+      const uint32_t c = row % sh.C;
+      const uint32_t ng = row / sh.D;
+      const A m = mu[ng];
+      const A r = rsig[ng];
+      const A g = gamma[c], b = beta[c];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) v[e] = (v[e] - m) * r * g + b;
+    } else {
+      const uint32_t c = i % sh.C;  // kVec divides C or is 1
+      const uint32_t n = i / (sh.S * sh.C);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const uint32_t ce = c + e;
+        const uint32_t ng = n * sh.G + (sh.G == 1 ? 0u : ce / sh.D);
+        v[e] = (v[e] - mu[ng]) * rsig[ng] * gamma[ce] + beta[ce];
+      }
+    }
+  }
+};
+
+// --------------------------------------------------------------------------
+// General backward: ds/db per group, dgamma/dbeta per channel, then dx
+// --------------------------------------------------------------------------
+template <typename T>
+struct InternalGradAccum {  // segments over one (n, g)
+  using A = typename IO<T>::Acc;
+  GroupShape sh;
+  const A* gamma;
+  uint32_t g;
+  __device__ __forceinline__ void begin(uint32_t o, uint32_t) { g = o % sh.G; }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t p, uint32_t, const A (&x)[V],
+                                      const A (&dy)[V], A& a, A& b) const {
+    if (sh.nchw) {
+      const A w = gamma[g * sh.D + p / sh.S];  // packet within one channel
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const A t = w * dy[e];
+        a += t * x[e];
+        b += t;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const A t = gamma[g * sh.D + p + e] * dy[e];
+        a += t * x[e];
+        b += t;
+      }
+    }
+  }
+};
+
+template <typename A>
+struct StorePairEpilogue {
+  A* out_a;
+  A* out_b;
+  __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
+    out_a[o] = a;
+    out_b[o] = b;
+  }
+};
+
+template <typename T>
+struct WGradAccumNCHW {  // segments: output c, segment n
+  using A = typename IO<T>::Acc;
+  GroupShape sh;
+  const A* mu;
+  const A* rsig;
+  uint32_t g;
+  __device__ __forceinline__ void begin(uint32_t c, uint32_t) { g = c / sh.D; }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t n, uint32_t, uint32_t, const A (&x)[V],
+                                      const A (&dy)[V], A& a, A& b) const {
+    const uint32_t ng = n * sh.G + g;
+    const A m = mu[ng], r = rsig[ng];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      a += dy[e] * (x[e] - m) * r;
+      b += dy[e];
+    }
+  }
+};
+
+template <typename T>
+struct WGradAccumNHWC {  // columns: rows = N*S, cols = C
+  using A = typename IO<T>::Acc;
+  GroupShape sh;
+  const A* mu;
+  const A* rsig;
+  uint32_t g;
+  __device__ __forceinline__ void begin(uint32_t c, uint32_t) { g = c / sh.D; }
+  __device__ __forceinline__ void add(uint32_t r, uint32_t, uint32_t, A x, A dy, A& a, A& b) const {
+    const uint32_t ng = (r / sh.S) * sh.G + g;
+    a += dy * (x - mu[ng]) * rsig[ng];
+    b += dy;
+  }
+};
+
+template <typename T, int kVec>
+struct GroupNormGradApply {
+  using A = typename IO<T>::Acc;
+  GroupShape sh;
+  const A* mu;
+  const A* rsig;
+  const A* gamma;
+  const A* ds;
+  const A* db;
+  A denom;
+  __device__ __forceinline__ A one(A x, A dy, uint32_t ng, uint32_t c) const {
+    const A m = mu[ng], r = rsig[ng], s = ds[ng], b = db[ng];
+    const A u = (b * m - s) * (x - m) * (r * r * r);
+    const A v = b * r;
+    return gamma[c] * dy * r + (u - v) * denom;
+  }
+  __device__ __forceinline__ void operator()(uint32_t i, A (&x)[kVec], const A (&dy)[kVec]) const {
+    if (sh.nchw) {
+      const uint32_t row = i / sh.S;
+      const uint32_t c = row % sh.C;
+      const uint32_t ng = row / sh.D;
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) x[e] = one(x[e], dy[e], ng, c);
+    } else {
+      const uint32_t c = i % sh.C;
+      const uint32_t n = i / (sh.S * sh.C);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const uint32_t ce = c + e;
+        x[e] = one(x[e], dy[e], n * sh.G + (sh.G == 1 ? 0u : ce / sh.D), ce);
+      }
+    }
+  }
+};
+
+// --------------------------------------------------------------------------
+// Fused row path (LayerNorm backward)
+// --------------------------------------------------------------------------
+constexpr int kGradThreads = 1024;
+
+// partial[blockIdx][c][{dgamma, dbeta}]
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(kGradThreads) void layer_norm_grad_rows(
+    const int64_t N, const int C, const T* __restrict__ x, const T* __restrict__ dy,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
+    const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
+    typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using Tile = RowTile<T, kTPR, kVPT, kGradThreads>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  constexpr int kGroups = Tile::kRowsPerBlock;
+  // A round of the final cross-group combine moves kChunk (dgamma, dbeta) pairs per thread.
+  constexpr int kChunk = kVec < 4 ? kVec : 4;
+  constexpr int kRedWords = kGroups > 1 ? (kGroups - 1) * kTPR * kChunk * 2 : 1;
+  __shared__ A slots[2 * Tile::kSlots];
+  __shared__ A red[kRedWords];
+  const int npackets = C / kVec;
+  const int lane = Tile::lane();
+  const int sub = Tile::sub_row();
+  const A inv_c = A(1) / A(C);
+
+  A g[kVPT][kVec], dg[kVPT][kVec], dbt[kVPT][kVec];
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) {
+    if (Tile::active(i, npackets)) {
+      load_params<kVec>(gamma + (i * kTPR + lane) * kVec, g[i]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) g[i][e] = A(0);
+    }
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) dg[i][e] = dbt[i][e] = A(0);
+  }
+
+  // Uniform trip count across the workgroup: the row reductions hold barriers.
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N;
+       base += static_cast<int64_t>(gridDim.x) * kGroups) {
+    const int64_t row = base + sub;
+    const bool valid = row < N;
+    Tile tx, tdy;
+    tx.load(x + row * C, npackets, A(0), valid);
+    tdy.load(dy + row * C, npackets, A(0), valid);
+    const A m = valid ? mu[row] : A(0);
+    const A r = valid ? rsig[row] : A(0);
+
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A t = g[i][e] * tdy.v[i][e];
+        s1 += t * tx.v[i][e];
+        s2 += t;
+      }
+    Tile::reduce_sum_pair(s1, s2, slots);
+    if (lane == 0 && valid) {
+      ds[row] = s1;
+      db[row] = s2;
+    }
+
+    const A u0 = (s2 * m - s1) * (r * r * r);
+    const A v0 = s2 * r;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A xc = tx.v[i][e] - m;
+        const A d = tdy.v[i][e];
+        dg[i][e] += d * xc * r;
+        dbt[i][e] += d;
+        tx.v[i][e] = g[i][e] * d * r + (u0 * xc - v0) * inv_c;
+      }
+    tx.store(dx + row * C, npackets, valid);
+    if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
+  }
+
+  // Combine the kGroups row groups of this workgroup, kChunk pairs at a time.
+  A* out = partial + static_cast<size_t>(blockIdx.x) * C * 2;
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) {
+#pragma unroll
+    for (int h = 0; h < kVec / kChunk; ++h) {
+      if (kGroups > 1) {
+        __syncthreads();
+        if (sub > 0) {
+          A* w = red + (static_cast<size_t>(sub - 1) * kTPR + lane) * kChunk * 2;
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) {
+            w[2 * e] = dg[i][h * kChunk + e];
+            w[2 * e + 1] = dbt[i][h * kChunk + e];
+          }
+        }
+        __syncthreads();
+      }
+      if (sub == 0 && Tile::active(i, npackets)) {
+        A pg[kChunk], pb[kChunk];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          pg[e] = dg[i][h * kChunk + e];
+          pb[e] = dbt[i][h * kChunk + e];
+        }
+        for (int q = 1; q < kGroups; ++q) {
+          const A* w = red + (static_cast<size_t>(q - 1) * kTPR + lane) * kChunk * 2;
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) {
+            pg[e] += w[2 * e];
+            pb[e] += w[2 * e + 1];
+          }
+        }
+        A* o = out + (static_cast<size_t>(i * kTPR + lane) * kVec + h * kChunk) * 2;
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {
+          o[2 * e] = pg[e];
+          o[2 * e + 1] = pb[e];
+        }
+      }
+    }
+  }
+}
+
+// Sums P partial rows of 2*C interleaved (dgamma, dbeta) words. A workgroup of
+// 16 wavefronts owns 64 adjacent words; wavefront w adds rows w, w+16, ...
+template <typename A>
+__global__ __launch_bounds__(1024) void sum_partial_rows(const uint32_t P, const uint32_t C,
+                                                         const A* __restrict__ partial,
+                                                         A* __restrict__ dgamma,
+                                                         A* __restrict__ dbeta) {
+  __shared__ A lds[16][kWaveSize];
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t word = blockIdx.x * kWaveSize + lane;
+  const uint32_t words = 2 * C;
+  A acc = A(0);
+  if (word < words) {
+#pragma unroll 8
+    for (uint32_t p = wave; p < P; p += 16) acc += partial[static_cast<size_t>(p) * words + word];
+  }
+  lds[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && word < words) {
+#pragma unroll
+    for (int w = 1; w < 16; ++w) acc += lds[w][lane];
+    if (word & 1) {
+      dbeta[word >> 1] = acc;
+    } else {
+      dgamma[word >> 1] = acc;
+    }
+  }
+}
+
+struct RowGradPlan {
+  bool use_rows;
+  RowConfig cfg;
+  unsigned grid;
+};
+
+// The fused row path holds x, dy, gamma and two gradient accumulators per
+// thread, and a 1024-thread workgroup leaves 128 registers per thread: tiles
+// are limited to 16 elements per thread (8 for fp64), fewest packets first.
+template <typename T>
+RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
+  RowGradPlan p = {false, {0, 0}, 0};
+  if (G != 1 || S != 1) return p;
+  constexpr int kVec = IO<T>::kVec;
+  constexpr int kMaxElems = sizeof(typename IO<T>::Acc) == 8 ? 8 : 16;
+  if (D % kVec != 0) return p;
+  static const RowConfig table[] = {{64, 1}, {64, 2}, {256, 1}, {256, 2}, {1024, 1}, {1024, 2}, {1024, 4}};
+  bool found = false;
+  for (const RowConfig& c : table) {
+    if (c.vpt * kVec <= kMaxElems && D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
+      p.cfg = c;
+      found = true;
+      break;
+    }
+  }
+  if (!found) return p;
+  const int64_t groups = kGradThreads / p.cfg.tpr;
+  const int64_t want = ceil_div(N, groups);
+  const int64_t cap = kNumCUs * 2;
+  p.grid = static_cast<unsigned>(want < cap ? want : cap);
+  p.use_rows = true;
+  return p;
+}
+
+template <typename T>
+size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
+  using A = typename IO<T>::Acc;
+  const RowGradPlan rp = plan_row_grad<T>(N, G, D, S);
+  if (rp.use_rows) return static_cast<size_t>(rp.grid) * D * 2 * sizeof(A);
+  const int64_t C = G * D;
+  const uint32_t split_g = pick_split(N * G, D * S);
+  size_t bytes = static_cast<size_t>(N) * G * split_g * 2 * sizeof(A);
+  const uint32_t split_c = layout == DRAGON_HIP_NCHW
+      ? pick_split(C, N * S)
+      : pick_split(ceil_div(C, kWaveSize), N * S * kWaveSize);
+  const size_t wbytes = static_cast<size_t>(C) * split_c * 2 * sizeof(A);
+  return bytes > wbytes ? bytes : wbytes;
+}
+
+template <typename T>
+int launch_group_norm(const GroupShape& sh, const void* x, const void* mu, const void* rsig,
+                      const void* gamma, const void* beta, void* y, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const uint32_t total = sh.N * sh.C * sh.S;
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  const bool vec_ok = aligned16(x) && aligned16(y) && (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
+  if (vec_ok) {
+    GroupNormApply<T, kVec> f{sh, static_cast<const A*>(mu), static_cast<const A*>(rsig),
+                              static_cast<const A*>(gamma), static_cast<const A*>(beta)};
+    hipLaunchKernelGGL((map_flat<T, 1, kVec, GroupNormApply<T, kVec>>), dim3(map_grid(total / kVec)),
+                       dim3(256), 0, stream, total, xp, xp, yp, f);
+  } else {
+    GroupNormApply<T, 1> f{sh, static_cast<const A*>(mu), static_cast<const A*>(rsig),
+                           static_cast<const A*>(gamma), static_cast<const A*>(beta)};
+    hipLaunchKernelGGL((map_flat<T, 1, 1, GroupNormApply<T, 1>>), dim3(map_grid(total)), dim3(256), 0,
+                       stream, total, xp, xp, yp, f);
+  }
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, const void* rsig,
+                           const void* gamma, const void* dy, void* ds, void* db, void* dgamma,
+                           void* dbeta, void* dx, void* scratch, size_t scratch_bytes,
+                           hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const T* xp = static_cast<const T*>(x);
+  const T* dyp = static_cast<const T*>(dy);
+  T* dxp = static_cast<T*>(dx);
+  const A* mup = static_cast<const A*>(mu);
+  const A* rsp = static_cast<const A*>(rsig);
+  const A* gp = static_cast<const A*>(gamma);
+  A* dsp = static_cast<A*>(ds);
+  A* dbp = static_cast<A*>(db);
+  A* dgp = static_cast<A*>(dgamma);
+  A* dbtp = static_cast<A*>(dbeta);
+  A* part = static_cast<A*>(scratch);
+  const int layout = sh.nchw ? DRAGON_HIP_NCHW : DRAGON_HIP_NHWC;
+  if (scratch_bytes < group_norm_grad_scratch<T>(sh.N, sh.G, sh.D, sh.S, layout) || !scratch) {
+    return DRAGON_HIP_ESCRATCH;
+  }
+
+  const RowGradPlan rp = plan_row_grad<T>(sh.N, sh.G, sh.D, sh.S);
+  if (rp.use_rows && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma)) {
+#define LAUNCH(TPR, VPT)                                                                         \
+  hipLaunchKernelGGL((layer_norm_grad_rows<T, TPR, VPT>), dim3(rp.grid), dim3(kGradThreads), 0, \
+                     stream, static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp,   \
+                     mup, rsp, dsp, dbp, dxp, part);
+    if (rp.cfg.tpr == 64 && rp.cfg.vpt == 1) LAUNCH(64, 1)
+    else if (rp.cfg.tpr == 64 && rp.cfg.vpt == 2) LAUNCH(64, 2)
+    else if (rp.cfg.tpr == 256 && rp.cfg.vpt == 1) LAUNCH(256, 1)
+    else if (rp.cfg.tpr == 256 && rp.cfg.vpt == 2) LAUNCH(256, 2)
+    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 1) LAUNCH(1024, 1)
+    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 2) LAUNCH(1024, 2)
+    else if constexpr (IO<T>::kVec <= 4) LAUNCH(1024, 4)
+#undef LAUNCH
+    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
+                       dim3(1024), 0, stream, rp.grid, sh.D, part, dgp, dbtp);
+    return status_of_launch();
+  }
+
+  const uint32_t total = sh.N * sh.C * sh.S;
+  const bool base_ok = aligned16(x) && aligned16(dy) && aligned16(dx);
+  // 1. ds, db per (n, g)
+  {
+    SegmentedReduce s;
+    s.n_out = sh.N * sh.G;
+    if (sh.nchw) {
+      s = SegmentedReduce{sh.N * sh.G, 1, sh.D * sh.S, 0, 1, sh.D * sh.S, 0, 1};
+    } else {
+      s = SegmentedReduce{sh.N * sh.G, sh.G, sh.S * sh.C, sh.D, sh.S, sh.D, sh.C, 1};
+    }
+    s.split = pick_split(s.n_out, static_cast<int64_t>(sh.D) * sh.S);
+    InternalGradAccum<T> f{sh, gp, 0};
+    const bool vec_ok = base_ok && (sh.nchw ? sh.S % kVec == 0 : sh.D % kVec == 0);
+    const dim3 grid(s.n_out * s.split);
+    if (vec_ok) {
+      hipLaunchKernelGGL((reduce2_segments<T, 2, kVec, InternalGradAccum<T>>), grid,
+                         dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
+    } else {
+      hipLaunchKernelGGL((reduce2_segments<T, 2, 1, InternalGradAccum<T>>), grid,
+                         dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
+    }
+    StorePairEpilogue<A> e{dsp, dbp};
+    hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
+                       dim3(static_cast<unsigned>(ceil_div(s.n_out, kReduceThreads))),
+                       dim3(kReduceThreads), 0, stream, s.n_out, s.split, true, part, e);
+  }
+  // 2. dgamma, dbeta per channel (scratch is reused: stream order keeps step 1 finished)
+  {
+    StorePairEpilogue<A> e{dgp, dbtp};
+    if (sh.nchw) {
+      SegmentedReduce s{sh.C, sh.C, 0, sh.S, sh.N, sh.S, sh.C * sh.S, 1};
+      s.split = pick_split(sh.C, static_cast<int64_t>(sh.N) * sh.S);
+      WGradAccumNCHW<T> f{sh, mup, rsp, 0};
+      const dim3 grid(s.n_out * s.split);
+      if (base_ok && sh.S % kVec == 0) {
+        hipLaunchKernelGGL((reduce2_segments<T, 2, kVec, WGradAccumNCHW<T>>), grid,
+                           dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
+      } else {
+        hipLaunchKernelGGL((reduce2_segments<T, 2, 1, WGradAccumNCHW<T>>), grid,
+                           dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
+      }
+      hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
+                         dim3(static_cast<unsigned>(ceil_div(sh.C, kReduceThreads))),
+                         dim3(kReduceThreads), 0, stream, sh.C, s.split, true, part, e);
+    } else {
+      ColumnReduce c{sh.N * sh.S, sh.C, 1};
+      c.split = pick_split(ceil_div(sh.C, kWaveSize), static_cast<int64_t>(sh.N) * sh.S * kWaveSize);
+      WGradAccumNHWC<T> f{sh, mup, rsp, 0};
+      const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
+      hipLaunchKernelGGL((reduce2_columns<T, 2, WGradAccumNHWC<T>>), grid, dim3(kReduceThreads), 0,
+                         stream, c, xp, dyp, f, part);
+      hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
+                         dim3(static_cast<unsigned>(ceil_div(sh.C, kReduceThreads))),
+                         dim3(kReduceThreads), 0, stream, sh.C, c.split, false, part, e);
+    }
+  }
+  // 3. dx
+  {
+    const A denom = A(1) / A(static_cast<int64_t>(sh.D) * sh.S);
+    const bool vec_ok = base_ok && (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
+    if (vec_ok) {
+      GroupNormGradApply<T, kVec> f{sh, mup, rsp, gp, dsp, dbp, denom};
+      hipLaunchKernelGGL((map_flat<T, 2, kVec, GroupNormGradApply<T, kVec>>),
+                         dim3(map_grid(total / kVec)), dim3(256), 0, stream, total, xp, dyp, dxp, f);
+    } else {
+      GroupNormGradApply<T, 1> f{sh, mup, rsp, gp, dsp, dbp, denom};
+      hipLaunchKernelGGL((map_flat<T, 2, 1, GroupNormGradApply<T, 1>>), dim3(map_grid(total)),
+                         dim3(256), 0, stream, total, xp, dyp, dxp, f);
+    }
+  }
+  return status_of_launch();
+}
+
+int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShape* sh) {
+  if (N < 0 || G <= 0 || D <= 0 || S < 0) return DRAGON_HIP_EINVAL;
+  if (layout != DRAGON_HIP_NCHW && layout != DRAGON_HIP_NHWC) return DRAGON_HIP_EINVAL;
+  if (!fits_int32(N * G * D * S)) return DRAGON_HIP_EINVAL;
+  sh->N = static_cast<uint32_t>(N), sh->G = static_cast<uint32_t>(G);
+  sh->D = static_cast<uint32_t>(D), sh->S = static_cast<uint32_t>(S);
+  sh->C = static_cast<uint32_t>(G * D);
+  sh->nchw = layout == DRAGON_HIP_NCHW;
+  return DRAGON_HIP_OK;
+}
+
+template <typename T>
+size_t grad_scratch_t(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
+  return group_norm_grad_scratch<T>(N, G, D, S, layout);
+}
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" {
+
+int dragon_hip_group_norm(int dtype, int64_t N, int64_t G, int64_t D, int64_t S, int layout,
+                          const void* x, const void* mu, const void* rsig, const void* gamma,
+                          const void* beta, void* y, void* stream) {
+  dragon_hip::GroupShape sh;
+  const int st = dragon_hip::make_shape(N, G, D, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!x || !mu || !rsig || !gamma || !beta || !y) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_group_norm, sh, x, mu, rsig, gamma, beta, y, s);
+}
+
+size_t dragon_hip_group_norm_grad_scratch_bytes(int dtype, int64_t N, int64_t G, int64_t D,
+                                                int64_t S, int layout) {
+  dragon_hip::GroupShape sh;
+  if (dragon_hip::make_shape(N, G, D, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  switch (dtype) {
+    case DRAGON_HIP_F16: return dragon_hip::grad_scratch_t<dragon_hip::f16_t>(N, G, D, S, layout);
+    case DRAGON_HIP_BF16: return dragon_hip::grad_scratch_t<dragon_hip::bf16_t>(N, G, D, S, layout);
+    case DRAGON_HIP_F32: return dragon_hip::grad_scratch_t<float>(N, G, D, S, layout);
+    case DRAGON_HIP_F64: return dragon_hip::grad_scratch_t<double>(N, G, D, S, layout);
+    default: return 0;
+  }
+}
+
+int dragon_hip_group_norm_grad(int dtype, int64_t N, int64_t G, int64_t D, int64_t S, int layout,
+                               const void* x, const void* mu, const void* rsig,
+                               const void* gamma, const void* dy, void* ds, void* db,
+                               void* dgamma, void* dbeta, void* dx, void* scratch,
+                               size_t scratch_bytes, void* stream) {
+  dragon_hip::GroupShape sh;
+  const int st = dragon_hip::make_shape(N, G, D, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (!dgamma || !dbeta) return DRAGON_HIP_EINVAL;
+  const size_t acc = dtype == DRAGON_HIP_F64 ? 8 : 4;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (N * S == 0) {
+    // Nothing to reduce: the reference still zero-fills the parameter gradients.
+    const int acc_tag = dtype == DRAGON_HIP_F64 ? DRAGON_HIP_F64 : DRAGON_HIP_F32;
+    const int e1 = dragon_hip_set(acc_tag, G * D, 0.f, dgamma, s);
+    return e1 != DRAGON_HIP_OK ? e1 : dragon_hip_set(acc_tag, G * D, 0.f, dbeta, s);
+  }
+  if (!x || !mu || !rsig || !gamma || !dy || !ds || !db || !dx) return DRAGON_HIP_EINVAL;
+  // ds == db selects the packed 2*N*G scratch convention of the operator.
+  void* db_eff = ds == db ? static_cast<char*>(ds) + acc * N * G : db;
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_group_norm_grad, sh, x, mu, rsig, gamma, dy,
+                            ds, db_eff, dgamma, dbeta, dx, scratch, scratch_bytes, s);
+}
+
+
+namespace {
+// Moments view of the group statistics: NCHW [N*G, D*S] over axis 1, NHWC
+// [N, S, G, D] over axes {1, 3} (dragon/operators/normalization/group_norm_op.cc:26-34).
+struct GroupMomentsView {
+  int num_dims, num_axes;
+  int64_t dims[4], axes[2];
+};
+GroupMomentsView group_moments_view(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
+  GroupMomentsView v;
+  if (layout == DRAGON_HIP_NCHW) {
+    v.num_dims = 2, v.num_axes = 1;
+    v.dims[0] = N * G, v.dims[1] = D * S, v.axes[0] = 1;
+  } else {
+    v.num_dims = 4, v.num_axes = 2;
+    v.dims[0] = N, v.dims[1] = S, v.dims[2] = G, v.dims[3] = D;
+    v.axes[0] = 1, v.axes[1] = 3;
+  }
+  return v;
+}
+} // namespace
+
+size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t G, int64_t D,
+                                                   int64_t S, int layout) {
+  dragon_hip::GroupShape sh;
+  if (dragon_hip::make_shape(N, G, D, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
+  return dragon_hip_moments_scratch_bytes(dtype, v.num_dims, v.dims, v.num_axes, v.axes);
+}
+
+int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
+                                  int layout, float eps, const void* x, const void* gamma,
+                                  const void* beta, void* mu, void* rsig, void* y,
+                                  void* scratch, size_t scratch_bytes, void* stream) {
+  dragon_hip::GroupShape sh;
+  int st = dragon_hip::make_shape(N, G, D, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!x || !gamma || !beta || !mu || !rsig || !y) return DRAGON_HIP_EINVAL;
+  const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
+  st = dragon_hip_moments(dtype, v.num_dims, v.dims, v.num_axes, v.axes, x, mu, rsig, scratch,
+                          scratch_bytes, stream);
+  if (st != DRAGON_HIP_OK) return st;
+  const int acc_tag = dtype == DRAGON_HIP_F64 ? DRAGON_HIP_F64 : DRAGON_HIP_F32;
+  st = dragon_hip_inv_std(acc_tag, N * G, eps, rsig, rsig, stream);
+  if (st != DRAGON_HIP_OK) return st;
+  return dragon_hip_group_norm(dtype, N, G, D, S, layout, x, mu, rsig, gamma, beta, y, stream);
+}
+
+} // extern "C"

@@ -1,0 +1,286 @@
+// kernels::Moments for gfx950: mean and biased variance over arbitrary axes.
+//
+// Replaces kernels::Moments<T, AccT, Context>
+// (dragon/kernels/math/op_kernels.h:106-115; CPU
+// dragon/kernels/math/cpu/moments_kernel.cc:10-189 with the axis utilities of
+// dragon/utils/math/reduce.h:96-198). As there, size-1 axes are dropped and
+// adjacent axes of the same kind are merged first; the collapsed pattern picks
+// the kernel:
+//   [K,R] [R] [R,K,R] [K,R,K,R]   segmented split reduction (contiguous runs)
+//   [R,K]                         column split reduction
+//   anything else                 one workgroup per output, strided gather
+// (K = kept extent, R = reduced extent).
+//
+// Variance uses sums shifted by one sample of the reduction set,
+//   mean = s + sum(x-s)/n,  var = sum((x-s)^2)/n - (sum(x-s)/n)^2,
+// which equals the reference's E[x^2]-E[x]^2 in exact arithmetic and keeps
+// Welford-class accuracy in fp32 when |mean| >> stddev, while partial sums
+// still combine by plain addition.
+#include <string>
+#include <vector>
+
+#include "reduce.h"
+
+namespace dragon_hip {
+namespace {
+
+template <typename T>
+struct MomentsAccum {
+  using A = typename IO<T>::Acc;
+  const T* x;
+  A shift;
+  __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
+    shift = IO<T>::load1(x + first_off);
+  }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x0)[V],
+                                      const A (&)[V], A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const A d = x0[e] - shift;
+      a += d;
+      b += d * d;
+    }
+  }
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, A x0, A, A& a, A& b) const {
+    const A d = x0 - shift;
+    a += d;
+    b += d * d;
+  }
+};
+
+template <typename T>
+struct MomentsSegEpilogue {
+  using A = typename IO<T>::Acc;
+  const T* x;
+  SegmentedReduce d;
+  A inv_n;
+  A* mean;
+  A* var;
+  __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
+    const uint32_t o1 = o / d.outer2;
+    const uint32_t o2 = o - o1 * d.outer2;
+    const A shift = IO<T>::load1(x + o1 * d.stride1 + o2 * d.stride2);
+    const A m = a * inv_n;
+    mean[o] = shift + m;
+    var[o] = b * inv_n - m * m;
+  }
+};
+
+template <typename T>
+struct MomentsColEpilogue {
+  using A = typename IO<T>::Acc;
+  const T* x;
+  A inv_n;
+  A* mean;
+  A* var;
+  __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
+    const A shift = IO<T>::load1(x + c);
+    const A m = a * inv_n;
+    mean[c] = shift + m;
+    var[c] = b * inv_n - m * m;
+  }
+};
+
+constexpr int kMaxDims = 8;
+struct GatherDims {
+  int n_keep, n_red;
+  uint32_t keep_dim[kMaxDims], keep_stride[kMaxDims];
+  uint32_t red_dim[kMaxDims], red_stride[kMaxDims];
+  uint32_t n_out, n_red_elems;
+};
+
+// One workgroup per output; the reduced index is unravelled over the reduced
+// extents (last fastest, the order the reference walks them in).
+template <typename T>
+__global__ __launch_bounds__(kReduceThreads) void moments_gather(
+    const GatherDims g, const T* __restrict__ x, typename IO<T>::Acc* __restrict__ mean,
+    typename IO<T>::Acc* __restrict__ var) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds[2 * kReduceWaves];
+  for (uint32_t o = blockIdx.x; o < g.n_out; o += gridDim.x) {
+    uint32_t base = 0, r = o;
+    for (int d = g.n_keep - 1; d >= 0; --d) {
+      base += (r % g.keep_dim[d]) * g.keep_stride[d];
+      r /= g.keep_dim[d];
+    }
+    const A shift = IO<T>::load1(x + base);
+    A a = A(0), b = A(0);
+    for (uint32_t j = threadIdx.x; j < g.n_red_elems; j += kReduceThreads) {
+      uint32_t off = base, q = j;
+      for (int d = g.n_red - 1; d >= 0; --d) {
+        off += (q % g.red_dim[d]) * g.red_stride[d];
+        q /= g.red_dim[d];
+      }
+      const A v = IO<T>::load1(x + off) - shift;
+      a += v;
+      b += v * v;
+    }
+    block_reduce_pair(a, b, lds);
+    if (threadIdx.x == 0) {
+      const A inv_n = A(1) / A(g.n_red_elems);
+      const A m = a * inv_n;
+      mean[o] = shift + m;
+      var[o] = b * inv_n - m * m;
+    }
+    __syncthreads();
+  }
+}
+
+enum PlanKind { kPlanSegments, kPlanColumns, kPlanGather };
+struct MomentsPlan {
+  PlanKind kind;
+  SegmentedReduce seg;
+  ColumnReduce col;
+  GatherDims gather;
+  int64_t n_out, n_red;
+  size_t scratch_bytes;
+};
+
+// Restates what CollapseReduceAxes does to the shape (drop extents of one,
+// merge neighbours of the same kind) and classifies the result.
+int make_plan(int dtype, int num_dims, const int64_t* dims, int num_axes, const int64_t* axes,
+              MomentsPlan* plan) {
+  if (num_dims < 0 || num_axes < 0 || (num_dims > 0 && !dims) || (num_axes > 0 && !axes)) {
+    return DRAGON_HIP_EINVAL;
+  }
+  std::vector<char> is_red(num_dims, 0);
+  for (int i = 0; i < num_axes; ++i) {
+    if (axes[i] < 0 || axes[i] >= num_dims) return DRAGON_HIP_EINVAL;
+    is_red[axes[i]] = 1;
+  }
+  std::vector<int64_t> ext;
+  std::vector<char> red;
+  int64_t total = 1;
+  for (int i = 0; i < num_dims; ++i) {
+    if (dims[i] < 0) return DRAGON_HIP_EINVAL;
+    total *= dims[i];
+    if (dims[i] == 1) continue;
+    if (!ext.empty() && red.back() == is_red[i]) {
+      ext.back() *= dims[i];
+    } else {
+      ext.push_back(dims[i]);
+      red.push_back(is_red[i]);
+    }
+  }
+  if (!fits_int32(total)) return DRAGON_HIP_EINVAL;
+  const size_t acc_bytes = dtype == DRAGON_HIP_F64 ? 8 : 4;
+  std::vector<int64_t> stride(ext.size(), 1);
+  for (int i = static_cast<int>(ext.size()) - 2; i >= 0; --i) stride[i] = stride[i + 1] * ext[i + 1];
+  plan->n_out = plan->n_red = 1;
+  for (size_t i = 0; i < ext.size(); ++i) (red[i] ? plan->n_red : plan->n_out) *= ext[i];
+  plan->scratch_bytes = 0;
+  std::string pat;
+  for (char r : red) pat.push_back(r ? 'R' : 'K');
+  SegmentedReduce& s = plan->seg;
+  s = SegmentedReduce{static_cast<uint32_t>(plan->n_out), 1, 0, 0, 1, 0, 0, 1};
+  auto u32 = [](int64_t v) { return static_cast<uint32_t>(v); };
+  if (pat == "R" || pat == "KR") {
+    plan->kind = kPlanSegments;
+    s.stride1 = u32(plan->n_red), s.seglen = u32(plan->n_red);
+  } else if (pat == "RKR") {
+    plan->kind = kPlanSegments;
+    s.outer2 = u32(ext[1]), s.stride2 = u32(ext[2]);
+    s.nseg = u32(ext[0]), s.seg_stride = u32(stride[0]), s.seglen = u32(ext[2]);
+  } else if (pat == "KRKR") {
+    plan->kind = kPlanSegments;
+    s.outer2 = u32(ext[2]), s.stride1 = u32(stride[0]), s.stride2 = u32(ext[3]);
+    s.nseg = u32(ext[1]), s.seg_stride = u32(stride[1]), s.seglen = u32(ext[3]);
+  } else if (pat == "RK") {
+    plan->kind = kPlanColumns;
+    plan->col = ColumnReduce{u32(ext[0]), u32(ext[1]), 1};
+    plan->col.split = pick_split(ceil_div(ext[1], kWaveSize), ext[0] * kWaveSize);
+    plan->scratch_bytes = static_cast<size_t>(plan->col.split) * ext[1] * 2 * acc_bytes;
+  } else {
+    if (ext.size() > kMaxDims) return DRAGON_HIP_EINVAL;
+    plan->kind = kPlanGather;
+    GatherDims& g = plan->gather;
+    g.n_keep = g.n_red = 0;
+    for (size_t i = 0; i < ext.size(); ++i) {
+      if (red[i]) {
+        g.red_dim[g.n_red] = u32(ext[i]), g.red_stride[g.n_red++] = u32(stride[i]);
+      } else {
+        g.keep_dim[g.n_keep] = u32(ext[i]), g.keep_stride[g.n_keep++] = u32(stride[i]);
+      }
+    }
+    g.n_out = u32(plan->n_out), g.n_red_elems = u32(plan->n_red);
+  }
+  if (plan->kind == kPlanSegments) {
+    s.split = pick_split(plan->n_out, plan->n_red);
+    plan->scratch_bytes = static_cast<size_t>(plan->n_out) * s.split * 2 * acc_bytes;
+  }
+  return DRAGON_HIP_OK;
+}
+
+template <typename T>
+int launch_moments(const MomentsPlan& plan, const void* x, void* mean, void* var, void* scratch,
+                   hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const T* xp = static_cast<const T*>(x);
+  A* mp = static_cast<A*>(mean);
+  A* vp = static_cast<A*>(var);
+  A* part = static_cast<A*>(scratch);
+  const A inv_n = A(1) / A(plan.n_red);
+  const unsigned fin_grid = static_cast<unsigned>(ceil_div(plan.n_out, kReduceThreads));
+  if (plan.kind == kPlanSegments) {
+    const SegmentedReduce& s = plan.seg;
+    const bool vec_ok = aligned16(x) && s.seglen % kVec == 0 && s.stride1 % kVec == 0 &&
+        s.stride2 % kVec == 0 && s.seg_stride % kVec == 0;
+    MomentsAccum<T> f{xp, A(0)};
+    const dim3 grid(s.n_out * s.split);
+    if (vec_ok) {
+      hipLaunchKernelGGL((reduce2_segments<T, 1, kVec, MomentsAccum<T>>), grid,
+                         dim3(kReduceThreads), 0, stream, s, xp, xp, f, part);
+    } else {
+      hipLaunchKernelGGL((reduce2_segments<T, 1, 1, MomentsAccum<T>>), grid, dim3(kReduceThreads),
+                         0, stream, s, xp, xp, f, part);
+    }
+    MomentsSegEpilogue<T> e{xp, s, inv_n, mp, vp};
+    hipLaunchKernelGGL((reduce2_finalize<A, MomentsSegEpilogue<T>>), dim3(fin_grid),
+                       dim3(kReduceThreads), 0, stream, s.n_out, s.split, true, part, e);
+  } else if (plan.kind == kPlanColumns) {
+    const ColumnReduce& c = plan.col;
+    MomentsAccum<T> f{xp, A(0)};
+    const dim3 grid(static_cast<unsigned>(ceil_div(c.cols, kWaveSize)) * c.split);
+    hipLaunchKernelGGL((reduce2_columns<T, 1, MomentsAccum<T>>), grid, dim3(kReduceThreads), 0,
+                       stream, c, xp, xp, f, part);
+    MomentsColEpilogue<T> e{xp, inv_n, mp, vp};
+    hipLaunchKernelGGL((reduce2_finalize<A, MomentsColEpilogue<T>>), dim3(fin_grid),
+                       dim3(kReduceThreads), 0, stream, c.cols, c.split, false, part, e);
+  } else {
+    const unsigned grid = static_cast<unsigned>(plan.n_out < 65536 ? plan.n_out : 65536);
+    hipLaunchKernelGGL((moments_gather<T>), dim3(grid), dim3(kReduceThreads), 0, stream,
+                       plan.gather, xp, mp, vp);
+  }
+  return status_of_launch();
+}
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" {
+
+size_t dragon_hip_moments_scratch_bytes(int dtype, int num_dims, const int64_t* dims,
+                                        int num_axes, const int64_t* axes) {
+  dragon_hip::MomentsPlan plan;
+  if (dragon_hip::make_plan(dtype, num_dims, dims, num_axes, axes, &plan) != DRAGON_HIP_OK) return 0;
+  return plan.scratch_bytes;
+}
+
+int dragon_hip_moments(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                       const int64_t* axes, const void* x, void* mean, void* var, void* scratch,
+                       size_t scratch_bytes, void* stream) {
+  dragon_hip::MomentsPlan plan;
+  const int st = dragon_hip::make_plan(dtype, num_dims, dims, num_axes, axes, &plan);
+  if (st != DRAGON_HIP_OK) return st;
+  if (plan.n_out * plan.n_red == 0) return DRAGON_HIP_OK;
+  if (!x || !mean || !var) return DRAGON_HIP_EINVAL;
+  if (plan.scratch_bytes > 0 && (!scratch || scratch_bytes < plan.scratch_bytes)) {
+    return DRAGON_HIP_ESCRATCH;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_moments, plan, x, mean, var, scratch, s);
+}
+
+} // extern "C"

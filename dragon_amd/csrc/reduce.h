@@ -1,0 +1,219 @@
+// Atomic-free two-stage reductions and flat element-wise maps shared by the
+// Moments, GroupNorm and BatchNorm kernels.
+//
+// Every reduction on this path is a pair of sums per output (sum x / sum x^2,
+// sum dy*(x-mu) / sum dy, sum gamma*dy*x / sum gamma*dy ...). Stage one spreads
+// each output over `split` workgroups so that a few hundred outputs still fill
+// 256 compute units; each workgroup tree-reduces its share in fp32 (fp64 for
+// double) and writes one pair to scratch. Stage two is a tiny kernel that adds
+// the `split` pairs of an output in a fixed order and applies the op's
+// epilogue. No atomics, so results are bit-reproducible run to run.
+//
+// Sizes: the reference's kernels:: interface carries `int` extents
+// (dragon/kernels/normalization/op_kernels.h:36-143), so every tensor on this
+// path has fewer than 2^31 elements and 32-bit index arithmetic is exact.
+#pragma once
+
+#include "common.h"
+
+namespace dragon_hip {
+
+constexpr int kReduceThreads = 256;
+constexpr int kReduceWaves = kReduceThreads / kWaveSize;
+
+// Reduction set of output o = (o1, o2), o = o1 * outer2 + o2: `nseg` segments
+// of `seglen` contiguous elements; element (seg, p) lives at
+//   o1 * stride1 + o2 * stride2 + seg * seg_stride + p.
+//   trailing-axis reduce [rows, cols]   outer2=1, stride1=cols, nseg=1, seglen=cols
+//   BatchNorm NCHW [N, C, S] per c      outer2=C, stride2=S, nseg=N, seg_stride=C*S, seglen=S
+//   GroupNorm NCHW per (n, g)           outer2=1, stride1=D*S, nseg=1, seglen=D*S
+//   GroupNorm NHWC per (n, g)           outer2=G, stride1=S*C, stride2=D, nseg=S, seg_stride=C, seglen=D
+struct SegmentedReduce {
+  uint32_t n_out, outer2;
+  uint32_t stride1, stride2;
+  uint32_t nseg, seglen, seg_stride;
+  uint32_t split;
+};
+
+// Leading-axis reduce of a [rows, cols] view, one output per column
+// (BatchNorm NHWC, parameter gradients of row-normalised tensors).
+struct ColumnReduce {
+  uint32_t rows, cols;
+  uint32_t split;
+};
+
+// How many workgroups share one output: enough to put ~8 workgroups on every
+// compute unit, but never less than ~16K elements per workgroup.
+inline uint32_t pick_split(int64_t n_out, int64_t elems_per_out) {
+  const int64_t want_blocks = static_cast<int64_t>(kNumCUs) * 8;
+  int64_t split = ceil_div(want_blocks, n_out > 0 ? n_out : 1);
+  const int64_t max_by_work = ceil_div(elems_per_out, 16384);
+  if (split > max_by_work) split = max_by_work;
+  if (split < 1) split = 1;
+  if (split > 1024) split = 1024;
+  return static_cast<uint32_t>(split);
+}
+
+template <typename A>
+__device__ __forceinline__ void block_reduce_pair(A& a, A& b, A* lds /*2*kReduceWaves*/) {
+  a = wave_allreduce(a, SumOp());
+  b = wave_allreduce(b, SumOp());
+  const int wave = threadIdx.x / kWaveSize;
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+    lds[2 * wave] = a;
+    lds[2 * wave + 1] = b;
+  }
+  __syncthreads();
+  a = lds[0], b = lds[1];
+#pragma unroll
+  for (int i = 1; i < kReduceWaves; ++i) {
+    a += lds[2 * i];
+    b += lds[2 * i + 1];
+  }
+}
+
+// Stage one over segments. F provides
+//   void begin(uint32_t o, uint32_t first_off)    per-output setup; first_off is
+//                                                 the offset of the output's first element
+//   void add(uint32_t o, uint32_t seg, uint32_t p, uint32_t off,
+//            const A (&x0)[V], const A (&x1)[V], A& a, A& b)
+// where `off` is the element offset of the packet; kVec == 1 is the scalar
+// variant for unaligned tensors. partial[(o * split + k) * 2 + {0,1}].
+template <typename T, int kIn, int kVec, typename F>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_segments(
+    const SegmentedReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds[2 * kReduceWaves];
+  const uint32_t o = blockIdx.x / d.split;
+  const uint32_t k = blockIdx.x - o * d.split;
+  const uint32_t o1 = o / d.outer2;
+  const uint32_t o2 = o - o1 * d.outer2;
+  const uint32_t base = o1 * d.stride1 + o2 * d.stride2;
+  const uint32_t packets_per_seg = d.seglen / kVec;  // kVec > 1 only when it divides seglen
+  const uint32_t npackets = d.nseg * packets_per_seg;
+  f.begin(o, base);
+  A a = A(0), b = A(0);
+#pragma unroll 4
+  for (uint32_t jp = k * kReduceThreads + threadIdx.x; jp < npackets;
+       jp += d.split * kReduceThreads) {
+    const uint32_t seg = jp / packets_per_seg;
+    const uint32_t p = (jp - seg * packets_per_seg) * kVec;
+    const uint32_t off = base + seg * d.seg_stride + p;
+    A x0[kVec], x1[kVec];
+    if constexpr (kVec == 1) {
+      x0[0] = IO<T>::load1(in0 + off);
+      x1[0] = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
+    } else {
+      IO<T>::load(in0 + off, x0);
+      if constexpr (kIn == 2) IO<T>::load(in1 + off, x1);
+    }
+    f.add(o, seg, p, off, x0, x1, a, b);
+  }
+  block_reduce_pair(a, b, lds);
+  if (threadIdx.x == 0) {
+    partial[(static_cast<size_t>(o) * d.split + k) * 2] = a;
+    partial[(static_cast<size_t>(o) * d.split + k) * 2 + 1] = b;
+  }
+}
+
+// Stage one over columns: a workgroup owns a tile of 64 adjacent columns
+// (one per lane, so a wavefront reads 64 adjacent elements) and its four
+// wavefronts stride over the rows of slice k. F provides
+//   void begin(uint32_t c, uint32_t first_off)
+//   void add(uint32_t r, uint32_t c, uint32_t off, A x0, A x1, A& a, A& b).
+// partial[(k * cols + c) * 2 + {0,1}].
+template <typename T, int kIn, typename F>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_columns(
+    const ColumnReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds[kReduceWaves][kWaveSize][2];
+  const uint32_t tiles = (d.cols + kWaveSize - 1) / kWaveSize;
+  const uint32_t tile = blockIdx.x % tiles;
+  const uint32_t k = blockIdx.x / tiles;
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t c = tile * kWaveSize + lane;
+  A a = A(0), b = A(0);
+  if (c < d.cols) {
+    f.begin(c, c);
+#pragma unroll 4
+    for (uint32_t r = k * kReduceWaves + wave; r < d.rows; r += d.split * kReduceWaves) {
+      const uint32_t off = r * d.cols + c;
+      const A x0 = IO<T>::load1(in0 + off);
+      const A x1 = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
+      f.add(r, c, off, x0, x1, a, b);
+    }
+  }
+  lds[wave][lane][0] = a;
+  lds[wave][lane][1] = b;
+  __syncthreads();
+  if (wave == 0 && c < d.cols) {
+#pragma unroll
+    for (int w = 1; w < kReduceWaves; ++w) {
+      a += lds[w][lane][0];
+      b += lds[w][lane][1];
+    }
+    partial[(static_cast<size_t>(k) * d.cols + c) * 2] = a;
+    partial[(static_cast<size_t>(k) * d.cols + c) * 2 + 1] = b;
+  }
+}
+
+// Stage two: one thread per output adds its `split` pairs in index order and
+// hands the totals to the epilogue E: void operator()(uint32_t o, A a, A b).
+// `segment_major` selects the scratch layout of reduce2_segments
+// ((o*split+k)*2) or of reduce2_columns ((k*n_out+o)*2).
+template <typename A, typename E>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_finalize(
+    const uint32_t n_out, const uint32_t split, const bool segment_major,
+    const A* __restrict__ partial, E e) {
+  const uint32_t o = blockIdx.x * kReduceThreads + threadIdx.x;
+  if (o >= n_out) return;
+  A a = A(0), b = A(0);
+  for (uint32_t k = 0; k < split; ++k) {
+    const size_t idx = segment_major ? (static_cast<size_t>(o) * split + k)
+                                     : (static_cast<size_t>(k) * n_out + o);
+    a += partial[idx * 2];
+    b += partial[idx * 2 + 1];
+  }
+  e(o, a, b);
+}
+
+// Flat element-wise map over `total` elements in packets of kVec. F provides
+//   void operator()(uint32_t i, A (&v0)[V], const A (&v1)[V])
+// which overwrites v0 (loaded from in0) with the result; v1 comes from in1
+// when kIn == 2.
+template <typename T, int kIn, int kVec, typename F>
+__global__ __launch_bounds__(256) void map_flat(const uint32_t total, const T* in0, const T* in1,
+                                                T* out, F f) {
+  using A = typename IO<T>::Acc;
+  const uint32_t npackets = total / kVec;  // kVec > 1 only when it divides total
+  for (uint32_t ip = blockIdx.x * 256 + threadIdx.x; ip < npackets; ip += gridDim.x * 256) {
+    const uint32_t i = ip * kVec;
+    A v0[kVec], v1[kVec];
+    if constexpr (kVec == 1) {
+      v0[0] = IO<T>::load1(in0 + i);
+      v1[0] = kIn == 2 ? IO<T>::load1(in1 + i) : A(0);
+    } else {
+      IO<T>::load(in0 + i, v0);
+      if constexpr (kIn == 2) IO<T>::load(in1 + i, v1);
+    }
+    f(i, v0, v1);
+    if constexpr (kVec == 1) {
+      IO<T>::store1(out + i, v0[0]);
+    } else {
+      IO<T>::store(out + i, v0);
+    }
+  }
+}
+
+inline unsigned map_grid(uint32_t npackets) {
+  const int64_t want = ceil_div(npackets, 256);
+  const int64_t cap = static_cast<int64_t>(kNumCUs) * 32;
+  return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
+}
+
+inline bool fits_int32(int64_t v) { return v >= 0 && v < (int64_t(1) << 31); }
+
+} // namespace dragon_hip

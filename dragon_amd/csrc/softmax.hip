@@ -1,0 +1,379 @@
+// Softmax / LogSoftmax forward and backward for gfx950.
+//
+// Replaces kernels::Softmax, LogSoftmax, SoftmaxGrad, LogSoftmaxGrad
+// (dragon/kernels/activation/op_kernels.h:211-247; CPU
+// dragon/kernels/activation/cpu/softmax_kernel.cc:10-108) over a tensor viewed
+// as [N, C, S] with the reduction along C:
+//   softmax       y  = exp(x - max) / sum exp(x - max)
+//   log_softmax   y  = (x - max) - log sum exp(x - max)
+//   softmax_grad      dx = (dy - sum(dy * y)) * y
+//   log_softmax_grad  dx = dy - exp(y) * sum(dy)
+//
+// S == 1 (reduction along the contiguous axis) keeps each row in registers:
+// every tensor is read once and written once. 16-bit I/O accumulates in fp32
+// and uses the hardware exp2 (relative error ~1e-7 near the row maximum,
+// below 3e-6 in the far tail, both far under one 16-bit ulp); fp32 / fp64 I/O
+// use the correctly-scaled library exp and a true division, which is what the
+// reference's CPU expression does.
+//
+// S > 1 assigns one thread to each (n, s) column so that neighbouring threads
+// read neighbouring addresses; the column is walked three times (max, sum,
+// write), the re-reads coming from L2.
+#include "row_tile.h"
+
+namespace dragon_hip {
+namespace {
+
+template <typename T>
+struct SoftmaxMath {
+  using A = typename IO<T>::Acc;
+  static constexpr bool kFast = sizeof(T) == 2;
+  static __device__ __forceinline__ A exp_of(A v) {
+    if constexpr (kFast) {
+      return __builtin_amdgcn_exp2f(v * 1.44269504088896340736f);
+    } else {
+      return acc_exp(v);
+    }
+  }
+  static __device__ __forceinline__ A normalise(A e, A sum, A inv_sum) {
+    if constexpr (kFast) {
+      return e * inv_sum;
+    } else {
+      return e / sum;
+    }
+  }
+};
+
+enum SoftmaxKind { kSoftmax = 0, kLogSoftmax = 1 };
+
+template <typename T, int kKind, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
+    const int64_t N, const int C, const T* x, T* y) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const int npackets = C / kVec;
+
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Tile t;
+    t.load(x + row * C, npackets, acc_neg_inf<A>());
+
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) m = MaxOp()(m, t.v[i][e]);
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+
+    A s = A(0);
+    if (kKind == kSoftmax) {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          t.v[i][e] = M::exp_of(t.v[i][e] - m);  // masked slots: exp(-inf) = 0
+          s += t.v[i][e];
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          t.v[i][e] = t.v[i][e] - m;
+          s += M::exp_of(t.v[i][e]);
+        }
+    }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+
+    if (kKind == kSoftmax) {
+      const A inv = A(1) / s;
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) t.v[i][e] = M::normalise(t.v[i][e], s, inv);
+    } else {
+      const A l = acc_log(s);
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) t.v[i][e] = t.v[i][e] - l;
+    }
+    t.store(y + row * C, npackets);
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+template <typename T, int kKind, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
+    const int64_t N, const int C, const T* dy, const T* y, T* dx) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[Tile::kSlots];
+  const int npackets = C / kVec;
+
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Tile g, o;
+    g.load(dy + row * C, npackets, A(0));
+    o.load(y + row * C, npackets, kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
+
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (kKind == kSoftmax) {
+          s += g.v[i][e] * o.v[i][e];
+        } else {
+          s += g.v[i][e];
+        }
+      }
+    s = Tile::reduce(s, SumOp(), slots);
+
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (kKind == kSoftmax) {
+          g.v[i][e] = (g.v[i][e] - s) * o.v[i][e];
+        } else {
+          g.v[i][e] = g.v[i][e] - M::exp_of(o.v[i][e]) * s;
+        }
+      }
+    g.store(dx + row * C, npackets);
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// One thread per (n, s) column, elements S apart. Also the fallback for S == 1
+// rows that are unaligned, not a whole number of packets, or too long for
+// registers (there a thread walks a contiguous row: correct, not fast).
+template <typename T, int kKind>
+__global__ __launch_bounds__(256) void softmax_columns(
+    const int64_t N, const int64_t S, const int64_t C, const T* x, T* y) {
+  using A = typename IO<T>::Acc;
+  const int64_t total = N * S;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * 256) {
+    const int64_t base = (i / S) * C * S + (i % S);
+    A m = acc_neg_inf<A>();
+    for (int64_t k = 0; k < C; ++k) m = MaxOp()(m, IO<T>::load1(x + base + k * S));
+    A s = A(0);
+    for (int64_t k = 0; k < C; ++k) s += acc_exp(IO<T>::load1(x + base + k * S) - m);
+    if (kKind == kSoftmax) {
+      for (int64_t k = 0; k < C; ++k) {
+        const A e = acc_exp(IO<T>::load1(x + base + k * S) - m);
+        IO<T>::store1(y + base + k * S, e / s);
+      }
+    } else {
+      const A l = acc_log(s);
+      for (int64_t k = 0; k < C; ++k) {
+        IO<T>::store1(y + base + k * S, (IO<T>::load1(x + base + k * S) - m) - l);
+      }
+    }
+  }
+}
+
+template <typename T, int kKind>
+__global__ __launch_bounds__(256) void softmax_grad_columns(
+    const int64_t N, const int64_t S, const int64_t C, const T* dy, const T* y, T* dx) {
+  using A = typename IO<T>::Acc;
+  const int64_t total = N * S;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * 256) {
+    const int64_t base = (i / S) * C * S + (i % S);
+    A s = A(0);
+    for (int64_t k = 0; k < C; ++k) {
+      const A g = IO<T>::load1(dy + base + k * S);
+      s += kKind == kSoftmax ? g * IO<T>::load1(y + base + k * S) : g;
+    }
+    for (int64_t k = 0; k < C; ++k) {
+      const A g = IO<T>::load1(dy + base + k * S);
+      const A o = IO<T>::load1(y + base + k * S);
+      IO<T>::store1(dx + base + k * S, kKind == kSoftmax ? (g - s) * o : g - acc_exp(o) * s);
+    }
+  }
+}
+
+// One workgroup per contiguous row of any length or alignment (S == 1 rows the
+// register tiles cannot take): strided element-wise passes over the row.
+template <typename T, int kKind>
+__global__ __launch_bounds__(256) void softmax_rows_looped(const int64_t N, const int64_t C,
+                                                           const T* x, T* y) {
+  using A = typename IO<T>::Acc;
+  __shared__ A slots[2][4];
+  for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
+    const T* xr = x + row * C;
+    T* yr = y + row * C;
+    A m = acc_neg_inf<A>();
+    for (int64_t j = threadIdx.x; j < C; j += 256) m = MaxOp()(m, IO<T>::load1(xr + j));
+    m = block_allreduce<4>(m, MaxOp(), slots[0]);
+    A s = A(0);
+    for (int64_t j = threadIdx.x; j < C; j += 256) s += acc_exp(IO<T>::load1(xr + j) - m);
+    s = block_allreduce<4>(s, SumOp(), slots[1]);
+    const A l = acc_log(s);
+    for (int64_t j = threadIdx.x; j < C; j += 256) {
+      const A d = IO<T>::load1(xr + j) - m;
+      IO<T>::store1(yr + j, kKind == kSoftmax ? acc_exp(d) / s : d - l);
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T, int kKind>
+__global__ __launch_bounds__(256) void softmax_grad_rows_looped(const int64_t N, const int64_t C,
+                                                                const T* dy, const T* y, T* dx) {
+  using A = typename IO<T>::Acc;
+  __shared__ A slots[4];
+  for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
+    const T* gr = dy + row * C;
+    const T* yr = y + row * C;
+    T* dr = dx + row * C;
+    A s = A(0);
+    for (int64_t j = threadIdx.x; j < C; j += 256) {
+      const A g = IO<T>::load1(gr + j);
+      s += kKind == kSoftmax ? g * IO<T>::load1(yr + j) : g;
+    }
+    s = block_allreduce<4>(s, SumOp(), slots);
+    for (int64_t j = threadIdx.x; j < C; j += 256) {
+      const A g = IO<T>::load1(gr + j);
+      const A o = IO<T>::load1(yr + j);
+      IO<T>::store1(dr + j, kKind == kSoftmax ? (g - s) * o : g - acc_exp(o) * s);
+    }
+    __syncthreads();
+  }
+}
+
+inline unsigned flat_grid(int64_t threads_needed) {
+  const int64_t want = ceil_div(threads_needed, 256);
+  const int64_t cap = static_cast<int64_t>(kNumCUs) * 64;
+  return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
+}
+
+template <typename T, int kKind>
+int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  RowConfig cfg;
+  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(y) && pick_row_config(C / kVec, &cfg)) {
+#define LAUNCH(TPR, VPT)                                                                     \
+  {                                                                                          \
+    using Tile = RowTile<T, TPR, VPT>;                                                       \
+    hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT>),                                   \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       N, static_cast<int>(C), xp, yp);                                      \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+  } else if (S == 1 && C >= 256) {
+    hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(row_grid(N, 1)), dim3(256), 0, stream,
+                       N, C, xp, yp);
+  } else {
+    hipLaunchKernelGGL((softmax_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0, stream, N,
+                       S, C, xp, yp);
+  }
+  return status_of_launch();
+}
+
+template <typename T, int kKind>
+int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const void* y, void* dx,
+                        hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const T* gp = static_cast<const T*>(dy);
+  const T* yp = static_cast<const T*>(y);
+  T* dp = static_cast<T*>(dx);
+  RowConfig cfg;
+  // Two tiles live at once: halve the packets a thread may hold.
+  if (S == 1 && C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx) &&
+      pick_row_config(C / kVec, &cfg) && !(cfg.tpr == 1024 && cfg.vpt == 8)) {
+#define LAUNCH(TPR, VPT)                                                                     \
+  {                                                                                          \
+    using Tile = RowTile<T, TPR, VPT>;                                                       \
+    hipLaunchKernelGGL((softmax_grad_rows<T, kKind, TPR, VPT>),                              \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       N, static_cast<int>(C), gp, yp, dp);                                  \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+  } else if (S == 1 && C >= 256) {
+    hipLaunchKernelGGL((softmax_grad_rows_looped<T, kKind>), dim3(row_grid(N, 1)), dim3(256), 0,
+                       stream, N, C, gp, yp, dp);
+  } else {
+    hipLaunchKernelGGL((softmax_grad_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0,
+                       stream, N, S, C, gp, yp, dp);
+  }
+  return status_of_launch();
+}
+
+template <typename T>
+int softmax_fwd(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipStream_t s) {
+  return launch_softmax<T, kSoftmax>(N, S, C, x, y, s);
+}
+template <typename T>
+int log_softmax_fwd(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipStream_t s) {
+  return launch_softmax<T, kLogSoftmax>(N, S, C, x, y, s);
+}
+template <typename T>
+int softmax_bwd(int64_t N, int64_t S, int64_t C, const void* dy, const void* y, void* dx,
+                hipStream_t s) {
+  return launch_softmax_grad<T, kSoftmax>(N, S, C, dy, y, dx, s);
+}
+template <typename T>
+int log_softmax_bwd(int64_t N, int64_t S, int64_t C, const void* dy, const void* y, void* dx,
+                    hipStream_t s) {
+  return launch_softmax_grad<T, kLogSoftmax>(N, S, C, dy, y, dx, s);
+}
+
+inline int check_softmax_args(int64_t N, int64_t S, int64_t C, const void* a, const void* b) {
+  if (N < 0 || S < 0 || C <= 0) return DRAGON_HIP_EINVAL;
+  if (N * S == 0) return 1;  // nothing to do
+  if (!a || !b) return DRAGON_HIP_EINVAL;
+  return 0;
+}
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" {
+
+int dragon_hip_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
+                       void* stream) {
+  const int c = dragon_hip::check_softmax_args(N, S, C, x, y);
+  if (c != 0) return c > 0 ? DRAGON_HIP_OK : c;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::softmax_fwd, N, S, C, x, y, s);
+}
+
+int dragon_hip_log_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
+                           void* stream) {
+  const int c = dragon_hip::check_softmax_args(N, S, C, x, y);
+  if (c != 0) return c > 0 ? DRAGON_HIP_OK : c;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::log_softmax_fwd, N, S, C, x, y, s);
+}
+
+int dragon_hip_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
+                            const void* y, void* dx, void* stream) {
+  const int c = dragon_hip::check_softmax_args(N, S, C, dy, y);
+  if (c != 0) return c > 0 ? DRAGON_HIP_OK : c;
+  if (!dx) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::softmax_bwd, N, S, C, dy, y, dx, s);
+}
+
+int dragon_hip_log_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
+                                const void* y, void* dx, void* stream) {
+  const int c = dragon_hip::check_softmax_args(N, S, C, dy, y);
+  if (c != 0) return c > 0 ? DRAGON_HIP_OK : c;
+  if (!dx) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::log_softmax_bwd, N, S, C, dy, y, dx, s);
+}
+
+} // extern "C"

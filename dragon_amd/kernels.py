@@ -1,0 +1,201 @@
+"""Python mirror of the reference's ``kernels::`` / ``math::`` free functions.
+
+Same names (snake-cased), argument order and aliasing conventions as the C++
+templates of dragon/kernels/normalization/op_kernels.h,
+dragon/kernels/activation/op_kernels.h and dragon/kernels/math/op_kernels.h;
+the trailing ``Context* ctx`` becomes the current torch stream. Tensors are
+torch CUDA tensors used purely as device memory: every function passes raw
+pointers through the C ABI (include/dragon_hip.h) to the gfx950 kernels.
+"""
+
+import ctypes
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2, torch.float64: 3}
+_LAYOUTS = {"NCHW": 0, "NHWC": 1}
+
+# Per-(device, stream) scratch, grown monotonically and never freed between
+# calls: the role of the "BufferShared" tensor of the context's scratch
+# workspace (dragon/core/workspace.h:81-92, dragon/core/context_cuda.cc:120-129).
+_scratch = {}
+
+
+def dtype_tag(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s" % t.dtype)
+
+
+def layout_tag(data_format):
+    if data_format not in _LAYOUTS:
+        raise ValueError("Unknown DataFormat: " + str(data_format))
+    return _LAYOUTS[data_format]
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("kernel arguments must live in device memory")
+    if not t.is_contiguous():
+        raise ValueError("kernel arguments must be contiguous")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def workspace(nbytes, device):
+    """Device scratch of at least ``nbytes`` for the current stream."""
+    if nbytes == 0:
+        return None
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _scratch[key] = buf
+    return buf
+
+
+def _call(name, *args):
+    _lib.check(name, getattr(_lib.lib(), name)(*args))
+
+
+def _dims(values):
+    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+
+
+# ---------------------------------------------------------------- math::
+
+def inv_std(N, eps, x, y):
+    _call("dragon_hip_inv_std", dtype_tag(x), N, eps, _ptr(x), _ptr(y), _stream())
+
+
+def axpby(N, alpha, x, beta, y):
+    _call("dragon_hip_axpby", dtype_tag(x), N, alpha, _ptr(x), beta, _ptr(y), _stream())
+
+
+def copy(N, x, y):
+    _call("dragon_hip_copy", dtype_tag(x), N, _ptr(x), _ptr(y), _stream())
+
+
+def set(N, value, y):  # noqa: A001 - the reference's name is math::Set
+    _call("dragon_hip_set", dtype_tag(y), N, value, _ptr(y), _stream())
+
+
+def square(N, x, y):
+    _call("dragon_hip_square", dtype_tag(x), N, _ptr(x), _ptr(y), _stream())
+
+
+def sub(N, a, b, y):
+    _call("dragon_hip_sub", dtype_tag(a), N, _ptr(a), _ptr(b), _ptr(y), _stream())
+
+
+# ---------------------------------------------------------------- kernels::
+
+def moments(dims, axes, x, mean, var):
+    d, a = _dims(dims), _dims(axes)
+    tag = dtype_tag(x)
+    need = _lib.lib().dragon_hip_moments_scratch_bytes(tag, len(dims), d, len(axes), a)
+    ws = workspace(need, x.device)
+    _call("dragon_hip_moments", tag, len(dims), d, len(axes), a, _ptr(x), _ptr(mean), _ptr(var),
+          _ptr(ws), need, _stream())
+
+
+def layer_norm(N, C, epsilon, x, gamma, beta, mu, rsig, y):
+    _call("dragon_hip_layer_norm", dtype_tag(x), N, C, epsilon, _ptr(x), _ptr(gamma), _ptr(beta),
+          _ptr(mu), _ptr(rsig), _ptr(y), _stream())
+
+
+def group_norm(N, G, D, S, data_format, x, mu, rsig, gamma, beta, y):
+    _call("dragon_hip_group_norm", dtype_tag(x), N, G, D, S, layout_tag(data_format), _ptr(x),
+          _ptr(mu), _ptr(rsig), _ptr(gamma), _ptr(beta), _ptr(y), _stream())
+
+
+def group_norm_grad(N, G, D, S, data_format, x, mu, rsig, gamma, dy, ds, db, dgamma, dbeta, dx):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    need = _lib.lib().dragon_hip_group_norm_grad_scratch_bytes(tag, N, G, D, S, lay)
+    ws = workspace(need, x.device)
+    _call("dragon_hip_group_norm_grad", tag, N, G, D, S, lay, _ptr(x), _ptr(mu), _ptr(rsig),
+          _ptr(gamma), _ptr(dy), _ptr(ds), _ptr(db), _ptr(dgamma), _ptr(dbeta), _ptr(dx),
+          _ptr(ws), need, _stream())
+
+
+def _bn_scratch(tag, N, C, S, lay, device):
+    need = _lib.lib().dragon_hip_batch_norm_reduce_scratch_bytes(tag, N, C, S, lay)
+    return workspace(need, device), need
+
+
+def batch_norm_expectation(N, C, S, normalizer, data_format, x, ex, ex2):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    ws, need = _bn_scratch(tag, N, C, S, lay, x.device)
+    _call("dragon_hip_batch_norm_expectation", tag, N, C, S, normalizer, lay, _ptr(x), _ptr(ex),
+          _ptr(ex2), _ptr(ws), need, _stream())
+
+
+def batch_norm(N, C, S, data_format, x, mu, rsig, gamma, beta, scale, bias, y):
+    _call("dragon_hip_batch_norm", dtype_tag(x), N, C, S, layout_tag(data_format), _ptr(x),
+          _ptr(mu), _ptr(rsig), _ptr(gamma), _ptr(beta), _ptr(scale), _ptr(bias), _ptr(y),
+          _stream())
+
+
+def batch_norm_wgrad(N, C, S, data_format, x, mu, rsig, dy, dgamma, dbeta):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    ws, need = _bn_scratch(tag, N, C, S, lay, x.device)
+    _call("dragon_hip_batch_norm_wgrad", tag, N, C, S, lay, _ptr(x), _ptr(mu), _ptr(rsig),
+          _ptr(dy), _ptr(dgamma), _ptr(dbeta), _ptr(ws), need, _stream())
+
+
+def batch_norm_training_grad(N, C, S, normalizer, data_format, x, mu, rsig, gamma, dgamma, dbeta,
+                             dy, dx):
+    _call("dragon_hip_batch_norm_training_grad", dtype_tag(x), N, C, S, normalizer,
+          layout_tag(data_format), _ptr(x), _ptr(mu), _ptr(rsig), _ptr(gamma), _ptr(dgamma),
+          _ptr(dbeta), _ptr(dy), _ptr(dx), _stream())
+
+
+def batch_norm_inference_grad(N, C, S, data_format, x, mu, rsig, gamma, dy, dgamma, dbeta, dx):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    ws, need = _bn_scratch(tag, N, C, S, lay, x.device)
+    _call("dragon_hip_batch_norm_inference_grad", tag, N, C, S, lay, _ptr(x), _ptr(mu), _ptr(rsig),
+          _ptr(gamma), _ptr(dy), _ptr(dgamma), _ptr(dbeta), _ptr(dx), _ptr(ws), need, _stream())
+
+
+def softmax(N, S, C, x, y):
+    _call("dragon_hip_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _stream())
+
+
+def log_softmax(N, S, C, x, y):
+    _call("dragon_hip_log_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _stream())
+
+
+def softmax_grad(N, S, C, dy, y, dx):
+    _call("dragon_hip_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx), _stream())
+
+
+def log_softmax_grad(N, S, C, dy, y, dx):
+    _call("dragon_hip_log_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx),
+          _stream())
+
+
+# ---------------------------------------------------------------- fused operator bodies
+
+def group_norm_forward(N, G, D, S, data_format, epsilon, x, gamma, beta, mu, rsig, y):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    need = _lib.lib().dragon_hip_group_norm_forward_scratch_bytes(tag, N, G, D, S, lay)
+    ws = workspace(need, x.device)
+    _call("dragon_hip_group_norm_forward", tag, N, G, D, S, lay, epsilon, _ptr(x), _ptr(gamma),
+          _ptr(beta), _ptr(mu), _ptr(rsig), _ptr(y), _ptr(ws), need, _stream())
+
+
+def batch_norm_training_forward(N, C, S, data_format, momentum, epsilon, x, gamma, beta,
+                                running_mean, running_var, mu, rsig, params, y):
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    ws, need = _bn_scratch(tag, N, C, S, lay, x.device)
+    _call("dragon_hip_batch_norm_training_forward", tag, N, C, S, lay, momentum, epsilon, _ptr(x),
+          _ptr(gamma), _ptr(beta), _ptr(running_mean), _ptr(running_var), _ptr(mu), _ptr(rsig),
+          _ptr(params), _ptr(y), _ptr(ws), need, _stream())

@@ -1,0 +1,251 @@
+/*
+ * dragon_hip.h - C ABI of the MI355X (gfx950) kernel library behind Dragon's
+ * kernels:: / math:: interface for LayerNorm, GroupNorm, BatchNorm, Moments and
+ * Softmax / LogSoftmax.
+ *
+ * Each entry point replaces one function template of the reference (cited as
+ * file:line relative to the reference tree). A `kernels::X<T, AccT, HIPContext>`
+ * specialisation is a one-line forward to the entry point of the same name:
+ * plain device pointers, 64-bit sizes, a dtype tag instead of the template
+ * arguments, a layout tag instead of the "NCHW"/"NHWC" string, the context's
+ * HIP stream, and (where a split reduction needs it) a scratch buffer the
+ * caller takes from the context's workspace.
+ *
+ * Conventions
+ *  - All tensor pointers are device pointers on the current device.
+ *  - `dtype` is the I/O type T. Statistics, affine parameters and parameter
+ *    gradients are AccT = float for f16/bf16/f32 and double for f64
+ *    (dragon/utils/math/types.h:69-152).
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *  - Kernels are enqueued asynchronously; nothing here allocates, frees or
+ *    synchronises, and every function is re-entrant.
+ *  - Return value: 0 on success, a negative dragon_hip_status on an argument
+ *    error (nothing was enqueued), a positive hipError_t when the runtime
+ *    refused a launch. The reference aborts through LOG(FATAL) on every error
+ *    (dragon/utils/logging.h:56-71); the HIPContext specialisation maps a
+ *    non-zero status to that.
+ *  - `scratch` may be NULL when the matching *_scratch_bytes() query returns 0;
+ *    otherwise it must hold at least that many bytes, 256-byte aligned, and
+ *    must not be shared by kernels running concurrently on other streams.
+ */
+#ifndef DRAGON_HIP_H_
+#define DRAGON_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  DRAGON_HIP_F16 = 0,  /* dragon::float16  (dragon/core/types.h:36-38) */
+  DRAGON_HIP_BF16 = 1, /* dragon::bfloat16 (dragon/core/types.h:40-42) */
+  DRAGON_HIP_F32 = 2,
+  DRAGON_HIP_F64 = 3
+} dragon_hip_dtype;
+
+typedef enum {
+  DRAGON_HIP_NCHW = 0, /* data_format == "NCHW": x is [N, C, S]  */
+  DRAGON_HIP_NHWC = 1  /* data_format == "NHWC": x is [N, S, C]  */
+} dragon_hip_layout;
+
+typedef enum {
+  DRAGON_HIP_OK = 0,
+  DRAGON_HIP_EINVAL = -1,   /* bad size, layout, null pointer or misalignment */
+  DRAGON_HIP_EDTYPE = -2,   /* dtype not in dragon_hip_dtype                  */
+  DRAGON_HIP_ESCRATCH = -3, /* scratch missing or too small                   */
+  DRAGON_HIP_ENODEVICE = -4 /* no gfx950 device visible                       */
+} dragon_hip_status;
+
+/* Human-readable text for a status returned by any function below. */
+const char* dragon_hip_status_string(int status);
+
+/* ------------------------------------------------------------------------ */
+/* Device-context plumbing: what a HIPContext needs so that the host layer   */
+/* includes no HIP header. Mirrors the static/member set every Dragon device */
+/* context provides (dragon/core/context_cuda.h:156-332; leanest precedent   */
+/* dragon/core/context_mlu.h:124-284).                                       */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_device_count(int* count);
+int dragon_hip_set_device(int device);
+int dragon_hip_get_device(int* device);
+int dragon_hip_device_name(int device, char* buf, size_t buf_bytes);
+int dragon_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
+/* Streams are non-blocking and all at the default priority. */
+int dragon_hip_stream_create(void** stream);
+int dragon_hip_stream_destroy(void* stream);
+int dragon_hip_stream_sync(void* stream);  /* Context::SynchronizeStream */
+int dragon_hip_malloc(void** ptr, size_t bytes);       /* Context::New    */
+int dragon_hip_free(void* ptr);                        /* Context::Delete */
+int dragon_hip_host_malloc(void** ptr, size_t bytes);  /* pinned host memory */
+int dragon_hip_host_free(void* ptr);
+int dragon_hip_memset_async(void* ptr, int value, size_t bytes, void* stream);
+/* kind: 0 host->host, 1 host->device, 2 device->host, 3 device->device */
+int dragon_hip_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
+int dragon_hip_event_create(void** event);
+int dragon_hip_event_destroy(void* event);
+int dragon_hip_event_record(void* event, void* stream);
+int dragon_hip_event_sync(void* event);
+int dragon_hip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ------------------------------------------------------------------------ */
+/* math:: helpers the operator bodies call on AccT buffers                   */
+/* ------------------------------------------------------------------------ */
+
+/* math::InvStd<T, Context>, dragon/utils/math/elementwise.h:48 (CPU
+ * dragon/utils/math/cpu/elementwise.cc:187-201): y = 1 / sqrt(x + eps).
+ * y may alias x (the operators run it in place on the variance buffer). */
+int dragon_hip_inv_std(int dtype, int64_t N, float eps, const void* x, void* y, void* stream);
+
+/* math::Axpby<T, Context>, dragon/utils/math/cpu/blas.cc:125-136:
+ * y = alpha * x + beta * y (running-statistics update, batch_norm_op.cc:60-63). */
+int dragon_hip_axpby(int dtype, int64_t N, float alpha, const void* x, float beta, void* y, void* stream);
+
+/* math::Copy / Set / Square / Sub as used at batch_norm_op.cc:45-47,148-165. */
+int dragon_hip_copy(int dtype, int64_t N, const void* x, void* y, void* stream);
+int dragon_hip_set(int dtype, int64_t N, float value, void* y, void* stream);
+int dragon_hip_square(int dtype, int64_t N, const void* x, void* y, void* stream);
+int dragon_hip_sub(int dtype, int64_t N, const void* a, const void* b, void* y, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* kernels::Moments, dragon/kernels/math/op_kernels.h:106-115                */
+/* (CPU dragon/kernels/math/cpu/moments_kernel.cc:10-189): mean and BIASED   */
+/* variance over `axes` of a row-major tensor of shape `dims`. mean / var    */
+/* are AccT with one element per kept index, in row-major order.             */
+/* ------------------------------------------------------------------------ */
+size_t dragon_hip_moments_scratch_bytes(int dtype, int num_dims, const int64_t* dims,
+                                        int num_axes, const int64_t* axes);
+int dragon_hip_moments(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                       const int64_t* axes, const void* x, void* mean, void* var,
+                       void* scratch, size_t scratch_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* kernels::LayerNorm, dragon/kernels/normalization/op_kernels.h:191-202     */
+/* (CPU dragon/kernels/normalization/cpu/layer_norm_kernel.cc:10-62).        */
+/* x, y: T[N, C]; gamma, beta: AccT[C]; mu, rsig: AccT[N].                   */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_layer_norm(int dtype, int64_t N, int64_t C, float eps, const void* x,
+                          const void* gamma, const void* beta, void* mu, void* rsig,
+                          void* y, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* kernels::GroupNorm, dragon/kernels/normalization/op_kernels.h:111-124     */
+/* (CPU dragon/kernels/normalization/cpu/group_norm_kernel.cc:11-31,88-110). */
+/* x, y: T[N,G,D,S] (NCHW) or T[N,S,G,D] (NHWC); mu, rsig: AccT[N*G];        */
+/* gamma, beta: AccT[G*D].                                                   */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_group_norm(int dtype, int64_t N, int64_t G, int64_t D, int64_t S, int layout,
+                          const void* x, const void* mu, const void* rsig, const void* gamma,
+                          const void* beta, void* y, void* stream);
+
+/* kernels::GroupNormGrad, dragon/kernels/normalization/op_kernels.h:126-143
+ * (CPU group_norm_kernel.cc:33-84,112-147). Also LayerNorm backward with
+ * G = S = 1, D = C, layout NHWC (dragon/operators/normalization/layer_norm_op.h:39-54).
+ * ds, db: AccT[N*G] each, written by the call; ds == db means db = ds + N*G
+ * (group_norm_kernel.cc:131). dgamma, dbeta: AccT[G*D]. All four are
+ * overwritten (the reference zero-fills them first, :132-135). */
+size_t dragon_hip_group_norm_grad_scratch_bytes(int dtype, int64_t N, int64_t G, int64_t D,
+                                                int64_t S, int layout);
+int dragon_hip_group_norm_grad(int dtype, int64_t N, int64_t G, int64_t D, int64_t S, int layout,
+                               const void* x, const void* mu, const void* rsig,
+                               const void* gamma, const void* dy, void* ds, void* db,
+                               void* dgamma, void* dbeta, void* dx, void* scratch,
+                               size_t scratch_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* BatchNorm family, dragon/kernels/normalization/op_kernels.h:36-109        */
+/* (CPU dragon/kernels/normalization/cpu/batch_norm_kernel.cc).              */
+/* x, y, dy, dx: T[N,C,S] (NCHW) or T[N,S,C] (NHWC); every [C] vector AccT.  */
+/* ------------------------------------------------------------------------ */
+
+/* kernels::BatchNormExpectation (op_kernels.h:36-46): ex = sum(x)/normalizer,
+ * ex2 = sum(x*x)/normalizer per channel. */
+size_t dragon_hip_batch_norm_reduce_scratch_bytes(int dtype, int64_t N, int64_t C, int64_t S,
+                                                  int layout);
+int dragon_hip_batch_norm_expectation(int dtype, int64_t N, int64_t C, int64_t S,
+                                      float normalizer, int layout, const void* x, void* ex,
+                                      void* ex2, void* scratch, size_t scratch_bytes,
+                                      void* stream);
+
+/* kernels::BatchNorm (op_kernels.h:48-62): scale = gamma*rsig,
+ * bias = beta - scale*mu, y = x*scale[c] + bias[c]. Aliasing conventions of
+ * batch_norm_kernel.cc:244-248: scale == rsig means a 3C buffer
+ * {rsig, scale, bias}; scale == bias means bias = scale + C. */
+int dragon_hip_batch_norm(int dtype, int64_t N, int64_t C, int64_t S, int layout, const void* x,
+                          const void* mu, const void* rsig, const void* gamma,
+                          const void* beta, void* scale, void* bias, void* y, void* stream);
+
+/* kernels::BatchNormWGrad (op_kernels.h:64-76): dgamma[c] = sum dy*(x-mu)*rsig,
+ * dbeta[c] = sum dy; dgamma == dbeta means dbeta = dgamma + C (:296).
+ * Scratch size: dragon_hip_batch_norm_reduce_scratch_bytes. */
+int dragon_hip_batch_norm_wgrad(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                const void* x, const void* mu, const void* rsig, const void* dy,
+                                void* dgamma, void* dbeta, void* scratch, size_t scratch_bytes,
+                                void* stream);
+
+/* kernels::BatchNormTrainingGrad (op_kernels.h:78-93):
+ * dx = gamma*rsig*(dy - ((x-mu)*rsig*dgamma + dbeta)/normalizer);
+ * dgamma == dbeta means dbeta = dgamma + C (:353). */
+int dragon_hip_batch_norm_training_grad(int dtype, int64_t N, int64_t C, int64_t S,
+                                        float normalizer, int layout, const void* x,
+                                        const void* mu, const void* rsig, const void* gamma,
+                                        const void* dgamma, const void* dbeta, const void* dy,
+                                        void* dx, void* stream);
+
+/* kernels::BatchNormInferenceGrad (op_kernels.h:95-109): dx = gamma*rsig*dy;
+ * dgamma != NULL additionally runs BatchNormWGrad (:406-409). */
+int dragon_hip_batch_norm_inference_grad(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                         const void* x, const void* mu, const void* rsig,
+                                         const void* gamma, const void* dy, void* dgamma,
+                                         void* dbeta, void* dx, void* scratch,
+                                         size_t scratch_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Softmax family, dragon/kernels/activation/op_kernels.h:211-247            */
+/* (CPU dragon/kernels/activation/cpu/softmax_kernel.cc:10-157).             */
+/* Tensors are T[N, C, S]: the reduced axis has length C and element stride  */
+/* S. y may alias x; dx may alias dy (softmax_op.cc:46-60).                  */
+/* 16-bit I/O accumulates in fp32.                                           */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
+                       void* stream);
+int dragon_hip_log_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
+                           void* stream);
+int dragon_hip_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
+                            const void* y, void* dx, void* stream);
+int dragon_hip_log_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
+                                const void* y, void* dx, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Operator-level fused entry points: one call for a kernel sequence that a  */
+/* Dragon operator body issues back to back, so that x is read once where    */
+/* the chip can hold the reduction unit on-die. Results equal the sequence.  */
+/* ------------------------------------------------------------------------ */
+
+/* GroupNormOp body, dragon/operators/normalization/group_norm_op.cc:26-51:
+ * Moments -> InvStd -> GroupNorm. Writes mu, rsig (AccT[N*G]) and y. */
+size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t G, int64_t D,
+                                                   int64_t S, int layout);
+int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
+                                  int layout, float eps, const void* x, const void* gamma,
+                                  const void* beta, void* mu, void* rsig, void* y,
+                                  void* scratch, size_t scratch_bytes, void* stream);
+
+/* BatchNormOp::RunTraining body without sync,
+ * dragon/operators/normalization/batch_norm_op.cc:49-82: Moments -> Axpby x2
+ * (running statistics, biased variance, y = (1-momentum)*stat + momentum*y)
+ * -> InvStd -> BatchNorm. Writes mu, rsig (AccT[C]), params (AccT[2C] =
+ * {scale, bias}), y, and updates running_mean / running_var in place. */
+int dragon_hip_batch_norm_training_forward(int dtype, int64_t N, int64_t C, int64_t S, int layout,
+                                           float momentum, float eps, const void* x,
+                                           const void* gamma, const void* beta,
+                                           void* running_mean, void* running_var, void* mu,
+                                           void* rsig, void* params, void* y, void* scratch,
+                                           size_t scratch_bytes, void* stream);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* DRAGON_HIP_H_ */

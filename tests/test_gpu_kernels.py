@@ -1,0 +1,425 @@
+"""GPU parity: every C-ABI kernel entry point against the CPU oracle on the same
+seeded inputs, at sizes the oracle finishes in seconds.
+
+Bar: normwise 1e-5 for fp32 I/O and 1e-2 for fp16 / bf16 I/O against the fp32
+oracle run on the 16-bit-rounded inputs (tests/util.py: TOL); fp64 to 1e-12.
+Where the reference's CPU kernel supports the 16-bit type itself (LayerNorm,
+GroupNorm forward, Moments) the oracle runs in that type.
+"""
+
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    import torch
+    assert torch.cuda.is_available()
+    from dragon_amd import kernels
+    return kernels
+
+
+def empty(shape, dtype):
+    import torch
+    return torch.empty(shape, dtype=U.torch_dtype(dtype), device="cuda")
+
+
+def acc_name(dtype):
+    return "float64" if dtype == "float64" else "float32"
+
+
+def oracle_dtype_inputs(bits, dtype):
+    """Inputs for an oracle kernel that only exists in fp32/fp64: widen 16-bit storage."""
+    if dtype in ("float16", "bfloat16"):
+        return R.from_bits(bits, dtype), "float32"
+    return bits, dtype
+
+
+# ---------------------------------------------------------------- LayerNorm forward
+
+LN_SHAPES = [(64, 1024), (33, 1000), (7, 12288), (5, 4096), (300, 48), (3, 37), (9, 8),
+             (2, 70000), (1, 1), (513, 256)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape", LN_SHAPES)
+def test_layer_norm_forward(K, dtype, shape):
+    N, C = shape
+    rng = U.rng_for(100 + C)
+    x = R.to_bits((rng.standard_normal(shape) * 2 + 0.5).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    y_ref, mu_ref, rsig_ref = R.layer_norm(dtype, x, g, b, 1e-5)
+    xd, gd, bd = U.to_device(x, dtype), U.to_device(g, acc_name(dtype)), U.to_device(b, acc_name(dtype))
+    y, mu, rsig = empty(shape, dtype), empty((N,), acc_name(dtype)), empty((N,), acc_name(dtype))
+    K.layer_norm(N, C, 1e-5, xd, gd, bd, mu, rsig, y)
+    stat_tol = 1e-12 if dtype == "float64" else 1e-5
+    assert U.normwise(U.to_host(mu), mu_ref) <= stat_tol
+    assert np.max(np.abs(U.to_host(rsig) / rsig_ref - 1)) <= stat_tol
+    assert U.normwise(U.widen(U.to_host(y), dtype), U.widen(y_ref, dtype)) <= U.TIGHT[dtype]
+
+
+def test_layer_norm_empty_and_errors(K):
+    import torch
+    from dragon_amd._lib import DragonHipError
+    z = torch.empty(0, device="cuda")
+    K.layer_norm(0, 16, 1e-5, z, z, z, z, z, z)  # no rows: nothing enqueued, no error
+    with pytest.raises(DragonHipError):
+        K.layer_norm(4, 0, 1e-5, z, z, z, z, z, z)
+    with pytest.raises(TypeError):
+        K.layer_norm(1, 1, 1e-5, z.to(torch.int32), z, z, z, z, z)
+
+
+def test_layer_norm_large_mean_stays_accurate(K):
+    """|mean| >> stddev: the centred variance must not cancel (fp64 is the judge)."""
+    rng = U.rng_for(7)
+    N, C = 16, 4096
+    x = (rng.standard_normal((N, C)) + 1000.0).astype(np.float32)
+    g, b = np.ones(C, np.float32), np.zeros(C, np.float32)
+    y, mu, rsig = empty((N, C), "float32"), empty((N,), "float32"), empty((N,), "float32")
+    K.layer_norm(N, C, 1e-5, U.to_device(x, "float32"), U.to_device(g, "float32"),
+                 U.to_device(b, "float32"), mu, rsig, y)
+    x64 = x.astype(np.float64)
+    r64 = 1 / np.sqrt(x64.var(1) + 1e-5)
+    assert np.max(np.abs(U.to_host(rsig) / r64 - 1)) < 1e-5
+
+
+# ---------------------------------------------------------------- Softmax family
+
+SM_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 100000), -1), ((5, 37), -1),
+             ((6, 300), -1), ((3, 7, 5), 1), ((2, 3, 4, 6), 2), ((4, 1), -1), ((2, 16, 8, 8), -1),
+             ((3, 8200), -1)]
+
+
+def _softmax_inputs(shape, dtype, seed):
+    rng = U.rng_for(seed)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    x[rng.random(shape) < 0.05] = -1e4
+    # keep one finite logit per reduced slice
+    dy = rng.standard_normal(shape).astype(np.float32)
+    return R.to_bits(x, dtype), R.to_bits(dy, dtype)
+
+
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape,axis", SM_SHAPES)
+def test_softmax_forward_backward(K, shape, axis, dtype, log):
+    x, dy = _softmax_inputs(shape, dtype, 200 + len(shape))
+    ax = axis % len(shape)
+    N = int(np.prod(shape[:ax] or (1,)))
+    C = shape[ax]
+    S = int(np.prod(shape[ax + 1:] or (1,)))
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    y_ref = R.op_softmax(od, xo, axis, log=log)
+    xd, dyd = U.to_device(x, dtype), U.to_device(dy, dtype)
+    y = empty(shape, dtype)
+    (K.log_softmax if log else K.softmax)(N, S, C, xd, y)
+    y_host = U.to_host(y)
+    yw = U.widen(y_host, dtype).reshape(shape)
+    if log:
+        finite = np.isfinite(y_ref) & (np.asarray(y_ref) > -5e3)
+        err = np.max(np.abs(yw[finite] - np.asarray(y_ref, np.float64)[finite]) /
+                     np.maximum(np.abs(np.asarray(y_ref, np.float64)[finite]), 1.0))
+        assert err <= U.TIGHT[dtype]
+    else:
+        assert U.rowwise_normwise(np.moveaxis(yw, ax, -1), np.moveaxis(np.asarray(y_ref), ax, -1)) \
+            <= U.TIGHT[dtype]
+        sums = yw.sum(ax)
+        assert np.max(np.abs(sums - 1)) <= {"float16": 2e-3, "bfloat16": 2e-2}.get(dtype, 1e-5)
+    # backward consumes the y the forward produced, as the operator graph does
+    yo, _ = oracle_dtype_inputs(y_host.reshape(shape), dtype)
+    dx_ref = R.op_softmax_grad(od, yo, dyo, axis, log=log)
+    dx = empty(shape, dtype)
+    (K.log_softmax_grad if log else K.softmax_grad)(N, S, C, dyd, y, dx)
+    dxw = U.widen(U.to_host(dx), dtype).reshape(shape)
+    ok = np.isfinite(np.asarray(dx_ref))
+    assert U.normwise(dxw[ok], np.asarray(dx_ref)[ok]) <= U.TIGHT[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_softmax_in_place(K, dtype):
+    shape = (64, 512)
+    x, dy = _softmax_inputs(shape, dtype, 5)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    y_ref = R.op_softmax(od, xo)
+    buf = U.to_device(x, dtype)
+    K.softmax(64, 1, 512, buf, buf)  # Y aliases X (AllowInplace {0,0})
+    assert U.rowwise_normwise(U.widen(U.to_host(buf), dtype), y_ref) <= U.TIGHT[dtype]
+    g = U.to_device(dy, dtype)
+    yo, _ = oracle_dtype_inputs(U.to_host(buf), dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    dx_ref = R.op_softmax_grad(od, yo, dyo)
+    K.softmax_grad(64, 1, 512, g, buf, g)  # dX aliases dY (AllowInplace {1,0})
+    assert U.normwise(U.widen(U.to_host(g), dtype), dx_ref) <= U.TIGHT[dtype]
+
+
+def test_softmax_masked_logits_are_exact_zero(K):
+    x = np.zeros((4, 512), np.float32)
+    x[:, ::2] = -1e4
+    xd = U.to_device(R.to_bits(x, "float16"), "float16")
+    y = empty((4, 512), "float16")
+    K.softmax(4, 1, 512, xd, y)
+    yw = U.widen(U.to_host(y), "float16")
+    assert np.all(yw[:, ::2] == 0)
+    assert np.allclose(yw[:, 1::2], 1 / 256, rtol=1e-3)
+
+
+# ---------------------------------------------------------------- LayerNorm backward
+
+LNB_SHAPES = [(64, 1024), (33, 1000), (16, 12288), (300, 48), (5, 37), (1100, 256), (40, 4096),
+              (3, 20000), (2, 8)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
+@pytest.mark.parametrize("shape", LNB_SHAPES)
+def test_layer_norm_backward(K, dtype, shape):
+    N, C = shape
+    rng = U.rng_for(300 + C)
+    x = (rng.standard_normal(shape)).astype(np.float32)
+    x[rng.random(shape) < 0.01] *= 50
+    x = R.to_bits(x, dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    an = acc_name(dtype)
+    _, mu, rsig = R.layer_norm(dtype, x, g, b, 1e-5)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    dx_ref, dg_ref, db_ref, ds_ref, dbb_ref = R.group_norm_grad(od, N, 1, C, 1, "NHWC", xo, mu, rsig, g, dyo)
+    params = empty((2 * N,), an)
+    dg, db, dx = empty((C,), an), empty((C,), an), empty(shape, dtype)
+    K.group_norm_grad(N, 1, C, 1, "NHWC", U.to_device(x, dtype), U.to_device(mu, an),
+                      U.to_device(rsig, an), U.to_device(g, an), U.to_device(dy, dtype),
+                      params, params, dg, db, dx)
+    tol = U.TIGHT[dtype]
+    assert U.normwise(U.widen(U.to_host(dx), dtype), dx_ref) <= tol
+    ptol = 1e-12 if dtype == "float64" else 2e-5
+    assert U.normwise(U.to_host(dg), dg_ref) <= ptol
+    assert U.normwise(U.to_host(db), db_ref) <= ptol
+    p = U.to_host(params)
+    assert U.normwise(p[:N], ds_ref) <= ptol and U.normwise(p[N:], dbb_ref) <= ptol
+
+
+# ---------------------------------------------------------------- GroupNorm
+
+GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), ((3, 5, 12), -1, 3),
+            ((2, 64, 16, 16), 1, 32), ((4, 8), -1, 2), ((2, 16, 4, 4), 1, 0), ((1, 4, 2), 1, 2)]
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
+@pytest.mark.parametrize("shape,axis,group", GN_CASES)
+def test_group_norm_forward_backward(K, shape, axis, group, dtype, fused):
+    rng = U.rng_for(400 + len(shape) + group)
+    ax = axis % len(shape)
+    N, C = shape[0], shape[ax]
+    S = int(np.prod(shape)) // N // C
+    G = group if group > 0 else C
+    D = C // G
+    layout = "NHWC" if ax + 1 == len(shape) else "NCHW"
+    an = acc_name(dtype)
+    x = R.to_bits((rng.standard_normal(shape) + 0.3).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    y_ref, mu_ref, rsig_ref = R.op_group_norm(dtype, x, g, b, axis, group, 1e-5)
+    xd, gd, bd = U.to_device(x, dtype), U.to_device(g, an), U.to_device(b, an)
+    mu, rsig, y = empty((N * G,), an), empty((N * G,), an), empty(shape, dtype)
+    if fused:
+        K.group_norm_forward(N, G, D, S, layout, 1e-5, xd, gd, bd, mu, rsig, y)
+    else:  # the operator's own sequence: Moments -> InvStd -> GroupNorm
+        if layout == "NCHW":
+            K.moments([N * G, D * S], [1], xd, mu, rsig)
+        else:
+            K.moments([N, S, G, D], [1, 3], xd, mu, rsig)
+        K.inv_std(N * G, 1e-5, rsig, rsig)
+        K.group_norm(N, G, D, S, layout, xd, mu, rsig, gd, bd, y)
+    stat_tol = 1e-12 if dtype == "float64" else 1e-5
+    assert U.normwise(U.to_host(mu), mu_ref) <= stat_tol
+    assert np.max(np.abs(U.to_host(rsig) / rsig_ref - 1)) <= stat_tol
+    assert U.normwise(U.widen(U.to_host(y), dtype), U.widen(y_ref, dtype)) <= U.TIGHT[dtype]
+    if fused:
+        return
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    dx_ref, dg_ref, db_ref, ds_ref, dbb_ref = R.group_norm_grad(
+        od, N, G, D, S, layout, xo, mu_ref, rsig_ref, g, dyo)
+    params = empty((2 * N * G,), an)
+    dg, db, dx = empty((C,), an), empty((C,), an), empty(shape, dtype)
+    K.group_norm_grad(N, G, D, S, layout, xd, U.to_device(mu_ref, an), U.to_device(rsig_ref, an), gd,
+                      U.to_device(dy, dtype), params, params, dg, db, dx)
+    ptol = 1e-12 if dtype == "float64" else 2e-5
+    assert U.normwise(U.widen(U.to_host(dx), dtype), dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(U.to_host(dg), dg_ref) <= ptol
+    assert U.normwise(U.to_host(db), db_ref) <= ptol
+    p = U.to_host(params)
+    assert U.normwise(p[:N * G], ds_ref) <= ptol and U.normwise(p[N * G:], dbb_ref) <= ptol
+
+
+# ---------------------------------------------------------------- BatchNorm
+
+BN_CASES = [((8, 16, 7, 7), 1), ((4, 3, 2), 1), ((16, 32), -1), ((4, 5, 5, 24), -1),
+            ((6, 64, 28, 28), 1), ((4, 2, 3), -1), ((3, 130, 4), 1), ((50, 70), -1)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16", "float16"])
+@pytest.mark.parametrize("shape,axis", BN_CASES)
+def test_batch_norm_training(K, shape, axis, dtype):
+    rng = U.rng_for(500 + len(shape))
+    ax = axis % len(shape)
+    N, C = shape[0], shape[ax]
+    S = int(np.prod(shape)) // N // C
+    layout = "NHWC" if ax + 1 == len(shape) else "NCHW"
+    an = acc_name(dtype)
+    x = R.to_bits((2 * rng.standard_normal(shape) + 0.5).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    rm0 = (rng.standard_normal(C) * 0.1).astype(U.acc_np(dtype))
+    rv0 = rng.uniform(0.5, 1.5, C).astype(U.acc_np(dtype))
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    rm_ref, rv_ref = rm0.copy(), rv0.copy()
+    y_ref, mu_ref, rsig_ref, params_ref = R.op_batch_norm_train(
+        od, np.asarray(xo).reshape(shape), g, b, rm_ref, rv_ref, axis, 0.9, 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_train_grad(
+        od, np.asarray(xo).reshape(shape), g, np.asarray(dyo).reshape(shape), mu_ref, rsig_ref, axis)
+
+    xd, gd, bd = U.to_device(x, dtype), U.to_device(g, an), U.to_device(b, an)
+    stat_tol = 1e-12 if dtype == "float64" else 1e-5
+
+    def check_forward(mu, rsig, params, rm, rv, y):
+        assert U.normwise(U.to_host(mu), mu_ref) <= stat_tol
+        assert np.max(np.abs(U.to_host(rsig) / rsig_ref - 1)) <= stat_tol
+        assert U.normwise(U.to_host(params), params_ref) <= stat_tol
+        assert U.normwise(U.to_host(rm), rm_ref) <= stat_tol
+        assert U.normwise(U.to_host(rv), rv_ref) <= stat_tol
+        # 16-bit y is compared with the fp32 reference result (the CPU has no 16-bit BatchNorm)
+        assert U.normwise(U.widen(U.to_host(y), dtype), y_ref) <= U.TIGHT[dtype]
+
+    # (a) the operator's own sequence: Moments, Axpby x2, InvStd, BatchNorm
+    mu, rsig, params = empty((C,), an), empty((C,), an), empty((2 * C,), an)
+    rm, rv, y = U.to_device(rm0, an), U.to_device(rv0, an), empty(shape, dtype)
+    if layout == "NCHW":
+        K.moments([N, C, S], [0, 2], xd, mu, rsig)
+    else:
+        K.moments([N * S, C], [0], xd, mu, rsig)
+    K.axpby(C, 1.0 - 0.9, mu, 0.9, rm)
+    K.axpby(C, 1.0 - 0.9, rsig, 0.9, rv)
+    K.inv_std(C, 1e-5, rsig, rsig)
+    K.batch_norm(N, C, S, layout, xd, mu, rsig, gd, bd, params, params, y)
+    check_forward(mu, rsig, params, rm, rv, y)
+
+    # (b) the fused training forward
+    mu2, rsig2, params2 = empty((C,), an), empty((C,), an), empty((2 * C,), an)
+    rm2, rv2, y2 = U.to_device(rm0, an), U.to_device(rv0, an), empty(shape, dtype)
+    K.batch_norm_training_forward(N, C, S, layout, 0.9, 1e-5, xd, gd, bd, rm2, rv2, mu2, rsig2,
+                                  params2, y2)
+    check_forward(mu2, rsig2, params2, rm2, rv2, y2)
+
+    # backward: WGrad into the packed params buffer, then TrainingGrad
+    dyd = U.to_device(dy, dtype)
+    mud, rsd = U.to_device(mu_ref, an), U.to_device(rsig_ref, an)
+    wg, dx = empty((2 * C,), an), empty(shape, dtype)
+    K.batch_norm_wgrad(N, C, S, layout, xd, mud, rsd, dyd, wg, wg)
+    ptol = 1e-12 if dtype == "float64" else 2e-5
+    w = U.to_host(wg)
+    assert U.normwise(w[:C], dg_ref) <= ptol and U.normwise(w[C:], db_ref) <= ptol
+    wref = U.to_device(np.concatenate([dg_ref, db_ref]).astype(U.acc_np(dtype)), an)
+    K.batch_norm_training_grad(N, C, S, float(N * S), layout, xd, mud, rsd, gd, wref, wref, dyd, dx)
+    assert U.normwise(U.widen(U.to_host(dx), dtype), dx_ref) <= U.TIGHT[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16"])
+@pytest.mark.parametrize("shape,axis", BN_CASES[:5])
+def test_batch_norm_inference_and_expectation(K, shape, axis, dtype):
+    rng = U.rng_for(600 + len(shape))
+    ax = axis % len(shape)
+    N, C = shape[0], shape[ax]
+    S = int(np.prod(shape)) // N // C
+    layout = "NHWC" if ax + 1 == len(shape) else "NCHW"
+    an = acc_name(dtype)
+    x = R.to_bits((2 * rng.standard_normal(shape) + 0.5).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    rm = (rng.standard_normal(C) * 0.1).astype(U.acc_np(dtype))
+    rv = rng.uniform(0.5, 1.5, C).astype(U.acc_np(dtype))
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    xo, dyo = np.asarray(xo).reshape(shape), np.asarray(dyo).reshape(shape)
+    y_ref = R.op_batch_norm_infer(od, xo, g, b, rm, rv, axis, 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_infer_grad(od, xo, g, rm, rv, dyo, axis, 1e-5)
+    xd, gd, bd = U.to_device(x, dtype), U.to_device(g, an), U.to_device(b, an)
+    rmd, rvd = U.to_device(rm, an), U.to_device(rv, an)
+    # RunInference: InvStd into params[0:C], BatchNorm with scale == bias == rsig (3C buffer)
+    params, y = empty((3 * C,), an), empty(shape, dtype)
+    K.inv_std(C, 1e-5, rvd, params)
+    K.batch_norm(N, C, S, layout, xd, rmd, params, gd, bd, params, params, y)
+    assert U.normwise(U.widen(U.to_host(y), dtype), y_ref) <= U.TIGHT[dtype]
+    p = U.to_host(params)
+    rs = 1 / np.sqrt(rv.astype(np.float64) + 1e-5)
+    assert np.max(np.abs(p[:C] / rs - 1)) < 1e-5 and np.max(np.abs(p[C:2 * C] / (g * rs) - 1)) < 1e-5
+    # RunInference gradient
+    dyd = U.to_device(dy, dtype)
+    rsd, dg, db, dx = empty((C,), an), empty((C,), an), empty((C,), an), empty(shape, dtype)
+    K.inv_std(C, 1e-5, rvd, rsd)
+    K.batch_norm_inference_grad(N, C, S, layout, xd, rmd, rsd, gd, dyd, dg, db, dx)
+    ptol = 1e-12 if dtype == "float64" else 2e-5
+    assert U.normwise(U.widen(U.to_host(dx), dtype), dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(U.to_host(dg), dg_ref) <= ptol and U.normwise(U.to_host(db), db_ref) <= ptol
+    dx2 = empty(shape, dtype)
+    K.batch_norm_inference_grad(N, C, S, layout, xd, rmd, rsd, gd, dyd, None, None, dx2)
+    assert np.array_equal(U.to_host(dx2), U.to_host(dx))
+    # SyncBN statistics kernel against E[x], E[x^2] with a doubled ("two rank") normaliser
+    ex, ex2 = empty((C,), an), empty((C,), an)
+    K.batch_norm_expectation(N, C, S, float(2 * N * S), layout, xd, ex, ex2)
+    ex_ref, ex2_ref = R.batch_norm_expectation(od, N, C, S, float(2 * N * S), layout, xo)
+    assert U.normwise(U.to_host(ex), ex_ref) <= ptol and U.normwise(U.to_host(ex2), ex2_ref) <= ptol
+
+
+# ---------------------------------------------------------------- Moments / math helpers
+
+MOMENT_CASES = [((4, 5, 6), (0, 2)), ((20, 5), (0,)), ((6, 35), (1,)), ((3, 4, 2, 5), (1, 3)),
+                ((3, 1, 4, 1, 5), (2, 4)), ((2, 3, 4), (0, 1, 2)), ((2, 3, 4), (1,)),
+                ((5, 4, 3, 2, 2), (0, 2, 4)), ((7,), ()), ((64, 40, 49), (0, 2)),
+                ((1000, 72), (0,)), ((16, 8192), (1,)), ((2, 3), (0,)), ((2, 3), (1,)),
+                ((2, 3), (0, 1))]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape,axes", MOMENT_CASES)
+def test_moments(K, shape, axes, dtype):
+    rng = U.rng_for(700 + len(shape))
+    x = R.to_bits((rng.standard_normal(shape) * 2 + 0.5).astype(np.float32), dtype)
+    mean_ref, var_ref = R.moments(dtype, x, list(axes))
+    an = acc_name(dtype)
+    mean, var = empty(mean_ref.shape, an), empty(var_ref.shape, an)
+    K.moments(list(shape), list(axes), U.to_device(x, dtype), mean, var)
+    tol = 1e-12 if dtype == "float64" else 1e-5
+    assert U.normwise(U.to_host(mean), mean_ref) <= tol
+    assert U.normwise(U.to_host(var), var_ref) <= tol * 2
+
+
+def test_math_helpers_bitwise(K):
+    rng = U.rng_for(9)
+    n = 1000
+    x = rng.uniform(0.1, 4, n).astype(np.float32)
+    y0 = rng.standard_normal(n).astype(np.float32)
+    xd, yd = U.to_device(x, "float32"), U.to_device(y0, "float32")
+    out = empty((n,), "float32")
+    K.inv_std(n, 1e-5, xd, out)
+    assert np.max(np.abs(U.to_host(out) / R.inv_std(x, 1e-5) - 1)) <= 1.2e-7
+    K.axpby(n, 0.1, xd, 0.9, yd)
+    y_ref = y0.copy()
+    R.axpby(0.1, x, 0.9, y_ref)
+    assert np.array_equal(U.to_host(yd), y_ref)  # two roundings, no fused multiply-add
+    K.copy(n, xd, out)
+    assert np.array_equal(U.to_host(out), x)
+    K.square(n, xd, out)
+    assert np.array_equal(U.to_host(out), x * x)
+    K.sub(n, xd, yd, out)
+    assert np.array_equal(U.to_host(out), x - U.to_host(yd))
+    K.set(n, 2.5, out)
+    assert np.all(U.to_host(out) == 2.5)
