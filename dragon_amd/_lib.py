@@ -90,6 +90,10 @@ def lib():
             raise RuntimeError(
                 "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "(there is no CPU fallback)" % LIB_PATH)
+        # torch ships its own HIP runtime and is the source of every device
+        # pointer: import it first so this library binds to that same runtime
+        # (one process must not hold two copies of libamdhip64).
+        import torch  # noqa: F401
         handle = ctypes.CDLL(LIB_PATH)
         for name, (restype, argtypes) in SIGNATURES.items():
             fn = getattr(handle, name)

@@ -80,20 +80,22 @@ struct IO<f16_t> {
   static constexpr int kVec = 8;
   static __device__ __forceinline__ void load(const f16_t* p, float (&v)[8]) {
     const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const h16x2 h = __builtin_bit_cast(h16x2, t[i]);
+      const h16x2 h = __builtin_bit_cast(h16x2, w[i]);
       v[2 * i] = static_cast<float>(h.x);
       v[2 * i + 1] = static_cast<float>(h.y);
     }
   }
   static __device__ __forceinline__ void store(f16_t* p, const float (&v)[8]) {
-    u32x4 t;
+    uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const f32x2 f = {v[2 * i], v[2 * i + 1]};
-      t[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
+      w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
     }
+    const u32x4 t = {w[0], w[1], w[2], w[3]};
     __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
   }
   static __device__ __forceinline__ float load1(const f16_t* p) {
@@ -110,19 +112,21 @@ struct IO<bf16_t> {
   static constexpr int kVec = 8;
   static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
     const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[2 * i] = __builtin_bit_cast(float, t[i] << 16);
-      v[2 * i + 1] = __builtin_bit_cast(float, t[i] & 0xffff0000u);
+      v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+      v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
     }
   }
   static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
-    u32x4 t;
+    uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const f32x2 f = {v[2 * i], v[2 * i + 1]};
-      t[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, b16x2));
+      w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, b16x2));
     }
+    const u32x4 t = {w[0], w[1], w[2], w[3]};
     __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
   }
   static __device__ __forceinline__ float load1(const bf16_t* p) {

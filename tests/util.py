@@ -78,3 +78,14 @@ def affine_params(rng, C, dtype):
     """gamma ~ U(0.5, 1.5), beta ~ N(0, 0.1) in the accumulator type."""
     a = acc_np(dtype)
     return (rng.uniform(0.5, 1.5, C).astype(a), (rng.standard_normal(C) * 0.1).astype(a))
+
+
+def close3(got, oracle, exact, tol):
+    """Three-way check for long reductions, where the oracle's strictly
+    sequential fp32 sums are themselves off: the distance to the oracle may
+    exceed ``tol`` only by the oracle's own distance to the fp64 result.
+    Returns (ok, gpu_vs_oracle, gpu_vs_exact, oracle_vs_exact), all normwise."""
+    e_go = normwise(got, oracle)
+    e_ge = normwise(got, exact)
+    e_oe = normwise(oracle, exact)
+    return e_go <= tol + e_oe and e_ge <= tol, e_go, e_ge, e_oe
