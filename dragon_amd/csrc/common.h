@@ -1,7 +1,6 @@
 // Shared device-side building blocks for the gfx950 norm / softmax kernels:
 // 16-byte packet I/O with conversion to the accumulator type, wave64 and
-// workgroup reductions, Chan/Welford partial-moment combination, and the
-// launch helpers every entry point uses.
+// workgroup reductions, and the launch helpers every entry point uses.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -35,7 +34,7 @@ typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
 //   Acc    accumulator type (math::Traits<T>::accumulator_type,
 //          dragon/utils/math/types.h:69-152)
 //   kVec   elements per 16-byte packet
-//   load / store   one aligned 16-byte packet <-> kVec accumulators
+//   unpack / pack  one 16-byte packet (four dwords) <-> kVec accumulators
 //   load1 / store1 one element (tails and unaligned tensors)
 // Rounding on store is round-to-nearest-even in hardware, which is what the
 // reference's software conversion implements (dragon/utils/conversions.h:42-106).
@@ -46,13 +45,17 @@ template <>
 struct IO<float> {
   using Acc = float;
   static constexpr int kVec = 4;
-  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
-    v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+  // Vector elements are copied to scalars before any bit cast: a bit cast
+  // applied directly to an element expression (t.x, t[i]) reads element 0.
+  static __device__ __forceinline__ void unpack(const u32x4 t, float (&v)[4]) {
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_bit_cast(float, w[i]);
   }
-  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
-    f32x4 t = {v[0], v[1], v[2], v[3]};
-    __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[4]) {
+    const u32x4 t = {__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
+                     __builtin_bit_cast(uint32_t, v[2]), __builtin_bit_cast(uint32_t, v[3])};
+    return t;
   }
   static __device__ __forceinline__ float load1(const float* p) { return *p; }
   static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
@@ -62,13 +65,13 @@ template <>
 struct IO<double> {
   using Acc = double;
   static constexpr int kVec = 2;
-  static __device__ __forceinline__ void load(const double* p, double (&v)[2]) {
-    const f64x2 t = *reinterpret_cast<const f64x2*>(p);
-    v[0] = t.x, v[1] = t.y;
+  static __device__ __forceinline__ void unpack(const u32x4 t, double (&v)[2]) {
+    const f64x2 d = __builtin_bit_cast(f64x2, t);
+    v[0] = d.x, v[1] = d.y;
   }
-  static __device__ __forceinline__ void store(double* p, const double (&v)[2]) {
-    f64x2 t = {v[0], v[1]};
-    __builtin_nontemporal_store(t, reinterpret_cast<f64x2*>(p));
+  static __device__ __forceinline__ u32x4 pack(const double (&v)[2]) {
+    const f64x2 d = {v[0], v[1]};
+    return __builtin_bit_cast(u32x4, d);
   }
   static __device__ __forceinline__ double load1(const double* p) { return *p; }
   static __device__ __forceinline__ void store1(double* p, double v) { *p = v; }
@@ -78,8 +81,7 @@ template <>
 struct IO<f16_t> {
   using Acc = float;
   static constexpr int kVec = 8;
-  static __device__ __forceinline__ void load(const f16_t* p, float (&v)[8]) {
-    const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+  static __device__ __forceinline__ void unpack(const u32x4 t, float (&v)[8]) {
     const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -88,7 +90,7 @@ struct IO<f16_t> {
       v[2 * i + 1] = static_cast<float>(h.y);
     }
   }
-  static __device__ __forceinline__ void store(f16_t* p, const float (&v)[8]) {
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -96,7 +98,7 @@ struct IO<f16_t> {
       w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
     }
     const u32x4 t = {w[0], w[1], w[2], w[3]};
-    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+    return t;
   }
   static __device__ __forceinline__ float load1(const f16_t* p) {
     return static_cast<float>(__builtin_bit_cast(_Float16, p->x));
@@ -110,8 +112,7 @@ template <>
 struct IO<bf16_t> {
   using Acc = float;
   static constexpr int kVec = 8;
-  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
-    const u32x4 t = *reinterpret_cast<const u32x4*>(p);
+  static __device__ __forceinline__ void unpack(const u32x4 t, float (&v)[8]) {
     const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -119,7 +120,7 @@ struct IO<bf16_t> {
       v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
     }
   }
-  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -127,7 +128,7 @@ struct IO<bf16_t> {
       w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, b16x2));
     }
     const u32x4 t = {w[0], w[1], w[2], w[3]};
-    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+    return t;
   }
   static __device__ __forceinline__ float load1(const bf16_t* p) {
     return __builtin_bit_cast(float, static_cast<uint32_t>(p->x) << 16);
@@ -136,6 +137,26 @@ struct IO<bf16_t> {
     p->x = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
   }
 };
+
+// One aligned 16-byte packet to and from HBM. Outputs are written once and not
+// read again by the same kernel, so stores carry the non-temporal hint.
+typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), may_alias));
+template <typename T>
+__device__ __forceinline__ u32x4 load_packet(const T* p) {
+  return *reinterpret_cast<const u32x4_any*>(p);
+}
+template <typename T>
+__device__ __forceinline__ void store_packet(T* p, const u32x4 t) {
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4_any*>(p));
+}
+template <typename T>
+__device__ __forceinline__ void load_unpack(const T* p, typename IO<T>::Acc (&v)[IO<T>::kVec]) {
+  IO<T>::unpack(load_packet(p), v);
+}
+template <typename T>
+__device__ __forceinline__ void pack_store(T* p, const typename IO<T>::Acc (&v)[IO<T>::kVec]) {
+  store_packet(p, IO<T>::pack(v));
+}
 
 // kVec consecutive accumulator-typed parameters (gamma, beta, ...), 16-byte
 // aligned at p.
@@ -192,55 +213,6 @@ __device__ __forceinline__ A block_allreduce(A v, Op op, A* slots) {
   A r = slots[0];
 #pragma unroll
   for (int i = 1; i < kWaves; ++i) r = op(r, slots[i]);
-  return r;
-}
-
-// Partial moments of a set of values: count, mean and M2 = sum (x - mean)^2.
-// merge() is Chan's pairwise update, the parallel form of Welford's
-// recurrence; it stays accurate when |mean| >> stddev, unlike E[x^2] - E[x]^2.
-template <typename A>
-struct Moments {
-  A n, mean, m2;
-  __device__ __forceinline__ void merge(const Moments& o) {
-    const A nn = n + o.n;
-    if (nn > A(0)) {
-      const A d = o.mean - mean;
-      const A f = o.n / nn;
-      mean += d * f;
-      m2 += o.m2 + d * d * n * f;
-      n = nn;
-    }
-  }
-};
-
-template <typename A, int kWidth = kWaveSize>
-__device__ __forceinline__ Moments<A> wave_allreduce_moments(Moments<A> v) {
-#pragma unroll
-  for (int o = kWidth / 2; o > 0; o >>= 1) {
-    Moments<A> t;
-    t.n = __shfl_xor(v.n, o, kWaveSize);
-    t.mean = __shfl_xor(v.mean, o, kWaveSize);
-    t.m2 = __shfl_xor(v.m2, o, kWaveSize);
-    v.merge(t);
-  }
-  return v;
-}
-
-template <int kWaves, typename A>
-__device__ __forceinline__ Moments<A> block_allreduce_moments(Moments<A> v, A* slots /*3*kWaves*/) {
-  v = wave_allreduce_moments(v);
-  if (kWaves == 1) return v;
-  const int wave = threadIdx.x / kWaveSize;
-  if ((threadIdx.x & (kWaveSize - 1)) == 0) {
-    slots[3 * wave] = v.n, slots[3 * wave + 1] = v.mean, slots[3 * wave + 2] = v.m2;
-  }
-  __syncthreads();
-  Moments<A> r = {slots[0], slots[1], slots[2]};
-#pragma unroll
-  for (int i = 1; i < kWaves; ++i) {
-    Moments<A> t = {slots[3 * i], slots[3 * i + 1], slots[3 * i + 2]};
-    r.merge(t);
-  }
   return r;
 }
 

@@ -185,82 +185,110 @@ struct GroupNormGradApply {
 // --------------------------------------------------------------------------
 // Fused row path (LayerNorm backward)
 // --------------------------------------------------------------------------
-constexpr int kGradThreads = 1024;
+constexpr int kGradThreads = 512;
 
-// partial[blockIdx][c][{dgamma, dbeta}]
+// Two 512-thread workgroups share a compute unit (128 registers per thread):
+// while one waits for its rows the other computes, which a single 1024-thread
+// workgroup with its barriers cannot do. gamma is staged in LDS once per
+// (persistent) workgroup; x and dy of a row are kept as raw packets;
+// dgamma / dbeta are accumulated per thread across the rows the workgroup
+// visits, combined across its row groups through LDS, and written as one
+// partial row per workgroup: partial[blockIdx][c][{dgamma, dbeta}].
+//
+// Per element, with the row scalars a = (db*mu - ds)*rsig^3/C, b = -db*rsig/C:
+//   xc = x - mu;  w = dy*rsig;  dgamma += w*xc;  dbeta += dy;
+//   dx = gamma*w + (a*xc + b)
 template <typename T, int kTPR, int kVPT>
-__global__ __launch_bounds__(kGradThreads) void layer_norm_grad_rows(
+__global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
     const int64_t N, const int C, const T* __restrict__ x, const T* __restrict__ dy,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
     const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
     typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
     typename IO<T>::Acc* __restrict__ partial) {
   using Tile = RowTile<T, kTPR, kVPT, kGradThreads>;
+  using Raw = RawRowTile<T, kTPR, kVPT, kGradThreads>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   constexpr int kGroups = Tile::kRowsPerBlock;
+  constexpr int kPerPacket = 16 / sizeof(A);
   // A round of the final cross-group combine moves kChunk (dgamma, dbeta) pairs per thread.
   constexpr int kChunk = kVec < 4 ? kVec : 4;
   constexpr int kRedWords = kGroups > 1 ? (kGroups - 1) * kTPR * kChunk * 2 : 1;
+  extern __shared__ u32x4 staged[];  // gamma[C]
   __shared__ A slots[2 * Tile::kSlots];
   __shared__ A red[kRedWords];
+  const A* lds_gamma = reinterpret_cast<const A*>(staged);
+  for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
+    staged[i] = load_packet(gamma + i * kPerPacket);
+  }
+  __syncthreads();
+
   const int npackets = C / kVec;
   const int lane = Tile::lane();
   const int sub = Tile::sub_row();
   const A inv_c = A(1) / A(C);
 
-  A g[kVPT][kVec], dg[kVPT][kVec], dbt[kVPT][kVec];
+  A dg[kVPT][kVec], dbt[kVPT][kVec];
 #pragma unroll
-  for (int i = 0; i < kVPT; ++i) {
-    if (Tile::active(i, npackets)) {
-      load_params<kVec>(gamma + (i * kTPR + lane) * kVec, g[i]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) g[i][e] = A(0);
-    }
+  for (int i = 0; i < kVPT; ++i)
 #pragma unroll
     for (int e = 0; e < kVec; ++e) dg[i][e] = dbt[i][e] = A(0);
-  }
 
   // Uniform trip count across the workgroup: the row reductions hold barriers.
   for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N;
        base += static_cast<int64_t>(gridDim.x) * kGroups) {
     const int64_t row = base + sub;
     const bool valid = row < N;
-    Tile tx, tdy;
-    tx.load(x + row * C, npackets, A(0), valid);
-    tdy.load(dy + row * C, npackets, A(0), valid);
+    Raw tx, tdy;
+    tx.load(x + row * C, npackets, valid);
+    tdy.load(dy + row * C, npackets, valid);
     const A m = valid ? mu[row] : A(0);
     const A r = valid ? rsig[row] : A(0);
 
     A s1 = A(0), s2 = A(0);
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i)
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        A xv[kVec], dv[kVec], g[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
+        load_params<kVec>(lds_gamma + (i * kTPR + lane) * kVec, g);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A t = g[i][e] * tdy.v[i][e];
-        s1 += t * tx.v[i][e];
-        s2 += t;
+        for (int e = 0; e < kVec; ++e) {
+          const A t = g[e] * dv[e];
+          s1 += t * xv[e];
+          s2 += t;
+        }
       }
+    }
     Tile::reduce_sum_pair(s1, s2, slots);
     if (lane == 0 && valid) {
       ds[row] = s1;
       db[row] = s2;
     }
 
-    const A u0 = (s2 * m - s1) * (r * r * r);
-    const A v0 = s2 * r;
+    const A a = (s2 * m - s1) * (r * r * r) * inv_c;
+    const A b = -(s2 * r) * inv_c;
+    tx.refresh();
+    tdy.refresh();
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i)
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        A xv[kVec], dv[kVec], g[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
+        load_params<kVec>(lds_gamma + (i * kTPR + lane) * kVec, g);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A xc = tx.v[i][e] - m;
-        const A d = tdy.v[i][e];
-        dg[i][e] += d * xc * r;
-        dbt[i][e] += d;
-        tx.v[i][e] = g[i][e] * d * r + (u0 * xc - v0) * inv_c;
+        for (int e = 0; e < kVec; ++e) {
+          const A xc = xv[e] - m;
+          const A w = dv[e] * r;
+          dg[i][e] += w * xc;
+          dbt[i][e] += dv[e];
+          xv[e] = g[e] * w + (a * xc + b);
+        }
+        if (valid) tx.store_slot(dx + row * C, i, xv);
       }
-    tx.store(dx + row * C, npackets, valid);
+    }
     if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
   }
 
@@ -308,6 +336,182 @@ __global__ __launch_bounds__(kGradThreads) void layer_norm_grad_rows(
   }
 }
 
+// --------------------------------------------------------------------------
+// Fused group paths (NCHW): a group's D*S elements are contiguous, so a group
+// is a row of width L = D*S whose affine parameters change every S elements.
+// --------------------------------------------------------------------------
+
+// Moments -> InvStd -> GroupNorm in one pass over x: the group stays in
+// registers between the statistics and the normalisation.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const int npackets = L / kVec;
+  const A inv_l = A(1) / A(L);
+  const int lane = Tile::lane();
+
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Raw t;
+    t.load(x + row * L, npackets);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      t.unpack(i, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += v[e];
+    }
+    const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_l;
+    t.refresh();
+    A q = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        A v[kVec];
+        t.unpack(i, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A d = v[e] - mean;
+          q += d * d;
+        }
+      }
+    }
+    const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_l;
+    const A rs = acc_rsqrt_exact(var + eps);
+    if (lane == 0) {
+      mu[row] = mean;
+      rsig[row] = rs;
+    }
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+    t.refresh();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
+        const uint32_t c = c0 + col / S;  // a packet lies in one channel: kVec divides S
+        const A gam = gamma[c] * rs, bet = beta[c];
+        A v[kVec];
+        t.unpack(i, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+        t.store_slot(y + row * L, i, v);
+      }
+    }
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// GroupNormGrad in one pass over x and dy: one workgroup per group keeps both
+// as raw packets. Requires S to be a multiple of 64 packets, so that every
+// (slot, wavefront) pair lies in one channel and the per-channel sums are a
+// wave reduction plus a fixed-order sum over LDS entries.
+// partial[(n*C + c)*2 + {0,1}] receives this group's share of dgamma / dbeta.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const T* __restrict__ x, const T* __restrict__ dy,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
+    const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
+    typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  constexpr int kWaves = kTPR / kWaveSize;
+  __shared__ A slots[2 * Tile::kSlots];
+  __shared__ A chan_part[kVPT][kWaves][2];
+  const int npackets = L / kVec;
+  const uint32_t packets_per_chan = S / kVec;
+  const A denom = A(1) / A(L);
+  const int lane = threadIdx.x;
+  const int wave = threadIdx.x / kWaveSize;
+
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    Raw tx, tdy;
+    tx.load(x + row * L, npackets);
+    tdy.load(dy + row * L, npackets);
+    const A m = mu[row], r = rsig[row];
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+
+    A gam[kVPT];
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const uint32_t chan = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) / packets_per_chan;
+      gam[i] = Tile::active(i, npackets) ? gamma[c0 + chan] : A(0);
+      A xv[kVec], dv[kVec];
+      tx.unpack(i, xv);
+      tdy.unpack(i, dv);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A t = gam[i] * dv[e];
+        s1 += t * xv[e];
+        s2 += t;
+      }
+    }
+    Tile::reduce_sum_pair(s1, s2, slots);
+    if (lane == 0) {
+      ds[row] = s1;
+      db[row] = s2;
+    }
+    const A u0 = (s2 * m - s1) * (r * r * r);
+    const A v0 = s2 * r;
+    tx.refresh();
+    tdy.refresh();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A xv[kVec], dv[kVec];
+      tx.unpack(i, xv);
+      tdy.unpack(i, dv);
+      A t1 = A(0), t2 = A(0);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A xc = xv[e] - m;
+        t1 += dv[e] * xc * r;
+        t2 += dv[e];
+        xv[e] = gam[i] * dv[e] * r + (u0 * xc - v0) * denom;
+      }
+      if (Tile::active(i, npackets)) tx.store_slot(dx + row * L, i, xv);
+      t1 = wave_allreduce(t1, SumOp());
+      t2 = wave_allreduce(t2, SumOp());
+      if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+        chan_part[i][wave][0] = t1;
+        chan_part[i][wave][1] = t2;
+      }
+    }
+    __syncthreads();
+    if (static_cast<uint32_t>(lane) < D) {
+      // Entry q = (slot, wavefront) covers packets [64 q, 64 q + 64); channel
+      // `lane` owns the entries [lane * waves_per_chan, (lane + 1) * waves_per_chan).
+      A a = A(0), b = A(0);
+      const A* entries = &chan_part[0][0][0];
+      const uint32_t waves_per_chan = packets_per_chan / kWaveSize;
+      const uint32_t q0 = static_cast<uint32_t>(lane) * waves_per_chan;
+#pragma nounroll
+      for (uint32_t q = q0; q < q0 + waves_per_chan; ++q) {
+        a += entries[2 * q];
+        b += entries[2 * q + 1];
+      }
+      const size_t n = static_cast<size_t>(row / G);
+      A* o = partial + (n * G * D + c0 + lane) * 2;
+      o[0] = a;
+      o[1] = b;
+    }
+    __syncthreads();  // chan_part and slots are reused by the next group
+  }
+}
+
 // Sums P partial rows of 2*C interleaved (dgamma, dbeta) words. A workgroup of
 // 16 wavefronts owns 64 adjacent words; wavefront w adds rows w, w+16, ...
 template <typename A>
@@ -344,20 +548,21 @@ struct RowGradPlan {
   unsigned grid;
 };
 
-// The fused row path holds x, dy, gamma and two gradient accumulators per
-// thread, and a 1024-thread workgroup leaves 128 registers per thread: tiles
-// are limited to 16 elements per thread (8 for fp64), fewest packets first.
+// Tiles of the fused row path: the fewest threads per row that hold it, at most
+// 32 accumulated elements per thread (two accumulators each).
 template <typename T>
 RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
   RowGradPlan p = {false, {0, 0}, 0};
   if (G != 1 || S != 1) return p;
   constexpr int kVec = IO<T>::kVec;
-  constexpr int kMaxElems = sizeof(typename IO<T>::Acc) == 8 ? 8 : 16;
-  if (D % kVec != 0) return p;
-  static const RowConfig table[] = {{64, 1}, {64, 2}, {256, 1}, {256, 2}, {1024, 1}, {1024, 2}, {1024, 4}};
+  if (D % kVec != 0 || static_cast<size_t>(D) * sizeof(typename IO<T>::Acc) > kMaxStagedParamBytes / 2) {
+    return p;
+  }
+  static const RowConfig table[] = {{64, 1}, {64, 2}, {256, 1}, {256, 2},
+                                    {512, 1}, {512, 2}, {512, 3}, {512, 4}};
   bool found = false;
   for (const RowConfig& c : table) {
-    if (c.vpt * kVec <= kMaxElems && D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
+    if (D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
       p.cfg = c;
       found = true;
       break;
@@ -366,10 +571,28 @@ RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
   if (!found) return p;
   const int64_t groups = kGradThreads / p.cfg.tpr;
   const int64_t want = ceil_div(N, groups);
-  const int64_t cap = kNumCUs * 2;
+  const int64_t cap = kNumCUs * 2;  // two resident workgroups per compute unit
   p.grid = static_cast<unsigned>(want < cap ? want : cap);
   p.use_rows = true;
   return p;
+}
+
+// Fused group backward applies to NCHW groups that fit a multi-wave register
+// tile and whose channels span whole wavefronts of packets.
+template <typename T>
+bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig* cfg) {
+  constexpr int kVec = IO<T>::kVec;
+  if (layout != DRAGON_HIP_NCHW || G * D == 1) return false;
+  if (S % (kWaveSize * kVec) != 0) return false;
+  static const RowConfig table[] = {{256, 2}, {256, 4}, {256, 8}, {1024, 4}, {1024, 8}};
+  const int64_t npackets = D * S / kVec;
+  for (const RowConfig& c : table) {
+    if (npackets <= static_cast<int64_t>(c.tpr) * c.vpt) {
+      *cfg = c;
+      return true;
+    }
+  }
+  return false;
 }
 
 template <typename T>
@@ -384,7 +607,42 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
       ? pick_split(C, N * S)
       : pick_split(ceil_div(C, kWaveSize), N * S * kWaveSize);
   const size_t wbytes = static_cast<size_t>(C) * split_c * 2 * sizeof(A);
-  return bytes > wbytes ? bytes : wbytes;
+  if (wbytes > bytes) bytes = wbytes;
+  RowConfig cfg;
+  if (plan_group_grad_rows<T>(G, D, S, layout, &cfg)) {
+    const size_t fbytes = static_cast<size_t>(N) * C * 2 * sizeof(A);
+    if (fbytes > bytes) bytes = fbytes;
+  }
+  return bytes;
+}
+
+// Fused forward: true when the register-resident kernel was launched.
+template <typename T>
+bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x, const void* gamma,
+                                 const void* beta, void* mu, void* rsig, void* y,
+                                 hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  RowConfig cfg;
+  const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
+  if (!sh.nchw || sh.S % kVec != 0 || !aligned16(x) || !aligned16(y) ||
+      !pick_row_config(L / kVec, 8, &cfg)) {
+    return false;
+  }
+  const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    using Tile = RowTile<T, TPR, VPT>;                                                          \
+    hipLaunchKernelGGL((group_norm_forward_rows<T, TPR, VPT>),                                  \
+                       dim3(row_grid(rows, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),                     \
+                       static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig), \
+                       static_cast<T*>(y));                                                     \
+  }
+  DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+  return true;
 }
 
 template <typename T>
@@ -435,20 +693,46 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 
   const RowGradPlan rp = plan_row_grad<T>(sh.N, sh.G, sh.D, sh.S);
   if (rp.use_rows && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma)) {
-#define LAUNCH(TPR, VPT)                                                                         \
-  hipLaunchKernelGGL((layer_norm_grad_rows<T, TPR, VPT>), dim3(rp.grid), dim3(kGradThreads), 0, \
-                     stream, static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp,   \
-                     mup, rsp, dsp, dbp, dxp, part);
+    const size_t staged_bytes = static_cast<size_t>(sh.D) * sizeof(A);
+#define LAUNCH(TPR, VPT)                                                                      \
+  {                                                                                           \
+    auto kernel = layer_norm_grad_rows<T, TPR, VPT>;                                          \
+    if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, kGradThreads, staged_bytes);    \
+    hipLaunchKernelGGL(kernel, dim3(rp.grid), dim3(kGradThreads), staged_bytes, stream,       \
+                       static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp, mup,  \
+                       rsp, dsp, dbp, dxp, part);                                             \
+  }
     if (rp.cfg.tpr == 64 && rp.cfg.vpt == 1) LAUNCH(64, 1)
     else if (rp.cfg.tpr == 64 && rp.cfg.vpt == 2) LAUNCH(64, 2)
     else if (rp.cfg.tpr == 256 && rp.cfg.vpt == 1) LAUNCH(256, 1)
     else if (rp.cfg.tpr == 256 && rp.cfg.vpt == 2) LAUNCH(256, 2)
-    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 1) LAUNCH(1024, 1)
-    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 2) LAUNCH(1024, 2)
-    else if constexpr (IO<T>::kVec <= 4) LAUNCH(1024, 4)
+    else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 1) LAUNCH(512, 1)
+    else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 2) LAUNCH(512, 2)
+    else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 3) LAUNCH(512, 3)
+    else LAUNCH(512, 4)
 #undef LAUNCH
     hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
                        dim3(1024), 0, stream, rp.grid, sh.D, part, dgp, dbtp);
+    return status_of_launch();
+  }
+
+  RowConfig gcfg;
+  if (plan_group_grad_rows<T>(sh.G, sh.D, sh.S, layout, &gcfg) && aligned16(x) && aligned16(dy) &&
+      aligned16(dx)) {
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+    const int L = static_cast<int>(sh.D * sh.S);
+    const unsigned grid = static_cast<unsigned>(rows < (1 << 20) ? rows : (1 << 20));
+#define LAUNCH(TPR, VPT)                                                                       \
+  hipLaunchKernelGGL((group_norm_grad_rows<T, TPR, VPT>), dim3(grid), dim3(TPR), 0, stream, rows, \
+                     L, sh.G, sh.D, sh.S, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);
+    if (gcfg.tpr == 256 && gcfg.vpt == 2) LAUNCH(256, 2)
+    else if (gcfg.tpr == 256 && gcfg.vpt == 4) LAUNCH(256, 4)
+    else if (gcfg.tpr == 256 && gcfg.vpt == 8) LAUNCH(256, 8)
+    else if (gcfg.tpr == 1024 && gcfg.vpt == 4) LAUNCH(1024, 4)
+    else LAUNCH(1024, 8)
+#undef LAUNCH
+    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.C, kWaveSize))),
+                       dim3(1024), 0, stream, sh.N, sh.C, part, dgp, dbtp);
     return status_of_launch();
   }
 
@@ -636,6 +920,25 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
   if (st != DRAGON_HIP_OK) return st;
   if (N * S == 0) return DRAGON_HIP_OK;
   if (!x || !gamma || !beta || !mu || !rsig || !y) return DRAGON_HIP_EINVAL;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  bool fused = false;
+  switch (dtype) {
+    case DRAGON_HIP_F16:
+      fused = dragon_hip::try_group_norm_forward_rows<dragon_hip::f16_t>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+      break;
+    case DRAGON_HIP_BF16:
+      fused = dragon_hip::try_group_norm_forward_rows<dragon_hip::bf16_t>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+      break;
+    case DRAGON_HIP_F32:
+      fused = dragon_hip::try_group_norm_forward_rows<float>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+      break;
+    case DRAGON_HIP_F64:
+      fused = dragon_hip::try_group_norm_forward_rows<double>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+      break;
+    default:
+      return DRAGON_HIP_EDTYPE;
+  }
+  if (fused) return dragon_hip::status_of_launch();
   const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
   st = dragon_hip_moments(dtype, v.num_dims, v.dims, v.num_axes, v.axes, x, mu, rsig, scratch,
                           scratch_bytes, stream);

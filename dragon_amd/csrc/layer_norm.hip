@@ -76,6 +76,90 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
   }
 }
 
+// Rows spanning several wavefronts: gamma and beta no longer fit the 32 KB L1
+// next to the streamed rows, and re-reading them from L2 for every row would
+// move more bytes than the row itself (fp32 parameters against 16-bit data).
+// A persistent workgroup stages both in LDS once and then walks its rows; the
+// 1024-thread tile, of which a compute unit holds few, also requests the next
+// row's packets before it reduces the current row.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
+    const int64_t N, const int C, const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  constexpr int kPerPacket = 16 / sizeof(A);  // parameters per 16-byte LDS word
+  constexpr bool kPrefetch = kTPR == 1024;
+  extern __shared__ u32x4 staged[];  // gamma[C] then beta[C]
+  __shared__ A slots[2][Tile::kSlots];
+  A* lds_gamma = reinterpret_cast<A*>(staged);
+  A* lds_beta = lds_gamma + C;
+  for (int i = threadIdx.x; i < C / kPerPacket; i += kTPR) {
+    staged[i] = load_packet(gamma + i * kPerPacket);
+    staged[C / kPerPacket + i] = load_packet(beta + i * kPerPacket);
+  }
+  __syncthreads();
+
+  const int npackets = C / kVec;
+  const A inv_c = A(1) / A(C);
+  const int lane = threadIdx.x;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  Raw cur;
+  if (kPrefetch) cur.load(x + row * C, npackets, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    if (kPrefetch) {
+      nxt.load(x + (row + stride) * C, npackets, row + stride < N);
+    } else {
+      cur.load(x + row * C, npackets);
+    }
+    Tile t;
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      cur.unpack(i, t.v[i]);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += t.v[i][e];
+    }
+    const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_c;
+    A q = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A d = t.v[i][e] - mean;
+          q += d * d;
+        }
+      }
+    }
+    const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_c;
+    const A rs = acc_rsqrt_exact(var + eps);
+    if (lane == 0) {
+      mu[row] = mean;
+      rsig[row] = rs;
+    }
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        const int col = (i * kTPR + lane) * kVec;
+        A g[kVec], b[kVec];
+        load_params<kVec>(lds_gamma + col, g);
+        load_params<kVec>(lds_beta + col, b);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * rs * g[e] + b[e];
+      }
+    }
+    t.store(y + row * C, npackets);
+    if (kPrefetch) cur = nxt;
+  }
+}
+
 // Any width, any alignment: one 256-thread workgroup per row, three strided
 // passes over the row with element-wise accesses (the second and third hit L2).
 template <typename T>
@@ -124,8 +208,33 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
   A* rp = static_cast<A*>(rsig);
   RowConfig cfg;
   const bool packets_ok = C % kVec == 0 && aligned16(x) && aligned16(y) && aligned16(gamma) &&
-      aligned16(beta) && pick_row_config(C / kVec, &cfg);
-  if (packets_ok) {
+      aligned16(beta) && pick_row_config(C / kVec, 8, &cfg);
+  const size_t staged_bytes = 2 * static_cast<size_t>(C) * sizeof(A);
+  if (packets_ok && cfg.tpr > kWaveSize && staged_bytes <= kMaxStagedParamBytes) {
+    // 256-thread tiles need several workgroups per compute unit to hide HBM
+    // latency; when the staged parameters leave room for fewer than four, use
+    // the 1024-thread tile (which prefetches instead).
+    if (cfg.tpr == 256 && staged_bytes * 4 > kMaxStagedParamBytes) {
+      const int64_t need = ceil_div(C / kVec, 1024);
+      cfg.tpr = 1024;
+      cfg.vpt = need <= 2 ? 2 : (need <= 4 ? 4 : 8);
+    }
+#define LAUNCH(TPR, VPT)                                                                     \
+  {                                                                                          \
+    auto kernel = layer_norm_wide_rows<T, TPR, VPT>;                                         \
+    const unsigned resident = resident_grid(kernel, TPR, staged_bytes);                      \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), staged_bytes, stream, N,               \
+                       static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);                 \
+  }
+    if (cfg.tpr == 256 && cfg.vpt == 2) LAUNCH(256, 2)
+    else if (cfg.tpr == 256 && cfg.vpt == 4) LAUNCH(256, 4)
+    else if (cfg.tpr == 256 && cfg.vpt == 8) LAUNCH(256, 8)
+    else if (cfg.tpr == 1024 && cfg.vpt == 2) LAUNCH(1024, 2)
+    else if (cfg.tpr == 1024 && cfg.vpt == 4) LAUNCH(1024, 4)
+    else LAUNCH(1024, 8)
+#undef LAUNCH
+  } else if (packets_ok) {
 #define LAUNCH(TPR, VPT)                                                                   \
   {                                                                                        \
     using Tile = RowTile<T, TPR, VPT>;                                                     \

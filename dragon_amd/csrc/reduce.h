@@ -105,8 +105,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_segments(
       x0[0] = IO<T>::load1(in0 + off);
       x1[0] = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
     } else {
-      IO<T>::load(in0 + off, x0);
-      if constexpr (kIn == 2) IO<T>::load(in1 + off, x1);
+      load_unpack<T>(in0 + off, x0);
+      if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
     }
     f.add(o, seg, p, off, x0, x1, a, b);
   }
@@ -196,14 +196,14 @@ __global__ __launch_bounds__(256) void map_flat(const uint32_t total, const T* i
       v0[0] = IO<T>::load1(in0 + i);
       v1[0] = kIn == 2 ? IO<T>::load1(in1 + i) : A(0);
     } else {
-      IO<T>::load(in0 + i, v0);
-      if constexpr (kIn == 2) IO<T>::load(in1 + i, v1);
+      load_unpack<T>(in0 + i, v0);
+      if constexpr (kIn == 2) load_unpack<T>(in1 + i, v1);
     }
     f(i, v0, v1);
     if constexpr (kVec == 1) {
       IO<T>::store1(out + i, v0[0]);
     } else {
-      IO<T>::store(out + i, v0);
+      pack_store<T>(out + i, v0);
     }
   }
 }

@@ -48,7 +48,7 @@ struct RowTile {
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       if (valid && active(s, npackets)) {
-        IO<T>::load(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
+        load_unpack<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
       } else {
 #pragma unroll
         for (int e = 0; e < kVec; ++e) v[s][e] = fill;
@@ -60,7 +60,7 @@ struct RowTile {
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       if (valid && active(s, npackets)) {
-        IO<T>::store(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
+        pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
       }
     }
   }
@@ -102,17 +102,59 @@ struct RowTile {
   }
 };
 
-// Picks the smallest tile that holds `npackets` packets. Returns false when
-// the row is too long for registers (the caller then uses its looping kernel).
-// Order: wave-per-row while a lane holds at most 4 packets, then a 256-thread
-// workgroup, then 1024 threads.
+// The same tile kept as raw packets (four dwords each): half the registers of
+// the unpacked form for 16-bit types, at the price of converting again on
+// every pass over the tile. Used where several tiles are live at once or the
+// next row is prefetched while the current one is processed.
+template <typename T, int kTPR, int kVPT, int kThreadsT = row_threads(kTPR)>
+struct RawRowTile {
+  using A = typename IO<T>::Acc;
+  static constexpr int kVec = IO<T>::kVec;
+  u32x4 p[kVPT];
+
+  static __device__ __forceinline__ int lane() { return threadIdx.x % kTPR; }
+  static __device__ __forceinline__ bool active(int slot, int npackets) {
+    return slot * kTPR + lane() < npackets;
+  }
+  // Inactive slots hold zero bits, i.e. +0.0 in every element type.
+  __device__ __forceinline__ void load(const T* row, int npackets, bool valid = true) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      if (valid && active(s, npackets)) {
+        p[s] = load_packet(row + static_cast<int64_t>(s * kTPR + lane()) * kVec);
+      } else {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        p[s] = z;
+      }
+    }
+  }
+  __device__ __forceinline__ void unpack(int s, A (&v)[kVec]) const { IO<T>::unpack(p[s], v); }
+  // Called between two passes over the tile: makes the compiler treat the
+  // packets as new values, so it converts them again in the next pass instead
+  // of keeping every converted element of the previous pass in registers.
+  __device__ __forceinline__ void refresh() {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) asm volatile("" : "+v"(p[s]));
+  }
+  __device__ __forceinline__ void store_slot(T* row, int s, const A (&v)[kVec]) const {
+    pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v);
+  }
+};
+
+// Picks the tile for a row of `npackets` packets: the fewest threads per row
+// whose tile still holds it, because short rows on few threads leave many rows
+// in flight per compute unit (wave-per-row up to 4 packets per lane, then a
+// 256-thread workgroup, then 1024 threads). `max_vpt` bounds the packets a
+// thread of a multi-wave tile may hold (kernels with two live tiles pass 4).
+// Returns false when the row is too long for registers.
 struct RowConfig {
   int tpr, vpt;
 };
-inline bool pick_row_config(int64_t npackets, RowConfig* cfg) {
-  static const RowConfig table[] = {{64, 1},  {64, 2},  {64, 4},   {256, 2},
-                                    {256, 4}, {1024, 2}, {1024, 4}, {1024, 8}};
+inline bool pick_row_config(int64_t npackets, int max_vpt, RowConfig* cfg) {
+  static const RowConfig table[] = {{64, 1},  {64, 2},  {64, 4},   {256, 2},  {256, 4},
+                                    {256, 8}, {1024, 2}, {1024, 4}, {1024, 8}};
   for (const RowConfig& c : table) {
+    if (c.vpt > max_vpt) continue;
     if (npackets <= static_cast<int64_t>(c.tpr) * c.vpt) {
       *cfg = c;
       return true;
@@ -121,16 +163,40 @@ inline bool pick_row_config(int64_t npackets, RowConfig* cfg) {
   return false;
 }
 
-// Instantiates LAUNCH(T, tpr, vpt) for the tile pick_row_config chose.
-#define DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH)                 \
-  if (cfg.tpr == 64 && cfg.vpt == 1) LAUNCH(64, 1)         \
-  else if (cfg.tpr == 64 && cfg.vpt == 2) LAUNCH(64, 2)    \
-  else if (cfg.tpr == 64 && cfg.vpt == 4) LAUNCH(64, 4)    \
-  else if (cfg.tpr == 256 && cfg.vpt == 2) LAUNCH(256, 2)  \
-  else if (cfg.tpr == 256 && cfg.vpt == 4) LAUNCH(256, 4)  \
+// Instantiates LAUNCH(tpr, vpt) for the tile pick_row_config chose.
+#define DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH)                  \
+  if (cfg.tpr == 64 && cfg.vpt == 1) LAUNCH(64, 1)          \
+  else if (cfg.tpr == 64 && cfg.vpt == 2) LAUNCH(64, 2)     \
+  else if (cfg.tpr == 64 && cfg.vpt == 4) LAUNCH(64, 4)     \
+  else if (cfg.tpr == 256 && cfg.vpt == 2) LAUNCH(256, 2)   \
+  else if (cfg.tpr == 256 && cfg.vpt == 4) LAUNCH(256, 4)   \
+  else if (cfg.tpr == 256 && cfg.vpt == 8) LAUNCH(256, 8)   \
   else if (cfg.tpr == 1024 && cfg.vpt == 2) LAUNCH(1024, 2) \
   else if (cfg.tpr == 1024 && cfg.vpt == 4) LAUNCH(1024, 4) \
   else LAUNCH(1024, 8)
+
+// Workgroups of `kernel` (block size `threads`, `dynamic_lds` bytes of dynamic
+// LDS) that can be resident on the whole device at once: the grid of a
+// persistent kernel. Also raises the kernel's dynamic-LDS limit when needed.
+template <typename Kernel>
+inline unsigned resident_grid(Kernel kernel, int threads, size_t dynamic_lds) {
+  if (dynamic_lds > 48 * 1024) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(dynamic_lds));
+  }
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) !=
+          hipSuccess ||
+      per_cu < 1) {
+    (void)hipGetLastError();
+    per_cu = 1;
+  }
+  return static_cast<unsigned>(per_cu) * kNumCUs;
+}
+
+// LDS a workgroup may use for staged parameters (of 160 KB per compute unit).
+constexpr size_t kMaxStagedParamBytes = 144 * 1024;
 
 // Workgroups for a row kernel: enough to cover every row once, capped so a
 // grid-stride loop picks up the rest.

@@ -261,7 +261,8 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   RowConfig cfg;
-  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(y) && pick_row_config(C / kVec, &cfg)) {
+  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(y) &&
+      pick_row_config(C / kVec, 8, &cfg)) {
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
@@ -291,7 +292,7 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   RowConfig cfg;
   // Two tiles live at once: halve the packets a thread may hold.
   if (S == 1 && C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx) &&
-      pick_row_config(C / kVec, &cfg) && !(cfg.tpr == 1024 && cfg.vpt == 8)) {
+      pick_row_config(C / kVec, 4, &cfg)) {
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \

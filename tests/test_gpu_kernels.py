@@ -228,7 +228,10 @@ def test_layer_norm_backward(K, dtype, shape):
 # ---------------------------------------------------------------- GroupNorm
 
 GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), ((3, 5, 12), -1, 3),
-            ((2, 64, 16, 16), 1, 32), ((4, 8), -1, 2), ((2, 16, 4, 4), 1, 0), ((1, 4, 2), 1, 2)]
+            ((2, 64, 16, 16), 1, 32), ((4, 8), -1, 2), ((2, 16, 4, 4), 1, 0), ((1, 4, 2), 1, 2),
+            # groups that take the register-resident fused kernels
+            ((2, 32, 32, 32), 1, 4), ((2, 16, 64, 64), 1, 2), ((3, 6, 32, 16), 1, 3),
+            ((2, 8, 64, 128), 1, 8), ((1, 4, 128, 128), 1, 2)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
