@@ -72,6 +72,7 @@ SIGNATURES = {
     "dragon_hip_batch_norm_training_forward": (_int, [_int, _i64, _i64, _i64, _int, _f32, _f32,
                                                       _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                                       _vp, _sz, _vp]),
+    "dragon_hip_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
 }
 
 _lib = None

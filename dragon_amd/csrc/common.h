@@ -192,12 +192,36 @@ struct MaxOp {
   }
 };
 
-// Butterfly all-reduce over the 64 lanes of a wavefront: every lane ends up
-// with the result. kWidth < 64 reduces within aligned lane groups.
-template <typename A, typename Op, int kWidth = kWaveSize>
-__device__ __forceinline__ A wave_allreduce(A v, Op op) {
+// One data-parallel-primitive step: every lane combines its value with the
+// value of the lane the DPP control selects (the cross-lane move happens in the
+// VALU operand path, without the LDS crossbar a shuffle would use).
+template <int kCtrl, typename Op>
+__device__ __forceinline__ float dpp_step(float v, Op op) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xf, 0xf, false);
+  return op(v, __builtin_bit_cast(float, moved));
+}
+
+// All-reduce over the 64 lanes of a wavefront: every lane ends up with the
+// result. fp32: four DPP steps reduce each row of 16 lanes (swap within pairs,
+// swap pairs within quads, mirror within 8, mirror within 16), then the four
+// row results are read into scalar registers and combined. fp64 uses the
+// butterfly of shuffles.
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v, Op op) {
+  v = dpp_step<0xB1>(v, op);   // quad_perm [1,0,3,2]
+  v = dpp_step<0x4E>(v, op);   // quad_perm [2,3,0,1]
+  v = dpp_step<0x141>(v, op);  // row_half_mirror
+  v = dpp_step<0x140>(v, op);  // row_mirror
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return op(op(r0, r1), op(r2, r3));
+}
+template <typename Op>
+__device__ __forceinline__ double wave_allreduce(double v, Op op) {
 #pragma unroll
-  for (int o = kWidth / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, kWaveSize));
+  for (int o = kWaveSize / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, kWaveSize));
   return v;
 }
 

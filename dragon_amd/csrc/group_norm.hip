@@ -23,6 +23,8 @@
 //          through LDS, written as one partial row per workgroup, and summed
 //          by a second small kernel (two-stage, no atomics).
 //   general  three split reductions / one flat map, any layout, any alignment.
+#include <cstdlib>
+
 #include "reduce.h"
 #include "row_tile.h"
 
@@ -185,7 +187,6 @@ struct GroupNormGradApply {
 // --------------------------------------------------------------------------
 // Fused row path (LayerNorm backward)
 // --------------------------------------------------------------------------
-constexpr int kGradThreads = 512;
 
 // Two 512-thread workgroups share a compute unit (128 registers per thread):
 // while one waits for its rows the other computes, which a single 1024-thread
@@ -198,7 +199,7 @@ constexpr int kGradThreads = 512;
 // Per element, with the row scalars a = (db*mu - ds)*rsig^3/C, b = -db*rsig/C:
 //   xc = x - mu;  w = dy*rsig;  dgamma += w*xc;  dbeta += dy;
 //   dx = gamma*w + (a*xc + b)
-template <typename T, int kTPR, int kVPT>
+template <typename T, int kTPR, int kVPT, int kGradThreads>
 __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
     const int64_t N, const int C, const T* __restrict__ x, const T* __restrict__ dy,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
@@ -234,16 +235,26 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
 #pragma unroll
     for (int e = 0; e < kVec; ++e) dg[i][e] = dbt[i][e] = A(0);
 
-  // Uniform trip count across the workgroup: the row reductions hold barriers.
-  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N;
-       base += static_cast<int64_t>(gridDim.x) * kGroups) {
-    const int64_t row = base + sub;
+  // The next row's packets are requested before the current row is reduced, so
+  // its HBM latency hides behind this row's arithmetic. Uniform trip count
+  // across the workgroup: the row reductions hold barriers.
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
+  int64_t row = static_cast<int64_t>(blockIdx.x) * kGroups + sub;
+  // Rows past the end are clamped to row 0 for addressing and masked off.
+  Raw tx, tdy;
+  tx.load(x + (row < N ? row : 0) * C, npackets, row < N);
+  tdy.load(dy + (row < N ? row : 0) * C, npackets, row < N);
+  A m = mu[row < N ? row : 0];
+  A r = rsig[row < N ? row : 0];
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N; base += stride) {
     const bool valid = row < N;
-    Raw tx, tdy;
-    tx.load(x + row * C, npackets, valid);
-    tdy.load(dy + row * C, npackets, valid);
-    const A m = valid ? mu[row] : A(0);
-    const A r = valid ? rsig[row] : A(0);
+    const int64_t next = row + stride;
+    const bool next_valid = next < N;
+    Raw nx, ndy;
+    nx.load(x + (next_valid ? next : 0) * C, npackets, next_valid);
+    ndy.load(dy + (next_valid ? next : 0) * C, npackets, next_valid);
+    const A nm = mu[next_valid ? next : 0];
+    const A nr = rsig[next_valid ? next : 0];
 
     A s1 = A(0), s2 = A(0);
 #pragma unroll
@@ -271,25 +282,40 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
     const A b = -(s2 * r) * inv_c;
     tx.refresh();
     tdy.refresh();
+    u32x4 out[kVPT];
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
+      A xv[kVec], dv[kVec], g[kVec];
+      tx.unpack(i, xv);
+      tdy.unpack(i, dv);
       if (Tile::active(i, npackets)) {
-        A xv[kVec], dv[kVec], g[kVec];
-        tx.unpack(i, xv);
-        tdy.unpack(i, dv);
         load_params<kVec>(lds_gamma + (i * kTPR + lane) * kVec, g);
+      } else {
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) {
-          const A xc = xv[e] - m;
-          const A w = dv[e] * r;
-          dg[i][e] += w * xc;
-          dbt[i][e] += dv[e];
-          xv[e] = g[e] * w + (a * xc + b);
-        }
-        if (valid) tx.store_slot(dx + row * C, i, xv);
+        for (int e = 0; e < kVec; ++e) g[e] = A(0);
+      }
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A xc = xv[e] - m;
+        const A w = dv[e] * r;
+        dg[i][e] += w * xc;  // masked slots hold dy = 0: they add nothing
+        dbt[i][e] += dv[e];
+        xv[e] = g[e] * w + (a * xc + b);
+      }
+      out[i] = IO<T>::pack(xv);
+    }
+    // Wait for the prefetched row here, before this row's stores are issued.
+    nx.wait_ready();
+    ndy.wait_ready();
+    T* dxr = dx + (valid ? row : 0) * C;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (valid && Tile::active(i, npackets)) {
+        store_packet(dxr + static_cast<int64_t>(i * kTPR + lane) * kVec, out[i]);
       }
     }
     if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
+    tx = nx, tdy = ndy, m = nm, r = nr, row = next;
   }
 
   // Combine the kGroups row groups of this workgroup, kChunk pairs at a time.
@@ -545,33 +571,37 @@ __global__ __launch_bounds__(1024) void sum_partial_rows(const uint32_t P, const
 struct RowGradPlan {
   bool use_rows;
   RowConfig cfg;
+  int threads;  // workgroup size: 512 (two per compute unit) or 1024 (one)
   unsigned grid;
 };
 
-// Tiles of the fused row path: the fewest threads per row that hold it, at most
-// 32 accumulated elements per thread (two accumulators each).
+// Tiles of the fused row path: the fewest threads per row that hold it with at
+// most 16 elements per thread (two raw tiles for the current row, two for the
+// prefetched one and two accumulator sets must fit 128 registers).
 template <typename T>
 RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
-  RowGradPlan p = {false, {0, 0}, 0};
+  RowGradPlan p = {false, {0, 0}, 512, 0};
   if (G != 1 || S != 1) return p;
   constexpr int kVec = IO<T>::kVec;
+  constexpr int kMaxVpt = kVec == 8 ? 2 : 4;
   if (D % kVec != 0 || static_cast<size_t>(D) * sizeof(typename IO<T>::Acc) > kMaxStagedParamBytes / 2) {
     return p;
   }
-  static const RowConfig table[] = {{64, 1}, {64, 2}, {256, 1}, {256, 2},
-                                    {512, 1}, {512, 2}, {512, 3}, {512, 4}};
+  static const RowConfig table[] = {{64, 1},  {64, 2},  {256, 1},  {256, 2}, {512, 1},
+                                    {512, 2}, {1024, 1}, {1024, 2}, {1024, 4}};
   bool found = false;
   for (const RowConfig& c : table) {
-    if (D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
+    if (!found && c.vpt <= kMaxVpt && D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
       p.cfg = c;
       found = true;
-      break;
     }
   }
   if (!found) return p;
-  const int64_t groups = kGradThreads / p.cfg.tpr;
+  p.threads = p.cfg.tpr == 1024 ? 1024 : 512;
+  const int per_cu = p.threads == 512 ? 2 : 1;
+  const int64_t groups = p.threads / p.cfg.tpr;
   const int64_t want = ceil_div(N, groups);
-  const int64_t cap = kNumCUs * 2;  // two resident workgroups per compute unit
+  const int64_t cap = kNumCUs * per_cu;
   p.grid = static_cast<unsigned>(want < cap ? want : cap);
   p.use_rows = true;
   return p;
@@ -694,13 +724,23 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   const RowGradPlan rp = plan_row_grad<T>(sh.N, sh.G, sh.D, sh.S);
   if (rp.use_rows && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma)) {
     const size_t staged_bytes = static_cast<size_t>(sh.D) * sizeof(A);
-#define LAUNCH(TPR, VPT)                                                                      \
+#define LAUNCH_T(TPR, VPT, THREADS)                                                           \
   {                                                                                           \
-    auto kernel = layer_norm_grad_rows<T, TPR, VPT>;                                          \
-    if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, kGradThreads, staged_bytes);    \
-    hipLaunchKernelGGL(kernel, dim3(rp.grid), dim3(kGradThreads), staged_bytes, stream,       \
+    auto kernel = layer_norm_grad_rows<T, TPR, VPT, THREADS>;                                 \
+    if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, THREADS, staged_bytes);         \
+    hipLaunchKernelGGL(kernel, dim3(rp.grid), dim3(THREADS), staged_bytes, stream,            \
                        static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp, mup,  \
                        rsp, dsp, dbp, dxp, part);                                             \
+  }
+#define LAUNCH(TPR, VPT)                                                    \
+  {                                                                         \
+    if constexpr (VPT * IO<T>::kVec <= 16 || sizeof(A) == 8) {              \
+      if constexpr (TPR == 1024) {                                          \
+        LAUNCH_T(TPR, VPT, 1024)                                            \
+      } else {                                                              \
+        LAUNCH_T(TPR, VPT, 512)                                             \
+      }                                                                     \
+    }                                                                       \
   }
     if (rp.cfg.tpr == 64 && rp.cfg.vpt == 1) LAUNCH(64, 1)
     else if (rp.cfg.tpr == 64 && rp.cfg.vpt == 2) LAUNCH(64, 2)
@@ -708,8 +748,10 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     else if (rp.cfg.tpr == 256 && rp.cfg.vpt == 2) LAUNCH(256, 2)
     else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 1) LAUNCH(512, 1)
     else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 2) LAUNCH(512, 2)
-    else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 3) LAUNCH(512, 3)
-    else LAUNCH(512, 4)
+    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 1) LAUNCH(1024, 1)
+    else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 2) LAUNCH(1024, 2)
+    else LAUNCH(1024, 4)
+#undef LAUNCH_T
 #undef LAUNCH
     hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
                        dim3(1024), 0, stream, rp.grid, sh.D, part, dgp, dbtp);

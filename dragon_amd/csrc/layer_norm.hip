@@ -110,11 +110,12 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
   Raw cur;
-  if (kPrefetch) cur.load(x + row * C, npackets, row < N);
+  if (kPrefetch) cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
   for (; row < N; row += stride) {
     Raw nxt;
     if (kPrefetch) {
-      nxt.load(x + (row + stride) * C, npackets, row + stride < N);
+      const bool more = row + stride < N;
+      nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
     } else {
       cur.load(x + row * C, npackets);
     }
@@ -155,8 +156,11 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
         for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * rs * g[e] + b[e];
       }
     }
+    if (kPrefetch) {
+      nxt.wait_ready();
+      cur = nxt;
+    }
     t.store(y + row * C, npackets);
-    if (kPrefetch) cur = nxt;
   }
 }
 

@@ -39,20 +39,29 @@ struct RowTile {
   A v[kVPT][kVec];
 
   static __device__ __forceinline__ int lane() { return threadIdx.x % kTPR; }
-  static __device__ __forceinline__ int sub_row() { return threadIdx.x / kTPR; }
+  // kTPR is a whole number of wavefronts, so the row-group index is uniform
+  // over a wavefront: reading it from the first lane keeps it, and every row
+  // base address derived from it, in scalar registers.
+  static __device__ __forceinline__ int sub_row() {
+    return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kTPR));
+  }
   static __device__ __forceinline__ bool active(int slot, int npackets) {
     return slot * kTPR + lane() < npackets;
   }
 
+  // Loads are unconditional (a masked slot reads packet 0 of the row and is
+  // then overwritten with `fill`): with no branch around a load the number of
+  // loads in flight is static, and the compiler can wait for exactly the ones a
+  // computation needs instead of draining the queue. `row` must point to
+  // readable memory even when `valid` is false.
   __device__ __forceinline__ void load(const T* row, int npackets, A fill, bool valid = true) {
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
-      if (valid && active(s, npackets)) {
-        load_unpack<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
-      } else {
+      const bool on = valid && active(s, npackets);
+      const int packet = on ? s * kTPR + lane() : 0;
+      load_unpack<T>(row + static_cast<int64_t>(packet) * kVec, v[s]);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) v[s][e] = fill;
-      }
+      for (int e = 0; e < kVec; ++e) v[s][e] = on ? v[s][e] : fill;
     }
   }
 
@@ -116,16 +125,17 @@ struct RawRowTile {
   static __device__ __forceinline__ bool active(int slot, int npackets) {
     return slot * kTPR + lane() < npackets;
   }
-  // Inactive slots hold zero bits, i.e. +0.0 in every element type.
+  // Inactive slots hold zero bits, i.e. +0.0 in every element type. The load
+  // itself is unconditional (see RowTile::load); `row` must be readable even
+  // when `valid` is false.
   __device__ __forceinline__ void load(const T* row, int npackets, bool valid = true) {
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
-      if (valid && active(s, npackets)) {
-        p[s] = load_packet(row + static_cast<int64_t>(s * kTPR + lane()) * kVec);
-      } else {
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        p[s] = z;
-      }
+      const bool on = valid && active(s, npackets);
+      const int packet = on ? s * kTPR + lane() : 0;
+      const u32x4 t = load_packet(row + static_cast<int64_t>(packet) * kVec);
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      p[s] = on ? t : z;
     }
   }
   __device__ __forceinline__ void unpack(int s, A (&v)[kVec]) const { IO<T>::unpack(p[s], v); }
@@ -135,6 +145,14 @@ struct RawRowTile {
   __device__ __forceinline__ void refresh() {
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) asm volatile("" : "+v"(p[s]));
+  }
+  // For a prefetched tile: pins the point where its loads must have landed.
+  // Placed after the current row's arithmetic and before the current row's
+  // stores, it makes the wait cover only loads (and the previous row's, by
+  // then old, stores), so the new stores stay in flight across the next row.
+  __device__ __forceinline__ void wait_ready() {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) asm volatile("" : "+v"(p[s])::"memory");
   }
   __device__ __forceinline__ void store_slot(T* row, int s, const A (&v)[kVec]) const {
     pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v);

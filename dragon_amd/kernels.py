@@ -199,3 +199,10 @@ def batch_norm_training_forward(N, C, S, data_format, momentum, epsilon, x, gamm
     _call("dragon_hip_batch_norm_training_forward", tag, N, C, S, lay, momentum, epsilon, _ptr(x),
           _ptr(gamma), _ptr(beta), _ptr(running_mean), _ptr(running_var), _ptr(mu), _ptr(rsig),
           _ptr(params), _ptr(y), _ptr(ws), need, _stream())
+
+
+# ---------------------------------------------------------------- measurement
+
+def stream_probe(mode, src, dst, nbytes):
+    """Streaming read (0), copy (1) or fill (2) of ``nbytes`` bytes."""
+    _call("dragon_hip_stream_probe", mode, _ptr(src), _ptr(dst), nbytes, _stream())

@@ -244,6 +244,15 @@ int dragon_hip_batch_norm_training_forward(int dtype, int64_t N, int64_t C, int6
                                            void* rsig, void* params, void* y, void* scratch,
                                            size_t scratch_bytes, void* stream);
 
+/* ------------------------------------------------------------------------ */
+/* Measurement utility (no counterpart in the reference): a streaming read    */
+/* (mode 0: dst receives at most one word), copy (mode 1) or fill (mode 2) of */
+/* `bytes` bytes (a multiple of 16, 16-byte aligned buffers) with 128-bit      */
+/* accesses. Gives the achieved streaming ceiling of the device and a         */
+/* known-size kernel for calibrating profiler byte counters.                  */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif
