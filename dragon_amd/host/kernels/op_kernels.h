@@ -1,0 +1,114 @@
+// The kernels:: and math:: function templates the operators call, declared
+// with the reference's signatures (dragon/kernels/normalization/op_kernels.h:36-202,
+// dragon/kernels/activation/op_kernels.h:211-247, dragon/kernels/math/op_kernels.h:106-115,
+// dragon/utils/math/elementwise.h:48, dragon/utils/math/blas.h) and explicitly
+// specialised for HIPContext in kernels_hip.cc, where each specialisation is a
+// forward to the C-ABI entry point of the same name.
+//
+// Two additions have no counterpart among the reference's kernels:: functions:
+// GroupNormForward and BatchNormTrainingForward run a sequence an operator
+// body issues (Moments, InvStd, ... ) as one call, so that x is read once
+// where the device can keep the reduction unit on-die.
+#pragma once
+
+#include "core/common.h"
+#include "core/context.h"
+
+namespace dragon {
+
+namespace math {
+
+template <typename T, class Context>
+void InvStd(const int N, const float eps, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void Axpby(const int N, const float alpha, const T* x, const float beta, T* y, Context* ctx);
+
+template <typename T, class Context>
+void Copy(const int N, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void Set(const int N, const T value, T* y, Context* ctx);
+
+template <typename T, class Context>
+void Square(const int N, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void Sub(const int N, const T* a, const T* b, T* y, Context* ctx);
+
+} // namespace math
+
+namespace kernels {
+
+template <typename T, typename AccT, class Context>
+void Moments(const int num_dims, const int64_t* dims, const int num_axes, const int64_t* axes,
+             const T* x, AccT* mean, AccT* var, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void LayerNorm(const int N, const int C, const float epsilon, const T* x, const AccT* gamma,
+               const AccT* beta, AccT* mu, AccT* rsig, T* y, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void GroupNorm(const int N, const int G, const int D, const int S, const string& data_format,
+               const T* x, const AccT* mu, const AccT* rsig, const AccT* gamma, const AccT* beta,
+               T* y, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void GroupNormGrad(const int N, const int G, const int D, const int S, const string& data_format,
+                   const T* x, const AccT* mu, const AccT* rsig, const AccT* gamma, const T* dy,
+                   AccT* ds, AccT* db, AccT* dgamma, AccT* dbeta, T* dx, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNormExpectation(const int N, const int C, const int S, const float normalizer,
+                          const string& data_format, const T* x, AccT* ex, AccT* ex2, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNorm(const int N, const int C, const int S, const string& data_format, const T* x,
+               const AccT* mu, const AccT* rsig, const AccT* gamma, const AccT* beta, AccT* scale,
+               AccT* bias, T* y, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNormWGrad(const int N, const int C, const int S, const string& data_format, const T* x,
+                    const AccT* mu, const AccT* rsig, const T* dy, AccT* dgamma, AccT* dbeta,
+                    Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNormTrainingGrad(const int N, const int C, const int S, const float normalizer,
+                           const string& data_format, const T* x, const AccT* mu, const AccT* rsig,
+                           const AccT* gamma, const AccT* dgamma, const AccT* dbeta, const T* dy,
+                           T* dx, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNormInferenceGrad(const int N, const int C, const int S, const string& data_format,
+                            const T* x, const AccT* mu, const AccT* rsig, const AccT* gamma,
+                            const T* dy, AccT* dgamma, AccT* dbeta, T* dx, Context* ctx);
+
+template <typename T, class Context>
+void Softmax(const int N, const int S, const int C, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void LogSoftmax(const int N, const int S, const int C, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void SoftmaxGrad(const int N, const int S, const int C, const T* dy, const T* y, T* dx, Context* ctx);
+
+template <typename T, class Context>
+void LogSoftmaxGrad(const int N, const int S, const int C, const T* dy, const T* y, T* dx,
+                    Context* ctx);
+
+// Fused operator bodies (see the header comment).
+template <typename T, typename AccT, class Context>
+void GroupNormForward(const int N, const int G, const int D, const int S, const string& data_format,
+                      const float epsilon, const T* x, const AccT* gamma, const AccT* beta,
+                      AccT* mu, AccT* rsig, T* y, Context* ctx);
+
+template <typename T, typename AccT, class Context>
+void BatchNormTrainingForward(const int N, const int C, const int S, const string& data_format,
+                              const float momentum, const float epsilon, const T* x,
+                              const AccT* gamma, const AccT* beta, AccT* running_mean,
+                              AccT* running_var, AccT* mu, AccT* rsig, AccT* params, T* y,
+                              Context* ctx);
+
+} // namespace kernels
+
+} // namespace dragon

@@ -1,0 +1,99 @@
+"""Host-layer logic that needs no GPU: operator definitions in text format, the
+HIP operator registry, schemas, gradient makers, tensor feed/fetch on the host
+side, and the error behaviour (the reference LOG(FATAL)s; the C API reports the
+same message as an exception)."""
+
+import numpy as np
+import pytest
+
+from dragon_amd import runtime as rt
+
+
+@pytest.fixture()
+def ws():
+    w = rt.Workspace("host_test")
+    yield w
+    w.close()
+
+
+def test_registry_holds_the_ten_operator_types_and_the_sync_aliases():
+    ops = set(rt.registered_operators())
+    assert {"LayerNorm", "LayerNormGradient", "GroupNorm", "GroupNormGradient", "BatchNorm",
+            "BatchNormGradient", "Softmax", "SoftmaxGradient", "LogSoftmax",
+            "LogSoftmaxGradient", "SyncBatchNorm", "SyncBatchNormGradient"} <= ops
+
+
+def test_feed_fetch_round_trip(ws):
+    rng = np.random.default_rng(0)
+    for dtype in (np.float32, np.float64, np.float16, np.int64):
+        a = (rng.standard_normal((3, 5)) * 4).astype(dtype)
+        ws.feed("t", a)
+        assert ws.info("t") == (np.dtype(dtype).name, (3, 5))
+        assert np.array_equal(ws.fetch("t"), a)
+    bits = rng.integers(0, 65535, (4, 2)).astype(np.uint16)
+    ws.feed("b", bits, dtype="bfloat16")
+    assert ws.info("b") == ("bfloat16", (4, 2))
+    assert np.array_equal(ws.fetch("b"), bits)
+    empty = np.zeros((0, 7), np.float32)
+    ws.feed("e", empty)
+    assert ws.fetch("e").shape == (0, 7)
+
+
+def test_gradient_definitions_follow_the_reference_makers(ws):
+    fwd = rt.make_def("LayerNorm", ["x", "w", "b"], ["y"], name="ln", axis=1, epsilon=1e-3)
+    defs, gis = ws.gradient_defs(fwd, ["dy"])
+    assert len(defs) == 1 and gis == ["x_grad", "w_grad", "b_grad"]
+    d = defs[0]
+    assert 'type: "LayerNormGradient"' in d
+    assert d.index('input: "x"') < d.index('input: "w"') < d.index('input: "dy"')
+    assert 'arg { name: "axis" i: 1 }' in d and 'arg { name: "name" s: "ln" }' in d
+    assert "device_type: 4" in d
+
+    fwd = rt.make_def("BatchNorm", ["x", "w", "b", "rm", "rv"], ["y"], name="bn", axis=1)
+    defs, gis = ws.gradient_defs(fwd, ["dy"])
+    d = defs[0]
+    assert 'type: "BatchNormGradient"' in d
+    order = [d.index('input: "%s"' % n) for n in ("x", "w", "rm", "rv", "dy")]
+    assert order == sorted(order) and 'input: "b"' not in d
+    assert gis == ["x_grad", "w_grad", "b_grad", "", ""]
+
+    fwd = rt.make_def("Softmax", ["x"], ["y"], name="sm", axis=-1)
+    defs, gis = ws.gradient_defs(fwd, ["dy"])
+    assert 'type: "SoftmaxGradient"' in defs[0]
+    assert defs[0].index('input: "y"') < defs[0].index('input: "dy"') and gis == ["x_grad"]
+
+    fwd = rt.make_def("SyncBatchNorm", ["x", "w", "b", "rm", "rv"], ["y"], name="sbn")
+    assert 'type: "SyncBatchNormGradient"' in ws.gradient_defs(fwd, ["dy"])[0][0]
+
+
+def test_schema_violations_and_unknown_operators_are_fatal(ws):
+    ws.feed("x", np.zeros((2, 4), np.float32))
+    with pytest.raises(rt.DragonError, match="inputs"):
+        ws.run_operator(rt.make_def("LayerNorm", ["x"], ["y"]))
+    with pytest.raises(rt.DragonError, match="not registered"):
+        ws.run_operator(rt.make_def("ChannelNorm", ["x"], ["y"]))
+    with pytest.raises(rt.DragonError, match="no gradient"):
+        ws.gradient_defs(rt.make_def("SoftmaxGradient", ["y", "dy"], ["dx"]), ["g"])
+    with pytest.raises(rt.DragonError, match="not in workspace"):
+        ws.run_operator(rt.make_def("Softmax", ["missing"], ["y"]))
+    # forward may only alias input 0 with output 0
+    ws.feed("w", np.zeros(4, np.float32))
+    ws.feed("b", np.zeros(4, np.float32))
+    with pytest.raises(rt.DragonError, match="inplace"):
+        ws.run_operator(rt.make_def("LayerNorm", ["x", "w", "b"], ["x"]))
+
+
+def test_cpu_device_is_reported_unavailable(ws):
+    ws.feed("x", np.zeros((2, 4), np.float32))
+    text = rt.make_def("Softmax", ["x"], ["y"]).replace("device_type: 4", "device_type: 0")
+    with pytest.raises(rt.DragonError, match="CPU operators are not part of this build"):
+        ws.run_operator(text)
+    with pytest.raises(rt.DragonError, match="Unknown device"):
+        ws.run_operator(text.replace("device_type: 0", "device_type: 9"))
+
+
+def test_malformed_definitions_are_fatal(ws):
+    for bad in ('type "Softmax"', 'type: "Softmax" arg { name: "axis" q: 1 }', 'bogus: 1',
+                'type: "Softmax" input: "x'):
+        with pytest.raises(rt.DragonError):
+            ws.run_operator(bad)
