@@ -31,6 +31,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE hardware counters, each
+# scaled by what it reads for the 1 GiB streaming-copy probe (figures and
+# commands: profiles/hbm_traffic_softmax_f16_16x32x512x512.txt).
+MEASURED_TRAFFIC_BYTES = {
+    ("softmax_f16_16x32x512x512", "softmax"): 536.9e6,
+    ("softmax_f16_16x32x512x512", "softmax_grad"): 805.4e6,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -332,7 +340,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dominant["kernel"],
                      "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dominant["GB/s"] / HBM_PEAK_GBS, 4),
-                     "avg_launch_us": dominant["us"], "traffic": None,
+                     "avg_launch_us": dominant["us"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((head, dominant["kernel"])),
                      "streaming_kernels_GB/s": ceiling},
         "cpu_baseline": cpu,
         "kernels": all_kernels,
