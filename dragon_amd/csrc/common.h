@@ -139,7 +139,10 @@ struct IO<bf16_t> {
 };
 
 // One aligned 16-byte packet to and from HBM. Outputs are written once and not
-// read again by the same kernel, so stores carry the non-temporal hint.
+// read again by the same kernel, so stores carry the non-temporal hint. Loads
+// do not: measured on MI355X, non-temporal loads slow every forward kernel
+// down (inputs that a previous kernel just produced, or that fit the 256 MB
+// last-level cache, are then fetched from HBM again).
 typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), may_alias));
 template <typename T>
 __device__ __forceinline__ u32x4 load_packet(const T* p) {

@@ -385,10 +385,21 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
   const A inv_l = A(1) / A(L);
   const int lane = Tile::lane();
 
-  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
-       row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
-    Raw t;
-    t.load(x + row * L, npackets);
+  // The 1024-thread tile (one or two workgroups per compute unit) requests the
+  // next group's packets before it reduces the current group.
+  constexpr bool kPrefetch = kTPR == 1024;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock;
+  int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+  Raw t;
+  if (kPrefetch) t.load(x + (row < rows ? row : 0) * L, npackets, row < rows);
+  for (; row < rows; row += stride) {
+    Raw nxt;
+    if (kPrefetch) {
+      const bool more = row + stride < rows;
+      nxt.load(x + (more ? row + stride : 0) * L, npackets, more);
+    } else {
+      t.load(x + row * L, npackets);
+    }
     A s = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
@@ -420,20 +431,28 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
     }
     const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
     t.refresh();
+    // Results replace the packets in place; they are stored after the wait for
+    // the prefetched group so that the stores overlap the next group's work.
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
+      const uint32_t c = c0 + (Tile::active(i, npackets) ? col / S : 0u);  // kVec divides S
+      const A gam = gamma[c] * rs, bet = beta[c];
+      A v[kVec];
+      t.unpack(i, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+      t.p[i] = IO<T>::pack(v);
+    }
+    if (kPrefetch) nxt.wait_ready();
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (Tile::active(i, npackets)) {
-        const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
-        const uint32_t c = c0 + col / S;  // a packet lies in one channel: kVec divides S
-        const A gam = gamma[c] * rs, bet = beta[c];
-        A v[kVec];
-        t.unpack(i, v);
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
-        t.store_slot(y + row * L, i, v);
+        store_packet(y + row * L + static_cast<int64_t>(i * kTPR + lane) * kVec, t.p[i]);
       }
     }
     if (kTPR != kWaveSize) __syncthreads();
+    if (kPrefetch) t = nxt;
   }
 }
 
@@ -663,8 +682,11 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
+    const unsigned one_shot = row_grid(rows, Tile::kRowsPerBlock);                              \
+    const unsigned resident =                                                                   \
+        TPR == 1024 ? resident_grid(group_norm_forward_rows<T, TPR, VPT>, TPR, 0) : one_shot;   \
     hipLaunchKernelGGL((group_norm_forward_rows<T, TPR, VPT>),                                  \
-                       dim3(row_grid(rows, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       dim3(one_shot < resident ? one_shot : resident), dim3(Tile::kThreads), 0, stream, \
                        rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),                     \
                        static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
                        static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig), \
