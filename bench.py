@@ -104,6 +104,23 @@ def wl_softmax(shape, dtype_name, seed=1):
     return kernels, {"rows": N, "width": C, "tensors": (x, dy, y, dx)}
 
 
+def wl_lp_norm(N, C, dtype_name, p=2, seed=5):
+    import torch
+    from dragon_amd import kernels as K
+    dtype = getattr(torch, dtype_name)
+    gen = _gen(seed)
+    x = _randn((N, C), dtype, gen)
+    dy = _randn((N, C), dtype, gen)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    nbytes = x.numel() * x.element_size()
+    fwd, bwd = (K.l1_norm, K.l1_norm_grad) if p == 1 else (K.l2_norm, K.l2_norm_grad)
+    kernels = [
+        ("l%d_norm" % p, lambda: fwd(N, 1, C, 1.0, 1e-12, x, y), 2 * nbytes),
+        ("l%d_norm_grad" % p, lambda: bwd(N, 1, C, 1.0, 1e-12, dy, x, dx), 3 * nbytes),
+    ]
+    return kernels, {"rows": N, "width": C}
+
+
 def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False):
     import torch
     from dragon_amd import kernels as K
@@ -205,6 +222,9 @@ WORKLOADS = {
     "layer_norm_f32_8192x4096": lambda: wl_layer_norm(8192, 4096, "float32", 4),
     "softmax_f16_8192x4096": lambda: wl_softmax((8192, 4096), "float16", 1),
     "softmax_f32_8192x4096": lambda: wl_softmax((8192, 4096), "float32", 1),
+    # sibling row reductions on the same skeleton
+    "l2_norm_bf16_8192x4096": lambda: wl_lp_norm(8192, 4096, "bfloat16", 2),
+    "l2_norm_f32_8192x4096": lambda: wl_lp_norm(8192, 4096, "float32", 2),
 }
 
 
@@ -333,9 +353,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate, f16 I/O" if "f16" in head else ("f32" if "f32" in head else "f32 accumulate, bf16 I/O"),
+        "dtype": "f32",  # every reduction and the element-wise math run in fp32; I/O type is in config
         "data": "synthetic",
-        "config": {"workload": head, "step": "forward + backward, inputs resident in HBM",
+        "config": {"workload": head, "io_dtype": "f16" if "f16" in head else ("bf16" if "bf16" in head else "f32"),
+                   "step": "forward + backward, inputs resident in HBM",
                    "algorithmic_bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "kernel": dominant["kernel"],
                      "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -66,6 +66,10 @@ SIGNATURES = {
     "dragon_hip_log_softmax": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "dragon_hip_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "dragon_hip_log_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "dragon_hip_l1_norm": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp]),
+    "dragon_hip_l2_norm": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp]),
+    "dragon_hip_l1_norm_grad": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp, _vp]),
+    "dragon_hip_l2_norm_grad": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp, _vp]),
     "dragon_hip_group_norm_forward_scratch_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int]),
     "dragon_hip_group_norm_forward": (_int, [_int, _i64, _i64, _i64, _i64, _int, _f32, _vp, _vp,
                                              _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -2,7 +2,7 @@
 // the gradient, from which tensors, into which. Follows the GradientMaker
 // classes registered next to each operator in the reference
 // (dragon/core/gradient.h:43-181; layer_norm_op.cc:60-74, group_norm_op.cc:112-126,
-// batch_norm_op.cc:254-268, softmax_op.cc:62, log_softmax_op.cc:62).
+// batch_norm_op.cc:254-268, softmax_op.cc:62, log_softmax_op.cc:62, lp_norm_op.cc:88).
 #pragma once
 
 #include "core/common.h"
@@ -54,6 +54,20 @@ class InplaceGradientMaker final : public GradientMakerBase {
   using GradientMakerBase::GradientMakerBase;
   void CreateGradientDefs() override {
     AddGradientDef(def().type + "Gradient", {O(0), GO(0)}, {GI(0)});
+  }
+};
+
+// Y1..Ym = f(X1..Xn) whose gradient operator takes (X1..Xn, dY1..dYm) and
+// produces (dX1..dXn) (dragon/core/gradient.h:132-150).
+class GenericGradientMaker final : public GradientMakerBase {
+ public:
+  using GradientMakerBase::GradientMakerBase;
+  void CreateGradientDefs() override {
+    vector<string> inputs(def().input.begin(), def().input.end());
+    vector<string> outputs;
+    for (size_t i = 0; i < def().output.size(); ++i) inputs.push_back(GO(static_cast<int>(i)));
+    for (size_t i = 0; i < def().input.size(); ++i) outputs.push_back(GI(static_cast<int>(i)));
+    AddGradientDef(def().type + "Gradient", inputs, outputs);
   }
 };
 

@@ -214,6 +214,38 @@ DEFINE_SOFTMAX_LAUNCHERS(float);
 DEFINE_SOFTMAX_LAUNCHERS(double);
 #undef DEFINE_SOFTMAX_LAUNCHERS
 
+#define DEFINE_LP_NORM_LAUNCHERS(T)                                                               \
+  template <>                                                                                     \
+  void L1Norm<T, HIPContext>(const int N, const int S, const int C, const float normalizer,       \
+                             const float epsilon, const T* x, T* y, HIPContext* ctx) {            \
+    HIP_CHECK(dragon_hip_l1_norm(Tag<T>(), N, S, C, normalizer, epsilon, x, y, ctx->hip_stream())); \
+  }                                                                                               \
+  template <>                                                                                     \
+  void L2Norm<T, HIPContext>(const int N, const int S, const int C, const float normalizer,       \
+                             const float epsilon, const T* x, T* y, HIPContext* ctx) {            \
+    HIP_CHECK(dragon_hip_l2_norm(Tag<T>(), N, S, C, normalizer, epsilon, x, y, ctx->hip_stream())); \
+  }                                                                                               \
+  template <>                                                                                     \
+  void L1NormGrad<T, HIPContext>(const int N, const int S, const int C, const float normalizer,   \
+                                 const float epsilon, const T* dy, const T* x, T* dx,             \
+                                 HIPContext* ctx) {                                               \
+    HIP_CHECK(dragon_hip_l1_norm_grad(Tag<T>(), N, S, C, normalizer, epsilon, dy, x, dx,          \
+                                      ctx->hip_stream()));                                        \
+  }                                                                                               \
+  template <>                                                                                     \
+  void L2NormGrad<T, HIPContext>(const int N, const int S, const int C, const float normalizer,   \
+                                 const float epsilon, const T* dy, const T* x, T* dx,             \
+                                 HIPContext* ctx) {                                               \
+    HIP_CHECK(dragon_hip_l2_norm_grad(Tag<T>(), N, S, C, normalizer, epsilon, dy, x, dx,          \
+                                      ctx->hip_stream()));                                        \
+  }
+
+DEFINE_LP_NORM_LAUNCHERS(float16);
+DEFINE_LP_NORM_LAUNCHERS(bfloat16);
+DEFINE_LP_NORM_LAUNCHERS(float);
+DEFINE_LP_NORM_LAUNCHERS(double);
+#undef DEFINE_LP_NORM_LAUNCHERS
+
 } // namespace kernels
 
 } // namespace dragon

@@ -96,6 +96,22 @@ template <typename T, class Context>
 void LogSoftmaxGrad(const int N, const int S, const int C, const T* dy, const T* y, T* dx,
                     Context* ctx);
 
+template <typename T, class Context>
+void L1Norm(const int N, const int S, const int C, const float normalizer, const float epsilon,
+            const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void L1NormGrad(const int N, const int S, const int C, const float normalizer, const float epsilon,
+                const T* dy, const T* x, T* dx, Context* ctx);
+
+template <typename T, class Context>
+void L2Norm(const int N, const int S, const int C, const float normalizer, const float epsilon,
+            const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void L2NormGrad(const int N, const int S, const int C, const float normalizer, const float epsilon,
+                const T* dy, const T* x, T* dx, Context* ctx);
+
 // Fused operator bodies (see the header comment).
 template <typename T, typename AccT, class Context>
 void GroupNormForward(const int N, const int G, const int D, const int S, const string& data_format,

@@ -1,7 +1,8 @@
 """Python mirror of the reference's ``kernels::`` / ``math::`` free functions.
 
 Same names (snake-cased), argument order and aliasing conventions as the C++
-templates of dragon/kernels/normalization/op_kernels.h,
+templates of dragon/kernels/normalization/op_kernels.h (LayerNorm, GroupNorm,
+BatchNorm, L1/L2Norm),
 dragon/kernels/activation/op_kernels.h and dragon/kernels/math/op_kernels.h;
 the trailing ``Context* ctx`` becomes the current torch stream. Tensors are
 torch CUDA tensors used purely as device memory: every function passes raw
@@ -180,6 +181,26 @@ def softmax_grad(N, S, C, dy, y, dx):
 def log_softmax_grad(N, S, C, dy, y, dx):
     _call("dragon_hip_log_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx),
           _stream())
+
+
+def l1_norm(N, S, C, normalizer, epsilon, x, y):
+    _call("dragon_hip_l1_norm", dtype_tag(x), N, S, C, normalizer, epsilon, _ptr(x), _ptr(y),
+          _stream())
+
+
+def l2_norm(N, S, C, normalizer, epsilon, x, y):
+    _call("dragon_hip_l2_norm", dtype_tag(x), N, S, C, normalizer, epsilon, _ptr(x), _ptr(y),
+          _stream())
+
+
+def l1_norm_grad(N, S, C, normalizer, epsilon, dy, x, dx):
+    _call("dragon_hip_l1_norm_grad", dtype_tag(x), N, S, C, normalizer, epsilon, _ptr(dy), _ptr(x),
+          _ptr(dx), _stream())
+
+
+def l2_norm_grad(N, S, C, normalizer, epsilon, dy, x, dx):
+    _call("dragon_hip_l2_norm_grad", dtype_tag(x), N, S, C, normalizer, epsilon, _ptr(dy), _ptr(x),
+          _ptr(dx), _stream())
 
 
 # ---------------------------------------------------------------- fused operator bodies

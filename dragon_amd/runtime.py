@@ -217,6 +217,11 @@ def batch_norm(tape, inputs, axis=-1, momentum=0.9, epsilon=1e-5, use_stats=-1, 
                     use_stats=int(use_stats))
 
 
+def lp_norm(tape, inputs, axis=-1, end_axis=None, p=2, epsilon=1e-12, reduction="sum"):
+    return tape.run("LpNorm", inputs, p=int(p), axis=axis, end_axis=end_axis, epsilon=float(epsilon),
+                    reduction=reduction.upper())
+
+
 def softmax(tape, inputs, axis=-1):
     return tape.run("Softmax", inputs, axis=axis)
 

@@ -218,6 +218,26 @@ int dragon_hip_log_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, cons
                                 const void* y, void* dx, void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* L1Norm / L2Norm, dragon/kernels/normalization/op_kernels.h:145-189        */
+/* (CPU dragon/kernels/normalization/cpu/lp_norm_kernel.cc:10-157).          */
+/* Tensors are T[N, C, S], reduction along C (element stride S):             */
+/*   l1  norm = max(sum|x| / normalizer, epsilon)                            */
+/*   l2  norm = max(sqrt(sum x^2 / normalizer), epsilon)                     */
+/*   y = x / norm;  dx = dy / norm - g(x) * (sum(dy*x) / normalizer) / norm^(p+1) */
+/* with g = sign for l1 and identity for l2. normalizer is C for the "MEAN"  */
+/* reduction and 1 for "SUM" (lp_norm_op.cc:14-35). y may alias x and dx may  */
+/* alias dy. 16-bit I/O accumulates in fp32.                                 */
+/* ------------------------------------------------------------------------ */
+int dragon_hip_l1_norm(int dtype, int64_t N, int64_t S, int64_t C, float normalizer, float epsilon,
+                       const void* x, void* y, void* stream);
+int dragon_hip_l2_norm(int dtype, int64_t N, int64_t S, int64_t C, float normalizer, float epsilon,
+                       const void* x, void* y, void* stream);
+int dragon_hip_l1_norm_grad(int dtype, int64_t N, int64_t S, int64_t C, float normalizer,
+                            float epsilon, const void* dy, const void* x, void* dx, void* stream);
+int dragon_hip_l2_norm_grad(int dtype, int64_t N, int64_t S, int64_t C, float normalizer,
+                            float epsilon, const void* dy, const void* x, void* dx, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Operator-level fused entry points: one call for a kernel sequence that a  */
 /* Dragon operator body issues back to back, so that x is read once where    */
 /* the chip can hold the reduction unit on-die. Results equal the sequence.  */

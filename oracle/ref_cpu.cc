@@ -1,5 +1,5 @@
 // CPU oracle: a loop-for-loop restatement of Dragon's CPU kernels for
-// LayerNorm, GroupNorm, BatchNorm, Moments and Softmax/LogSoftmax.
+// LayerNorm, GroupNorm, BatchNorm, Moments, Softmax/LogSoftmax and L1/L2Norm.
 //
 // THIS FILE IS TEST INFRASTRUCTURE. It is the checker the HIP kernels are
 // compared against and the CPU baseline that is timed beside them. Nothing in
@@ -17,6 +17,8 @@
 //   layer_norm, group_norm_grad    reference test literals, test_ops.py:4232-4291,4303-4351,4363-4397
 //   moments                        numpy mean/var closed form, test_ops.py:3489-3511
 //   batch_norm fwd/bwd             numpy closed forms,  test_ops.py:4127-4181
+//   lp_norm (+grad)                reference test literals and the numpy closed
+//                                  form of test_ops.py:4480-4512
 //   f16 / bf16 conversions         exhaustive comparison against numpy float16 and
 //                                  a bit-level bf16 RNE over all 2^16 encodings
 //   running-stat update (axpby)    PARITY UNPINNED by any reference test; pinned
@@ -679,6 +681,71 @@ void log_softmax_grad(
   }
 }
 
+// ---------------------------------------------------------------------------
+// L1Norm / L2Norm and gradients over [N, C, S], reduction along C.
+// dragon/kernels/normalization/cpu/lp_norm_kernel.cc:10-101. The reference
+// evaluates Eigen expressions (lpNorm<1>, squaredNorm, dot, array().sign());
+// each is restated as a sequential scalar loop with the same data flow: the
+// norm is narrowed to float, divided by the normalizer, clamped from below by
+// epsilon and narrowed to T before the element-wise division.
+// ---------------------------------------------------------------------------
+template <typename T>
+inline T sign_of(T v) {
+  return T((T(0) < v) - (v < T(0)));
+}
+
+template <typename T, int kP>
+void lp_norm(const int N, const int S, const int C, const float normalizer,
+             const float epsilon, const T* x, T* y) {
+  // :10-49
+  for (int i = 0; i < N; ++i) {
+    for (int j = 0; j < S; ++j) {
+      const int64_t base = int64_t(i) * C * S + j;
+      T acc = T(0);
+      for (int k = 0; k < C; ++k) {
+        const T v = x[base + int64_t(k) * S];
+        acc += kP == 1 ? std::abs(v) : v * v;
+      }
+      const float norm = kP == 1 ? float(acc) / normalizer
+                                 : std::sqrt(float(acc) / normalizer);
+      const T div = T(std::max(norm, epsilon));
+      for (int k = 0; k < C; ++k) {
+        const int64_t o = base + int64_t(k) * S;
+        y[o] = x[o] / div;
+      }
+    }
+  }
+}
+
+template <typename T, int kP>
+void lp_norm_grad(const int N, const int S, const int C, const float normalizer,
+                  const float eps, const T* dy, const T* x, T* dx) {
+  // :51-101 : dx = dy / norm - sign(x) / (norm^2 / sum)   (p = 1)
+  //           dx = dy / norm -      x  / (norm^3 / sum)   (p = 2)
+  // with sum = dot(dy, x) / normalizer.
+  for (int i = 0; i < N; ++i) {
+    for (int j = 0; j < S; ++j) {
+      const int64_t base = int64_t(i) * C * S + j;
+      T acc = T(0), dot = T(0);
+      for (int k = 0; k < C; ++k) {
+        const int64_t o = base + int64_t(k) * S;
+        acc += kP == 1 ? std::abs(x[o]) : x[o] * x[o];
+        dot += dy[o] * x[o];
+      }
+      const float norm =
+          std::max(kP == 1 ? float(acc) / normalizer
+                           : std::sqrt(float(acc) / normalizer), eps);
+      const float sum = float(dot) / normalizer;
+      const float powed = kP == 1 ? norm * norm : std::pow(norm, 3.f);
+      const T a = T(norm), b = T(powed / sum);
+      for (int k = 0; k < C; ++k) {
+        const int64_t o = base + int64_t(k) * S;
+        dx[o] = dy[o] / a - (kP == 1 ? sign_of(x[o]) : x[o]) / b;
+      }
+    }
+  }
+}
+
 enum { kF16 = 0, kBF16 = 1, kF32 = 2, kF64 = 3 };
 enum { kNCHWLayout = 0, kNHWCLayout = 1 };
 enum { kOk = 0, kBadArg = -1, kUnsupportedDtype = -2 };
@@ -1038,5 +1105,40 @@ REF_SM_BWD(ref_softmax_grad, softmax_grad)
 REF_SM_BWD(ref_log_softmax_grad, log_softmax_grad)
 #undef REF_SM_FWD
 #undef REF_SM_BWD
+
+// kernels::L1Norm / L2Norm / L1NormGrad / L2NormGrad launchers,
+// lp_norm_kernel.cc:105-157. p is 1 or 2. f32 and f64 only, as for softmax.
+int ref_lp_norm(int dtype, int p, int64_t N, int64_t S, int64_t C,
+                float normalizer, float epsilon, const void* x, void* y) {
+  if (p != 1 && p != 2) return kBadArg;
+  if (dtype == kF32) {
+    if (p == 1) lp_norm<float, 1>(int(N), int(S), int(C), normalizer, epsilon, (const float*)x, (float*)y);
+    else lp_norm<float, 2>(int(N), int(S), int(C), normalizer, epsilon, (const float*)x, (float*)y);
+    return kOk;
+  }
+  if (dtype == kF64) {
+    if (p == 1) lp_norm<double, 1>(int(N), int(S), int(C), normalizer, epsilon, (const double*)x, (double*)y);
+    else lp_norm<double, 2>(int(N), int(S), int(C), normalizer, epsilon, (const double*)x, (double*)y);
+    return kOk;
+  }
+  return kUnsupportedDtype;
+}
+
+int ref_lp_norm_grad(int dtype, int p, int64_t N, int64_t S, int64_t C,
+                     float normalizer, float epsilon, const void* dy,
+                     const void* x, void* dx) {
+  if (p != 1 && p != 2) return kBadArg;
+  if (dtype == kF32) {
+    if (p == 1) lp_norm_grad<float, 1>(int(N), int(S), int(C), normalizer, epsilon, (const float*)dy, (const float*)x, (float*)dx);
+    else lp_norm_grad<float, 2>(int(N), int(S), int(C), normalizer, epsilon, (const float*)dy, (const float*)x, (float*)dx);
+    return kOk;
+  }
+  if (dtype == kF64) {
+    if (p == 1) lp_norm_grad<double, 1>(int(N), int(S), int(C), normalizer, epsilon, (const double*)dy, (const double*)x, (double*)dx);
+    else lp_norm_grad<double, 2>(int(N), int(S), int(C), normalizer, epsilon, (const double*)dy, (const double*)x, (double*)dx);
+    return kOk;
+  }
+  return kUnsupportedDtype;
+}
 
 } // extern "C"

@@ -12,6 +12,7 @@ kernels the way the reference's operator bodies do:
 * ``op_group_norm`` / ``_grad``  dragon/operators/normalization/group_norm_op.cc:8-85
 * ``op_batch_norm_train`` / ``op_batch_norm_infer`` / ``*_grad``
                                dragon/operators/normalization/batch_norm_op.cc:8-226
+* ``op_lp_norm`` / ``_grad``     dragon/operators/normalization/lp_norm_op.cc:8-72
 
 16-bit tensors travel as ``numpy.uint16`` bit patterns together with a dtype
 name (``"float16"`` / ``"bfloat16"``); ``to_bits`` / ``from_bits`` use the
@@ -277,6 +278,28 @@ def log_softmax_grad(dtype, N, S, C, dy, y):
     return _softmax_grad_like("ref_log_softmax_grad", dtype, N, S, C, dy, y)
 
 
+def lp_norm(dtype, p, N, S, C, normalizer, epsilon, x):
+    """kernels::L1Norm (p=1) / L2Norm (p=2), lp_norm_kernel.cc:10-49."""
+    t = storage_dtype(dtype)
+    x = _c(x, t)
+    y = np.empty_like(x)
+    _check(lib().ref_lp_norm(
+        DTYPES[dtype], int(p), _i64(N), _i64(S), _i64(C), ctypes.c_float(normalizer),
+        ctypes.c_float(epsilon), _p(x), _p(y)), "lp_norm")
+    return y
+
+
+def lp_norm_grad(dtype, p, N, S, C, normalizer, epsilon, dy, x):
+    """kernels::L1NormGrad / L2NormGrad, lp_norm_kernel.cc:51-101."""
+    t = storage_dtype(dtype)
+    dy, x = _c(dy, t), _c(x, t)
+    dx = np.empty_like(x)
+    _check(lib().ref_lp_norm_grad(
+        DTYPES[dtype], int(p), _i64(N), _i64(S), _i64(C), ctypes.c_float(normalizer),
+        ctypes.c_float(epsilon), _p(dy), _p(x), _p(dx)), "lp_norm_grad")
+    return dx
+
+
 # ---------------------------------------------------------------------------
 # Operator-level sequences (what the reference's op bodies run)
 # ---------------------------------------------------------------------------
@@ -299,6 +322,30 @@ def op_softmax_grad(dtype, y, dy, axis=-1, log=False):
     _, N, C, S = _axis_split(y.shape, axis)
     fn = log_softmax_grad if log else softmax_grad
     return fn(dtype, N, S, C, dy, y).reshape(y.shape)
+
+
+def _lp_args(shape, axis, end_axis):
+    """LpNormOp: N=count(0,axis), C=count(axis,end_axis+1), S=count(end_axis+1)."""
+    axis = axis % len(shape)
+    end_axis = axis if end_axis is None else end_axis % len(shape)
+    N = int(np.prod(shape[:axis] or (1,)))
+    C = int(np.prod(shape[axis:end_axis + 1]))
+    S = int(np.prod(shape[end_axis + 1:] or (1,)))
+    return N, C, S
+
+
+def op_lp_norm(dtype, x, axis=-1, end_axis=None, p=2, eps=1e-12, reduction="sum"):
+    """LpNormOp, dragon/operators/normalization/lp_norm_op.cc:8-38."""
+    N, C, S = _lp_args(x.shape, axis, end_axis)
+    normalizer = float(C) if reduction.upper() == "MEAN" else 1.0
+    return lp_norm(dtype, p, N, S, C, normalizer, eps, x).reshape(x.shape)
+
+
+def op_lp_norm_grad(dtype, x, dy, axis=-1, end_axis=None, p=2, eps=1e-12, reduction="sum"):
+    """LpNormGradientOp, dragon/operators/normalization/lp_norm_op.cc:40-72."""
+    N, C, S = _lp_args(x.shape, axis, end_axis)
+    normalizer = float(C) if reduction.upper() == "MEAN" else 1.0
+    return lp_norm_grad(dtype, p, N, S, C, normalizer, eps, dy, x).reshape(x.shape)
 
 
 def op_layer_norm(dtype, x, gamma, beta, axis=-1, eps=1e-5):

@@ -448,3 +448,102 @@ def test_math_helpers_bitwise(K):
     assert np.array_equal(U.to_host(out), x - U.to_host(yd))
     K.set(n, 2.5, out)
     assert np.all(U.to_host(out) == 2.5)
+
+
+# ---------------------------------------------------------------- L1Norm / L2Norm
+
+LP_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 70000), -1), ((5, 37), -1),
+             ((6, 300), -1), ((3, 7, 5), 1), ((2, 3, 4, 16), 2), ((4, 1), -1), ((2, 16, 8, 8), 1),
+             ((3, 8200), -1), ((2, 40, 24), 1)]
+
+
+def _lp_fp64(x, dy, ax, p, normalizer, eps):
+    x64, dy64 = np.asarray(x, np.float64), np.asarray(dy, np.float64)
+    if p == 1:
+        norm = np.maximum(np.abs(x64).sum(ax, keepdims=True) / normalizer, eps)
+        g = np.sign(x64)
+    else:
+        norm = np.maximum(np.sqrt(np.square(x64).sum(ax, keepdims=True) / normalizer), eps)
+        g = x64
+    dot = (dy64 * x64).sum(ax, keepdims=True) / normalizer
+    # third value: size of the two terms that cancel in dx
+    return x64 / norm, dy64 / norm - g * dot / norm ** (p + 1), float(np.max(np.abs(dy64 / norm)))
+
+
+@pytest.mark.parametrize("reduction", ["sum", "mean"])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape,axis", LP_SHAPES)
+def test_lp_norm_forward_backward(K, shape, axis, dtype, p, reduction):
+    rng = U.rng_for(900 + len(shape) + p)
+    x = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    ax = axis % len(shape)
+    N = int(np.prod(shape[:ax] or (1,)))
+    C = shape[ax]
+    S = int(np.prod(shape[ax + 1:] or (1,)))
+    normalizer = float(C) if reduction == "mean" else 1.0
+    eps = 1e-12
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    y_ref = R.op_lp_norm(od, xo, axis, None, p, eps, reduction)
+    dx_ref = R.op_lp_norm_grad(od, xo, dyo, axis, None, p, eps, reduction)
+    y64, dx64, term = _lp_fp64(xo, dyo, ax, p, normalizer, eps)
+    xd, dyd = U.to_device(x, dtype), U.to_device(dy, dtype)
+    y, dx = empty(shape, dtype), empty(shape, dtype)
+    fwd = K.l1_norm if p == 1 else K.l2_norm
+    bwd = K.l1_norm_grad if p == 1 else K.l2_norm_grad
+    fwd(N, S, C, normalizer, eps, xd, y)
+    bwd(N, S, C, normalizer, eps, dyd, xd, dx)
+    yw = U.widen(U.to_host(y), dtype).reshape(shape)
+    dxw = U.widen(U.to_host(dx), dtype).reshape(shape)
+    # rows of 70000 put the oracle's sequential fp32 sums themselves off: three-way check
+    ok, *errs = U.close3(yw, y_ref, y64, U.TIGHT[dtype])
+    assert ok, errs
+    # dx is a difference of two terms of size `term` (it vanishes for C == 1):
+    # errors are measured against that size
+    e_go = np.max(np.abs(dxw - np.asarray(dx_ref, np.float64))) / term
+    e_ge = np.max(np.abs(dxw - dx64)) / term
+    e_oe = np.max(np.abs(np.asarray(dx_ref, np.float64) - dx64)) / term
+    assert e_ge <= U.TIGHT[dtype] and e_go <= U.TIGHT[dtype] + e_oe, (e_go, e_ge, e_oe)
+
+
+@pytest.mark.parametrize("p", [1, 2])
+def test_lp_norm_reference_literals_on_device(K, p):
+    # test/dragon/test_ops.py:4480-4512
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_test_vectors.json")) as f:
+        g = json.load(f)["lp_norm"]
+    data1 = np.arange(6, dtype=np.float32)
+    data2 = (np.arange(6, dtype=np.float32) / 10 + 1).astype(np.float32)
+    for e in g["entries"]:
+        if e["p"] != p:
+            continue
+        normalizer = 6.0 if e["reduction"] == "mean" else 1.0
+        xd, dyd = U.to_device(data1, "float32"), U.to_device(data2, "float32")
+        y, dx = empty((6,), "float32"), empty((6,), "float32")
+        (K.l1_norm if p == 1 else K.l2_norm)(1, 1, 6, normalizer, e["eps"], xd, y)
+        (K.l1_norm_grad if p == 1 else K.l2_norm_grad)(1, 1, 6, normalizer, e["eps"], dyd, xd, dx)
+        norm = np.abs(data1) if p == 1 else np.square(data1)
+        norm = norm.sum() if e["reduction"] == "sum" else norm.mean()
+        norm = norm if p == 1 else np.sqrt(norm)
+        assert np.max(np.abs(U.to_host(y) - data1 / max(norm, e["eps"]))) <= g["prec"]
+        assert np.max(np.abs(U.to_host(dx) - np.array(e["dx"], np.float32))) <= g["prec"]
+
+
+def test_lp_norm_in_place_epsilon_clamp_and_empty(K):
+    x = np.zeros((4, 512), np.float32)
+    x[1] = np.linspace(-1, 1, 512)
+    x[2, 7] = 3.0
+    dy = np.ones((4, 512), np.float32)
+    y_ref = R.op_lp_norm("float32", x, -1, None, 2, 0.5, "sum")
+    dx_ref = R.op_lp_norm_grad("float32", x, dy, -1, None, 2, 0.5, "sum")
+    buf, g = U.to_device(x, "float32"), U.to_device(dy, "float32")
+    K.l2_norm_grad(4, 1, 512, 1.0, 0.5, g, buf, g)   # dX aliases dY
+    K.l2_norm(4, 1, 512, 1.0, 0.5, buf, buf)         # Y aliases X
+    assert U.normwise(U.to_host(buf), y_ref) <= 1e-6
+    assert U.normwise(U.to_host(g), dx_ref) <= 1e-6
+    assert np.all(U.to_host(buf)[0] == 0)            # 0 / max(0, eps)
+    e = empty((0, 8), "float32")
+    K.l1_norm(0, 1, 8, 1.0, 1e-12, e, e)             # no rows: nothing to do, no error

@@ -76,6 +76,33 @@ def test_log_softmax(rt, ws):
     assert_equal(ws.fetch(dx), g["dx_with_dy_eq_x"], g["prec"])
 
 
+def test_lp_norm(rt, ws):
+    g = GOLD["lp_norm"]
+    for e in g["entries"]:
+        data1, data2 = arange((6,)), arange((6,)) / 10 + 1
+        tape = rt.Tape(ws)
+        x, dy = ws.feed("x", data1), ws.feed("dy", data2)
+        y = rt.lp_norm(tape, [x], e["axis"], p=e["p"], epsilon=e["eps"], reduction=e["reduction"])
+        (dx,) = tape.gradient(y, [x], output_gradient=dy)
+        norm = np.abs(data1) if e["p"] == 1 else np.square(data1)
+        norm = norm.sum() if e["reduction"] == "sum" else norm.mean()
+        norm = norm if e["p"] == 1 else np.sqrt(norm)
+        assert_equal(ws.fetch(y), data1 / max(norm, e["eps"]), g["prec"])
+        assert_equal(ws.fetch(dx), e["dx"], g["prec"])
+
+
+def test_lp_norm_axis_range_and_bad_order(rt, ws):
+    rng = np.random.default_rng(3)
+    data = rng.standard_normal((3, 4, 5, 6)).astype("float32")
+    x = ws.feed("x", data)
+    tape = rt.Tape(ws)
+    y = rt.lp_norm(tape, [x], axis=1, end_axis=2, p=2, reduction="mean")
+    norm = np.sqrt(np.square(data.astype(np.float64)).mean((1, 2), keepdims=True))
+    assert_equal(ws.fetch(y), data / norm, 1e-5)
+    with pytest.raises(rt.DragonError, match="Unsupported order"):
+        ws.run_operator(rt.make_def("LpNorm", [x], ["y_bad"], p=3))
+
+
 def test_layer_norm(rt, ws):
     g = GOLD["layer_norm"]
     x_shape, w_shape = tuple(g["x_shape"]), (g["x_shape"][-1],)

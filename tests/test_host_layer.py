@@ -20,7 +20,8 @@ def test_registry_holds_the_ten_operator_types_and_the_sync_aliases():
     ops = set(rt.registered_operators())
     assert {"LayerNorm", "LayerNormGradient", "GroupNorm", "GroupNormGradient", "BatchNorm",
             "BatchNormGradient", "Softmax", "SoftmaxGradient", "LogSoftmax",
-            "LogSoftmaxGradient", "SyncBatchNorm", "SyncBatchNormGradient"} <= ops
+            "LogSoftmaxGradient", "SyncBatchNorm", "SyncBatchNormGradient", "LpNorm",
+            "LpNormGradient"} <= ops
 
 
 def test_feed_fetch_round_trip(ws):

@@ -416,3 +416,62 @@ def test_inv_std_and_axpby_closed_forms():
     # exactly: round(round(0.9f*y) + round(0.1f*x))
     expect = (np.float32(0.9) * y0).astype(np.float32) + (np.float32(0.1) * x).astype(np.float32)
     assert np.array_equal(y, expect.astype(np.float32))
+
+
+# ---------------------------------------------------------------- lp norm
+
+@pytest.mark.parametrize("idx", range(4))
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_lp_norm_reference_literals(idx, dtype):
+    g = GOLD["lp_norm"]
+    e = g["entries"][idx]
+    data1 = arange(tuple(g["x_shape"])).astype(dtype)
+    data2 = (arange(tuple(g["x_shape"])) / 10 + 1).astype(dtype)
+    y = R.op_lp_norm(dtype, data1, e["axis"], None, e["p"], e["eps"], e["reduction"])
+    dx = R.op_lp_norm_grad(dtype, data1, data2, e["axis"], None, e["p"], e["eps"], e["reduction"])
+    norm = np.abs(data1) if e["p"] == 1 else np.square(data1)
+    norm = norm.sum() if e["reduction"] == "sum" else norm.mean()
+    norm = norm if e["p"] == 1 else np.sqrt(norm)
+    assert maxabs(y, data1 / max(norm, e["eps"])) <= g["prec"]
+    assert maxabs(dx, e["dx"]) <= g["prec"]
+
+
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("reduction", ["sum", "mean"])
+@pytest.mark.parametrize("shape,axis,end_axis", [((5, 7), -1, None), ((3, 6, 4), 1, None),
+                                                 ((2, 3, 4, 5), 1, 2), ((4, 1), -1, None)])
+def test_lp_norm_vs_fp64_bruteforce(p, reduction, shape, axis, end_axis):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(shape).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    eps = 1e-12
+    a = axis % len(shape)
+    b = a if end_axis is None else end_axis
+    red = tuple(range(a, b + 1))
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    n = float(np.prod([shape[i] for i in red])) if reduction == "mean" else 1.0
+    if p == 1:
+        norm = np.maximum(np.abs(x64).sum(red, keepdims=True) / n, eps)
+        dx64 = dy64 / norm - np.sign(x64) * ((dy64 * x64).sum(red, keepdims=True) / n) / norm ** 2
+    else:
+        norm = np.maximum(np.sqrt(np.square(x64).sum(red, keepdims=True) / n), eps)
+        dx64 = dy64 / norm - x64 * ((dy64 * x64).sum(red, keepdims=True) / n) / norm ** 3
+    y = R.op_lp_norm("float32", x, axis, end_axis, p, eps, reduction)
+    dx = R.op_lp_norm_grad("float32", x, dy, axis, end_axis, p, eps, reduction)
+    scale = float(np.max(np.abs(dy64 / norm)))  # size of the terms that cancel in dx
+    assert maxabs(y, x64 / norm) < 2e-6 * (float(np.max(np.abs(x64 / norm))) + 1e-30)
+    assert maxabs(dx, dx64) < 5e-6 * scale
+
+
+def test_lp_norm_epsilon_clamp_and_zero_rows():
+    x = np.zeros((2, 4), np.float32)
+    x[1] = [3.0, -4.0, 0.0, 0.0]
+    dy = np.ones((2, 4), np.float32)
+    y = R.op_lp_norm("float32", x, -1, None, 2, 0.5, "sum")
+    assert np.all(y[0] == 0.0)                       # 0 / max(0, eps)
+    assert maxabs(y[1], x[1] / 5.0) < 1e-7
+    dx = R.op_lp_norm_grad("float32", x, dy, -1, None, 2, 0.5, "sum")
+    assert maxabs(dx[0], dy[0] / 0.5) < 1e-7          # sum == 0: second term vanishes
+    # d/dx of x/|x| is orthogonal to x when dy is parallel to x
+    dxp = R.op_lp_norm_grad("float32", x[1:], x[1:].copy(), -1, None, 2, 1e-12, "sum")
+    assert maxabs(dxp, 0.0) < 1e-6
