@@ -121,6 +121,29 @@ def wl_lp_norm(N, C, dtype_name, p=2, seed=5):
     return kernels, {"rows": N, "width": C}
 
 
+def wl_softmax_cross_entropy(N, C, seed=6):
+    """fp32 logits [N, C], int64 class indices, VALID reduction, 1 in 16 targets ignored."""
+    import torch
+    from dragon_amd import kernels as K
+    gen = _gen(seed)
+    x = _randn((N, C), torch.float32, gen, scale=2.0)
+    target = torch.randint(0, C, (N,), generator=gen, device="cuda", dtype=torch.int64)
+    target[::16] = 255 if C > 255 else -1
+    ignore = 255 if C > 255 else -1
+    prob, dx = torch.empty_like(x), torch.empty_like(x)
+    loss, dl = torch.empty(1, device="cuda"), torch.ones(1, device="cuda")
+    nbytes = x.numel() * 4
+    kernels = [
+        ("softmax_cross_entropy_loss_forward",
+         lambda: K.softmax_cross_entropy_loss_forward(N, 1, C, ignore, "valid", x, target, prob, loss),
+         2 * nbytes + N * 8),
+        ("softmax_cross_entropy_loss_backward",
+         lambda: K.softmax_cross_entropy_loss_backward(N, 1, C, ignore, "valid", prob, target, dl, dx),
+         2 * nbytes + N * 8),
+    ]
+    return kernels, {"rows": N, "width": C}
+
+
 def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False):
     import torch
     from dragon_amd import kernels as K
@@ -223,6 +246,7 @@ WORKLOADS = {
     "softmax_f16_8192x4096": lambda: wl_softmax((8192, 4096), "float16", 1),
     "softmax_f32_8192x4096": lambda: wl_softmax((8192, 4096), "float32", 1),
     # sibling row reductions on the same skeleton
+    "softmax_cross_entropy_f32_8192x4096": lambda: wl_softmax_cross_entropy(8192, 4096),
     "l2_norm_bf16_8192x4096": lambda: wl_lp_norm(8192, 4096, "bfloat16", 2),
     "l2_norm_f32_8192x4096": lambda: wl_lp_norm(8192, 4096, "float32", 2),
 }

@@ -45,6 +45,11 @@ SIGNATURES = {
     "dragon_hip_sub": (_int, [_int, _i64, _vp, _vp, _vp, _vp]),
     "dragon_hip_moments_scratch_bytes": (_sz, [_int, _int, _i64p, _int, _i64p]),
     "dragon_hip_moments": (_int, [_int, _int, _i64p, _int, _i64p, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_reduce_scratch_bytes": (_sz, [_int, _int, _i64p, _int, _i64p]),
+    "dragon_hip_reduce_sum": (_int, [_int, _int, _i64p, _int, _i64p, _f32, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_reduce_sum_sqr": (_int, [_int, _int, _i64p, _int, _i64p, _f32, _vp, _vp, _vp, _sz,
+                                         _vp]),
+    "dragon_hip_reduce_l1": (_int, [_int, _int, _i64p, _int, _i64p, _f32, _vp, _vp, _vp, _sz, _vp]),
     "dragon_hip_layer_norm": (_int, [_int, _i64, _i64, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dragon_hip_group_norm": (_int, [_int, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp,
                                      _vp, _vp]),
@@ -70,6 +75,22 @@ SIGNATURES = {
     "dragon_hip_l2_norm": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp]),
     "dragon_hip_l1_norm_grad": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp, _vp]),
     "dragon_hip_l2_norm_grad": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp, _vp]),
+    "dragon_hip_cross_entropy": (_int, [_int, _i64, _vp, _vp, _vp, _vp]),
+    "dragon_hip_sparse_cross_entropy": (_int, [_int, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp,
+                                               _vp, _vp]),
+    "dragon_hip_softmax_cross_entropy_grad": (_int, [_int, _int, _i64, _i64, _i64, _i64, _vp, _vp,
+                                                     _vp, _vp, _vp]),
+    "dragon_hip_reduce_loss_scratch_bytes": (_sz, [_int]),
+    "dragon_hip_reduce_loss": (_int, [_int, _i64, _i64, _f32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_reduce_loss_grad": (_int, [_int, _i64, _i64, _f32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_broadcast_loss_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "dragon_hip_softmax_cross_entropy_loss_scratch_bytes": (_sz, [_int, _i64, _i64]),
+    "dragon_hip_softmax_cross_entropy_loss_forward": (_int, [_int, _int, _i64, _i64, _i64, _i64,
+                                                             _int, _vp, _vp, _vp, _vp, _vp, _sz,
+                                                             _vp]),
+    "dragon_hip_softmax_cross_entropy_loss_backward": (_int, [_int, _int, _i64, _i64, _i64, _i64,
+                                                              _int, _vp, _vp, _vp, _vp, _vp, _sz,
+                                                              _vp]),
     "dragon_hip_group_norm_forward_scratch_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int]),
     "dragon_hip_group_norm_forward": (_int, [_int, _i64, _i64, _i64, _i64, _int, _f32, _vp, _vp,
                                              _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -1,0 +1,724 @@
+// Softmax cross-entropy loss kernels for gfx950.
+//
+// Replaces, for float and double (dtypes::Loss, dragon/core/types.h:90):
+//   kernels::CrossEntropy (dense and sparse targets), SoftmaxCrossEntropyGrad
+//     dragon/kernels/loss/op_kernels.h:51-69,179-189;
+//     CPU dragon/kernels/loss/cpu/cross_entropy_kernel.cc:10-42,80-108
+//   kernels::ReduceLoss, ReduceLossGrad, BroadcastLossGrad
+//     dragon/kernels/loss/op_kernels.h:25-32,95-113;
+//     CPU dragon/kernels/loss/cpu/generic_loss_kernel.cc:10-73
+// and fuses the bodies of SoftmaxCrossEntropyLossOp / ...GradientOp
+// (dragon/operators/loss/cross_entropy_softmax_loss_op.cc:8-143) for sparse
+// targets:
+//   forward   one pass over the logits writes the probabilities (the op's
+//             "X_norm" output), the per-position loss and the validity mask,
+//             where the reference runs Softmax, then a gather kernel;
+//   backward  one pass over the probabilities writes
+//             dx = (p - onehot(target)) * mask * scale, where the reference
+//             copies p, patches it per position and rescales it (three passes).
+//
+// A target outside [0, C) that is not ignore_index is treated as ignored
+// (loss 0, mask 0, zero gradient); the reference would read out of bounds.
+#include <cfloat>
+
+#include "row_tile.h"
+
+namespace dragon_hip {
+namespace {
+
+constexpr int kLossThreads = 256;
+constexpr int kLossWaves = kLossThreads / kWaveSize;
+constexpr int kMaxPartials = 1024;  // stage-one workgroups of a loss reduction
+
+template <typename A>
+__device__ __forceinline__ A neg_log_clamped(A p) {
+  const A lo = static_cast<A>(FLT_MIN);
+  return -acc_log(p > lo ? p : lo);
+}
+
+// ------------------------------------------------------------------ CrossEntropy
+
+template <typename T>
+__global__ __launch_bounds__(kLossThreads) void cross_entropy_dense(
+    const int64_t N, const T* __restrict__ input, const T* __restrict__ target,
+    T* __restrict__ loss) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < N;
+       i += static_cast<int64_t>(gridDim.x) * kLossThreads) {
+    loss[i] = target[i] * neg_log_clamped(input[i]);
+  }
+}
+
+template <typename TargetT>
+__device__ __forceinline__ bool target_valid(TargetT tgt, int64_t ignore_index, int64_t C) {
+  const int64_t t = static_cast<int64_t>(tgt);
+  return t != ignore_index && t >= 0 && t < C;
+}
+
+template <typename T, typename TargetT>
+__global__ __launch_bounds__(kLossThreads) void cross_entropy_sparse(
+    const int64_t NxS, const int64_t S, const int64_t C, const int64_t ignore_index,
+    const T* __restrict__ input, const TargetT* __restrict__ target, T* __restrict__ loss,
+    T* __restrict__ mask) {
+  for (int64_t index = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x;
+       index < NxS; index += static_cast<int64_t>(gridDim.x) * kLossThreads) {
+    const int64_t i = index / S, j = index - i * S;
+    const TargetT tgt = target[index];
+    if (target_valid(tgt, ignore_index, C)) {
+      loss[index] = neg_log_clamped(input[(i * C + static_cast<int64_t>(tgt)) * S + j]);
+      mask[index] = T(1);
+    } else {
+      loss[index] = mask[index] = T(0);
+    }
+  }
+}
+
+// S > 1: a thread per (n, s) position, neighbouring threads neighbouring s.
+template <typename T, typename TargetT>
+__global__ __launch_bounds__(kLossThreads) void softmax_ce_grad_positions(
+    const int64_t NxS, const int64_t S, const int64_t C, const int64_t ignore_index,
+    const TargetT* __restrict__ target, T* __restrict__ dx, T* __restrict__ mask) {
+  for (int64_t index = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x;
+       index < NxS; index += static_cast<int64_t>(gridDim.x) * kLossThreads) {
+    const int64_t i = index / S, j = index - i * S;
+    const TargetT tgt = target[index];
+    if (target_valid(tgt, ignore_index, C)) {
+      dx[(i * C + static_cast<int64_t>(tgt)) * S + j] -= T(1);
+      mask[index] = T(1);
+    } else {
+      T* col = dx + i * C * S + j;
+      for (int64_t k = 0; k < C; ++k) col[k * S] = T(0);
+      mask[index] = T(0);
+    }
+  }
+}
+
+// S == 1: a wavefront per row, so that an ignored row is cleared with
+// coalesced stores.
+template <typename T, typename TargetT>
+__global__ __launch_bounds__(kLossThreads) void softmax_ce_grad_rows(
+    const int64_t N, const int64_t C, const int64_t ignore_index,
+    const TargetT* __restrict__ target, T* __restrict__ dx, T* __restrict__ mask) {
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * kLossWaves + threadIdx.x / kWaveSize;
+       row < N; row += static_cast<int64_t>(gridDim.x) * kLossWaves) {
+    const TargetT tgt = target[row];
+    if (target_valid(tgt, ignore_index, C)) {
+      if (lane == 0) {
+        dx[row * C + static_cast<int64_t>(tgt)] -= T(1);
+        mask[row] = T(1);
+      }
+    } else {
+      for (int64_t k = lane; k < C; k += kWaveSize) dx[row * C + k] = T(0);
+      if (lane == 0) mask[row] = T(0);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ loss reductions
+
+template <typename T, int kWaves = kLossWaves>
+__device__ __forceinline__ T block_sum(T v, T* lds /*kWaves*/) {
+  v = wave_allreduce(v, SumOp());
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) lds[threadIdx.x / kWaveSize] = v;
+  __syncthreads();
+  T r = lds[0];
+#pragma unroll
+  for (int i = 1; i < kWaves; ++i) r += lds[i];
+  __syncthreads();
+  return r;
+}
+
+// Stage one: workgroup b adds its slice of x[0, n_x) and of mask[0, n_mask)
+// and writes partial[2b], partial[2b+1]. Either array may be absent (n == 0).
+template <typename T>
+__global__ __launch_bounds__(kLossThreads) void loss_partial_sums(
+    const int64_t n_x, const T* __restrict__ x, const int64_t n_mask, const T* __restrict__ mask,
+    T* __restrict__ partial) {
+  __shared__ T lds[kLossWaves];
+  T a = T(0), b = T(0);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kLossThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < n_x;
+       i += stride)
+    a += x[i];
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < n_mask;
+       i += stride)
+    b += mask[i];
+  a = block_sum(a, lds);
+  b = block_sum(b, lds);
+  if (threadIdx.x == 0) {
+    partial[2 * blockIdx.x] = a;
+    partial[2 * blockIdx.x + 1] = b;
+  }
+}
+
+// Stage one of counting valid targets: partial[2b] = 0, partial[2b+1] = count.
+template <typename T, typename TargetT>
+__global__ __launch_bounds__(kLossThreads) void valid_target_partial_counts(
+    const int64_t NxS, const int64_t C, const int64_t ignore_index,
+    const TargetT* __restrict__ target, T* __restrict__ partial) {
+  __shared__ T lds[kLossWaves];
+  T b = T(0);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < NxS;
+       i += static_cast<int64_t>(gridDim.x) * kLossThreads)
+    b += target_valid(target[i], ignore_index, C) ? T(1) : T(0);
+  b = block_sum(b, lds);
+  if (threadIdx.x == 0) {
+    partial[2 * blockIdx.x] = T(0);
+    partial[2 * blockIdx.x + 1] = b;
+  }
+}
+
+// Stage two (one workgroup): totals of the partial pairs in index order, then
+//   kReduce   y[0] = sum_x * (1 / max(inv_scale, 1))              (ReduceLoss)
+//   kGradScale  y[0] = dl[0] / max(inv_scale, 0.5)                (ReduceLossGrad)
+// with inv_scale = sum_mask when `by_mask`, else `normalizer`.
+enum LossFinal { kReduce = 0, kGradScale = 1 };
+template <typename T, int kMode>
+__global__ __launch_bounds__(kLossThreads) void loss_finalize(
+    const int nparts, const T* __restrict__ partial, const bool by_mask, const float normalizer,
+    const T* __restrict__ dl, T* __restrict__ y) {
+  __shared__ T lds[kLossWaves];
+  T a = T(0), b = T(0);
+  for (int i = threadIdx.x; i < nparts; i += kLossThreads) {
+    a += partial[2 * i];
+    b += partial[2 * i + 1];
+  }
+  a = block_sum(a, lds);
+  b = block_sum(b, lds);
+  if (threadIdx.x == 0) {
+    const float inv_scale = by_mask ? static_cast<float>(b) : normalizer;
+    if (kMode == kReduce) {
+      const float scale = 1.f / (inv_scale > 1.f ? inv_scale : 1.f);
+      y[0] = a * static_cast<T>(scale);
+    } else {
+      y[0] = static_cast<T>(static_cast<float>(dl[0]) / (inv_scale > 0.5f ? inv_scale : 0.5f));
+    }
+  }
+}
+
+// Both stages in one workgroup, for reductions short enough that a second
+// launch would cost more than the loop: sums x[0, n_x) and mask[0, n_mask)
+// (or, with kCountTargets, counts the valid targets) and applies the epilogue
+// of loss_finalize.
+constexpr int kDirectThreads = 1024;
+constexpr int64_t kDirectReduceMax = 16 * 1024;
+template <typename T, typename TargetT, int kMode, bool kCountTargets>
+__global__ __launch_bounds__(kDirectThreads) void loss_reduce_direct(
+    const int64_t n_x, const T* __restrict__ x, const int64_t n_mask, const T* __restrict__ mask,
+    const TargetT* __restrict__ target, const int64_t C, const int64_t ignore_index,
+    const bool by_mask, const float normalizer, const T* __restrict__ dl, T* __restrict__ y) {
+  constexpr int kWaves = kDirectThreads / kWaveSize;
+  constexpr int kSteps = static_cast<int>(kDirectReduceMax / kDirectThreads);
+  __shared__ T lds[kWaves];
+  T a = T(0), b = T(0);
+  // fixed trip count with guarded, independent loads: all of them are in flight at once
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) {
+    const int64_t i = static_cast<int64_t>(k) * kDirectThreads + threadIdx.x;
+    if (i < n_x) a += x[i];
+    if (i < n_mask) {
+      if constexpr (kCountTargets) {
+        b += target_valid(target[i], ignore_index, C) ? T(1) : T(0);
+      } else {
+        b += mask[i];
+      }
+    }
+  }
+  a = block_sum<T, kWaves>(a, lds);
+  b = block_sum<T, kWaves>(b, lds);
+  if (threadIdx.x == 0) {
+    const float inv_scale = by_mask ? static_cast<float>(b) : normalizer;
+    if (kMode == kReduce) {
+      const float scale = 1.f / (inv_scale > 1.f ? inv_scale : 1.f);
+      y[0] = a * static_cast<T>(scale);
+    } else {
+      y[0] = static_cast<T>(static_cast<float>(dl[0]) / (inv_scale > 0.5f ? inv_scale : 0.5f));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLossThreads) void scale_by_device_scalar(
+    const int64_t N, const T* __restrict__ scale, T* __restrict__ dx) {
+  const T alpha = scale[0];
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < N;
+       i += static_cast<int64_t>(gridDim.x) * kLossThreads)
+    dx[i] *= alpha;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLossThreads) void broadcast_loss_grad(
+    const int64_t NxCxS, const int64_t CxS, const int64_t S, const T* __restrict__ dl,
+    T* __restrict__ dx) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; i < NxCxS;
+       i += static_cast<int64_t>(gridDim.x) * kLossThreads)
+    dx[i] *= dl[i / CxS * S + i % S];
+}
+
+// ------------------------------------------------------------------ fused forward (S == 1)
+
+// softmax_rows with the loss gather folded in: the thread whose tile slot holds
+// column `target[row]` writes -log(max(p, FLT_MIN)).
+template <typename T, typename TargetT, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void softmax_ce_rows(
+    const int64_t N, const int C, const int64_t ignore_index, const T* __restrict__ x,
+    const TargetT* __restrict__ target, T* __restrict__ prob, T* __restrict__ loss,
+    T* __restrict__ mask) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const int npackets = C / kVec;
+
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Tile t;
+    t.load(x + row * C, npackets, acc_neg_inf<A>());
+    const TargetT tgt = target[row];
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) m = MaxOp()(m, t.v[i][e]);
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = acc_exp(t.v[i][e] - m);
+        s += t.v[i][e];
+      }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    const bool valid = target_valid(tgt, ignore_index, C);
+    const int col = valid ? static_cast<int>(tgt) : -1;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = t.v[i][e] / s;
+        if ((i * kTPR + Tile::lane()) * kVec + e == col) {
+          loss[row] = neg_log_clamped(t.v[i][e]);
+          mask[row] = T(1);
+        }
+      }
+    if (!valid && Tile::lane() == 0) loss[row] = mask[row] = T(0);
+    t.store(prob + row * C, npackets);
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------ fused backward
+
+// dx = (p - [k == target]) * w over [N, C, S], with w = 0 where the target is
+// ignored, else dl[n * S + s] (kPerPosition) or the scalar scale[0]. kAlongC:
+// the packet runs along C (S == 1), else along S.
+template <typename T, typename TargetT, int kVec, bool kAlongC, bool kPerPosition>
+__global__ __launch_bounds__(kLossThreads) void softmax_ce_backward(
+    const int64_t npackets, const int64_t S, const int64_t C, const int64_t ignore_index,
+    const T* __restrict__ prob, const TargetT* __restrict__ target, const T* __restrict__ dl,
+    const T* __restrict__ scale, T* __restrict__ dx) {
+  using A = typename IO<T>::Acc;
+  const A alpha = kPerPosition ? A(0) : static_cast<A>(scale[0]);
+  for (int64_t ip = static_cast<int64_t>(blockIdx.x) * kLossThreads + threadIdx.x; ip < npackets;
+       ip += static_cast<int64_t>(gridDim.x) * kLossThreads) {
+    const int64_t i = ip * kVec;
+    A v[kVec];
+    if constexpr (kVec == 1) {
+      v[0] = IO<T>::load1(prob + i);
+    } else {
+      load_unpack<T>(prob + i, v);
+    }
+    if constexpr (kAlongC) {
+      const int64_t n = i / C, k0 = i - n * C;
+      const TargetT tgt = target[n];
+      const bool valid = target_valid(tgt, ignore_index, C);
+      const A w = valid ? (kPerPosition ? static_cast<A>(dl[n]) : alpha) : A(0);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A hot = (valid && k0 + e == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+        v[e] = (v[e] - hot) * w;
+      }
+    } else {
+      const int64_t n = i / (C * S);
+      const int64_t rem = i - n * C * S;
+      const int64_t k = rem / S, s0 = rem - k * S;
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const int64_t pos = n * S + s0 + e;
+        const TargetT tgt = target[pos];
+        const bool valid = target_valid(tgt, ignore_index, C);
+        const A w = valid ? (kPerPosition ? static_cast<A>(dl[pos]) : alpha) : A(0);
+        const A hot = (valid && k == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+        v[e] = (v[e] - hot) * w;
+      }
+    }
+    if constexpr (kVec == 1) {
+      IO<T>::store1(dx + i, v[0]);
+    } else {
+      pack_store<T>(dx + i, v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ launchers
+
+inline unsigned loss_grid(int64_t work_items) {
+  const int64_t want = ceil_div(work_items, kLossThreads);
+  const int64_t cap = static_cast<int64_t>(kNumCUs) * 32;
+  return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
+}
+
+// Stage-one workgroups of a reduction over n elements (at most kMaxPartials).
+inline int partial_blocks(int64_t n) {
+  const int64_t want = ceil_div(n, static_cast<int64_t>(kLossThreads) * 8);
+  return static_cast<int>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+}
+
+// Scratch of a loss reduction: the partial pairs plus one scalar.
+inline size_t reduce_loss_scratch(size_t elem) { return (2 * kMaxPartials + 1) * elem; }
+
+template <typename T>
+int launch_cross_entropy(int64_t N, const void* input, const void* target, void* loss,
+                         hipStream_t stream) {
+  hipLaunchKernelGGL((cross_entropy_dense<T>), dim3(loss_grid(N)), dim3(kLossThreads), 0, stream,
+                     N, static_cast<const T*>(input), static_cast<const T*>(target),
+                     static_cast<T*>(loss));
+  return status_of_launch();
+}
+
+template <typename T, typename TargetT>
+int launch_sparse_cross_entropy(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
+                                const void* input, const void* target, void* loss, void* mask,
+                                hipStream_t stream) {
+  hipLaunchKernelGGL((cross_entropy_sparse<T, TargetT>), dim3(loss_grid(N * S)),
+                     dim3(kLossThreads), 0, stream, N * S, S, C, ignore_index,
+                     static_cast<const T*>(input), static_cast<const TargetT*>(target),
+                     static_cast<T*>(loss), static_cast<T*>(mask));
+  return status_of_launch();
+}
+
+template <typename T, typename TargetT>
+int launch_softmax_ce_grad(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
+                           const void* target, void* dx, void* mask, hipStream_t stream) {
+  const TargetT* tp = static_cast<const TargetT*>(target);
+  if (S == 1) {
+    hipLaunchKernelGGL((softmax_ce_grad_rows<T, TargetT>), dim3(loss_grid(N * kWaveSize)),
+                       dim3(kLossThreads), 0, stream, N, C, ignore_index, tp, static_cast<T*>(dx),
+                       static_cast<T*>(mask));
+  } else {
+    hipLaunchKernelGGL((softmax_ce_grad_positions<T, TargetT>), dim3(loss_grid(N * S)),
+                       dim3(kLossThreads), 0, stream, N * S, S, C, ignore_index, tp,
+                       static_cast<T*>(dx), static_cast<T*>(mask));
+  }
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_reduce_loss(int64_t N, int64_t num_masks, float normalizer, const void* x,
+                       const void* mask, void* y, void* scratch, hipStream_t stream) {
+  const bool by_mask = num_masks > 0 && normalizer < 0.f;
+  T* part = static_cast<T*>(scratch);
+  const int64_t n_mask = by_mask ? num_masks : 0;
+  if (N <= kDirectReduceMax && n_mask <= kDirectReduceMax) {
+    hipLaunchKernelGGL((loss_reduce_direct<T, int32_t, kReduce, false>), dim3(1),
+                       dim3(kDirectThreads), 0, stream, N, static_cast<const T*>(x), n_mask,
+                       static_cast<const T*>(mask), static_cast<const int32_t*>(nullptr),
+                       static_cast<int64_t>(0), static_cast<int64_t>(0), by_mask, normalizer,
+                       static_cast<const T*>(nullptr), static_cast<T*>(y));
+    return status_of_launch();
+  }
+  const int nparts = partial_blocks(N > n_mask ? N : n_mask);
+  hipLaunchKernelGGL((loss_partial_sums<T>), dim3(nparts), dim3(kLossThreads), 0, stream, N,
+                     static_cast<const T*>(x), n_mask, static_cast<const T*>(mask), part);
+  hipLaunchKernelGGL((loss_finalize<T, kReduce>), dim3(1), dim3(kLossThreads), 0, stream, nparts,
+                     part, by_mask, normalizer, static_cast<const T*>(nullptr),
+                     static_cast<T*>(y));
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_reduce_loss_grad(int64_t N, int64_t num_masks, float normalizer, const void* dl,
+                            const void* mask, void* dx, void* scratch, hipStream_t stream) {
+  const bool by_mask = num_masks > 0 && normalizer < 0.f;
+  T* part = static_cast<T*>(scratch);
+  T* scalar = part + 2 * kMaxPartials;
+  if (!by_mask || num_masks <= kDirectReduceMax) {
+    hipLaunchKernelGGL((loss_reduce_direct<T, int32_t, kGradScale, false>), dim3(1),
+                       dim3(kDirectThreads), 0, stream, static_cast<int64_t>(0),
+                       static_cast<const T*>(nullptr), by_mask ? num_masks : static_cast<int64_t>(0),
+                       static_cast<const T*>(mask), static_cast<const int32_t*>(nullptr),
+                       static_cast<int64_t>(0), static_cast<int64_t>(0), by_mask, normalizer,
+                       static_cast<const T*>(dl), scalar);
+  } else {
+    const int nparts = partial_blocks(num_masks);
+    hipLaunchKernelGGL((loss_partial_sums<T>), dim3(nparts), dim3(kLossThreads), 0, stream,
+                       static_cast<int64_t>(0), static_cast<const T*>(nullptr), num_masks,
+                       static_cast<const T*>(mask), part);
+    hipLaunchKernelGGL((loss_finalize<T, kGradScale>), dim3(1), dim3(kLossThreads), 0, stream,
+                       nparts, part, by_mask, normalizer, static_cast<const T*>(dl), scalar);
+  }
+  hipLaunchKernelGGL((scale_by_device_scalar<T>), dim3(loss_grid(N)), dim3(kLossThreads), 0,
+                     stream, N, scalar, static_cast<T*>(dx));
+  return status_of_launch();
+}
+
+template <typename T>
+int launch_broadcast_loss_grad(int64_t N, int64_t S, int64_t C, const void* dl, void* dx,
+                               hipStream_t stream) {
+  hipLaunchKernelGGL((broadcast_loss_grad<T>), dim3(loss_grid(N * C * S)), dim3(kLossThreads), 0,
+                     stream, N * C * S, C * S, S, static_cast<const T*>(dl), static_cast<T*>(dx));
+  return status_of_launch();
+}
+
+enum Reduction { kNone = 0, kSum = 1, kMean = 2, kBatchMean = 3, kValid = 4 };
+
+// The normalizer the operator bodies derive from the reduction
+// (cross_entropy_softmax_loss_op.cc:69-78); -1 selects the mask count.
+inline float loss_normalizer(int reduction, int64_t N, int64_t S, bool has_mask) {
+  switch (reduction) {
+    case kValid: return has_mask ? -1.f : static_cast<float>(N * S);
+    case kBatchMean: return static_cast<float>(N);
+    case kMean: return static_cast<float>(N * S);
+    default: return 1.f;
+  }
+}
+
+template <typename T, typename TargetT>
+int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, int reduction,
+                         const void* x, const void* target, void* prob, void* out, void* scratch,
+                         hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const T* xp = static_cast<const T*>(x);
+  const TargetT* tp = static_cast<const TargetT*>(target);
+  T* pp = static_cast<T*>(prob);
+  const int64_t NxS = N * S;
+  // reduction == NONE writes the per-position loss straight to the output
+  T* loss = reduction == kNone ? static_cast<T*>(out) : static_cast<T*>(scratch);
+  T* mask = static_cast<T*>(scratch) + NxS;
+  T* part = mask + NxS;
+  RowConfig cfg;
+  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(prob) &&
+      pick_row_config(C / kVec, 8, &cfg)) {
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    using Tile = RowTile<T, TPR, VPT>;                                                          \
+    hipLaunchKernelGGL((softmax_ce_rows<T, TargetT, TPR, VPT>),                                 \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       N, static_cast<int>(C), ignore_index, xp, tp, pp, loss, mask);           \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+  } else {
+    const int st = dragon_hip_softmax(sizeof(T) == 8 ? DRAGON_HIP_F64 : DRAGON_HIP_F32, N, S, C, x, prob, stream);
+    if (st != DRAGON_HIP_OK) return st;
+    hipLaunchKernelGGL((cross_entropy_sparse<T, TargetT>), dim3(loss_grid(NxS)),
+                       dim3(kLossThreads), 0, stream, NxS, S, C, ignore_index, pp, tp, loss, mask);
+  }
+  if (reduction != kNone) {
+    const float normalizer = loss_normalizer(reduction, N, S, true);
+    const bool by_mask = normalizer < 0.f;
+    const int64_t n_mask = by_mask ? NxS : static_cast<int64_t>(0);
+    if (NxS <= kDirectReduceMax) {
+      hipLaunchKernelGGL((loss_reduce_direct<T, TargetT, kReduce, false>), dim3(1),
+                         dim3(kDirectThreads), 0, stream, NxS, loss, n_mask, mask,
+                         static_cast<const TargetT*>(nullptr), static_cast<int64_t>(0),
+                         static_cast<int64_t>(0), by_mask, normalizer,
+                         static_cast<const T*>(nullptr), static_cast<T*>(out));
+    } else {
+      const int nparts = partial_blocks(NxS);
+      hipLaunchKernelGGL((loss_partial_sums<T>), dim3(nparts), dim3(kLossThreads), 0, stream, NxS,
+                         loss, n_mask, mask, part);
+      hipLaunchKernelGGL((loss_finalize<T, kReduce>), dim3(1), dim3(kLossThreads), 0, stream,
+                         nparts, part, by_mask, normalizer, static_cast<const T*>(nullptr),
+                         static_cast<T*>(out));
+    }
+  }
+  return status_of_launch();
+}
+
+template <typename T, typename TargetT>
+int launch_fused_backward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, int reduction,
+                          const void* prob, const void* target, const void* dl, void* dx,
+                          void* scratch, hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const T* pp = static_cast<const T*>(prob);
+  const TargetT* tp = static_cast<const TargetT*>(target);
+  const T* dlp = static_cast<const T*>(dl);
+  T* dp = static_cast<T*>(dx);
+  T* part = static_cast<T*>(scratch);
+  T* scalar = part + 2 * kMaxPartials;
+  const int64_t NxS = N * S, total = N * C * S;
+  if (reduction != kNone) {
+    const float normalizer = loss_normalizer(reduction, N, S, true);
+    const bool by_mask = normalizer < 0.f;
+    if (!by_mask || NxS <= kDirectReduceMax) {
+      hipLaunchKernelGGL((loss_reduce_direct<T, TargetT, kGradScale, true>), dim3(1),
+                         dim3(kDirectThreads), 0, stream, static_cast<int64_t>(0),
+                         static_cast<const T*>(nullptr), by_mask ? NxS : static_cast<int64_t>(0),
+                         static_cast<const T*>(nullptr), tp, C, ignore_index, by_mask, normalizer,
+                         dlp, scalar);
+    } else {
+      const int nparts = partial_blocks(NxS);
+      hipLaunchKernelGGL((valid_target_partial_counts<T, TargetT>), dim3(nparts),
+                         dim3(kLossThreads), 0, stream, NxS, C, ignore_index, tp, part);
+      hipLaunchKernelGGL((loss_finalize<T, kGradScale>), dim3(1), dim3(kLossThreads), 0, stream,
+                         nparts, part, by_mask, normalizer, dlp, scalar);
+    }
+  }
+  const bool aligned = aligned16(prob) && aligned16(dx);
+#define LAUNCH(VEC, ALONG_C, PER_POS)                                                          \
+  hipLaunchKernelGGL((softmax_ce_backward<T, TargetT, VEC, ALONG_C, PER_POS>),                 \
+                     dim3(loss_grid(total / VEC)), dim3(kLossThreads), 0, stream, total / VEC, \
+                     S, C, ignore_index, pp, tp, dlp, scalar, dp)
+  if (S == 1 && C % kVec == 0 && aligned) {
+    if (reduction == kNone) LAUNCH(kVec, true, true); else LAUNCH(kVec, true, false);
+  } else if (S > 1 && S % kVec == 0 && aligned) {
+    if (reduction == kNone) LAUNCH(kVec, false, true); else LAUNCH(kVec, false, false);
+  } else {
+    if (reduction == kNone) LAUNCH(1, false, true); else LAUNCH(1, false, false);
+  }
+#undef LAUNCH
+  return status_of_launch();
+}
+
+inline bool loss_dtype_ok(int dtype) { return dtype == DRAGON_HIP_F32 || dtype == DRAGON_HIP_F64; }
+inline bool target_dtype_ok(int t) { return t == DRAGON_HIP_I32 || t == DRAGON_HIP_I64; }
+inline size_t loss_elem(int dtype) { return dtype == DRAGON_HIP_F64 ? 8 : 4; }
+
+// Calls FN<T, TargetT>(args...) for T in {float, double}, TargetT in {int32, int64}.
+#define DRAGON_HIP_DISPATCH_LOSS(dtype, target_dtype, FN, ...)                      \
+  if (dtype == DRAGON_HIP_F32) {                                                    \
+    return target_dtype == DRAGON_HIP_I32 ? FN<float, int32_t>(__VA_ARGS__)         \
+                                          : FN<float, int64_t>(__VA_ARGS__);        \
+  }                                                                                 \
+  return target_dtype == DRAGON_HIP_I32 ? FN<double, int32_t>(__VA_ARGS__)          \
+                                        : FN<double, int64_t>(__VA_ARGS__)
+
+#define DRAGON_HIP_DISPATCH_LOSS_T(dtype, FN, ...)         \
+  if (dtype == DRAGON_HIP_F32) return FN<float>(__VA_ARGS__); \
+  return FN<double>(__VA_ARGS__)
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" {
+
+using namespace dragon_hip;
+
+int dragon_hip_cross_entropy(int dtype, int64_t N, const void* input, const void* target,
+                             void* loss, void* stream) {
+  if (!loss_dtype_ok(dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0) return DRAGON_HIP_EINVAL;
+  if (N == 0) return DRAGON_HIP_OK;
+  if (!input || !target || !loss) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS_T(dtype, launch_cross_entropy, N, input, target, loss, s);
+}
+
+int dragon_hip_sparse_cross_entropy(int dtype, int target_dtype, int64_t N, int64_t S, int64_t C,
+                                    int64_t ignore_index, const void* input, const void* target,
+                                    void* loss, void* mask, void* stream) {
+  if (!loss_dtype_ok(dtype) || !target_dtype_ok(target_dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || S < 0 || C <= 0) return DRAGON_HIP_EINVAL;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!input || !target || !loss || !mask) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS(dtype, target_dtype, launch_sparse_cross_entropy, N, S, C, ignore_index,
+                           input, target, loss, mask, s);
+}
+
+int dragon_hip_softmax_cross_entropy_grad(int dtype, int target_dtype, int64_t N, int64_t S,
+                                          int64_t C, int64_t ignore_index, const void* input,
+                                          const void* target, void* dx, void* mask, void* stream) {
+  (void)input;  // the probabilities are already in dx (cross_entropy_kernel.cc:80-108)
+  if (!loss_dtype_ok(dtype) || !target_dtype_ok(target_dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || S < 0 || C <= 0) return DRAGON_HIP_EINVAL;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!target || !dx || !mask) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS(dtype, target_dtype, launch_softmax_ce_grad, N, S, C, ignore_index,
+                           target, dx, mask, s);
+}
+
+size_t dragon_hip_reduce_loss_scratch_bytes(int dtype) {
+  return loss_dtype_ok(dtype) ? reduce_loss_scratch(loss_elem(dtype)) : 0;
+}
+
+int dragon_hip_reduce_loss(int dtype, int64_t N, int64_t num_masks, float normalizer,
+                           const void* x, const void* mask, void* y, void* scratch,
+                           size_t scratch_bytes, void* stream) {
+  if (!loss_dtype_ok(dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || num_masks < 0 || !y || (N > 0 && !x)) return DRAGON_HIP_EINVAL;
+  if (num_masks > 0 && normalizer < 0.f && !mask) return DRAGON_HIP_EINVAL;
+  if (!scratch || scratch_bytes < reduce_loss_scratch(loss_elem(dtype))) return DRAGON_HIP_ESCRATCH;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS_T(dtype, launch_reduce_loss, N, num_masks, normalizer, x, mask, y,
+                             scratch, s);
+}
+
+int dragon_hip_reduce_loss_grad(int dtype, int64_t N, int64_t num_masks, float normalizer,
+                                const void* dl, const void* mask, void* dx, void* scratch,
+                                size_t scratch_bytes, void* stream) {
+  if (!loss_dtype_ok(dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || num_masks < 0 || !dl) return DRAGON_HIP_EINVAL;
+  if (N == 0) return DRAGON_HIP_OK;
+  if (!dx || (num_masks > 0 && normalizer < 0.f && !mask)) return DRAGON_HIP_EINVAL;
+  if (!scratch || scratch_bytes < reduce_loss_scratch(loss_elem(dtype))) return DRAGON_HIP_ESCRATCH;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS_T(dtype, launch_reduce_loss_grad, N, num_masks, normalizer, dl, mask, dx,
+                             scratch, s);
+}
+
+int dragon_hip_broadcast_loss_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dl,
+                                   void* dx, void* stream) {
+  if (!loss_dtype_ok(dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || S < 0 || C < 0) return DRAGON_HIP_EINVAL;
+  if (N * S * C == 0) return DRAGON_HIP_OK;
+  if (!dl || !dx) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS_T(dtype, launch_broadcast_loss_grad, N, S, C, dl, dx, s);
+}
+
+size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S) {
+  if (!loss_dtype_ok(dtype) || N < 0 || S < 0) return 0;
+  // loss[NxS], mask[NxS], then the reduction's partial pairs and scalar
+  return (static_cast<size_t>(2 * N * S)) * loss_elem(dtype) + reduce_loss_scratch(loss_elem(dtype));
+}
+
+int dragon_hip_softmax_cross_entropy_loss_forward(int dtype, int target_dtype, int64_t N, int64_t S,
+                                                  int64_t C, int64_t ignore_index, int reduction,
+                                                  const void* x, const void* target, void* prob,
+                                                  void* loss, void* scratch, size_t scratch_bytes,
+                                                  void* stream) {
+  if (!loss_dtype_ok(dtype) || !target_dtype_ok(target_dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || S < 0 || C <= 0 || reduction < kNone || reduction > kValid) return DRAGON_HIP_EINVAL;
+  if (!loss) return DRAGON_HIP_EINVAL;
+  if (N * S > 0 && (!x || !target || !prob)) return DRAGON_HIP_EINVAL;
+  if (N * S == 0 && reduction == kNone) return DRAGON_HIP_OK;
+  if (!scratch ||
+      scratch_bytes < dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S)) {
+    return DRAGON_HIP_ESCRATCH;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS(dtype, target_dtype, launch_fused_forward, N, S, C, ignore_index,
+                           reduction, x, target, prob, loss, scratch, s);
+}
+
+int dragon_hip_softmax_cross_entropy_loss_backward(int dtype, int target_dtype, int64_t N,
+                                                   int64_t S, int64_t C, int64_t ignore_index,
+                                                   int reduction, const void* prob,
+                                                   const void* target, const void* dl, void* dx,
+                                                   void* scratch, size_t scratch_bytes,
+                                                   void* stream) {
+  if (!loss_dtype_ok(dtype) || !target_dtype_ok(target_dtype)) return DRAGON_HIP_EDTYPE;
+  if (N < 0 || S < 0 || C <= 0 || reduction < kNone || reduction > kValid) return DRAGON_HIP_EINVAL;
+  if (N * S == 0) return DRAGON_HIP_OK;
+  if (!prob || !target || !dl || !dx) return DRAGON_HIP_EINVAL;
+  if (!scratch || scratch_bytes < reduce_loss_scratch(loss_elem(dtype))) return DRAGON_HIP_ESCRATCH;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DRAGON_HIP_DISPATCH_LOSS(dtype, target_dtype, launch_fused_backward, N, S, C, ignore_index,
+                           reduction, prob, target, dl, dx, scratch, s);
+}
+
+} // extern "C"

@@ -1,9 +1,12 @@
-// kernels::Moments for gfx950: mean and biased variance over arbitrary axes.
+// kernels::Moments (mean and biased variance) and math::ReduceSum /
+// ReduceSumSqr / ReduceL1 over arbitrary axes for gfx950.
 //
 // Replaces kernels::Moments<T, AccT, Context>
 // (dragon/kernels/math/op_kernels.h:106-115; CPU
 // dragon/kernels/math/cpu/moments_kernel.cc:10-189 with the axis utilities of
-// dragon/utils/math/reduce.h:96-198). As there, size-1 axes are dropped and
+// dragon/utils/math/reduce.h:96-198) and math::ReduceSum / ReduceSumSqr /
+// ReduceL1 (dragon/utils/math/reduce.h:50-80; CPU
+// dragon/utils/math/cpu/reduce.cc:10-236). As there, size-1 axes are dropped and
 // adjacent axes of the same kind are merged first; the collapsed pattern picks
 // the kernel:
 //   [K,R] [R] [R,K,R] [K,R,K,R]   segmented split reduction (contiguous runs)
@@ -24,61 +27,95 @@
 namespace dragon_hip {
 namespace {
 
+// What is accumulated and what is written is a policy, so that Moments and
+// the plain sums (math::ReduceSum / ReduceSumSqr / ReduceL1,
+// dragon/utils/math/reduce.h:50-80) share the planner and the kernels.
+//   kShift            subtract the first element of the reduction set first
+//   term(d, a, b)     fold one (shifted) element into the pair of sums
+//   Out / finish      outputs and the per-output epilogue
 template <typename T>
-struct MomentsAccum {
+struct MomentsPolicy {
+  using A = typename IO<T>::Acc;
+  static constexpr bool kShift = true;
+  struct Out {
+    A* mean;
+    A* var;
+  };
+  static __device__ __forceinline__ void term(A d, A& a, A& b) {
+    a += d;
+    b += d * d;
+  }
+  static __device__ __forceinline__ void finish(const Out& out, uint32_t o, A shift, A a, A b,
+                                                A inv_n) {
+    const A m = a * inv_n;
+    out.mean[o] = shift + m;
+    out.var[o] = b * inv_n - m * m;
+  }
+};
+
+enum SumKind { kSumPlain = 0, kSumSqr = 1, kSumAbs = 2 };
+
+// y[o] = scale * sum f(x) with f = identity, square or absolute value; the sum
+// is kept in the accumulator type and rounded to T once.
+template <typename T, int kKind>
+struct SumPolicy {
+  using A = typename IO<T>::Acc;
+  static constexpr bool kShift = false;
+  struct Out {
+    T* y;
+    A scale;
+  };
+  static __device__ __forceinline__ void term(A d, A& a, A&) {
+    a += kKind == kSumPlain ? d : (kKind == kSumSqr ? d * d : (d < A(0) ? -d : d));
+  }
+  static __device__ __forceinline__ void finish(const Out& out, uint32_t o, A, A a, A, A) {
+    IO<T>::store1(out.y + o, a * out.scale);
+  }
+};
+
+template <typename T, typename P>
+struct ReduceAccum {
   using A = typename IO<T>::Acc;
   const T* x;
   A shift;
   __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
-    shift = IO<T>::load1(x + first_off);
+    shift = P::kShift ? IO<T>::load1(x + first_off) : A(0);
   }
   template <int V>
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x0)[V],
                                       const A (&)[V], A& a, A& b) const {
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const A d = x0[e] - shift;
-      a += d;
-      b += d * d;
-    }
+    for (int e = 0; e < V; ++e) P::term(P::kShift ? x0[e] - shift : x0[e], a, b);
   }
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, A x0, A, A& a, A& b) const {
-    const A d = x0 - shift;
-    a += d;
-    b += d * d;
+    P::term(P::kShift ? x0 - shift : x0, a, b);
   }
 };
 
-template <typename T>
-struct MomentsSegEpilogue {
+template <typename T, typename P>
+struct ReduceSegEpilogue {
   using A = typename IO<T>::Acc;
   const T* x;
   SegmentedReduce d;
   A inv_n;
-  A* mean;
-  A* var;
+  typename P::Out out;
   __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
     const uint32_t o1 = o / d.outer2;
     const uint32_t o2 = o - o1 * d.outer2;
-    const A shift = IO<T>::load1(x + o1 * d.stride1 + o2 * d.stride2);
-    const A m = a * inv_n;
-    mean[o] = shift + m;
-    var[o] = b * inv_n - m * m;
+    const A shift = P::kShift ? IO<T>::load1(x + o1 * d.stride1 + o2 * d.stride2) : A(0);
+    P::finish(out, o, shift, a, b, inv_n);
   }
 };
 
-template <typename T>
-struct MomentsColEpilogue {
+template <typename T, typename P>
+struct ReduceColEpilogue {
   using A = typename IO<T>::Acc;
   const T* x;
   A inv_n;
-  A* mean;
-  A* var;
+  typename P::Out out;
   __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
-    const A shift = IO<T>::load1(x + c);
-    const A m = a * inv_n;
-    mean[c] = shift + m;
-    var[c] = b * inv_n - m * m;
+    const A shift = P::kShift ? IO<T>::load1(x + c) : A(0);
+    P::finish(out, c, shift, a, b, inv_n);
   }
 };
 
@@ -92,10 +129,9 @@ struct GatherDims {
 
 // One workgroup per output; the reduced index is unravelled over the reduced
 // extents (last fastest, the order the reference walks them in).
-template <typename T>
-__global__ __launch_bounds__(kReduceThreads) void moments_gather(
-    const GatherDims g, const T* __restrict__ x, typename IO<T>::Acc* __restrict__ mean,
-    typename IO<T>::Acc* __restrict__ var) {
+template <typename T, typename P>
+__global__ __launch_bounds__(kReduceThreads) void reduce_gather(
+    const GatherDims g, const T* __restrict__ x, const typename P::Out out) {
   using A = typename IO<T>::Acc;
   __shared__ A lds[2 * kReduceWaves];
   for (uint32_t o = blockIdx.x; o < g.n_out; o += gridDim.x) {
@@ -104,7 +140,7 @@ __global__ __launch_bounds__(kReduceThreads) void moments_gather(
       base += (r % g.keep_dim[d]) * g.keep_stride[d];
       r /= g.keep_dim[d];
     }
-    const A shift = IO<T>::load1(x + base);
+    const A shift = P::kShift ? IO<T>::load1(x + base) : A(0);
     A a = A(0), b = A(0);
     for (uint32_t j = threadIdx.x; j < g.n_red_elems; j += kReduceThreads) {
       uint32_t off = base, q = j;
@@ -112,17 +148,10 @@ __global__ __launch_bounds__(kReduceThreads) void moments_gather(
         off += (q % g.red_dim[d]) * g.red_stride[d];
         q /= g.red_dim[d];
       }
-      const A v = IO<T>::load1(x + off) - shift;
-      a += v;
-      b += v * v;
+      P::term(IO<T>::load1(x + off) - shift, a, b);
     }
     block_reduce_pair(a, b, lds);
-    if (threadIdx.x == 0) {
-      const A inv_n = A(1) / A(g.n_red_elems);
-      const A m = a * inv_n;
-      mean[o] = shift + m;
-      var[o] = b * inv_n - m * m;
-    }
+    if (threadIdx.x == 0) P::finish(out, o, shift, a, b, A(1) / A(g.n_red_elems));
     __syncthreads();
   }
 }
@@ -212,48 +241,97 @@ int make_plan(int dtype, int num_dims, const int64_t* dims, int num_axes, const 
   return DRAGON_HIP_OK;
 }
 
-template <typename T>
-int launch_moments(const MomentsPlan& plan, const void* x, void* mean, void* var, void* scratch,
-                   hipStream_t stream) {
+template <typename T, typename P>
+int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out& out, void* scratch,
+                  hipStream_t stream) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
   const T* xp = static_cast<const T*>(x);
-  A* mp = static_cast<A*>(mean);
-  A* vp = static_cast<A*>(var);
   A* part = static_cast<A*>(scratch);
   const A inv_n = A(1) / A(plan.n_red);
   const unsigned fin_grid = static_cast<unsigned>(ceil_div(plan.n_out, kReduceThreads));
+  using Accum = ReduceAccum<T, P>;
   if (plan.kind == kPlanSegments) {
     const SegmentedReduce& s = plan.seg;
     const bool vec_ok = aligned16(x) && s.seglen % kVec == 0 && s.stride1 % kVec == 0 &&
         s.stride2 % kVec == 0 && s.seg_stride % kVec == 0;
-    MomentsAccum<T> f{xp, A(0)};
+    Accum f{xp, A(0)};
     const dim3 grid(s.n_out * s.split);
     if (vec_ok) {
-      hipLaunchKernelGGL((reduce2_segments<T, 1, kVec, MomentsAccum<T>>), grid,
-                         dim3(kReduceThreads), 0, stream, s, xp, xp, f, part);
+      hipLaunchKernelGGL((reduce2_segments<T, 1, kVec, Accum>), grid, dim3(kReduceThreads), 0,
+                         stream, s, xp, xp, f, part);
     } else {
-      hipLaunchKernelGGL((reduce2_segments<T, 1, 1, MomentsAccum<T>>), grid, dim3(kReduceThreads),
-                         0, stream, s, xp, xp, f, part);
+      hipLaunchKernelGGL((reduce2_segments<T, 1, 1, Accum>), grid, dim3(kReduceThreads), 0, stream,
+                         s, xp, xp, f, part);
     }
-    MomentsSegEpilogue<T> e{xp, s, inv_n, mp, vp};
-    hipLaunchKernelGGL((reduce2_finalize<A, MomentsSegEpilogue<T>>), dim3(fin_grid),
+    ReduceSegEpilogue<T, P> e{xp, s, inv_n, out};
+    hipLaunchKernelGGL((reduce2_finalize<A, ReduceSegEpilogue<T, P>>), dim3(fin_grid),
                        dim3(kReduceThreads), 0, stream, s.n_out, s.split, true, part, e);
   } else if (plan.kind == kPlanColumns) {
     const ColumnReduce& c = plan.col;
-    MomentsAccum<T> f{xp, A(0)};
+    Accum f{xp, A(0)};
     const dim3 grid(static_cast<unsigned>(ceil_div(c.cols, kWaveSize)) * c.split);
-    hipLaunchKernelGGL((reduce2_columns<T, 1, MomentsAccum<T>>), grid, dim3(kReduceThreads), 0,
-                       stream, c, xp, xp, f, part);
-    MomentsColEpilogue<T> e{xp, inv_n, mp, vp};
-    hipLaunchKernelGGL((reduce2_finalize<A, MomentsColEpilogue<T>>), dim3(fin_grid),
+    hipLaunchKernelGGL((reduce2_columns<T, 1, Accum>), grid, dim3(kReduceThreads), 0, stream, c, xp,
+                       xp, f, part);
+    ReduceColEpilogue<T, P> e{xp, inv_n, out};
+    hipLaunchKernelGGL((reduce2_finalize<A, ReduceColEpilogue<T, P>>), dim3(fin_grid),
                        dim3(kReduceThreads), 0, stream, c.cols, c.split, false, part, e);
   } else {
     const unsigned grid = static_cast<unsigned>(plan.n_out < 65536 ? plan.n_out : 65536);
-    hipLaunchKernelGGL((moments_gather<T>), dim3(grid), dim3(kReduceThreads), 0, stream,
-                       plan.gather, xp, mp, vp);
+    hipLaunchKernelGGL((reduce_gather<T, P>), dim3(grid), dim3(kReduceThreads), 0, stream,
+                       plan.gather, xp, out);
   }
   return status_of_launch();
+}
+
+template <typename T>
+int launch_moments(const MomentsPlan& plan, const void* x, void* mean, void* var, void* scratch,
+                   hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  using P = MomentsPolicy<T>;
+  return launch_reduce<T, P>(plan, x, typename P::Out{static_cast<A*>(mean), static_cast<A*>(var)},
+                             scratch, stream);
+}
+
+template <typename T>
+int launch_sum(int kind, const MomentsPlan& plan, float scale, const void* x, void* y,
+               void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  T* yp = static_cast<T*>(y);
+  const A sc = static_cast<A>(scale);
+  switch (kind) {
+    case kSumPlain: {
+      using P = SumPolicy<T, kSumPlain>;
+      return launch_reduce<T, P>(plan, x, typename P::Out{yp, sc}, scratch, stream);
+    }
+    case kSumSqr: {
+      using P = SumPolicy<T, kSumSqr>;
+      return launch_reduce<T, P>(plan, x, typename P::Out{yp, sc}, scratch, stream);
+    }
+    default: {
+      using P = SumPolicy<T, kSumAbs>;
+      return launch_reduce<T, P>(plan, x, typename P::Out{yp, sc}, scratch, stream);
+    }
+  }
+}
+
+// Shared body of the three sum entry points. A reduction over no element (an
+// extent of zero among the reduced axes) writes zeros, the reducer's identity.
+int reduce_sum_entry(int kind, int dtype, int num_dims, const int64_t* dims, int num_axes,
+                     const int64_t* axes, float scale, const void* x, void* y, void* scratch,
+                     size_t scratch_bytes, void* stream) {
+  MomentsPlan plan;
+  const int st = make_plan(dtype, num_dims, dims, num_axes, axes, &plan);
+  if (st != DRAGON_HIP_OK) return st;
+  if (plan.n_out == 0) return DRAGON_HIP_OK;
+  if (!y) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan.n_red == 0) return dragon_hip_set(dtype, plan.n_out, 0.f, y, stream);
+  if (!x) return DRAGON_HIP_EINVAL;
+  if (plan.scratch_bytes > 0 && (!scratch || scratch_bytes < plan.scratch_bytes)) {
+    return DRAGON_HIP_ESCRATCH;
+  }
+  DRAGON_HIP_DISPATCH_DTYPE(dtype, launch_sum, kind, plan, scale, x, y, scratch, s);
 }
 
 } // namespace
@@ -281,6 +359,32 @@ int dragon_hip_moments(int dtype, int num_dims, const int64_t* dims, int num_axe
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_moments, plan, x, mean, var, scratch, s);
+}
+
+size_t dragon_hip_reduce_scratch_bytes(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                                       const int64_t* axes) {
+  return dragon_hip_moments_scratch_bytes(dtype, num_dims, dims, num_axes, axes);
+}
+
+int dragon_hip_reduce_sum(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                          const int64_t* axes, float scale, const void* x, void* y, void* scratch,
+                          size_t scratch_bytes, void* stream) {
+  return dragon_hip::reduce_sum_entry(dragon_hip::kSumPlain, dtype, num_dims, dims, num_axes, axes,
+                                      scale, x, y, scratch, scratch_bytes, stream);
+}
+
+int dragon_hip_reduce_sum_sqr(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                              const int64_t* axes, float scale, const void* x, void* y,
+                              void* scratch, size_t scratch_bytes, void* stream) {
+  return dragon_hip::reduce_sum_entry(dragon_hip::kSumSqr, dtype, num_dims, dims, num_axes, axes,
+                                      scale, x, y, scratch, scratch_bytes, stream);
+}
+
+int dragon_hip_reduce_l1(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                         const int64_t* axes, float scale, const void* x, void* y, void* scratch,
+                         size_t scratch_bytes, void* stream) {
+  return dragon_hip::reduce_sum_entry(dragon_hip::kSumAbs, dtype, num_dims, dims, num_axes, axes,
+                                      scale, x, y, scratch, scratch_bytes, stream);
 }
 
 } // extern "C"

@@ -90,6 +90,7 @@ int dragon_c_feed_tensor(void* ws, const char* name, const char* dtype, int ndim
       case dragon::DType::kFloat32: dst = t->mutable_data<float, dragon::CPUContext>(); break;
       case dragon::DType::kFloat64: dst = t->mutable_data<double, dragon::CPUContext>(); break;
       case dragon::DType::kInt64: dst = t->mutable_data<int64_t, dragon::CPUContext>(); break;
+      case dragon::DType::kInt32: dst = t->mutable_data<int, dragon::CPUContext>(); break;
       default: LOG(FATAL) << "Unsupported dtype: " << dtype;
     }
     if (t->nbytes() > 0) std::memcpy(dst, host_data, t->nbytes());

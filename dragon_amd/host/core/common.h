@@ -39,6 +39,7 @@ enum class DType : int {
   kFloat64 = 3,
   kInt64 = 4,
   kUInt8 = 5,
+  kInt32 = 6,
   kUndefined = -1
 };
 
@@ -68,12 +69,17 @@ template <>
 struct TypeOf<uint8_t> {
   static constexpr DType value = DType::kUInt8;
 };
+template <>
+struct TypeOf<int> {
+  static constexpr DType value = DType::kInt32;
+};
 
 inline size_t SizeOf(DType t) {
   switch (t) {
     case DType::kFloat16:
     case DType::kBFloat16: return 2;
-    case DType::kFloat32: return 4;
+    case DType::kFloat32:
+    case DType::kInt32: return 4;
     case DType::kFloat64:
     case DType::kInt64: return 8;
     case DType::kUInt8: return 1;
@@ -89,6 +95,7 @@ inline const char* NameOf(DType t) {
     case DType::kFloat64: return "float64";
     case DType::kInt64: return "int64";
     case DType::kUInt8: return "uint8";
+    case DType::kInt32: return "int32";
     default: return "unknown";
   }
 }
@@ -100,6 +107,7 @@ inline DType DTypeFromName(const string& s) {
   if (s == "float64") return DType::kFloat64;
   if (s == "int64") return DType::kInt64;
   if (s == "uint8") return DType::kUInt8;
+  if (s == "int32") return DType::kInt32;
   return DType::kUndefined;
 }
 

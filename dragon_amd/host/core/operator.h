@@ -138,6 +138,19 @@ struct FloatingDispatch {
   }
 };
 
+// DispatchHelper<dtypes::Loss> (dragon/core/types.h:90): float and double.
+struct LossDispatch {
+  template <class Op>
+  static void Call(Op* op, const Tensor& tensor) {
+    switch (tensor.meta()) {
+      case DType::kFloat32: op->template DoRunWithType<float>(); break;
+      case DType::kFloat64: op->template DoRunWithType<double>(); break;
+      default:
+        LOG(FATAL) << op->MessageForUnsupported(NameOf(tensor.meta()), {"float32", "float64"});
+    }
+  }
+};
+
 // Input/output arity and in-place permissions of an operator type
 // (dragon/core/operator_schema.h, operator_schema.cc:5-28).
 class OpSchema {

@@ -246,6 +246,128 @@ DEFINE_LP_NORM_LAUNCHERS(float);
 DEFINE_LP_NORM_LAUNCHERS(double);
 #undef DEFINE_LP_NORM_LAUNCHERS
 
+namespace {
+
+template <typename T>
+constexpr int TargetTag() {
+  return sizeof(T) == 4 ? DRAGON_HIP_I32 : DRAGON_HIP_I64;
+}
+
+int ReductionTag(const string& r) {
+  if (r == "NONE") return 0;
+  if (r == "SUM") return 1;
+  if (r == "MEAN") return 2;
+  if (r == "BATCH_MEAN") return 3;
+  if (r == "VALID") return 4;
+  LOG(FATAL) << "Unknown reduction: " << r;
+  return -1;
+}
+
+} // namespace
+
+#define DEFINE_LOSS_LAUNCHERS(T)                                                                  \
+  template <>                                                                                     \
+  void CrossEntropy<T, HIPContext>(const int N, const T* input, const T* target, T* loss,         \
+                                   HIPContext* ctx) {                                             \
+    HIP_CHECK(dragon_hip_cross_entropy(Tag<T>(), N, input, target, loss, ctx->hip_stream()));     \
+  }                                                                                               \
+  template <>                                                                                     \
+  void ReduceLoss<T, HIPContext>(const int N, const int num_masks, const float normalizer,        \
+                                 const T* x, const T* mask, T* y, HIPContext* ctx) {              \
+    const size_t bytes = dragon_hip_reduce_loss_scratch_bytes(Tag<T>());                          \
+    HIP_CHECK(dragon_hip_reduce_loss(Tag<T>(), N, num_masks, normalizer, x, mask, y,              \
+                                     Scratch(ctx, bytes), bytes, ctx->hip_stream()));             \
+  }                                                                                               \
+  template <>                                                                                     \
+  void ReduceLossGrad<T, HIPContext>(const int N, const int num_masks, const float normalizer,    \
+                                     const T* dl, const T* mask, T* dx, HIPContext* ctx) {        \
+    const size_t bytes = dragon_hip_reduce_loss_scratch_bytes(Tag<T>());                          \
+    HIP_CHECK(dragon_hip_reduce_loss_grad(Tag<T>(), N, num_masks, normalizer, dl, mask, dx,       \
+                                          Scratch(ctx, bytes), bytes, ctx->hip_stream()));        \
+  }                                                                                               \
+  template <>                                                                                     \
+  void BroadcastLossGrad<T, HIPContext>(const int N, const int S, const int C, const T* dl,       \
+                                        T* dx, HIPContext* ctx) {                                 \
+    HIP_CHECK(dragon_hip_broadcast_loss_grad(Tag<T>(), N, S, C, dl, dx, ctx->hip_stream()));      \
+  }
+
+DEFINE_LOSS_LAUNCHERS(float);
+DEFINE_LOSS_LAUNCHERS(double);
+#undef DEFINE_LOSS_LAUNCHERS
+
+#define DEFINE_SPARSE_LOSS_LAUNCHERS(InputT, TargetT)                                             \
+  template <>                                                                                     \
+  void CrossEntropy<InputT, TargetT, HIPContext>(                                                 \
+      const int N, const int S, const int C, const int ignore_index, const InputT* input,         \
+      const TargetT* target, InputT* loss, InputT* mask, HIPContext* ctx) {                       \
+    HIP_CHECK(dragon_hip_sparse_cross_entropy(Tag<InputT>(), TargetTag<TargetT>(), N, S, C,       \
+                                              ignore_index, input, target, loss, mask,            \
+                                              ctx->hip_stream()));                                \
+  }                                                                                               \
+  template <>                                                                                     \
+  void SoftmaxCrossEntropyGrad<InputT, TargetT, HIPContext>(                                      \
+      const int N, const int S, const int C, const int ignore_index, const InputT* input,         \
+      const TargetT* target, InputT* dx, InputT* mask, HIPContext* ctx) {                         \
+    HIP_CHECK(dragon_hip_softmax_cross_entropy_grad(Tag<InputT>(), TargetTag<TargetT>(), N, S, C, \
+                                                    ignore_index, input, target, dx, mask,        \
+                                                    ctx->hip_stream()));                          \
+  }                                                                                               \
+  template <>                                                                                     \
+  void SoftmaxCrossEntropyLossForward<InputT, TargetT, HIPContext>(                               \
+      const int N, const int S, const int C, const int ignore_index, const string& reduction,     \
+      const InputT* x, const TargetT* target, InputT* prob, InputT* loss, HIPContext* ctx) {      \
+    const size_t bytes = dragon_hip_softmax_cross_entropy_loss_scratch_bytes(Tag<InputT>(), N, S); \
+    HIP_CHECK(dragon_hip_softmax_cross_entropy_loss_forward(                                      \
+        Tag<InputT>(), TargetTag<TargetT>(), N, S, C, ignore_index, ReductionTag(reduction), x,   \
+        target, prob, loss, Scratch(ctx, bytes), bytes, ctx->hip_stream()));                      \
+  }                                                                                               \
+  template <>                                                                                     \
+  void SoftmaxCrossEntropyLossBackward<InputT, TargetT, HIPContext>(                              \
+      const int N, const int S, const int C, const int ignore_index, const string& reduction,     \
+      const InputT* prob, const TargetT* target, const InputT* dl, InputT* dx, HIPContext* ctx) { \
+    const size_t bytes = dragon_hip_reduce_loss_scratch_bytes(Tag<InputT>());                     \
+    HIP_CHECK(dragon_hip_softmax_cross_entropy_loss_backward(                                     \
+        Tag<InputT>(), TargetTag<TargetT>(), N, S, C, ignore_index, ReductionTag(reduction),      \
+        prob, target, dl, dx, Scratch(ctx, bytes), bytes, ctx->hip_stream()));                    \
+  }
+
+DEFINE_SPARSE_LOSS_LAUNCHERS(float, int);
+DEFINE_SPARSE_LOSS_LAUNCHERS(float, int64_t);
+DEFINE_SPARSE_LOSS_LAUNCHERS(double, int);
+DEFINE_SPARSE_LOSS_LAUNCHERS(double, int64_t);
+#undef DEFINE_SPARSE_LOSS_LAUNCHERS
+
 } // namespace kernels
+
+namespace math {
+
+#define DEFINE_REDUCE_FUNCS(T)                                                                    \
+  template <>                                                                                     \
+  void ReduceSum<T, HIPContext>(const int num_dims, const int64_t* dims, const int num_axes,      \
+                                const int64_t* axes, const float scale, const T* x, T* y,         \
+                                HIPContext* ctx) {                                                \
+    const size_t bytes = dragon_hip_reduce_scratch_bytes(Tag<T>(), num_dims, dims,       \
+                                                         num_axes, axes);                         \
+    HIP_CHECK(dragon_hip_reduce_sum(Tag<T>(), num_dims, dims, num_axes, axes, scale, x,  \
+                                    y, Scratch(ctx, bytes), bytes, ctx->hip_stream()));  \
+  }                                                                                               \
+  template <>                                                                                     \
+  void ReduceSumSqr<T, HIPContext>(const int num_dims, const int64_t* dims, const int num_axes,   \
+                                   const int64_t* axes, const float scale, const T* x, T* y,      \
+                                   HIPContext* ctx) {                                             \
+    const size_t bytes = dragon_hip_reduce_scratch_bytes(Tag<T>(), num_dims, dims,       \
+                                                         num_axes, axes);                         \
+    HIP_CHECK(dragon_hip_reduce_sum_sqr(Tag<T>(), num_dims, dims, num_axes, axes, scale, \
+                                        x, y, Scratch(ctx, bytes), bytes,                \
+                                        ctx->hip_stream()));                                      \
+  }
+
+DEFINE_REDUCE_FUNCS(float16);
+DEFINE_REDUCE_FUNCS(bfloat16);
+DEFINE_REDUCE_FUNCS(float);
+DEFINE_REDUCE_FUNCS(double);
+#undef DEFINE_REDUCE_FUNCS
+
+} // namespace math
 
 } // namespace dragon

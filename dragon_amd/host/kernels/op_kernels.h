@@ -36,6 +36,15 @@ void Square(const int N, const T* x, T* y, Context* ctx);
 template <typename T, class Context>
 void Sub(const int N, const T* a, const T* b, T* y, Context* ctx);
 
+// y = scale * sum(x) over `axes` (dragon/utils/math/reduce.h:50-58).
+template <typename T, class Context>
+void ReduceSum(const int num_dims, const int64_t* dims, const int num_axes, const int64_t* axes,
+               const float scale, const T* x, T* y, Context* ctx);
+
+template <typename T, class Context>
+void ReduceSumSqr(const int num_dims, const int64_t* dims, const int num_axes, const int64_t* axes,
+                  const float scale, const T* x, T* y, Context* ctx);
+
 } // namespace math
 
 namespace kernels {
@@ -112,11 +121,49 @@ template <typename T, class Context>
 void L2NormGrad(const int N, const int S, const int C, const float normalizer, const float epsilon,
                 const T* dy, const T* x, T* dx, Context* ctx);
 
+// Loss kernels (dragon/kernels/loss/op_kernels.h:25-32,51-69,95-113,179-189).
+template <typename T, class Context>
+void CrossEntropy(const int N, const T* input, const T* target, T* loss, Context* ctx);
+
+template <typename InputT, typename TargetT, class Context>
+void CrossEntropy(const int N, const int S, const int C, const int ignore_index,
+                  const InputT* input, const TargetT* target, InputT* loss, InputT* mask,
+                  Context* ctx);
+
+template <typename InputT, typename TargetT, class Context>
+void SoftmaxCrossEntropyGrad(const int N, const int S, const int C, const int ignore_index,
+                             const InputT* input, const TargetT* target, InputT* dx, InputT* mask,
+                             Context* ctx);
+
+template <typename T, class Context>
+void ReduceLoss(const int N, const int num_masks, const float normalizer, const T* x, const T* mask,
+                T* y, Context* ctx);
+
+template <typename T, class Context>
+void ReduceLossGrad(const int N, const int num_masks, const float normalizer, const T* dl,
+                    const T* mask, T* dx, Context* ctx);
+
+template <typename T, class Context>
+void BroadcastLossGrad(const int N, const int S, const int C, const T* dl, T* dx, Context* ctx);
+
 // Fused operator bodies (see the header comment).
 template <typename T, typename AccT, class Context>
 void GroupNormForward(const int N, const int G, const int D, const int S, const string& data_format,
                       const float epsilon, const T* x, const AccT* gamma, const AccT* beta,
                       AccT* mu, AccT* rsig, T* y, Context* ctx);
+
+// SoftmaxCrossEntropyLossOp / ...GradientOp bodies for class-index targets;
+// reduction is "NONE", "SUM", "MEAN", "BATCH_MEAN" or "VALID".
+template <typename InputT, typename TargetT, class Context>
+void SoftmaxCrossEntropyLossForward(const int N, const int S, const int C, const int ignore_index,
+                                    const string& reduction, const InputT* x, const TargetT* target,
+                                    InputT* prob, InputT* loss, Context* ctx);
+
+template <typename InputT, typename TargetT, class Context>
+void SoftmaxCrossEntropyLossBackward(const int N, const int S, const int C, const int ignore_index,
+                                     const string& reduction, const InputT* prob,
+                                     const TargetT* target, const InputT* dl, InputT* dx,
+                                     Context* ctx);
 
 template <typename T, typename AccT, class Context>
 void BatchNormTrainingForward(const int N, const int C, const int S, const string& data_format,

@@ -2,7 +2,7 @@
 
 Same names (snake-cased), argument order and aliasing conventions as the C++
 templates of dragon/kernels/normalization/op_kernels.h (LayerNorm, GroupNorm,
-BatchNorm, L1/L2Norm),
+BatchNorm, L1/L2Norm), dragon/kernels/loss/op_kernels.h (softmax cross-entropy),
 dragon/kernels/activation/op_kernels.h and dragon/kernels/math/op_kernels.h;
 the trailing ``Context* ctx`` becomes the current torch stream. Tensors are
 torch CUDA tensors used purely as device memory: every function passes raw
@@ -16,6 +16,8 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2, torch.float64: 3}
+_TARGET_DTYPES = {torch.int32: 4, torch.int64: 5}
+REDUCTIONS = {"NONE": 0, "SUM": 1, "MEAN": 2, "BATCH_MEAN": 3, "VALID": 4}
 _LAYOUTS = {"NCHW": 0, "NHWC": 1}
 
 # Per-(device, stream) scratch, grown monotonically and never freed between
@@ -29,6 +31,13 @@ def dtype_tag(t):
         return _DTYPES[t.dtype]
     except KeyError:
         raise TypeError("unsupported dtype %s" % t.dtype)
+
+
+def target_tag(t):
+    try:
+        return _TARGET_DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("unsupported target dtype %s" % t.dtype)
 
 
 def layout_tag(data_format):
@@ -95,6 +104,30 @@ def square(N, x, y):
 
 def sub(N, a, b, y):
     _call("dragon_hip_sub", dtype_tag(a), N, _ptr(a), _ptr(b), _ptr(y), _stream())
+
+
+def _reduce(name, dims, axes, scale, x, y):
+    d, a = _dims(dims), _dims(axes)
+    tag = dtype_tag(x)
+    need = _lib.lib().dragon_hip_reduce_scratch_bytes(tag, len(dims), d, len(axes), a)
+    ws = workspace(need, x.device)
+    _call(name, tag, len(dims), d, len(axes), a, scale, _ptr(x), _ptr(y), _ptr(ws), need, _stream())
+
+
+def reduce_sum(dims, axes, scale, x, y):
+    _reduce("dragon_hip_reduce_sum", dims, axes, scale, x, y)
+
+
+def reduce_sum_sqr(dims, axes, scale, x, y):
+    _reduce("dragon_hip_reduce_sum_sqr", dims, axes, scale, x, y)
+
+
+def reduce_l1(dims, axes, scale, x, y):
+    _reduce("dragon_hip_reduce_l1", dims, axes, scale, x, y)
+
+
+def sum(N, scale, x, y):  # noqa: A001 - the reference's name is math::Sum
+    reduce_sum([N], [0], scale, x, y)
 
 
 # ---------------------------------------------------------------- kernels::
@@ -203,7 +236,64 @@ def l2_norm_grad(N, S, C, normalizer, epsilon, dy, x, dx):
           _ptr(dx), _stream())
 
 
+# ---------------------------------------------------------------- kernels:: (loss)
+
+def _loss_scratch(tag, device):
+    need = _lib.lib().dragon_hip_reduce_loss_scratch_bytes(tag)
+    return workspace(need, device), need
+
+
+def cross_entropy(N, input, target, loss):  # dense targets
+    _call("dragon_hip_cross_entropy", dtype_tag(input), N, _ptr(input), _ptr(target), _ptr(loss),
+          _stream())
+
+
+def sparse_cross_entropy(N, S, C, ignore_index, input, target, loss, mask):
+    _call("dragon_hip_sparse_cross_entropy", dtype_tag(input), target_tag(target), N, S, C,
+          ignore_index, _ptr(input), _ptr(target), _ptr(loss), _ptr(mask), _stream())
+
+
+def softmax_cross_entropy_grad(N, S, C, ignore_index, input, target, dx, mask):
+    _call("dragon_hip_softmax_cross_entropy_grad", dtype_tag(dx), target_tag(target), N, S, C,
+          ignore_index, _ptr(input), _ptr(target), _ptr(dx), _ptr(mask), _stream())
+
+
+def reduce_loss(N, num_masks, normalizer, x, mask, y):
+    tag = dtype_tag(x)
+    ws, need = _loss_scratch(tag, x.device)
+    _call("dragon_hip_reduce_loss", tag, N, num_masks, normalizer, _ptr(x), _ptr(mask), _ptr(y),
+          _ptr(ws), need, _stream())
+
+
+def reduce_loss_grad(N, num_masks, normalizer, dl, mask, dx):
+    tag = dtype_tag(dx)
+    ws, need = _loss_scratch(tag, dx.device)
+    _call("dragon_hip_reduce_loss_grad", tag, N, num_masks, normalizer, _ptr(dl), _ptr(mask),
+          _ptr(dx), _ptr(ws), need, _stream())
+
+
+def broadcast_loss_grad(N, S, C, dl, dx):
+    _call("dragon_hip_broadcast_loss_grad", dtype_tag(dx), N, S, C, _ptr(dl), _ptr(dx), _stream())
+
+
 # ---------------------------------------------------------------- fused operator bodies
+
+def softmax_cross_entropy_loss_forward(N, S, C, ignore_index, reduction, x, target, prob, loss):
+    tag = dtype_tag(x)
+    need = _lib.lib().dragon_hip_softmax_cross_entropy_loss_scratch_bytes(tag, N, S)
+    ws = workspace(need, x.device)
+    _call("dragon_hip_softmax_cross_entropy_loss_forward", tag, target_tag(target), N, S, C,
+          ignore_index, REDUCTIONS[reduction.upper()], _ptr(x), _ptr(target), _ptr(prob),
+          _ptr(loss), _ptr(ws), need, _stream())
+
+
+def softmax_cross_entropy_loss_backward(N, S, C, ignore_index, reduction, prob, target, dl, dx):
+    tag = dtype_tag(prob)
+    ws, need = _loss_scratch(tag, prob.device)
+    _call("dragon_hip_softmax_cross_entropy_loss_backward", tag, target_tag(target), N, S, C,
+          ignore_index, REDUCTIONS[reduction.upper()], _ptr(prob), _ptr(target), _ptr(dl),
+          _ptr(dx), _ptr(ws), need, _stream())
+
 
 def group_norm_forward(N, G, D, S, data_format, epsilon, x, gamma, beta, mu, rsig, y):
     tag, lay = dtype_tag(x), layout_tag(data_format)

@@ -53,7 +53,7 @@ def registered_operators():
 
 def _np_storage(dtype):
     return {"float16": np.uint16, "bfloat16": np.uint16, "float32": np.float32,
-            "float64": np.float64, "int64": np.int64}[dtype]
+            "float64": np.float64, "int64": np.int64, "int32": np.int32}[dtype]
 
 
 def _quote(s):
@@ -115,7 +115,8 @@ class Workspace:
         """Feed a numpy array; 16-bit floats travel as uint16 bit patterns with ``dtype`` given."""
         if dtype is None:
             dtype = {np.dtype(np.float16): "float16", np.dtype(np.float32): "float32",
-                     np.dtype(np.float64): "float64", np.dtype(np.int64): "int64"}[array.dtype]
+                     np.dtype(np.float64): "float64", np.dtype(np.int64): "int64",
+                     np.dtype(np.int32): "int32"}[array.dtype]
             if dtype == "float16":
                 array = array.view(np.uint16)
         a = np.ascontiguousarray(array, dtype=_np_storage(dtype))
@@ -219,6 +220,12 @@ def batch_norm(tape, inputs, axis=-1, momentum=0.9, epsilon=1e-5, use_stats=-1, 
 
 def lp_norm(tape, inputs, axis=-1, end_axis=None, p=2, epsilon=1e-12, reduction="sum"):
     return tape.run("LpNorm", inputs, p=int(p), axis=axis, end_axis=end_axis, epsilon=float(epsilon),
+                    reduction=reduction.upper())
+
+
+def softmax_cross_entropy_loss(tape, inputs, axis=-1, ignore_index=None, reduction="valid"):
+    """dragon.losses.softmax_cross_entropy_loss (dragon/python/core/ops/loss_ops.py:301-340)."""
+    return tape.run("SoftmaxCrossEntropyLoss", inputs, axis=axis, ignore_index=ignore_index,
                     reduction=reduction.upper())
 
 

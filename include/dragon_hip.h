@@ -1,7 +1,8 @@
 /*
  * dragon_hip.h - C ABI of the MI355X (gfx950) kernel library behind Dragon's
- * kernels:: / math:: interface for LayerNorm, GroupNorm, BatchNorm, Moments and
- * Softmax / LogSoftmax.
+ * kernels:: / math:: interface for LayerNorm, GroupNorm, BatchNorm, Moments,
+ * Softmax / LogSoftmax and their siblings on the same reduction skeleton
+ * (L1/L2Norm, ReduceSum, softmax cross-entropy loss).
  *
  * Each entry point replaces one function template of the reference (cited as
  * file:line relative to the reference tree). A `kernels::X<T, AccT, HIPContext>`
@@ -42,7 +43,9 @@ typedef enum {
   DRAGON_HIP_F16 = 0,  /* dragon::float16  (dragon/core/types.h:36-38) */
   DRAGON_HIP_BF16 = 1, /* dragon::bfloat16 (dragon/core/types.h:40-42) */
   DRAGON_HIP_F32 = 2,
-  DRAGON_HIP_F64 = 3
+  DRAGON_HIP_F64 = 3,
+  DRAGON_HIP_I32 = 4, /* class-index targets of the loss kernels only */
+  DRAGON_HIP_I64 = 5
 } dragon_hip_dtype;
 
 typedef enum {
@@ -119,6 +122,23 @@ size_t dragon_hip_moments_scratch_bytes(int dtype, int num_dims, const int64_t* 
 int dragon_hip_moments(int dtype, int num_dims, const int64_t* dims, int num_axes,
                        const int64_t* axes, const void* x, void* mean, void* var,
                        void* scratch, size_t scratch_bytes, void* stream);
+
+/* math::ReduceSum / ReduceSumSqr / ReduceL1, dragon/utils/math/reduce.h:50-80
+ * (CPU dragon/utils/math/cpu/reduce.cc:62-236): y = scale * sum f(x) over
+ * `axes` with f = identity, square or absolute value. y is T with the kept
+ * extents in order (as Moments); the sum is held in AccT and rounded once.
+ * Scratch: dragon_hip_reduce_scratch_bytes (same planner as Moments). */
+size_t dragon_hip_reduce_scratch_bytes(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                                       const int64_t* axes);
+int dragon_hip_reduce_sum(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                          const int64_t* axes, float scale, const void* x, void* y, void* scratch,
+                          size_t scratch_bytes, void* stream);
+int dragon_hip_reduce_sum_sqr(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                              const int64_t* axes, float scale, const void* x, void* y,
+                              void* scratch, size_t scratch_bytes, void* stream);
+int dragon_hip_reduce_l1(int dtype, int num_dims, const int64_t* dims, int num_axes,
+                         const int64_t* axes, float scale, const void* x, void* y, void* scratch,
+                         size_t scratch_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* kernels::LayerNorm, dragon/kernels/normalization/op_kernels.h:191-202     */
@@ -236,6 +256,73 @@ int dragon_hip_l1_norm_grad(int dtype, int64_t N, int64_t S, int64_t C, float no
                             float epsilon, const void* dy, const void* x, void* dx, void* stream);
 int dragon_hip_l2_norm_grad(int dtype, int64_t N, int64_t S, int64_t C, float normalizer,
                             float epsilon, const void* dy, const void* x, void* dx, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Softmax cross-entropy loss, dragon/kernels/loss/op_kernels.h              */
+/* (CPU dragon/kernels/loss/cpu/cross_entropy_kernel.cc,                     */
+/* generic_loss_kernel.cc). dtype is F32 or F64 (dtypes::Loss,               */
+/* dragon/core/types.h:90); target_dtype is I32 or I64. A target outside     */
+/* [0, C) other than ignore_index is treated as ignored.                     */
+/* ------------------------------------------------------------------------ */
+
+/* CrossEntropy, dense targets (op_kernels.h:51-57; cpu :10-15):
+ * loss[i] = -target[i] * log(max(input[i], FLT_MIN)). */
+int dragon_hip_cross_entropy(int dtype, int64_t N, const void* input, const void* target,
+                             void* loss, void* stream);
+
+/* CrossEntropy, class-index targets over input T[N, C, S] (op_kernels.h:59-69;
+ * cpu :17-42): per (n, s) loss = -log(max(input[n, target, s], FLT_MIN)) and
+ * mask = 1, or loss = mask = 0 where target == ignore_index. loss, mask: T[N*S]. */
+int dragon_hip_sparse_cross_entropy(int dtype, int target_dtype, int64_t N, int64_t S, int64_t C,
+                                    int64_t ignore_index, const void* input, const void* target,
+                                    void* loss, void* mask, void* stream);
+
+/* SoftmaxCrossEntropyGrad (op_kernels.h:179-189; cpu :80-108): dx holds a copy
+ * of the probabilities on entry; subtracts 1 at the target class, or clears
+ * the whole class axis where the target is ignored; writes mask T[N*S]. */
+int dragon_hip_softmax_cross_entropy_grad(int dtype, int target_dtype, int64_t N, int64_t S,
+                                          int64_t C, int64_t ignore_index, const void* input,
+                                          const void* target, void* dx, void* mask, void* stream);
+
+/* ReduceLoss / ReduceLossGrad (op_kernels.h:95-113; generic_loss_kernel.cc:31-60):
+ *   inv_scale = sum(mask[0, num_masks)) if num_masks > 0 and normalizer < 0, else normalizer
+ *   ReduceLoss      y[0] = sum(x[0, N)) * (1 / max(inv_scale, 1))
+ *   ReduceLossGrad  dx[0, N) *= dl[0] / max(inv_scale, 0.5)
+ * Scratch: dragon_hip_reduce_loss_scratch_bytes(dtype). */
+size_t dragon_hip_reduce_loss_scratch_bytes(int dtype);
+int dragon_hip_reduce_loss(int dtype, int64_t N, int64_t num_masks, float normalizer,
+                           const void* x, const void* mask, void* y, void* scratch,
+                           size_t scratch_bytes, void* stream);
+int dragon_hip_reduce_loss_grad(int dtype, int64_t N, int64_t num_masks, float normalizer,
+                                const void* dl, const void* mask, void* dx, void* scratch,
+                                size_t scratch_bytes, void* stream);
+
+/* BroadcastLossGrad (op_kernels.h:25-32; generic_loss_kernel.cc:10-25):
+ * dx[n, c, s] *= dl[n, s]. */
+int dragon_hip_broadcast_loss_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dl,
+                                   void* dx, void* stream);
+
+/* SoftmaxCrossEntropyLossOp / ...GradientOp bodies for class-index targets
+ * (dragon/operators/loss/cross_entropy_softmax_loss_op.cc:8-143) as one call
+ * each. reduction: 0 NONE, 1 SUM, 2 MEAN, 3 BATCH_MEAN, 4 VALID.
+ *   forward   prob = softmax(x) (the op's "X_norm"), loss = T[N*S] for NONE,
+ *             else the reduced scalar T[1]
+ *   backward  dx = (prob - onehot(target)) * w, w = 0 at ignored positions,
+ *             dl[n, s] for NONE, else dl[0] / max(normalizer or valid count, 0.5)
+ * Scratch: forward dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S),
+ * backward dragon_hip_reduce_loss_scratch_bytes(dtype). */
+size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S);
+int dragon_hip_softmax_cross_entropy_loss_forward(int dtype, int target_dtype, int64_t N, int64_t S,
+                                                  int64_t C, int64_t ignore_index, int reduction,
+                                                  const void* x, const void* target, void* prob,
+                                                  void* loss, void* scratch, size_t scratch_bytes,
+                                                  void* stream);
+int dragon_hip_softmax_cross_entropy_loss_backward(int dtype, int target_dtype, int64_t N,
+                                                   int64_t S, int64_t C, int64_t ignore_index,
+                                                   int reduction, const void* prob,
+                                                   const void* target, const void* dl, void* dx,
+                                                   void* scratch, size_t scratch_bytes,
+                                                   void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Operator-level fused entry points: one call for a kernel sequence that a  */

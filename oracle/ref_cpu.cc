@@ -1,5 +1,6 @@
 // CPU oracle: a loop-for-loop restatement of Dragon's CPU kernels for
-// LayerNorm, GroupNorm, BatchNorm, Moments, Softmax/LogSoftmax and L1/L2Norm.
+// LayerNorm, GroupNorm, BatchNorm, Moments, Softmax/LogSoftmax, L1/L2Norm,
+// ReduceSum and the softmax cross-entropy loss.
 //
 // THIS FILE IS TEST INFRASTRUCTURE. It is the checker the HIP kernels are
 // compared against and the CPU baseline that is timed beside them. Nothing in
@@ -17,6 +18,13 @@
 //   layer_norm, group_norm_grad    reference test literals, test_ops.py:4232-4291,4303-4351,4363-4397
 //   moments                        numpy mean/var closed form, test_ops.py:3489-3511
 //   batch_norm fwd/bwd             numpy closed forms,  test_ops.py:4127-4181
+//   reduce_sum / _sum_sqr / _l1    numpy sum closed forms (the reference's reduce
+//                                  tests compare with numpy, test_ops.py TestReduceOps)
+//   cross_entropy*, reduce_loss*,  the numpy closed form of test_ops.py:2260-2296 (sparse
+//   broadcast_loss_grad            and dense targets, reductions mean / sum / none);
+//                                  ignore_index and VALID / BATCH_MEAN normalisation are
+//                                  PARITY UNPINNED by any reference test, checked against
+//                                  the formulas of the operator body only
 //   lp_norm (+grad)                reference test literals and the numpy closed
 //                                  form of test_ops.py:4480-4512
 //   f16 / bf16 conversions         exhaustive comparison against numpy float16 and
@@ -31,6 +39,7 @@
 
 #include <algorithm>
 #include <array>
+#include <cfloat>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -343,26 +352,17 @@ bool is_colwise_reduce(
   return true;
 }
 
-template <typename T, typename AccT>
-void moments(
-    const int num_dims_in, const int64_t* dims_in, const int num_axes_in,
-    const int64_t* axes_in, const T* x, AccT* mean, AccT* var) {
-  // moments_kernel.cc:160-183 then :86-135
-  std::vector<int64_t> dims, axes;
-  collapse_reduce_axes(num_dims_in, dims_in, num_axes_in, axes_in, dims, axes);
+// reduce.h:140-158 (TransposeAxesForReduce) and the stride computation of
+// ComputeTransposeStrides: kept axes first, reduced axes last, each keeping
+// its source stride.
+void transposed_reduce_plan(
+    const std::vector<int64_t>& dims, const std::vector<int64_t>& axes,
+    int64_t* rows, int64_t* cols, std::vector<int64_t>& t_dims,
+    std::vector<int64_t>& t_strides) {
   const int num_dims = int(dims.size()), num_axes = int(axes.size());
-  int64_t rows, cols;
-  std::vector<int64_t> out_dims(dims);
-  for (int i = 0; i < num_axes; ++i) out_dims[axes[i]] = 1;
-  if (is_rowwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
-    return rowwise_moments(rows, cols, x, mean, var);
-  }
-  if (is_colwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
-    return colwise_moments(rows, cols, x, mean, var);
-  }
-  // reduce.h:140-158 (TransposeAxesForReduce) and the stride computation:
-  // kept axes first, reduced axes last, each keeping its source stride.
-  std::vector<int64_t> t_axes(num_dims), t_dims(num_dims), t_strides(num_dims);
+  std::vector<int64_t> t_axes(num_dims);
+  t_dims.assign(num_dims, 0);
+  t_strides.assign(num_dims, 0);
   const int d = num_dims - num_axes;
   std::copy_n(axes.begin(), num_axes, t_axes.begin() + d);
   std::sort(t_axes.begin() + d, t_axes.end());
@@ -380,15 +380,102 @@ void moments(
     strides[i] = acc;
     acc *= dims[i];
   }
-  rows = cols = 1;
-  for (int i = 0; i < d; ++i) rows *= dims[t_axes[i]];
-  for (int i = d; i < num_dims; ++i) cols *= dims[t_axes[i]];
+  *rows = *cols = 1;
+  for (int i = 0; i < d; ++i) *rows *= dims[t_axes[i]];
+  for (int i = d; i < num_dims; ++i) *cols *= dims[t_axes[i]];
   for (int i = 0; i < num_dims; ++i) {
     t_dims[i] = dims[t_axes[i]];
     t_strides[i] = strides[t_axes[i]];
   }
+}
+
+template <typename T, typename AccT>
+void moments(
+    const int num_dims_in, const int64_t* dims_in, const int num_axes_in,
+    const int64_t* axes_in, const T* x, AccT* mean, AccT* var) {
+  // moments_kernel.cc:160-183 then :86-135
+  std::vector<int64_t> dims, axes;
+  collapse_reduce_axes(num_dims_in, dims_in, num_axes_in, axes_in, dims, axes);
+  const int num_dims = int(dims.size()), num_axes = int(axes.size());
+  int64_t rows, cols;
+  std::vector<int64_t> out_dims(dims);
+  for (int i = 0; i < num_axes; ++i) out_dims[axes[i]] = 1;
+  if (is_rowwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
+    return rowwise_moments(rows, cols, x, mean, var);
+  }
+  if (is_colwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
+    return colwise_moments(rows, cols, x, mean, var);
+  }
+  std::vector<int64_t> t_dims, t_strides;
+  transposed_reduce_plan(dims, axes, &rows, &cols, t_dims, t_strides);
   generic_moments(
       rows, cols, num_dims, t_dims.data(), t_strides.data(), x, mean, var);
+}
+
+// ---------------------------------------------------------------------------
+// math::ReduceSum / ReduceSumSqr / ReduceL1, dragon/utils/math/cpu/reduce.cc.
+// The global, rowwise ("leading axes") and colwise ("trailing axes") cases are
+// Eigen reductions there (:12-61), restated as sequential sums in T; the
+// generic case is the strided walk of :62-88 in AccT = T. y = T(sum) * T(scale)
+// where scale != 1 (:17,:36,:54), y = T(sum * scale) in the generic case (:86).
+// kKind: 0 identity, 1 square, 2 absolute value.
+// ---------------------------------------------------------------------------
+template <typename T, int kKind>
+inline T reduce_term(T v) {
+  return kKind == 0 ? v : (kKind == 1 ? v * v : std::abs(v));
+}
+
+template <typename T, int kKind>
+void reduce_sum(
+    const int num_dims_in, const int64_t* dims_in, const int num_axes_in,
+    const int64_t* axes_in, const float scale, const T* x, T* y) {
+  // :188-212 (CollapseReduceAxes) then the dispatcher :90-160
+  std::vector<int64_t> dims, axes;
+  collapse_reduce_axes(num_dims_in, dims_in, num_axes_in, axes_in, dims, axes);
+  const int num_dims = int(dims.size()), num_axes = int(axes.size());
+  if (num_dims == num_axes) {
+    int64_t n = 1;
+    for (int64_t d : dims) n *= d;
+    T acc = T(0);
+    for (int64_t i = 0; i < n; ++i) acc += reduce_term<T, kKind>(x[i]);
+    y[0] = acc;
+    if (scale != 1.f) y[0] *= T(scale);
+    return;
+  }
+  int64_t rows, cols;
+  std::vector<int64_t> out_dims(dims);
+  for (int i = 0; i < num_axes; ++i) out_dims[axes[i]] = 1;
+  if (is_rowwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
+    for (int64_t i = 0; i < cols; ++i) {
+      T acc = T(0);
+      for (int64_t j = 0; j < rows; ++j) acc += reduce_term<T, kKind>(x[j * cols + i]);
+      y[i] = scale != 1.f ? acc * T(scale) : acc;
+    }
+    return;
+  }
+  if (is_colwise_reduce(num_dims, dims.data(), out_dims.data(), &rows, &cols)) {
+    for (int64_t i = 0; i < rows; ++i) {
+      T acc = T(0);
+      for (int64_t j = 0; j < cols; ++j) acc += reduce_term<T, kKind>(x[i * cols + j]);
+      y[i] = scale != 1.f ? acc * T(scale) : acc;
+    }
+    return;
+  }
+  std::vector<int64_t> t_dims, t_strides;
+  transposed_reduce_plan(dims, axes, &rows, &cols, t_dims, t_strides);
+  for (int64_t i = 0; i < rows; ++i) {
+    T val = T(0);
+    for (int64_t j = 0; j < cols; ++j) {
+      int64_t xi = 0, c = i * cols + j;
+      for (int d = num_dims - 1; d >= 0; --d) {
+        const int64_t r = c % t_dims[d];
+        c = c / t_dims[d];
+        xi += r * t_strides[d];
+      }
+      val += reduce_term<T, kKind>(x[xi]);
+    }
+    y[i] = val * T(scale);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -744,6 +831,112 @@ void lp_norm_grad(const int N, const int S, const int C, const float normalizer,
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Softmax cross-entropy loss kernels.
+// dragon/kernels/loss/cpu/cross_entropy_kernel.cc:10-42,80-108 and
+// dragon/kernels/loss/cpu/generic_loss_kernel.cc:10-60. math::Sum inside
+// ReduceLoss is the global Eigen sum followed by `*= T(scale)` (reduce.cc:12-19),
+// restated as a sequential sum.
+// ---------------------------------------------------------------------------
+template <typename T>
+void cross_entropy_dense(const int64_t N, const T* input, const T* target, T* loss) {
+  // :10-15
+  for (int64_t i = 0; i < N; ++i) {
+    loss[i] = -target[i] * std::log(std::max(input[i], T(FLT_MIN)));
+  }
+}
+
+template <typename InputT, typename TargetT>
+void cross_entropy_sparse(
+    const int N, const int S, const int C, const int ignore_index,
+    const InputT* input, const TargetT* target, InputT* loss, InputT* mask) {
+  // :17-42 : positions are walked n-major, s-minor.
+  for (int n = 0; n < N; ++n) {
+    for (int sidx = 0; sidx < S; ++sidx) {
+      const int64_t i = int64_t(n) * S + sidx;
+      const int tgt = int(target[i]);
+      if (tgt == ignore_index) {
+        loss[i] = mask[i] = InputT(0);
+      } else {
+        const int64_t j = (int64_t(n) * C + tgt) * S + sidx;
+        loss[i] = -std::log(std::max(input[j], InputT(FLT_MIN)));
+        mask[i] = InputT(1);
+      }
+    }
+  }
+}
+
+template <typename InputT, typename TargetT>
+void softmax_cross_entropy_grad(
+    const int N, const int S, const int C, const int ignore_index,
+    const TargetT* target, InputT* grad, InputT* mask) {
+  // :80-108
+  for (int n = 0; n < N; ++n) {
+    for (int sidx = 0; sidx < S; ++sidx) {
+      const int64_t i = int64_t(n) * S + sidx;
+      const int tgt = int(target[i]);
+      if (tgt == ignore_index) {
+        InputT* g = grad + int64_t(n) * C * S + sidx;
+        for (int k = 0; k < C; ++k) {
+          *g = InputT(0);
+          g += S;
+        }
+        mask[i] = InputT(0);
+      } else {
+        grad[(int64_t(n) * C + tgt) * S + sidx] -= InputT(1);
+        mask[i] = InputT(1);
+      }
+    }
+  }
+}
+
+template <typename T>
+T scaled_sum(const int64_t N, const float scale, const T* x) {
+  T acc = T(0);
+  for (int64_t i = 0; i < N; ++i) acc += x[i];
+  if (scale != 1.f) acc *= T(scale);
+  return acc;
+}
+
+template <typename T>
+void reduce_loss(const int64_t N, const int64_t num_masks, const float normalizer,
+                 const T* x, const T* mask, T* y) {
+  // generic_loss_kernel.cc:31-44
+  const float inv_scale = num_masks > 0 && normalizer < 0.f
+      ? float(scaled_sum(num_masks, 1.f, mask)) : normalizer;
+  y[0] = scaled_sum(N, 1.f / std::max(inv_scale, 1.f), x);
+}
+
+template <typename T>
+void reduce_loss_grad(const int64_t N, const int64_t num_masks, const float normalizer,
+                      const T* dl, const T* mask, T* dx) {
+  // generic_loss_kernel.cc:46-60 ; math::Scale is x * T(scale) (blas.cc:87-97)
+  const float inv_scale = num_masks > 0 && normalizer < 0.f
+      ? float(scaled_sum(num_masks, 1.f, mask)) : normalizer;
+  const float scale = float(dl[0]) / std::max(inv_scale, 0.5f);
+  for (int64_t i = 0; i < N; ++i) dx[i] = dx[i] * T(scale);
+}
+
+template <typename T>
+void broadcast_loss_grad(const int N, const int S, const int C, const T* dl, T* dx) {
+  // generic_loss_kernel.cc:10-25
+  for (int n = 0; n < N; ++n)
+    for (int c = 0; c < C; ++c)
+      for (int sidx = 0; sidx < S; ++sidx) {
+        const int64_t i = (int64_t(n) * C + c) * S + sidx;
+        dx[i] = dx[i] * dl[int64_t(n) * S + sidx];
+      }
+}
+
+template <typename I, typename Tg>
+void sparse_ce_erased(int N, int S, int C, int ig, const void* in, const void* tg, void* loss, void* mask) {
+  cross_entropy_sparse(N, S, C, ig, (const I*)in, (const Tg*)tg, (I*)loss, (I*)mask);
+}
+template <typename I, typename Tg>
+void sce_grad_erased(int N, int S, int C, int ig, const void* tg, void* dx, void* mask) {
+  softmax_cross_entropy_grad(N, S, C, ig, (const Tg*)tg, (I*)dx, (I*)mask);
 }
 
 enum { kF16 = 0, kBF16 = 1, kF32 = 2, kF64 = 3 };
@@ -1138,6 +1331,84 @@ int ref_lp_norm_grad(int dtype, int p, int64_t N, int64_t S, int64_t C,
     else lp_norm_grad<double, 2>(int(N), int(S), int(C), normalizer, epsilon, (const double*)dy, (const double*)x, (double*)dx);
     return kOk;
   }
+  return kUnsupportedDtype;
+}
+
+// math::ReduceSum (kind 0) / ReduceSumSqr (1) / ReduceL1 (2), reduce.cc:162-236.
+// float16 / bfloat16 are CPU_UNSUPPORTED_DTYPE there (:162-186).
+int ref_reduce_sum(int dtype, int kind, int num_dims, const int64_t* dims,
+                   int num_axes, const int64_t* axes, float scale,
+                   const void* x, void* y) {
+  if (kind < 0 || kind > 2) return kBadArg;
+  if (dtype == kF32) {
+    const float* xp = (const float*)x;
+    float* yp = (float*)y;
+    if (kind == 0) reduce_sum<float, 0>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    else if (kind == 1) reduce_sum<float, 1>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    else reduce_sum<float, 2>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    return kOk;
+  }
+  if (dtype == kF64) {
+    const double* xp = (const double*)x;
+    double* yp = (double*)y;
+    if (kind == 0) reduce_sum<double, 0>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    else if (kind == 1) reduce_sum<double, 1>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    else reduce_sum<double, 2>(num_dims, dims, num_axes, axes, scale, xp, yp);
+    return kOk;
+  }
+  return kUnsupportedDtype;
+}
+
+// Loss kernels: dtype f32 / f64 only (cross_entropy_kernel.cc:110-165,
+// generic_loss_kernel.cc:27-81 instantiate the 16-bit types for the reductions
+// only; the softmax loss operators dispatch on float and double).
+// target_dtype: 4 = int32, 5 = int64.
+int ref_cross_entropy(int dtype, int64_t N, const void* input,
+                      const void* target, void* loss) {
+  if (dtype == kF32) { cross_entropy_dense(N, (const float*)input, (const float*)target, (float*)loss); return kOk; }
+  if (dtype == kF64) { cross_entropy_dense(N, (const double*)input, (const double*)target, (double*)loss); return kOk; }
+  return kUnsupportedDtype;
+}
+
+#define REF_LOSS_DISPATCH(FN, ...)                                              \
+  if (dtype == kF32 && target_dtype == 4) { FN<float, int32_t>(__VA_ARGS__); return kOk; }  \
+  if (dtype == kF32 && target_dtype == 5) { FN<float, int64_t>(__VA_ARGS__); return kOk; }  \
+  if (dtype == kF64 && target_dtype == 4) { FN<double, int32_t>(__VA_ARGS__); return kOk; } \
+  if (dtype == kF64 && target_dtype == 5) { FN<double, int64_t>(__VA_ARGS__); return kOk; } \
+  return kUnsupportedDtype;
+
+int ref_sparse_cross_entropy(int dtype, int target_dtype, int64_t N, int64_t S,
+                             int64_t C, int64_t ignore_index, const void* input,
+                             const void* target, void* loss, void* mask) {
+  REF_LOSS_DISPATCH(sparse_ce_erased, int(N), int(S), int(C), int(ignore_index), input, target, loss, mask)
+}
+
+int ref_softmax_cross_entropy_grad(int dtype, int target_dtype, int64_t N,
+                                   int64_t S, int64_t C, int64_t ignore_index,
+                                   const void* target, void* dx, void* mask) {
+  REF_LOSS_DISPATCH(sce_grad_erased, int(N), int(S), int(C), int(ignore_index), target, dx, mask)
+}
+#undef REF_LOSS_DISPATCH
+
+int ref_reduce_loss(int dtype, int64_t N, int64_t num_masks, float normalizer,
+                    const void* x, const void* mask, void* y) {
+  if (dtype == kF32) { reduce_loss(N, num_masks, normalizer, (const float*)x, (const float*)mask, (float*)y); return kOk; }
+  if (dtype == kF64) { reduce_loss(N, num_masks, normalizer, (const double*)x, (const double*)mask, (double*)y); return kOk; }
+  return kUnsupportedDtype;
+}
+
+int ref_reduce_loss_grad(int dtype, int64_t N, int64_t num_masks,
+                         float normalizer, const void* dl, const void* mask,
+                         void* dx) {
+  if (dtype == kF32) { reduce_loss_grad(N, num_masks, normalizer, (const float*)dl, (const float*)mask, (float*)dx); return kOk; }
+  if (dtype == kF64) { reduce_loss_grad(N, num_masks, normalizer, (const double*)dl, (const double*)mask, (double*)dx); return kOk; }
+  return kUnsupportedDtype;
+}
+
+int ref_broadcast_loss_grad(int dtype, int64_t N, int64_t S, int64_t C,
+                            const void* dl, void* dx) {
+  if (dtype == kF32) { broadcast_loss_grad(int(N), int(S), int(C), (const float*)dl, (float*)dx); return kOk; }
+  if (dtype == kF64) { broadcast_loss_grad(int(N), int(S), int(C), (const double*)dl, (double*)dx); return kOk; }
   return kUnsupportedDtype;
 }
 

@@ -13,6 +13,8 @@ kernels the way the reference's operator bodies do:
 * ``op_batch_norm_train`` / ``op_batch_norm_infer`` / ``*_grad``
                                dragon/operators/normalization/batch_norm_op.cc:8-226
 * ``op_lp_norm`` / ``_grad``     dragon/operators/normalization/lp_norm_op.cc:8-72
+* ``op_softmax_cross_entropy_loss`` / ``_grad``
+                               dragon/operators/loss/cross_entropy_softmax_loss_op.cc:8-143
 
 16-bit tensors travel as ``numpy.uint16`` bit patterns together with a dtype
 name (``"float16"`` / ``"bfloat16"``); ``to_bits`` / ``from_bits`` use the
@@ -130,6 +132,24 @@ def moments(dtype, x, axes):
         DTYPES[dtype], x.ndim, dims, len(axes), ax, _p(x), _p(mean), _p(var)),
         "moments")
     return mean, var
+
+
+REDUCE_KINDS = {"sum": 0, "sum_sqr": 1, "l1": 2}
+
+
+def reduce_sum(dtype, x, axes, scale=1.0, kind="sum"):
+    """math::ReduceSum / ReduceSumSqr / ReduceL1 over ``axes`` of ``x``; returns y flat."""
+    t = storage_dtype(dtype)
+    x = _c(x, t)
+    dims = (ctypes.c_int64 * x.ndim)(*x.shape)
+    axes = [a % x.ndim for a in axes]
+    ax = (ctypes.c_int64 * len(axes))(*axes)
+    n_out = int(np.prod([d for i, d in enumerate(x.shape) if i not in axes] or [1]))
+    y = np.empty(n_out, t)
+    _check(lib().ref_reduce_sum(
+        DTYPES[dtype], REDUCE_KINDS[kind], x.ndim, dims, len(axes), ax, ctypes.c_float(scale),
+        _p(x), _p(y)), "reduce_sum")
+    return y
 
 
 def inv_std(x, eps):
@@ -300,6 +320,75 @@ def lp_norm_grad(dtype, p, N, S, C, normalizer, epsilon, dy, x):
     return dx
 
 
+TARGET_DTYPES = {np.dtype(np.int32): 4, np.dtype(np.int64): 5}
+
+
+def cross_entropy(dtype, inp, target):
+    """kernels::CrossEntropy with dense targets, cross_entropy_kernel.cc:10-15."""
+    t = storage_dtype(dtype)
+    inp, target = _c(inp, t), _c(target, t)
+    loss = np.empty_like(inp)
+    _check(lib().ref_cross_entropy(DTYPES[dtype], _i64(inp.size), _p(inp), _p(target), _p(loss)),
+           "cross_entropy")
+    return loss
+
+
+def sparse_cross_entropy(dtype, N, S, C, ignore_index, inp, target):
+    """kernels::CrossEntropy with class-index targets; returns (loss, mask), each [N*S]."""
+    t = storage_dtype(dtype)
+    inp = _c(inp, t)
+    target = np.ascontiguousarray(target)
+    loss, mask = np.empty(N * S, t), np.empty(N * S, t)
+    _check(lib().ref_sparse_cross_entropy(
+        DTYPES[dtype], TARGET_DTYPES[target.dtype], _i64(N), _i64(S), _i64(C), _i64(ignore_index),
+        _p(inp), _p(target), _p(loss), _p(mask)), "sparse_cross_entropy")
+    return loss, mask
+
+
+def softmax_cross_entropy_grad(dtype, N, S, C, ignore_index, target, dx):
+    """kernels::SoftmaxCrossEntropyGrad: patches ``dx`` IN PLACE, returns mask [N*S]."""
+    t = storage_dtype(dtype)
+    assert dx.dtype == t and dx.flags.c_contiguous
+    target = np.ascontiguousarray(target)
+    mask = np.empty(N * S, t)
+    _check(lib().ref_softmax_cross_entropy_grad(
+        DTYPES[dtype], TARGET_DTYPES[target.dtype], _i64(N), _i64(S), _i64(C), _i64(ignore_index),
+        _p(target), _p(dx), _p(mask)), "softmax_cross_entropy_grad")
+    return mask
+
+
+def reduce_loss(dtype, normalizer, x, mask=None):
+    """kernels::ReduceLoss: returns the scalar as a 0-d array."""
+    t = storage_dtype(dtype)
+    x = _c(x, t)
+    y = np.empty(1, t)
+    m = None if mask is None else _c(mask, t)
+    _check(lib().ref_reduce_loss(
+        DTYPES[dtype], _i64(x.size), _i64(0 if m is None else m.size), ctypes.c_float(normalizer),
+        _p(x), _p(m), _p(y)), "reduce_loss")
+    return y.reshape(())
+
+
+def reduce_loss_grad(dtype, normalizer, dl, dx, mask=None):
+    """kernels::ReduceLossGrad: scales ``dx`` IN PLACE."""
+    t = storage_dtype(dtype)
+    assert dx.dtype == t and dx.flags.c_contiguous
+    m = None if mask is None else _c(mask, t)
+    _check(lib().ref_reduce_loss_grad(
+        DTYPES[dtype], _i64(dx.size), _i64(0 if m is None else m.size), ctypes.c_float(normalizer),
+        _p(_c(dl, t)), _p(m), _p(dx)), "reduce_loss_grad")
+    return dx
+
+
+def broadcast_loss_grad(dtype, N, S, C, dl, dx):
+    """kernels::BroadcastLossGrad: ``dx[n, c, s] *= dl[n, s]`` IN PLACE."""
+    t = storage_dtype(dtype)
+    assert dx.dtype == t and dx.flags.c_contiguous
+    _check(lib().ref_broadcast_loss_grad(
+        DTYPES[dtype], _i64(N), _i64(S), _i64(C), _p(_c(dl, t)), _p(dx)), "broadcast_loss_grad")
+    return dx
+
+
 # ---------------------------------------------------------------------------
 # Operator-level sequences (what the reference's op bodies run)
 # ---------------------------------------------------------------------------
@@ -346,6 +435,62 @@ def op_lp_norm_grad(dtype, x, dy, axis=-1, end_axis=None, p=2, eps=1e-12, reduct
     N, C, S = _lp_args(x.shape, axis, end_axis)
     normalizer = float(C) if reduction.upper() == "MEAN" else 1.0
     return lp_norm_grad(dtype, p, N, S, C, normalizer, eps, dy, x).reshape(x.shape)
+
+
+def _loss_normalizer(reduction, N, S, dim0, has_mask):
+    """cross_entropy_softmax_loss_op.cc:69-78."""
+    reduction = reduction.upper()
+    if reduction == "VALID":
+        return -1.0 if has_mask else float(N * S)
+    if reduction == "BATCH_MEAN":
+        return float(dim0)
+    if reduction == "MEAN":
+        return float(N * S)
+    return 1.0
+
+
+def op_softmax_cross_entropy_loss(dtype, x, target, axis=-1, ignore_index=None,
+                                  reduction="valid"):
+    """SoftmaxCrossEntropyLossOp, cross_entropy_softmax_loss_op.cc:8-88.
+
+    ``target`` is dense when it has the dtype of ``x`` and class indices when it
+    is int32 / int64. Returns (loss, prob) with prob the op's "X_norm" output.
+    """
+    ax, N, C, S = _axis_split(x.shape, axis)
+    ignore = 2 ** 31 - 1 if ignore_index is None else int(ignore_index)
+    prob = softmax(dtype, N, S, C, x)
+    dense = np.asarray(target).dtype == storage_dtype(dtype)
+    out_shape = tuple(d for i, d in enumerate(x.shape) if i != ax)
+    if dense:
+        loss, mask = cross_entropy(dtype, prob, target).ravel(), None
+    else:
+        loss, mask = sparse_cross_entropy(dtype, N, S, C, ignore, prob, target)
+    if reduction.upper() == "NONE":
+        if dense:
+            loss = reduce_sum(dtype, loss.reshape(N, C, S), [1])
+        return loss.reshape(out_shape), prob.reshape(x.shape)
+    normalizer = _loss_normalizer(reduction, N, S, x.shape[0], mask is not None)
+    return reduce_loss(dtype, normalizer, loss, mask), prob.reshape(x.shape)
+
+
+def op_softmax_cross_entropy_loss_grad(dtype, prob, target, dl, axis=-1, ignore_index=None,
+                                       reduction="valid"):
+    """SoftmaxCrossEntropyLossGradientOp, cross_entropy_softmax_loss_op.cc:90-143."""
+    ax, N, C, S = _axis_split(prob.shape, axis)
+    ignore = 2 ** 31 - 1 if ignore_index is None else int(ignore_index)
+    t = storage_dtype(dtype)
+    dx = np.array(prob, dtype=t, order="C", copy=True)
+    mask = None
+    if np.asarray(target).dtype == t:
+        dx -= _c(target, t).reshape(dx.shape)       # math::Axpy(-1)
+    else:
+        mask = softmax_cross_entropy_grad(dtype, N, S, C, ignore, target, dx)
+    if reduction.upper() == "NONE":
+        broadcast_loss_grad(dtype, N, S, C, dl, dx)
+    else:
+        normalizer = _loss_normalizer(reduction, N, S, prob.shape[0], mask is not None)
+        reduce_loss_grad(dtype, normalizer, dl, dx, mask)
+    return dx
 
 
 def op_layer_norm(dtype, x, gamma, beta, axis=-1, eps=1e-5):

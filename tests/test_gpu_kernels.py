@@ -547,3 +547,161 @@ def test_lp_norm_in_place_epsilon_clamp_and_empty(K):
     assert np.all(U.to_host(buf)[0] == 0)            # 0 / max(0, eps)
     e = empty((0, 8), "float32")
     K.l1_norm(0, 1, 8, 1.0, 1e-12, e, e)             # no rows: nothing to do, no error
+
+
+# ---------------------------------------------------------------- ReduceSum / ReduceSumSqr / ReduceL1
+
+@pytest.mark.parametrize("kind", ["sum", "sum_sqr", "l1"])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape,axes", MOMENT_CASES)
+def test_reduce_sums(K, shape, axes, dtype, kind):
+    rng = U.rng_for(1100 + len(shape))
+    x = R.to_bits((rng.standard_normal(shape) * 2 + 0.5).astype(np.float32), dtype)
+    xo, od = oracle_dtype_inputs(x, dtype)   # the reference's CPU has these for fp32/fp64 only
+    scale = 0.5
+    y_ref = R.reduce_sum(od, xo, list(axes), scale, kind)
+    f = {"sum": lambda v: v, "sum_sqr": np.square, "l1": np.abs}[kind]
+    y64 = (f(np.asarray(xo, np.float64)).sum(tuple(axes)) * scale).ravel()
+    y = empty(y_ref.shape, dtype)
+    fn = {"sum": K.reduce_sum, "sum_sqr": K.reduce_sum_sqr, "l1": K.reduce_l1}[kind]
+    fn(list(shape), list(axes), scale, U.to_device(x, dtype), y)
+    yw = U.widen(U.to_host(y), dtype)
+    # plain sums cancel: errors are measured against the sum of magnitudes
+    mag = (np.abs(f(np.asarray(xo, np.float64))).sum(tuple(axes)) * scale).ravel()
+    mag = float(np.max(mag)) if mag.size else 1.0
+    e_go = np.max(np.abs(yw - np.asarray(y_ref, np.float64))) / mag if yw.size else 0.0
+    e_ge = np.max(np.abs(yw - y64)) / mag if yw.size else 0.0
+    e_oe = np.max(np.abs(np.asarray(y_ref, np.float64) - y64)) / mag if yw.size else 0.0
+    assert e_ge <= U.TIGHT[dtype] and e_go <= U.TIGHT[dtype] + e_oe, (e_go, e_ge, e_oe)
+
+
+def test_sum_of_a_large_vector_and_empty_reduction(K):
+    rng = U.rng_for(12)
+    n = 3_000_001
+    x = rng.standard_normal(n).astype(np.float32)
+    y = empty((1,), "float32")
+    K.sum(n, 1.0, U.to_device(x, "float32"), y)
+    want = float(x.astype(np.float64).sum())
+    assert abs(float(U.to_host(y)[0]) - want) <= 1e-5 * float(np.abs(x).sum())
+    # a reduced extent of zero yields the sum's identity
+    out = U.to_device(np.full(3, 7.0, np.float32), "float32")
+    K.reduce_sum([3, 0], [1], 1.0, empty((3, 0), "float32"), out)
+    assert np.all(U.to_host(out) == 0)
+
+
+# ---------------------------------------------------------------- softmax cross-entropy loss
+
+SCE_SHAPES = [((64, 512), -1), ((10, 1000), -1), ((5, 37), -1), ((6, 4096), -1), ((3, 7, 5), 1),
+              ((2, 19, 8, 8), 1), ((4, 1), -1), ((3, 40000), -1), ((2, 6, 16), 1),
+              # more than 16384 positions: the two-stage loss reductions
+              ((70000, 8), -1), ((2, 5, 40000), 1)]
+
+
+def _sce_case(shape, axis, dtype, tdtype, seed):
+    rng = U.rng_for(seed)
+    ax = axis % len(shape)
+    x = (rng.standard_normal(shape) * 2).astype(dtype)
+    C = shape[ax]
+    tshape = tuple(d for i, d in enumerate(shape) if i != ax)
+    target = rng.integers(0, C, tshape).astype(tdtype)
+    target.ravel()[::4] = 255
+    N = int(np.prod(shape[:ax] or (1,)))
+    S = int(np.prod(shape[ax + 1:] or (1,)))
+    return x, target, tshape, N, C, S
+
+
+@pytest.mark.parametrize("dtype,tdtype", [("float32", "int64"), ("float32", "int32"),
+                                          ("float64", "int64")])
+@pytest.mark.parametrize("shape,axis", SCE_SHAPES)
+def test_loss_kernels_one_by_one(K, shape, axis, dtype, tdtype):
+    import torch
+    x, target, tshape, N, C, S = _sce_case(shape, axis, dtype, tdtype, 1300 + len(shape))
+    tol = U.TIGHT[dtype]
+    prob = R.softmax(dtype, N, S, C, x)
+    pd, td = U.to_device(prob, dtype), torch.from_numpy(target).cuda()
+    # CrossEntropy with class indices
+    loss_ref, mask_ref = R.sparse_cross_entropy(dtype, N, S, C, 255, prob, target)
+    loss, mask = empty((N * S,), dtype), empty((N * S,), dtype)
+    K.sparse_cross_entropy(N, S, C, 255, pd, td, loss, mask)
+    assert np.array_equal(U.to_host(mask), mask_ref)
+    assert U.normwise(U.to_host(loss), loss_ref) <= tol
+    # CrossEntropy with dense targets
+    dense = U.rng_for(5).random(prob.shape).astype(dtype)
+    dl_ref = R.cross_entropy(dtype, prob, dense)
+    dloss = empty(prob.shape, dtype)
+    K.cross_entropy(prob.size, pd, U.to_device(dense, dtype), dloss)
+    assert U.normwise(U.to_host(dloss), dl_ref) <= tol
+    # SoftmaxCrossEntropyGrad patches a copy of the probabilities in place
+    dx_ref = prob.copy()
+    gmask_ref = R.softmax_cross_entropy_grad(dtype, N, S, C, 255, target, dx_ref)
+    dx, gmask = pd.clone(), empty((N * S,), dtype)
+    K.softmax_cross_entropy_grad(N, S, C, 255, pd, td, dx, gmask)
+    assert np.array_equal(U.to_host(gmask), gmask_ref)
+    assert np.array_equal(U.to_host(dx), dx_ref)       # subtracting 1 and clearing are exact
+    # ReduceLoss / ReduceLossGrad with every normalisation, BroadcastLossGrad
+    for normalizer, use_mask in ((-1.0, True), (float(N * S), True), (1.0, False), (3.0, False)):
+        m_ref = mask_ref if use_mask else None
+        y_ref = R.reduce_loss(dtype, normalizer, loss_ref, m_ref)
+        y = empty((1,), dtype)
+        K.reduce_loss(N * S, N * S if use_mask else 0, normalizer, loss, mask if use_mask else None, y)
+        assert abs(float(U.to_host(y)[0]) - float(y_ref)) <= tol * max(1.0, abs(float(y_ref)))
+        dlv = np.array([1.7], dtype)
+        g_ref = R.reduce_loss_grad(dtype, normalizer, dlv, dx_ref.copy(), m_ref)
+        g = dx.clone()
+        K.reduce_loss_grad(g.numel(), N * S if use_mask else 0, normalizer,
+                           U.to_device(dlv, dtype), gmask if use_mask else None, g)
+        assert U.normwise(U.to_host(g), g_ref) <= tol
+    dlp = U.rng_for(6).standard_normal(N * S).astype(dtype)
+    b_ref = R.broadcast_loss_grad(dtype, N, S, C, dlp, dx_ref.copy())
+    b = dx.clone()
+    K.broadcast_loss_grad(N, S, C, U.to_device(dlp, dtype), b)
+    assert U.normwise(U.to_host(b), b_ref) <= tol
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean", "batch_mean", "valid"])
+@pytest.mark.parametrize("dtype,tdtype", [("float32", "int64"), ("float32", "int32"),
+                                          ("float64", "int64")])
+@pytest.mark.parametrize("shape,axis", SCE_SHAPES)
+def test_fused_softmax_cross_entropy_loss(K, shape, axis, dtype, tdtype, reduction):
+    import torch
+    x, target, tshape, N, C, S = _sce_case(shape, axis, dtype, tdtype, 1400 + len(shape))
+    tol = U.TIGHT[dtype]
+    loss_ref, prob_ref = R.op_softmax_cross_entropy_loss(dtype, x, target, axis, 255, reduction)
+    xd, td = U.to_device(x, dtype), torch.from_numpy(target).cuda()
+    prob = empty(shape, dtype)
+    loss = empty(tshape if reduction == "none" else (1,), dtype)
+    # BATCH_MEAN divides by the leading extent of x, which is N only for a 2-d view
+    if reduction == "batch_mean" and shape[0] != N:
+        pytest.skip("the fused entry point takes N as the batch extent")
+    K.softmax_cross_entropy_loss_forward(N, S, C, 255, reduction, xd, td, prob, loss)
+    # the oracle's sequential fp32 sums over 40000 classes are themselves ~1e-5 off
+    x64 = np.moveaxis(np.asarray(x, np.float64), axis % len(shape), -1)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    p64 = np.moveaxis(e / e.sum(-1, keepdims=True), -1, axis % len(shape))
+    ok, *errs = U.close3(U.to_host(prob), prob_ref, p64, tol)
+    assert ok, errs
+    got = U.to_host(loss).reshape(np.shape(loss_ref))
+    assert np.max(np.abs(got - loss_ref)) <= 4 * tol * max(1.0, float(np.max(np.abs(loss_ref))))
+    # backward from the probabilities the forward produced
+    ph = U.to_host(prob)
+    dl = (U.rng_for(7).standard_normal(tshape).astype(dtype) if reduction == "none"
+          else np.array(1.7, dtype))
+    dx_ref = R.op_softmax_cross_entropy_loss_grad(dtype, ph, target, dl, axis, 255, reduction)
+    dx = empty(shape, dtype)
+    K.softmax_cross_entropy_loss_backward(N, S, C, 255, reduction, prob, td,
+                                          U.to_device(np.atleast_1d(dl), dtype), dx)
+    assert U.normwise(U.to_host(dx), dx_ref) <= tol
+    ignored = np.expand_dims(target == 255, axis % len(shape))
+    assert np.all(U.to_host(dx)[np.broadcast_to(ignored, shape)] == 0)
+
+
+def test_fused_softmax_cross_entropy_loss_out_of_range_target_is_ignored(K):
+    import torch
+    x = np.zeros((4, 8), np.float32)
+    target = np.array([1, 8, -3, 2], np.int64)     # 8 and -3 are outside [0, 8)
+    xd, td = U.to_device(x, "float32"), torch.from_numpy(target).cuda()
+    prob, loss = empty((4, 8), "float32"), empty((4,), "float32")
+    K.softmax_cross_entropy_loss_forward(4, 1, 8, 2 ** 31 - 1, "none", xd, td, prob, loss)
+    got = U.to_host(loss)
+    assert got[1] == 0 and got[2] == 0
+    assert np.allclose(got[[0, 3]], np.log(8.0), rtol=1e-6)

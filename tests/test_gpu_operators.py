@@ -103,6 +103,51 @@ def test_lp_norm_axis_range_and_bad_order(rt, ws):
         ws.run_operator(rt.make_def("LpNorm", [x], ["y_bad"], p=3))
 
 
+def test_softmax_cross_entropy_loss(rt, ws):
+    g = GOLD["softmax_cross_entropy_loss"]
+    for reduction in g["reductions"]:
+        data1 = np.log(np.array(g["probs"], "float32"))
+        data2 = np.array(g["target"], "int32")
+        data3 = np.eye(3, dtype="float32")[data2]
+        scale = (np.exp(data1) - data3) / (data1.shape[0] if reduction == "mean" else 1)
+        picked = -data1[np.arange(2), data2]
+        result = {"mean": picked.mean(), "sum": picked.sum(), "none": picked}[reduction]
+        for target in (data2, data2.astype("int64"), data3):
+            tape = rt.Tape(ws)
+            x, y = ws.feed("x", data1), ws.feed("y", target)
+            loss = rt.softmax_cross_entropy_loss(tape, [x, y], reduction=reduction)
+            data4 = arange(np.shape(result), 2)
+            dl = ws.feed("dl", data4)
+            (dx,) = tape.gradient(loss, [x], output_gradient=dl)
+            assert_equal(ws.fetch(loss), result, g["prec"])
+            assert_equal(ws.fetch(dx), np.expand_dims(data4, -1) * scale, g["prec"])
+
+
+def test_softmax_cross_entropy_loss_ignore_index_axis_and_valid(rt, ws):
+    rng = np.random.default_rng(8)
+    data = rng.standard_normal((4, 6, 5)).astype("float32")
+    target = rng.integers(0, 6, (4, 5)).astype("int64")
+    target[0, :] = 255
+    for reduction in ("valid", "batch_mean", "mean", "sum", "none"):
+        tape = rt.Tape(ws)
+        x, y = ws.feed("x", data), ws.feed("y", target)
+        loss = rt.softmax_cross_entropy_loss(tape, [x, y], axis=1, ignore_index=255,
+                                             reduction=reduction)
+        want, prob = R.op_softmax_cross_entropy_loss("float32", data, target, 1, 255, reduction)
+        assert_equal(ws.fetch(loss), want, 1e-5)
+        dl_np = (rng.standard_normal((4, 5)).astype("float32") if reduction == "none"
+                 else np.array(0.7, "float32"))
+        dl = ws.feed("dl", dl_np)
+        (dx,) = tape.gradient(loss, [x], output_gradient=dl)
+        want_dx = R.op_softmax_cross_entropy_loss_grad("float32", prob, target, dl_np, 1, 255,
+                                                       reduction)
+        assert_equal(ws.fetch(dx), want_dx, 1e-6)
+        assert np.all(ws.fetch(dx)[0] == 0)
+    with pytest.raises(rt.DragonError, match="Numel of X and Y"):
+        ws.run_operator(rt.make_def("SoftmaxCrossEntropyLoss", [ws.feed("x", data),
+                                                                ws.feed("y", target[:2])], ["l"], axis=1))
+
+
 def test_layer_norm(rt, ws):
     g = GOLD["layer_norm"]
     x_shape, w_shape = tuple(g["x_shape"]), (g["x_shape"][-1],)

@@ -21,7 +21,7 @@ def test_registry_holds_the_ten_operator_types_and_the_sync_aliases():
     assert {"LayerNorm", "LayerNormGradient", "GroupNorm", "GroupNormGradient", "BatchNorm",
             "BatchNormGradient", "Softmax", "SoftmaxGradient", "LogSoftmax",
             "LogSoftmaxGradient", "SyncBatchNorm", "SyncBatchNormGradient", "LpNorm",
-            "LpNormGradient"} <= ops
+            "LpNormGradient", "SoftmaxCrossEntropyLoss", "SoftmaxCrossEntropyLossGradient"} <= ops
 
 
 def test_feed_fetch_round_trip(ws):

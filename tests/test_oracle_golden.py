@@ -475,3 +475,103 @@ def test_lp_norm_epsilon_clamp_and_zero_rows():
     # d/dx of x/|x| is orthogonal to x when dy is parallel to x
     dxp = R.op_lp_norm_grad("float32", x[1:], x[1:].copy(), -1, None, 2, 1e-12, "sum")
     assert maxabs(dxp, 0.0) < 1e-6
+
+
+# ---------------------------------------------------------------- reduce sums
+
+REDUCE_CASES = [((2, 3, 3), (0,)), ((2, 3, 3), (1,)), ((2, 3, 3), (1, 2)), ((2, 3, 3), (0, 1, 2)),
+                ((4, 5, 6, 7), (1, 3)), ((4, 5, 6, 7), (0, 2)), ((3, 1, 5), (1,)), ((7,), (0,)),
+                ((6, 5), (0,)), ((2, 3, 4, 5), (0, 3))]
+
+
+@pytest.mark.parametrize("kind", ["sum", "sum_sqr", "l1"])
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+@pytest.mark.parametrize("shape,axes", REDUCE_CASES)
+def test_reduce_sum_against_numpy(shape, axes, dtype, kind):
+    # the reference's own reduce tests compare with numpy (test_ops.py:4047-4073 for sum)
+    if shape == (2, 3, 3):
+        data = arange(shape).astype(dtype) - 4
+    else:
+        data = np.random.default_rng(21).standard_normal(shape).astype(dtype)
+    f = {"sum": lambda v: v, "sum_sqr": np.square, "l1": np.abs}[kind]
+    for scale in (1.0, 0.25):
+        want = f(data.astype(np.float64)).sum(axes) * scale
+        got = R.reduce_sum(dtype, data, list(axes), scale, kind)
+        assert got.shape == (want.size,)
+        tol = 1e-12 if dtype == "float64" else 2e-6
+        assert maxabs(got, want.ravel()) <= tol * max(1.0, float(np.max(np.abs(want))))
+
+
+def test_reduce_sum_rejects_16_bit_like_the_reference_cpu():
+    x = np.zeros(4, np.uint16)
+    with pytest.raises(RuntimeError):
+        R.reduce_sum("float16", x, [0])
+
+
+# ---------------------------------------------------------------- softmax cross-entropy loss
+
+def _sce_numpy(x, target, dl, axis, ignore_index, reduction):
+    """fp64 closed form of the operator pair for class-index targets."""
+    x64 = np.moveaxis(np.asarray(x, np.float64), axis, -1)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    p = e / e.sum(-1, keepdims=True)
+    tgt = np.asarray(target)
+    valid = tgt != ignore_index if ignore_index is not None else np.ones(tgt.shape, bool)
+    safe = np.where(valid, tgt, 0)
+    picked = np.take_along_axis(p, safe[..., None], -1)[..., 0]
+    loss = np.where(valid, -np.log(np.maximum(picked, np.finfo(np.float32).tiny)), 0.0)
+    onehot = np.zeros_like(p)
+    np.put_along_axis(onehot, safe[..., None], 1.0, -1)
+    g = (p - onehot) * valid[..., None]
+    r = reduction.lower()
+    if r == "none":
+        return loss, np.moveaxis(g * np.asarray(dl, np.float64)[..., None], -1, axis)
+    n = {"sum": 1.0, "mean": float(tgt.size), "batch_mean": float(x.shape[0]),
+         "valid": float(valid.sum())}[r]
+    return loss.sum() / max(n, 1.0), np.moveaxis(g * float(dl) / max(n, 0.5), -1, axis)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+@pytest.mark.parametrize("target_kind", ["int32", "int64", "dense"])
+def test_softmax_cross_entropy_loss_reference_closed_form(dtype, target_kind):
+    g = GOLD["softmax_cross_entropy_loss"]
+    data1 = np.log(np.array(g["probs"], "float32")).astype(dtype)
+    data2 = np.array(g["target"], "int32")
+    data3 = np.eye(3, dtype=dtype)[data2]
+    tgt = data3 if target_kind == "dense" else data2.astype(target_kind)
+    for reduction in g["reductions"]:
+        scale = (np.exp(data1) - data3) / (data1.shape[0] if reduction == "mean" else 1)
+        picked = -data1[np.arange(2), data2]
+        result = {"mean": picked.mean(), "sum": picked.sum(), "none": picked}[reduction]
+        loss, prob = R.op_softmax_cross_entropy_loss(dtype, data1, tgt, reduction=reduction)
+        data4 = arange(loss.shape, 2).astype(dtype)
+        dx = R.op_softmax_cross_entropy_loss_grad(dtype, prob, tgt, data4, reduction=reduction)
+        assert maxabs(loss, result) <= g["prec"]
+        assert maxabs(dx, np.expand_dims(data4, -1) * scale) <= g["prec"]
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean", "batch_mean", "valid"])
+@pytest.mark.parametrize("shape,axis", [((6, 7), -1), ((3, 5, 4), 1), ((2, 4, 3, 3), 1)])
+def test_softmax_cross_entropy_loss_ignore_index_vs_fp64(shape, axis, reduction):
+    rng = np.random.default_rng(31)
+    x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    C = shape[axis]
+    tshape = tuple(d for i, d in enumerate(shape) if i != axis % len(shape))
+    target = rng.integers(0, C, tshape).astype(np.int64)
+    target.ravel()[::3] = 255                                  # ignored positions
+    loss, prob = R.op_softmax_cross_entropy_loss("float32", x, target, axis, 255, reduction)
+    dl = rng.standard_normal(tshape).astype(np.float32) if reduction == "none" else np.float32(1.7)
+    dx = R.op_softmax_cross_entropy_loss_grad("float32", prob, target, np.asarray(dl, np.float32),
+                                              axis, 255, reduction)
+    want_loss, want_dx = _sce_numpy(x, target, dl, axis % len(shape), 255, reduction)
+    assert maxabs(loss, want_loss) <= 2e-6 * max(1.0, float(np.max(np.abs(want_loss))))
+    assert maxabs(dx, want_dx) <= 2e-6 * max(1.0, float(np.max(np.abs(want_dx))))
+
+
+def test_softmax_cross_entropy_loss_all_ignored_is_zero():
+    x = np.zeros((3, 4), np.float32)
+    target = np.full(3, 9, np.int32)
+    loss, prob = R.op_softmax_cross_entropy_loss("float32", x, target, -1, 9, "valid")
+    assert float(loss) == 0.0                                   # sum 0 / max(0, 1)
+    dx = R.op_softmax_cross_entropy_loss_grad("float32", prob, target, np.float32(1), -1, 9, "valid")
+    assert np.all(dx == 0)
