@@ -22,10 +22,13 @@ SIGNATURES = {
     "dragon_hip_set_device": (_int, [_int]),
     "dragon_hip_get_device": (_int, [ctypes.POINTER(_int)]),
     "dragon_hip_device_name": (_int, [_int, ctypes.c_char_p, _sz]),
+    "dragon_hip_device_capability": (_int, [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
+    "dragon_hip_device_sync": (_int, []),
     "dragon_hip_mem_info": (_int, [ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
     "dragon_hip_stream_create": (_int, [ctypes.POINTER(_vp)]),
     "dragon_hip_stream_destroy": (_int, [_vp]),
     "dragon_hip_stream_sync": (_int, [_vp]),
+    "dragon_hip_stream_query": (_int, [_vp, ctypes.POINTER(_int)]),
     "dragon_hip_malloc": (_int, [ctypes.POINTER(_vp), _sz]),
     "dragon_hip_free": (_int, [_vp]),
     "dragon_hip_host_malloc": (_int, [ctypes.POINTER(_vp), _sz]),

@@ -41,6 +41,15 @@ int dragon_hip_device_name(int device, char* buf, size_t buf_bytes) {
   snprintf(buf, buf_bytes, "%s (%s)", prop.name, prop.gcnArchName);
   return DRAGON_HIP_OK;
 }
+int dragon_hip_device_capability(int device, int* major, int* minor) {
+  if (!major || !minor) return DRAGON_HIP_EINVAL;
+  hipDeviceProp_t prop;
+  const hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return st(e);
+  *major = prop.major, *minor = prop.minor;
+  return DRAGON_HIP_OK;
+}
+int dragon_hip_device_sync(void) { return st(hipDeviceSynchronize()); }
 int dragon_hip_mem_info(size_t* free_bytes, size_t* total_bytes) {
   if (!free_bytes || !total_bytes) return DRAGON_HIP_EINVAL;
   return st(hipMemGetInfo(free_bytes, total_bytes));
@@ -53,6 +62,16 @@ int dragon_hip_stream_create(void** stream) {
   return st(e);
 }
 int dragon_hip_stream_destroy(void* stream) { return st(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
+int dragon_hip_stream_query(void* stream, int* done) {
+  if (!done) return DRAGON_HIP_EINVAL;
+  const hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
+  if (e == hipErrorNotReady) {
+    *done = 0;
+    return DRAGON_HIP_OK;
+  }
+  *done = e == hipSuccess ? 1 : 0;
+  return st(e);
+}
 int dragon_hip_stream_sync(void* stream) { return st(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
 int dragon_hip_malloc(void** ptr, size_t bytes) {
   if (!ptr) return DRAGON_HIP_EINVAL;

@@ -74,11 +74,14 @@ int dragon_hip_device_count(int* count);
 int dragon_hip_set_device(int device);
 int dragon_hip_get_device(int* device);
 int dragon_hip_device_name(int device, char* buf, size_t buf_bytes);
+int dragon_hip_device_capability(int device, int* major, int* minor);
+int dragon_hip_device_sync(void);  /* every stream of the current device */
 int dragon_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
 /* Streams are non-blocking and all at the default priority. */
 int dragon_hip_stream_create(void** stream);
 int dragon_hip_stream_destroy(void* stream);
 int dragon_hip_stream_sync(void* stream);  /* Context::SynchronizeStream */
+int dragon_hip_stream_query(void* stream, int* done); /* 1 when all work on it has finished */
 int dragon_hip_malloc(void** ptr, size_t bytes);       /* Context::New    */
 int dragon_hip_free(void* ptr);                        /* Context::Delete */
 int dragon_hip_host_malloc(void** ptr, size_t bytes);  /* pinned host memory */

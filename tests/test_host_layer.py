@@ -98,3 +98,18 @@ def test_malformed_definitions_are_fatal(ws):
                 'type: "Softmax" input: "x'):
         with pytest.raises(rt.DragonError):
             ws.run_operator(bad)
+
+
+def test_hip_module_without_a_device():
+    """Without a GPU the count is zero and every per-device query fails loudly."""
+    import torch
+    from dragon_amd import _lib, hip
+    hip.set_default_device(0)
+    assert hip.default_device() == {"device_type": "hip", "device_index": 0}
+    hip.set_default_device(-1)
+    assert hip.default_device()["device_type"] == "cpu"
+    if not torch.cuda.is_available():
+        assert hip.is_available() is False
+        assert hip.get_device_count() == 0
+        with pytest.raises(_lib.DragonHipError):
+            hip.get_device_name(0)
