@@ -152,6 +152,19 @@ template <typename T>
 __device__ __forceinline__ void store_packet(T* p, const u32x4 t) {
   __builtin_nontemporal_store(t, reinterpret_cast<u32x4_any*>(p));
 }
+// The same packet at an address that is only element-aligned (rows whose byte
+// length is not a multiple of 16): still one 128-bit access, the memory system
+// splits it where it straddles a cache line.
+typedef uint32_t u32x4_unaligned __attribute__((ext_vector_type(4), may_alias, aligned(2)));
+template <typename T>
+__device__ __forceinline__ u32x4 load_packet_unaligned(const T* p) {
+  return *reinterpret_cast<const u32x4_unaligned*>(p);
+}
+template <typename T>
+__device__ __forceinline__ void store_packet_unaligned(T* p, const u32x4 t) {
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4_unaligned*>(p));
+}
+
 template <typename T>
 __device__ __forceinline__ void load_unpack(const T* p, typename IO<T>::Acc (&v)[IO<T>::kVec]) {
   IO<T>::unpack(load_packet(p), v);

@@ -11,22 +11,23 @@
 // once. Variance is the centred sum sum((x-mu)^2)/C computed from the
 // register copy: same quantity as the reference's E[x^2]-E[x]^2 without its
 // cancellation.
+#include "row_loop.h"
 #include "row_tile.h"
 
 namespace dragon_hip {
 namespace {
 
-template <typename T, int kTPR, int kVPT>
+template <typename T, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
     const int64_t N, const int C, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
     T* __restrict__ y) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
   const A inv_c = A(1) / A(C);
   const int lane = Tile::lane();
 
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
           const A d = t.v[i][e] - mean;
-          q += d * d;
+          if (Tile::elem_active(i, e, npackets)) q += d * d;
         }
       }
     }
@@ -65,8 +66,16 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
       if (Tile::active(i, npackets)) {
         const int col = (i * kTPR + lane) * kVec;
         A g[kVec], b[kVec];
-        load_params<kVec>(gamma + col, g);
-        load_params<kVec>(beta + col, b);
+        if constexpr (kRagged) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            g[e] = col + e < C ? gamma[col + e] : A(0);
+            b[e] = col + e < C ? beta[col + e] : A(0);
+          }
+        } else {
+          load_params<kVec>(gamma + col, g);
+          load_params<kVec>(beta + col, b);
+        }
 #pragma unroll
         for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * rs * g[e] + b[e];
       }
@@ -164,38 +173,54 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
   }
 }
 
-// Any width, any alignment: one 256-thread workgroup per row, three strided
-// passes over the row with element-wise accesses (the second and third hit L2).
+// Rows too long for the register tiles: two passes per row. Pass one
+// accumulates sums shifted by the row's first element (mean = s + sum(x-s)/C,
+// var = sum((x-s)^2)/C - (sum(x-s)/C)^2: no cancellation against a large mean),
+// pass two normalises; gamma and beta are read element-wise (any alignment).
 template <typename T>
-__global__ __launch_bounds__(256) void layer_norm_rows_looped(
+__global__ __launch_bounds__(kLoopThreads) void layer_norm_rows_looped(
     const int64_t N, const int64_t C, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
     T* __restrict__ y) {
   using A = typename IO<T>::Acc;
-  __shared__ A slots[2][4];
+  using Loop = RowLoop<T>;
+  constexpr int kVec = Loop::kVec;
+  __shared__ A slots[2][kLoopWaves];
   const A inv_c = A(1) / A(C);
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const T* xr = x + row * C;
     T* yr = y + row * C;
-    A s = A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) s += IO<T>::load1(xr + j);
-    const A mean = block_allreduce<4>(s, SumOp(), slots[0]) * inv_c;
-    A q = A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A d = IO<T>::load1(xr + j) - mean;
-      q += d * d;
-    }
-    const A var = block_allreduce<4>(q, SumOp(), slots[1]) * inv_c;
-    const A rs = acc_rsqrt_exact(var + eps);
+    const A shift = IO<T>::load1(xr);
+    A s = A(0), q = A(0);
+    Loop::visit(xr, C, shift, [&](int64_t, const A(&v)[kVec], int) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A d = v[e] - shift;  // padding holds `shift`: adds nothing
+        s += d;
+        q += d * d;
+      }
+    });
+    s = block_allreduce<kLoopWaves>(s, SumOp(), slots[0]);
+    q = block_allreduce<kLoopWaves>(q, SumOp(), slots[1]);
+    const A dm = s * inv_c;
+    const A mean = shift + dm;
+    const A rs = acc_rsqrt_exact((q * inv_c - dm * dm) + eps);
     if (threadIdx.x == 0) {
       mu[row] = mean;
       rsig[row] = rs;
     }
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      IO<T>::store1(yr + j, (IO<T>::load1(xr + j) - mean) * rs * gamma[j] + beta[j]);
-    }
-    __syncthreads();
+    Loop::visit(xr, C, A(0), [&](int64_t col, const A(&v)[kVec], int n) {
+      A o[kVec];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A g = e < n ? gamma[col + e] : A(0);
+        const A b = e < n ? beta[col + e] : A(0);
+        o[e] = (v[e] - mean) * rs * g + b;
+      }
+      Loop::store(yr, col, o, n);
+    });
+    __syncthreads();  // slots are reused by the next row
   }
 }
 
@@ -211,8 +236,9 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
   A* mp = static_cast<A*>(mu);
   A* rp = static_cast<A*>(rsig);
   RowConfig cfg;
-  const bool packets_ok = C % kVec == 0 && aligned16(x) && aligned16(y) && aligned16(gamma) &&
-      aligned16(beta) && pick_row_config(C / kVec, 8, &cfg);
+  const bool fits = pick_row_config(ceil_div(C, kVec), 8, &cfg);
+  const bool packets_ok = fits && C % kVec == 0 && aligned16(x) && aligned16(y) &&
+      aligned16(gamma) && aligned16(beta);
   const size_t staged_bytes = 2 * static_cast<size_t>(C) * sizeof(A);
   if (packets_ok && cfg.tpr > kWaveSize && staged_bytes <= kMaxStagedParamBytes) {
     // 256-thread tiles need several workgroups per compute unit to hide HBM
@@ -242,15 +268,26 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
 #define LAUNCH(TPR, VPT)                                                                   \
   {                                                                                        \
     using Tile = RowTile<T, TPR, VPT>;                                                     \
-    hipLaunchKernelGGL((layer_norm_rows<T, TPR, VPT>), dim3(row_grid(N, Tile::kRowsPerBlock)), \
-                       dim3(Tile::kThreads), 0, stream, N, static_cast<int>(C), A(eps), xp, gp, \
-                       bp, mp, rp, yp);                                                    \
+    hipLaunchKernelGGL((layer_norm_rows<T, TPR, VPT, false>),                              \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       N, static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);            \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+  } else if (fits) {
+    // any width, any alignment: ragged tiles, parameters read element-wise
+#define LAUNCH(TPR, VPT)                                                                   \
+  {                                                                                        \
+    using Tile = RowTile<T, TPR, VPT>;                                                     \
+    hipLaunchKernelGGL((layer_norm_rows<T, TPR, VPT, true>),                               \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       N, static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);            \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
   } else {
-    hipLaunchKernelGGL((layer_norm_rows_looped<T>), dim3(row_grid(N, 1)), dim3(256), 0, stream, N,
-                       C, A(eps), xp, gp, bp, mp, rp, yp);
+    hipLaunchKernelGGL((layer_norm_rows_looped<T>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
+                       stream, N, C, A(eps), xp, gp, bp, mp, rp, yp);
   }
   return status_of_launch();
 }

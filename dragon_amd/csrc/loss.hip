@@ -259,16 +259,16 @@ __global__ __launch_bounds__(kLossThreads) void broadcast_loss_grad(
 
 // softmax_rows with the loss gather folded in: the thread whose tile slot holds
 // column `target[row]` writes -log(max(p, FLT_MIN)).
-template <typename T, typename TargetT, int kTPR, int kVPT>
+template <typename T, typename TargetT, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_ce_rows(
     const int64_t N, const int C, const int64_t ignore_index, const T* __restrict__ x,
     const TargetT* __restrict__ target, T* __restrict__ prob, T* __restrict__ loss,
     T* __restrict__ mask) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
 
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
@@ -498,14 +498,19 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
   T* mask = static_cast<T*>(scratch) + NxS;
   T* part = mask + NxS;
   RowConfig cfg;
-  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(prob) &&
-      pick_row_config(C / kVec, 8, &cfg)) {
+  if (S == 1 && pick_row_config(ceil_div(C, kVec), 8, &cfg)) {
+    const bool regular = C % kVec == 0 && aligned16(x) && aligned16(prob);  // else ragged tiles
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
-    hipLaunchKernelGGL((softmax_ce_rows<T, TargetT, TPR, VPT>),                                 \
-                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
-                       N, static_cast<int>(C), ignore_index, xp, tp, pp, loss, mask);           \
+    const dim3 grid(row_grid(N, Tile::kRowsPerBlock)), block(Tile::kThreads);                   \
+    if (regular) {                                                                              \
+      hipLaunchKernelGGL((softmax_ce_rows<T, TargetT, TPR, VPT, false>), grid, block, 0, stream, \
+                         N, static_cast<int>(C), ignore_index, xp, tp, pp, loss, mask);         \
+    } else {                                                                                    \
+      hipLaunchKernelGGL((softmax_ce_rows<T, TargetT, TPR, VPT, true>), grid, block, 0, stream, \
+                         N, static_cast<int>(C), ignore_index, xp, tp, pp, loss, mask);         \
+    }                                                                                           \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH

@@ -20,6 +20,7 @@
 // 16-bit I/O accumulates in fp32 as the reference's CUDA kernels do; fp32 and
 // fp64 I/O divide by the norm exactly as the reference's CPU expression does,
 // 16-bit I/O multiplies by its reciprocal (error far below one 16-bit ulp).
+#include "row_loop.h"
 #include "row_tile.h"
 
 namespace dragon_hip {
@@ -66,16 +67,16 @@ struct LpMath {
   }
 };
 
-template <typename T, int kP, int kTPR, int kVPT>
+template <typename T, int kP, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void lp_norm_rows(
     const int64_t N, const int C, const typename IO<T>::Acc normalizer,
     const typename IO<T>::Acc eps, const T* x, T* y) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = LpMath<T, kP>;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
 
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
@@ -98,16 +99,16 @@ __global__ __launch_bounds__(row_threads(kTPR)) void lp_norm_rows(
   }
 }
 
-template <typename T, int kP, int kTPR, int kVPT>
+template <typename T, int kP, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void lp_norm_grad_rows(
     const int64_t N, const int C, const typename IO<T>::Acc normalizer,
     const typename IO<T>::Acc eps, const T* dy, const T* x, T* dx) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = LpMath<T, kP>;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2 * Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
 
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
@@ -136,38 +137,56 @@ __global__ __launch_bounds__(row_threads(kTPR)) void lp_norm_grad_rows(
   }
 }
 
-// One workgroup per contiguous row of any length or alignment.
+// S == 1 rows too long for the register tiles: two passes per row.
 template <typename T, int kP, bool kGrad>
-__global__ __launch_bounds__(256) void lp_norm_rows_looped(
+__global__ __launch_bounds__(kLoopThreads) void lp_norm_rows_looped(
     const int64_t N, const int64_t C, const typename IO<T>::Acc normalizer,
     const typename IO<T>::Acc eps, const T* dy, const T* x, T* out) {
   using A = typename IO<T>::Acc;
   using M = LpMath<T, kP>;
-  __shared__ A slots[2][4];
+  using Loop = RowLoop<T>;
+  constexpr int kVec = Loop::kVec;
+  __shared__ A slots[2][kLoopWaves];
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const T* xr = x + row * C;
-    const T* gr = kGrad ? dy + row * C : nullptr;
+    const T* gr = kGrad ? dy + row * C : xr;
     T* outr = out + row * C;
     A acc = A(0), dot = A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A v = IO<T>::load1(xr + j);
-      acc += M::term(v);
-      if (kGrad) dot += IO<T>::load1(gr + j) * v;
+    if constexpr (kGrad) {
+      Loop::visit2(gr, xr, C, A(0), [&](int64_t, const A(&g)[kVec], const A(&v)[kVec], int) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          acc += M::term(v[e]);
+          dot += g[e] * v[e];
+        }
+      });
+    } else {
+      Loop::visit(xr, C, A(0), [&](int64_t, const A(&v)[kVec], int) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) acc += M::term(v[e]);
+      });
     }
-    acc = block_allreduce<4>(acc, SumOp(), slots[0]);
-    if (kGrad) dot = block_allreduce<4>(dot, SumOp(), slots[1]);
+    acc = block_allreduce<kLoopWaves>(acc, SumOp(), slots[0]);
+    if (kGrad) dot = block_allreduce<kLoopWaves>(dot, SumOp(), slots[1]);
     const A norm = M::norm_of(acc, normalizer, eps);
     const A inv = A(1) / norm;
     const A coef = kGrad ? M::coef_of(dot, normalizer, norm) : A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A v = IO<T>::load1(xr + j);
-      if (kGrad) {
-        IO<T>::store1(outr + j, M::backward(IO<T>::load1(gr + j), v, norm, inv, coef));
-      } else {
-        IO<T>::store1(outr + j, M::forward(v, norm, inv));
-      }
+    if constexpr (kGrad) {
+      Loop::visit2(gr, xr, C, A(0), [&](int64_t col, const A(&g)[kVec], const A(&v)[kVec], int n) {
+        A o[kVec];
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) o[e] = M::backward(g[e], v[e], norm, inv, coef);
+        Loop::store(outr, col, o, n);
+      });
+    } else {
+      Loop::visit(xr, C, A(0), [&](int64_t col, const A(&v)[kVec], int n) {
+        A o[kVec];
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) o[e] = M::forward(v[e], norm, inv);
+        Loop::store(outr, col, o, n);
+      });
     }
-    __syncthreads();
+    __syncthreads();  // slots are reused by the next row
   }
 }
 
@@ -251,25 +270,32 @@ int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsi
   const bool packets_ok = aligned16(x) && aligned16(out) && (!kGrad || aligned16(dy));
   RowConfig cfg;
   // The gradient holds two tiles at once: halve the packets a thread may hold.
-  if (S == 1 && C % kVec == 0 && packets_ok && pick_row_config(C / kVec, kGrad ? 4 : 8, &cfg)) {
-#define LAUNCH(TPR, VPT)                                                                        \
+  if (S == 1 && pick_row_config(ceil_div(C, kVec), kGrad ? 4 : 8, &cfg)) {
+    const bool regular = C % kVec == 0 && packets_ok;  // else ragged tiles
+#define LAUNCH_FLAVOUR(TPR, VPT, RAGGED)                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
     if constexpr (kGrad) {                                                                      \
-      hipLaunchKernelGGL((lp_norm_grad_rows<T, kP, TPR, VPT>),                                  \
+      hipLaunchKernelGGL((lp_norm_grad_rows<T, kP, TPR, VPT, RAGGED>),                          \
                          dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,       \
                          stream, N, static_cast<int>(C), nrm, eps, gp, xp, op);                 \
     } else {                                                                                    \
-      hipLaunchKernelGGL((lp_norm_rows<T, kP, TPR, VPT>),                                       \
+      hipLaunchKernelGGL((lp_norm_rows<T, kP, TPR, VPT, RAGGED>),                               \
                          dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,       \
                          stream, N, static_cast<int>(C), nrm, eps, xp, op);                     \
     }                                                                                           \
   }
+#define LAUNCH(TPR, VPT)                                          \
+  {                                                               \
+    if (regular) LAUNCH_FLAVOUR(TPR, VPT, false)                  \
+    else LAUNCH_FLAVOUR(TPR, VPT, true)                           \
+  }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
-  } else if (S == 1 && C >= 256) {
-    hipLaunchKernelGGL((lp_norm_rows_looped<T, kP, kGrad>), dim3(row_grid(N, 1)), dim3(256), 0,
-                       stream, N, C, nrm, eps, gp, xp, op);
+#undef LAUNCH_FLAVOUR
+  } else if (S == 1) {
+    hipLaunchKernelGGL((lp_norm_rows_looped<T, kP, kGrad>), dim3(loop_grid(N)), dim3(kLoopThreads),
+                       0, stream, N, C, nrm, eps, gp, xp, op);
   } else if (kVec > 1 && S % kVec == 0 && packets_ok) {
     hipLaunchKernelGGL((lp_norm_columns<T, kP, kGrad, kVec>), dim3(flat_grid(N * (S / kVec))),
                        dim3(256), 0, stream, N, S, C, nrm, eps, gp, xp, op);

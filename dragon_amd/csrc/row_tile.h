@@ -12,6 +12,12 @@
 // A tile covers rows of up to kTPR * kVPT packets; slots beyond the row's
 // packet count are masked off, which is how widths that are not a multiple of
 // the tile (e.g. 1000 = 125 packets of 8) are handled.
+//
+// Ragged tiles (kRagged) take rows of any width and alignment: packets are
+// counted from the row's first element, so a packet may sit at an address that
+// is only element-aligned, and the last packet of a row may be partial (it is
+// then read and written element by element). Their `extent` argument is the
+// row's element count; for regular tiles it is the row's packet count.
 #pragma once
 
 #include "common.h"
@@ -25,7 +31,7 @@ constexpr int row_threads(int tpr) { return tpr == kWaveSize ? 256 : tpr; }
 // time. Kernels whose rows span several wavefronts and that run more than one
 // row per workgroup must keep their row loop uniform across the workgroup
 // (reductions contain a barrier).
-template <typename T, int kTPR, int kVPT, int kThreadsT = row_threads(kTPR)>
+template <typename T, int kTPR, int kVPT, int kThreadsT = row_threads(kTPR), bool kRagged = false>
 struct RowTile {
   using A = typename IO<T>::Acc;
   static constexpr int kVec = IO<T>::kVec;
@@ -45,9 +51,17 @@ struct RowTile {
   static __device__ __forceinline__ int sub_row() {
     return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kTPR));
   }
-  static __device__ __forceinline__ bool active(int slot, int npackets) {
-    return slot * kTPR + lane() < npackets;
+  // Whether slot `slot` of this thread holds any element of the row.
+  static __device__ __forceinline__ bool active(int slot, int extent) {
+    return kRagged ? (slot * kTPR + lane()) * kVec < extent : slot * kTPR + lane() < extent;
   }
+  // Whether element `e` of slot `slot` lies inside the row (always true for a
+  // regular tile's active slot).
+  static __device__ __forceinline__ bool elem_active(int slot, int e, int extent) {
+    return kRagged ? (slot * kTPR + lane()) * kVec + e < extent : true;
+  }
+  // The extent argument of this tile flavour for a row of C elements.
+  static __host__ __device__ __forceinline__ int extent_of(int C) { return kRagged ? C : C / kVec; }
 
   // Loads are unconditional (a masked slot reads packet 0 of the row and is
   // then overwritten with `fill`): with no branch around a load the number of
@@ -55,6 +69,10 @@ struct RowTile {
   // computation needs instead of draining the queue. `row` must point to
   // readable memory even when `valid` is false.
   __device__ __forceinline__ void load(const T* row, int npackets, A fill, bool valid = true) {
+    if constexpr (kRagged) {
+      load_ragged(row, npackets, fill, valid);
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       const bool on = valid && active(s, npackets);
@@ -66,10 +84,45 @@ struct RowTile {
   }
 
   __device__ __forceinline__ void store(T* row, int npackets, bool valid = true) const {
+    if constexpr (kRagged) {
+      store_ragged(row, npackets, valid);
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       if (valid && active(s, npackets)) {
         pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void load_ragged(const T* row, int ncols, A fill, bool valid) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int col = (s * kTPR + lane()) * kVec;
+      if (valid && col + kVec <= ncols) {
+        IO<T>::unpack(load_packet_unaligned(row + col), v[s]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          v[s][e] = (valid && col + e < ncols) ? IO<T>::load1(row + col + e) : fill;
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store_ragged(T* row, int ncols, bool valid) const {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int col = (s * kTPR + lane()) * kVec;
+      if (!valid) continue;
+      if (col + kVec <= ncols) {
+        store_packet_unaligned(row + col, IO<T>::pack(v[s]));
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (col + e < ncols) IO<T>::store1(row + col + e, v[s][e]);
+        }
       }
     }
   }

@@ -10,7 +10,8 @@
 //   log_softmax_grad  dx = dy - exp(y) * sum(dy)
 //
 // S == 1 (reduction along the contiguous axis) keeps each row in registers:
-// every tensor is read once and written once. 16-bit I/O accumulates in fp32
+// every tensor is read once and written once, whatever the row width and
+// alignment (ragged tiles take widths that are not whole 16-byte packets). 16-bit I/O accumulates in fp32
 // and uses the hardware exp2 (relative error ~1e-7 near the row maximum,
 // below 3e-6 in the far tail, both far under one 16-bit ulp); fp32 / fp64 I/O
 // use the correctly-scaled library exp and a true division, which is what the
@@ -19,6 +20,7 @@
 // S > 1 assigns one thread to each (n, s) column so that neighbouring threads
 // read neighbouring addresses; the column is walked three times (max, sum,
 // write), the re-reads coming from L2.
+#include "row_loop.h"
 #include "row_tile.h"
 
 namespace dragon_hip {
@@ -46,15 +48,15 @@ struct SoftmaxMath {
 
 enum SoftmaxKind { kSoftmax = 0, kLogSoftmax = 1 };
 
-template <typename T, int kKind, int kTPR, int kVPT>
+template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
     const int64_t N, const int C, const T* x, T* y) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
 
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
@@ -106,15 +108,15 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
   }
 }
 
-template <typename T, int kKind, int kTPR, int kVPT>
+template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
     const int64_t N, const int C, const T* dy, const T* y, T* dx) {
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);
 
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
@@ -150,9 +152,7 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
   }
 }
 
-// One thread per (n, s) column, elements S apart. Also the fallback for S == 1
-// rows that are unaligned, not a whole number of packets, or too long for
-// registers (there a thread walks a contiguous row: correct, not fast).
+// One thread per (n, s) column, elements S apart.
 template <typename T, int kKind>
 __global__ __launch_bounds__(256) void softmax_columns(
     const int64_t N, const int64_t S, const int64_t C, const T* x, T* y) {
@@ -200,51 +200,79 @@ __global__ __launch_bounds__(256) void softmax_grad_columns(
   }
 }
 
-// One workgroup per contiguous row of any length or alignment (S == 1 rows the
-// register tiles cannot take): strided element-wise passes over the row.
+// S == 1 rows too long for the register tiles. Pass one keeps a running
+// maximum and a sum rescaled to it per thread (one extra exponential per
+// packet), so the row is walked twice, not three times.
 template <typename T, int kKind>
-__global__ __launch_bounds__(256) void softmax_rows_looped(const int64_t N, const int64_t C,
-                                                           const T* x, T* y) {
+__global__ __launch_bounds__(kLoopThreads) void softmax_rows_looped(const int64_t N,
+                                                                    const int64_t C, const T* x,
+                                                                    T* y) {
   using A = typename IO<T>::Acc;
-  __shared__ A slots[2][4];
+  using M = SoftmaxMath<T>;
+  using Loop = RowLoop<T>;
+  constexpr int kVec = Loop::kVec;
+  __shared__ A slots[2][kLoopWaves];
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const T* xr = x + row * C;
     T* yr = y + row * C;
-    A m = acc_neg_inf<A>();
-    for (int64_t j = threadIdx.x; j < C; j += 256) m = MaxOp()(m, IO<T>::load1(xr + j));
-    m = block_allreduce<4>(m, MaxOp(), slots[0]);
-    A s = A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) s += acc_exp(IO<T>::load1(xr + j) - m);
-    s = block_allreduce<4>(s, SumOp(), slots[1]);
+    A m = acc_neg_inf<A>(), s = A(0);
+    Loop::visit(xr, C, acc_neg_inf<A>(), [&](int64_t, const A(&v)[kVec], int) {
+      A pm = v[0];
+#pragma unroll
+      for (int e = 1; e < kVec; ++e) pm = MaxOp()(pm, v[e]);
+      if (pm > m) {
+        s *= M::exp_of(m - pm);  // m == -inf on the first finite packet: s is 0 and stays 0
+        m = pm;
+      }
+      if (m > acc_neg_inf<A>()) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) s += M::exp_of(v[e] - m);
+      }
+    });
+    const A row_max = block_allreduce<kLoopWaves>(m, MaxOp(), slots[0]);
+    s = m > acc_neg_inf<A>() ? s * M::exp_of(m - row_max) : A(0);
+    s = block_allreduce<kLoopWaves>(s, SumOp(), slots[1]);
+    const A inv = A(1) / s;
     const A l = acc_log(s);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A d = IO<T>::load1(xr + j) - m;
-      IO<T>::store1(yr + j, kKind == kSoftmax ? acc_exp(d) / s : d - l);
-    }
-    __syncthreads();
+    Loop::visit(xr, C, acc_neg_inf<A>(), [&](int64_t col, const A(&v)[kVec], int n) {
+      A o[kVec];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A d = v[e] - row_max;
+        o[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), s, inv) : d - l;
+      }
+      Loop::store(yr, col, o, n);
+    });
+    __syncthreads();  // slots are reused by the next row
   }
 }
 
 template <typename T, int kKind>
-__global__ __launch_bounds__(256) void softmax_grad_rows_looped(const int64_t N, const int64_t C,
-                                                                const T* dy, const T* y, T* dx) {
+__global__ __launch_bounds__(kLoopThreads) void softmax_grad_rows_looped(
+    const int64_t N, const int64_t C, const T* dy, const T* y, T* dx) {
   using A = typename IO<T>::Acc;
-  __shared__ A slots[4];
+  using M = SoftmaxMath<T>;
+  using Loop = RowLoop<T>;
+  constexpr int kVec = Loop::kVec;
+  __shared__ A slots[kLoopWaves];
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const T* gr = dy + row * C;
     const T* yr = y + row * C;
     T* dr = dx + row * C;
     A s = A(0);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A g = IO<T>::load1(gr + j);
-      s += kKind == kSoftmax ? g * IO<T>::load1(yr + j) : g;
-    }
-    s = block_allreduce<4>(s, SumOp(), slots);
-    for (int64_t j = threadIdx.x; j < C; j += 256) {
-      const A g = IO<T>::load1(gr + j);
-      const A o = IO<T>::load1(yr + j);
-      IO<T>::store1(dr + j, kKind == kSoftmax ? (g - s) * o : g - acc_exp(o) * s);
-    }
+    Loop::visit2(gr, yr, C, A(0), [&](int64_t, const A(&g)[kVec], const A(&o)[kVec], int) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += kKind == kSoftmax ? g[e] * o[e] : g[e];
+    });
+    s = block_allreduce<kLoopWaves>(s, SumOp(), slots);
+    Loop::visit2(gr, yr, C, A(0), [&](int64_t col, const A(&g)[kVec], const A(&o)[kVec], int n) {
+      A r[kVec];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        r[e] = kKind == kSoftmax ? (g[e] - s) * o[e] : g[e] - M::exp_of(o[e]) * s;
+      }
+      Loop::store(dr, col, r, n);
+    });
     __syncthreads();
   }
 }
@@ -261,20 +289,27 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   RowConfig cfg;
-  if (S == 1 && C % kVec == 0 && aligned16(x) && aligned16(y) &&
-      pick_row_config(C / kVec, 8, &cfg)) {
+  if (S == 1 && pick_row_config(ceil_div(C, kVec), 8, &cfg)) {
+    // rows that are whole, aligned packets take the regular tiles, any other
+    // width or base address the ragged ones
+    const bool regular = C % kVec == 0 && aligned16(x) && aligned16(y);
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
-    hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT>),                                   \
-                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
-                       N, static_cast<int>(C), xp, yp);                                      \
+    const dim3 grid(row_grid(N, Tile::kRowsPerBlock)), block(Tile::kThreads);                \
+    if (regular) {                                                                           \
+      hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT, false>), grid, block, 0, stream, N, \
+                         static_cast<int>(C), xp, yp);                                       \
+    } else {                                                                                 \
+      hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT, true>), grid, block, 0, stream, N, \
+                         static_cast<int>(C), xp, yp);                                       \
+    }                                                                                        \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
-  } else if (S == 1 && C >= 256) {
-    hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(row_grid(N, 1)), dim3(256), 0, stream,
-                       N, C, xp, yp);
+  } else if (S == 1) {
+    hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
+                       stream, N, C, xp, yp);
   } else {
     hipLaunchKernelGGL((softmax_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0, stream, N,
                        S, C, xp, yp);
@@ -291,20 +326,25 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   T* dp = static_cast<T*>(dx);
   RowConfig cfg;
   // Two tiles live at once: halve the packets a thread may hold.
-  if (S == 1 && C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx) &&
-      pick_row_config(C / kVec, 4, &cfg)) {
+  if (S == 1 && pick_row_config(ceil_div(C, kVec), 4, &cfg)) {
+    const bool regular = C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx);
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
-    hipLaunchKernelGGL((softmax_grad_rows<T, kKind, TPR, VPT>),                              \
-                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
-                       N, static_cast<int>(C), gp, yp, dp);                                  \
+    const dim3 grid(row_grid(N, Tile::kRowsPerBlock)), block(Tile::kThreads);                \
+    if (regular) {                                                                           \
+      hipLaunchKernelGGL((softmax_grad_rows<T, kKind, TPR, VPT, false>), grid, block, 0,     \
+                         stream, N, static_cast<int>(C), gp, yp, dp);                        \
+    } else {                                                                                 \
+      hipLaunchKernelGGL((softmax_grad_rows<T, kKind, TPR, VPT, true>), grid, block, 0,      \
+                         stream, N, static_cast<int>(C), gp, yp, dp);                        \
+    }                                                                                        \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
-  } else if (S == 1 && C >= 256) {
-    hipLaunchKernelGGL((softmax_grad_rows_looped<T, kKind>), dim3(row_grid(N, 1)), dim3(256), 0,
-                       stream, N, C, gp, yp, dp);
+  } else if (S == 1) {
+    hipLaunchKernelGGL((softmax_grad_rows_looped<T, kKind>), dim3(loop_grid(N)),
+                       dim3(kLoopThreads), 0, stream, N, C, gp, yp, dp);
   } else {
     hipLaunchKernelGGL((softmax_grad_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0,
                        stream, N, S, C, gp, yp, dp);

@@ -705,3 +705,69 @@ def test_fused_softmax_cross_entropy_loss_out_of_range_target_is_ignored(K):
     got = U.to_host(loss)
     assert got[1] == 0 and got[2] == 0
     assert np.allclose(got[[0, 3]], np.log(8.0), rtol=1e-6)
+
+
+# ---------------------------------------------------------------- unaligned bases, ragged widths
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
+@pytest.mark.parametrize("shape", [(7, 197), (5, 1001), (3, 4099), (2, 66001)])
+def test_rows_at_element_aligned_addresses(K, dtype, shape):
+    """Tensors that start one element past a 16-byte boundary, with widths that
+    are not whole packets: the ragged tiles and the looped kernels."""
+    import torch
+    N, C = shape
+    rng = U.rng_for(1500 + C)
+    x = R.to_bits(rng.standard_normal(shape).astype(np.float32) * 2, dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    x64 = np.asarray(xo, np.float64)
+
+    def shifted(bits):
+        buf = empty((N * C + 1,), dtype)
+        view = buf[1:].view(N, C)
+        view.copy_(U.to_device(bits, dtype))
+        assert view.data_ptr() % 16 != 0
+        return view
+
+    def out():
+        return empty((N * C + 1,), dtype)[1:].view(N, C)
+
+    xd, dyd = shifted(x), shifted(dy)
+    tol = U.TIGHT[dtype]
+    # softmax forward / backward
+    y = out()
+    K.softmax(N, 1, C, xd, y)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    y64 = e / e.sum(1, keepdims=True)
+    yw = U.widen(U.to_host(y.contiguous()), dtype).reshape(shape)
+    assert U.rowwise_normwise(yw, y64) <= tol
+    dx = out()
+    K.softmax_grad(N, 1, C, dyd, y, dx)
+    yo, _ = oracle_dtype_inputs(U.to_host(y.contiguous()).reshape(shape), dtype)
+    dx_ref = R.op_softmax_grad(od, yo, dyo)
+    assert U.normwise(U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape), dx_ref) <= tol
+    # log-softmax forward
+    K.log_softmax(N, 1, C, xd, y)
+    ly64 = (x64 - x64.max(1, keepdims=True)) - np.log(e.sum(1, keepdims=True))
+    lyw = U.widen(U.to_host(y.contiguous()), dtype).reshape(shape)
+    assert np.max(np.abs(lyw - ly64) / np.maximum(np.abs(ly64), 1.0)) <= tol
+    # layer norm forward (gamma / beta element-aligned too)
+    an = acc_name(dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    gbuf, bbuf = empty((C + 1,), an), empty((C + 1,), an)
+    gbuf[1:].copy_(U.to_device(g, an))
+    bbuf[1:].copy_(U.to_device(b, an))
+    mu, rsig = empty((N,), an), empty((N,), an)
+    K.layer_norm(N, C, 1e-5, xd, gbuf[1:], bbuf[1:], mu, rsig, y)
+    mean64 = x64.mean(1, keepdims=True)
+    ln64 = (x64 - mean64) / np.sqrt(x64.var(1, keepdims=True) + 1e-5) * g + b
+    assert U.normwise(U.widen(U.to_host(y.contiguous()), dtype).reshape(shape), ln64) <= tol
+    assert U.normwise(U.to_host(mu), mean64.ravel()) <= (1e-12 if dtype == "float64" else 1e-5)
+    # l2 normalisation forward / backward
+    K.l2_norm(N, 1, C, 1.0, 1e-12, xd, y)
+    y64n, dx64n, term = _lp_fp64(xo, dyo, 1, 2, 1.0, 1e-12)
+    assert U.normwise(U.widen(U.to_host(y.contiguous()), dtype).reshape(shape), y64n) <= tol
+    K.l2_norm_grad(N, 1, C, 1.0, 1e-12, dyd, xd, dx)
+    dxw = U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape)
+    assert np.max(np.abs(dxw - dx64n)) / term <= tol
