@@ -192,6 +192,27 @@ __device__ __forceinline__ void load_params(const double* p, double (&v)[kVec]) 
   v[0] = t.x, v[1] = t.y;
 }
 
+// The same for parameters at an element-aligned address, of which only the
+// first n (n <= kVec) exist: whole groups as one unaligned access, the rest
+// element by element, absent ones as zero.
+template <int kVec, typename A>
+__device__ __forceinline__ void load_params_ragged(const A* p, int n, A (&v)[kVec]) {
+  constexpr int kPer = 16 / sizeof(A);
+  if (n >= kVec) {
+#pragma unroll
+    for (int i = 0; i < kVec / kPer; ++i) {
+      const u32x4 t = load_packet_unaligned(p + kPer * i);
+      A w[kPer];
+      IO<A>::unpack(t, w);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) v[kPer * i + e] = w[e];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) v[e] = e < n ? p[e] : A(0);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Reductions
 // ---------------------------------------------------------------------------

@@ -67,11 +67,8 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
         const int col = (i * kTPR + lane) * kVec;
         A g[kVec], b[kVec];
         if constexpr (kRagged) {
-#pragma unroll
-          for (int e = 0; e < kVec; ++e) {
-            g[e] = col + e < C ? gamma[col + e] : A(0);
-            b[e] = col + e < C ? beta[col + e] : A(0);
-          }
+          load_params_ragged<kVec>(gamma + col, C - col, g);
+          load_params_ragged<kVec>(beta + col, C - col, b);
         } else {
           load_params<kVec>(gamma + col, g);
           load_params<kVec>(beta + col, b);
@@ -211,13 +208,11 @@ __global__ __launch_bounds__(kLoopThreads) void layer_norm_rows_looped(
       rsig[row] = rs;
     }
     Loop::visit(xr, C, A(0), [&](int64_t col, const A(&v)[kVec], int n) {
-      A o[kVec];
+      A o[kVec], g[kVec], b[kVec];
+      load_params_ragged<kVec>(gamma + col, n, g);
+      load_params_ragged<kVec>(beta + col, n, b);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A g = e < n ? gamma[col + e] : A(0);
-        const A b = e < n ? beta[col + e] : A(0);
-        o[e] = (v[e] - mean) * rs * g + b;
-      }
+      for (int e = 0; e < kVec; ++e) o[e] = (v[e] - mean) * rs * g[e] + b[e];
       Loop::store(yr, col, o, n);
     });
     __syncthreads();  // slots are reused by the next row

@@ -12,14 +12,16 @@
 //               with g(x) = sign(x) for p = 1 and g(x) = x for p = 2
 //
 // S == 1 keeps each row in registers (one read, one write per tensor), with
-// the same tiles as the softmax kernels. S > 1 gives each thread a strip of
-// adjacent (n, s) columns one 16-byte packet wide, so that every access is a
-// full-width coalesced packet; the strip is walked twice (reduce, write), the
-// second walk re-reading what the first left in L2.
+// the same tiles as the softmax kernels. S > 1 keeps a [C, columns] tile in
+// the registers of a workgroup (col_tile.h) when C <= 1024; beyond that each
+// thread owns a strip of adjacent (n, s) columns one 16-byte packet wide and
+// walks it twice (reduce, write), the second walk re-reading what the first
+// left in L2.
 //
 // 16-bit I/O accumulates in fp32 as the reference's CUDA kernels do; fp32 and
 // fp64 I/O divide by the norm exactly as the reference's CPU expression does,
 // 16-bit I/O multiplies by its reciprocal (error far below one 16-bit ulp).
+#include "col_tile.h"
 #include "row_loop.h"
 #include "row_tile.h"
 
@@ -190,6 +192,71 @@ __global__ __launch_bounds__(kLoopThreads) void lp_norm_rows_looped(
   }
 }
 
+// S > 1 with the whole reduced axis in one register tile (col_tile.h): one
+// read of every tensor.
+template <typename T, int kP, bool kGrad, int kTW, int kR>
+__global__ __launch_bounds__(kColThreads) void lp_norm_col_tiles(
+    const ColGrid g, const typename IO<T>::Acc normalizer, const typename IO<T>::Acc eps,
+    const T* dy, const T* x, T* out) {
+  using Tile = ColTile<T, kTW, kR>;
+  using A = typename Tile::A;
+  using M = LpMath<T, kP>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A lds[Tile::kLdsWords];
+  const int nr = Tile::rows_used(g.C);  // uniform: later packets are padding
+  for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
+    const int64_t n = tile / g.strips;
+    const int64_t s0 = (tile - n * g.strips) * Tile::kCols + Tile::tw() * kVec;
+    const int64_t left = g.S - s0;
+    const int nvalid = left >= kVec ? kVec : (left > 0 ? static_cast<int>(left) : 0);
+    const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
+    Tile tx, tg;
+    tx.load(x + base, g.S, g.C, nvalid, A(0));
+    if (kGrad) tg.load(dy + base, g.S, g.C, nvalid, A(0));
+    A acc[kVec], dot[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) acc[e] = dot[e] = A(0);
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A v[kVec], gv[kVec];
+        tx.unpack(r, v);
+        if (kGrad) tg.unpack(r, gv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          acc[e] += M::term(v[e]);
+          if (kGrad) dot[e] += gv[e] * v[e];
+        }
+      }
+    }
+    Tile::reduce_rows(acc, SumOp(), lds);
+    if (kGrad) Tile::reduce_rows(dot, SumOp(), lds);
+    tx.refresh();
+    if (kGrad) tg.refresh();
+    A norm[kVec], inv[kVec], coef[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      norm[e] = M::norm_of(acc[e], normalizer, eps);
+      inv[e] = A(1) / norm[e];
+      coef[e] = kGrad ? M::coef_of(dot[e], normalizer, norm[e]) : A(0);
+    }
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A v[kVec], gv[kVec];
+        tx.unpack(r, v);
+        if (kGrad) tg.unpack(r, gv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          v[e] = kGrad ? M::backward(gv[e], v[e], norm[e], inv[e], coef[e])
+                       : M::forward(v[e], norm[e], inv[e]);
+        }
+        Tile::store(out + base, g.S, g.C, nvalid, r, v);
+      }
+    }
+  }
+}
+
 // Reduction along a strided axis: a thread owns kW adjacent columns of one n
 // (kW = 1, or one 16-byte packet when S is a multiple of it and the tensors are
 // aligned) and walks its C elements S apart.
@@ -296,6 +363,23 @@ int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsi
   } else if (S == 1) {
     hipLaunchKernelGGL((lp_norm_rows_looped<T, kP, kGrad>), dim3(loop_grid(N)), dim3(kLoopThreads),
                        0, stream, N, C, nrm, eps, gp, xp, op);
+  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+    // the gradient holds two tiles: 8 packets per thread each where that holds C rows
+    const bool small = kGrad && C <= static_cast<int64_t>(kColThreads / tw) * 8;
+#define LAUNCH(TW)                                                                            \
+  {                                                                                           \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                      \
+    const dim3 grid(col_launch_grid(g.tiles)), block(kColThreads);                            \
+    if (small) {                                                                              \
+      hipLaunchKernelGGL((lp_norm_col_tiles<T, kP, kGrad, TW, 8>), grid, block, 0, stream, g, \
+                         nrm, eps, gp, xp, op);                                               \
+    } else {                                                                                  \
+      hipLaunchKernelGGL((lp_norm_col_tiles<T, kP, kGrad, TW, 16>), grid, block, 0, stream, g, \
+                         nrm, eps, gp, xp, op);                                               \
+    }                                                                                         \
+  }
+    if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
   } else if (kVec > 1 && S % kVec == 0 && packets_ok) {
     hipLaunchKernelGGL((lp_norm_columns<T, kP, kGrad, kVec>), dim3(flat_grid(N * (S / kVec))),
                        dim3(256), 0, stream, N, S, C, nrm, eps, gp, xp, op);

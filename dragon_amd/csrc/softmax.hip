@@ -17,9 +17,11 @@
 // use the correctly-scaled library exp and a true division, which is what the
 // reference's CPU expression does.
 //
-// S > 1 assigns one thread to each (n, s) column so that neighbouring threads
-// read neighbouring addresses; the column is walked three times (max, sum,
-// write), the re-reads coming from L2.
+// S > 1 keeps a [C, columns] tile in the registers of a workgroup (col_tile.h)
+// when C <= 1024: one read, one write. Longer strided
+// axes assign one thread to each (n, s) column and walk it three times (max,
+// sum, write), the re-reads coming from L2.
+#include "col_tile.h"
 #include "row_loop.h"
 #include "row_tile.h"
 
@@ -149,6 +151,121 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
       }
     g.store(dx + row * C, npackets);
     if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// S > 1 with the whole reduced axis in one register tile (col_tile.h): every
+// tensor is read once. 16-bit types evaluate the exponential twice (statistics
+// and output) instead of keeping fp32 copies of the tile.
+template <typename T, int kKind, int kTW, int kR>
+__global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g, const T* x,
+                                                                 T* y) {
+  using Tile = ColTile<T, kTW, kR>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A lds[Tile::kLdsWords];
+  const int nr = Tile::rows_used(g.C);  // uniform: later packets are padding
+  for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
+    const int64_t n = tile / g.strips;
+    const int64_t s0 = (tile - n * g.strips) * Tile::kCols + Tile::tw() * kVec;
+    const int64_t left = g.S - s0;
+    const int nvalid = left >= kVec ? kVec : (left > 0 ? static_cast<int>(left) : 0);
+    const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
+    Tile t;
+    t.load(x + base, g.S, g.C, nvalid, acc_neg_inf<A>());
+    A m[kVec], sum[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) m[e] = acc_neg_inf<A>(), sum[e] = A(0);
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) m[e] = MaxOp()(m[e], v[e]);
+      }
+    }
+    Tile::reduce_rows(m, MaxOp(), lds);
+    t.refresh();
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) sum[e] += M::exp_of(v[e] - m[e]);  // padding: exp(-inf) = 0
+      }
+    }
+    Tile::reduce_rows(sum, SumOp(), lds);
+    t.refresh();
+    A inv[kVec], l[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) inv[e] = A(1) / sum[e], l[e] = acc_log(sum[e]);
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A d = v[e] - m[e];
+          v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), sum[e], inv[e]) : d - l[e];
+        }
+        Tile::store(y + base, g.S, g.C, nvalid, r, v);
+      }
+    }
+  }
+}
+
+template <typename T, int kKind, int kTW, int kR>
+__global__ __launch_bounds__(kColThreads) void softmax_grad_col_tiles(const ColGrid g,
+                                                                      const T* dy, const T* y,
+                                                                      T* dx) {
+  using Tile = ColTile<T, kTW, kR>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A lds[Tile::kLdsWords];
+  const int nr = Tile::rows_used(g.C);  // uniform: later packets are padding
+  for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
+    const int64_t n = tile / g.strips;
+    const int64_t s0 = (tile - n * g.strips) * Tile::kCols + Tile::tw() * kVec;
+    const int64_t left = g.S - s0;
+    const int nvalid = left >= kVec ? kVec : (left > 0 ? static_cast<int>(left) : 0);
+    const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
+    Tile tg, to;
+    tg.load(dy + base, g.S, g.C, nvalid, A(0));
+    to.load(y + base, g.S, g.C, nvalid, kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
+    A sum[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) sum[e] = A(0);
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A gv[kVec], ov[kVec];
+        tg.unpack(r, gv);
+        to.unpack(r, ov);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) sum[e] += kKind == kSoftmax ? gv[e] * ov[e] : gv[e];
+      }
+    }
+    Tile::reduce_rows(sum, SumOp(), lds);
+    tg.refresh();
+    to.refresh();
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      if (r < nr) {
+        A gv[kVec], ov[kVec];
+        tg.unpack(r, gv);
+        to.unpack(r, ov);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          gv[e] = kKind == kSoftmax ? (gv[e] - sum[e]) * ov[e] : gv[e] - M::exp_of(ov[e]) * sum[e];
+        }
+        Tile::store(dx + base, g.S, g.C, nvalid, r, gv);
+      }
+    }
   }
 }
 
@@ -310,6 +427,15 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
   } else if (S == 1) {
     hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
                        stream, N, C, xp, yp);
+  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+#define LAUNCH(TW)                                                                        \
+  {                                                                                       \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                  \
+    hipLaunchKernelGGL((softmax_col_tiles<T, kKind, TW, 16>), dim3(col_launch_grid(g.tiles)), \
+                       dim3(kColThreads), 0, stream, g, xp, yp);                          \
+  }
+    if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
   } else {
     hipLaunchKernelGGL((softmax_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0, stream, N,
                        S, C, xp, yp);
@@ -345,6 +471,23 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   } else if (S == 1) {
     hipLaunchKernelGGL((softmax_grad_rows_looped<T, kKind>), dim3(loop_grid(N)),
                        dim3(kLoopThreads), 0, stream, N, C, gp, yp, dp);
+  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+    // two tiles live at once: 8 packets per thread each where that holds C rows
+    const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
+#define LAUNCH(TW)                                                                        \
+  {                                                                                       \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                  \
+    const dim3 grid(col_launch_grid(g.tiles)), block(kColThreads);                        \
+    if (small) {                                                                          \
+      hipLaunchKernelGGL((softmax_grad_col_tiles<T, kKind, TW, 8>), grid, block, 0, stream, g, \
+                         gp, yp, dp);                                                     \
+    } else {                                                                              \
+      hipLaunchKernelGGL((softmax_grad_col_tiles<T, kKind, TW, 16>), grid, block, 0, stream, g, \
+                         gp, yp, dp);                                                     \
+    }                                                                                     \
+  }
+    if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
   } else {
     hipLaunchKernelGGL((softmax_grad_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0,
                        stream, N, S, C, gp, yp, dp);
