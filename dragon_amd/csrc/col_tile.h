@@ -63,6 +63,7 @@ struct ColTile {
   }
 
   __device__ __forceinline__ void unpack(int r, A (&v)[kVec]) const { IO<T>::unpack(p[r], v); }
+  __device__ __forceinline__ void set(int r, const A (&v)[kVec]) { p[r] = IO<T>::pack(v); }
   // Between two passes over the tile: makes the compiler convert the packets
   // again in the next pass instead of keeping every converted element live.
   __device__ __forceinline__ void refresh() {

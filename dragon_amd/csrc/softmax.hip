@@ -164,6 +164,13 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
   constexpr int kVec = Tile::kVec;
+  // Up to 8 packets per thread are converted once and held as accumulator
+  // values; longer tiles stay raw packets and are converted in every pass.
+  constexpr bool kHold = kR <= 8;
+  // The exponentials of the statistics pass are kept where the tile holds
+  // accumulator-typed values (held tiles; raw fp32 / fp64 packets); raw 16-bit
+  // packets evaluate them again for the output.
+  constexpr bool kKeepExp = kKind == kSoftmax && (kHold || sizeof(T) == sizeof(A));
   __shared__ A lds[Tile::kLdsWords];
   const int nr = Tile::rows_used(g.C);  // uniform: later packets are padding
   for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
@@ -174,6 +181,27 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
     const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
     Tile t;
     t.load(x + base, g.S, g.C, nvalid, acc_neg_inf<A>());
+    A held[kHold ? kR : 1][kVec];
+    if constexpr (kHold) {
+#pragma unroll
+      for (int r = 0; r < kR; ++r) t.unpack(r, held[r]);
+    }
+    auto get = [&](int r, A(&v)[kVec]) {
+      if constexpr (kHold) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = held[r][e];
+      } else {
+        t.unpack(r, v);
+      }
+    };
+    auto put = [&](int r, const A(&v)[kVec]) {
+      if constexpr (kHold) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) held[r][e] = v[e];
+      } else {
+        t.set(r, v);
+      }
+    };
     A m[kVec], sum[kVec];
 #pragma unroll
     for (int e = 0; e < kVec; ++e) m[e] = acc_neg_inf<A>(), sum[e] = A(0);
@@ -181,24 +209,28 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
     for (int r = 0; r < kR; ++r) {
       if (r < nr) {
         A v[kVec];
-        t.unpack(r, v);
+        get(r, v);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) m[e] = MaxOp()(m[e], v[e]);
       }
     }
     Tile::reduce_rows(m, MaxOp(), lds);
-    t.refresh();
+    if (!kHold) t.refresh();
 #pragma unroll
     for (int r = 0; r < kR; ++r) {
       if (r < nr) {
         A v[kVec];
-        t.unpack(r, v);
+        get(r, v);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) sum[e] += M::exp_of(v[e] - m[e]);  // padding: exp(-inf) = 0
+        for (int e = 0; e < kVec; ++e) {
+          v[e] = kKind == kSoftmax ? M::exp_of(v[e] - m[e]) : v[e] - m[e];  // padding: exp(-inf) = 0
+          sum[e] += kKind == kSoftmax ? v[e] : M::exp_of(v[e]);
+        }
+        if (kKeepExp || (kHold && kKind == kLogSoftmax)) put(r, v);
       }
     }
     Tile::reduce_rows(sum, SumOp(), lds);
-    t.refresh();
+    if (!kHold) t.refresh();
     A inv[kVec], l[kVec];
 #pragma unroll
     for (int e = 0; e < kVec; ++e) inv[e] = A(1) / sum[e], l[e] = acc_log(sum[e]);
@@ -206,11 +238,17 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
     for (int r = 0; r < kR; ++r) {
       if (r < nr) {
         A v[kVec];
-        t.unpack(r, v);
+        get(r, v);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const A d = v[e] - m[e];
-          v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), sum[e], inv[e]) : d - l[e];
+          if (kKeepExp) {
+            v[e] = M::normalise(v[e], sum[e], inv[e]);
+          } else if (kHold) {  // log-softmax: the held value is x - max
+            v[e] = v[e] - l[e];
+          } else {
+            const A d = v[e] - m[e];
+            v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), sum[e], inv[e]) : d - l[e];
+          }
         }
         Tile::store(y + base, g.S, g.C, nvalid, r, v);
       }
@@ -428,11 +466,20 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
     hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
                        stream, N, C, xp, yp);
   } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+    // the widest tile wins (narrow row segments cost more than a second
+    // exponential); within it, up to 8 packets per thread are held converted
+    const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
 #define LAUNCH(TW)                                                                        \
   {                                                                                       \
     const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                  \
-    hipLaunchKernelGGL((softmax_col_tiles<T, kKind, TW, 16>), dim3(col_launch_grid(g.tiles)), \
-                       dim3(kColThreads), 0, stream, g, xp, yp);                          \
+    const dim3 grid(col_launch_grid(g.tiles)), block(kColThreads);                        \
+    if (small) {                                                                          \
+      hipLaunchKernelGGL((softmax_col_tiles<T, kKind, TW, 8>), grid, block, 0, stream, g, xp, \
+                         yp);                                                             \
+    } else {                                                                              \
+      hipLaunchKernelGGL((softmax_col_tiles<T, kKind, TW, 16>), grid, block, 0, stream, g, xp, \
+                         yp);                                                             \
+    }                                                                                     \
   }
     if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
 #undef LAUNCH
