@@ -69,8 +69,7 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
     const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
     hipLaunchKernelGGL((reduce2_columns<T, kIn, F>), grid, dim3(kReduceThreads), 0, stream, c, in0,
                        in1, f, part);
-    hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3(fin_grid), dim3(kReduceThreads), 0, stream,
-                       sh.C, c.split, false, part, e);
+    launch_reduce2_finalize<A, E>(sh.C, c.split, false, part, e, stream);
   }
 }
 

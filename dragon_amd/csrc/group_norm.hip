@@ -61,6 +61,17 @@ struct GroupNormApply {
     } else {
       const uint32_t c = i % sh.C;  // kVec divides C or is 1
       const uint32_t n = i / (sh.S * sh.C);
+      if (kVec > 1 && sh.D % kVec == 0) {
+        // the packet lies within one group: one pair of statistics, parameters as packets
+        const uint32_t ng = n * sh.G + c / sh.D;
+        const A m = mu[ng], r = rsig[ng];
+        A g[kVec], b[kVec];
+        load_params_ragged<kVec>(gamma + c, kVec, g);
+        load_params_ragged<kVec>(beta + c, kVec, b);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - m) * r * g[e] + b[e];
+        return;
+      }
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
         const uint32_t ce = c + e;
@@ -175,6 +186,18 @@ struct GroupNormGradApply {
     } else {
       const uint32_t c = i % sh.C;
       const uint32_t n = i / (sh.S * sh.C);
+      if (kVec > 1 && sh.D % kVec == 0) {
+        // the packet lies within one group: the group's scalars once, gamma as a packet
+        const uint32_t ng = n * sh.G + c / sh.D;
+        const A m = mu[ng], r = rsig[ng], s = ds[ng], b = db[ng];
+        const A ku = (b * m - s) * (r * r * r) * denom;
+        const A kv = b * r * denom;
+        A g[kVec];
+        load_params_ragged<kVec>(gamma + c, kVec, g);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) x[e] = g[e] * dy[e] * r + (ku * (x[e] - m) - kv);
+        return;
+      }
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
         const uint32_t ce = c + e;
@@ -852,9 +875,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
       hipLaunchKernelGGL((reduce2_columns<T, 2, WGradAccumNHWC<T>>), grid, dim3(kReduceThreads), 0,
                          stream, c, xp, dyp, f, part);
-      hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
-                         dim3(static_cast<unsigned>(ceil_div(sh.C, kReduceThreads))),
-                         dim3(kReduceThreads), 0, stream, sh.C, c.split, false, part, e);
+      launch_reduce2_finalize<A, StorePairEpilogue<A>>(sh.C, c.split, false, part, e, stream);
     }
   }
   // 3. dx

@@ -274,8 +274,7 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
     hipLaunchKernelGGL((reduce2_columns<T, 1, Accum>), grid, dim3(kReduceThreads), 0, stream, c, xp,
                        xp, f, part);
     ReduceColEpilogue<T, P> e{xp, inv_n, out};
-    hipLaunchKernelGGL((reduce2_finalize<A, ReduceColEpilogue<T, P>>), dim3(fin_grid),
-                       dim3(kReduceThreads), 0, stream, c.cols, c.split, false, part, e);
+    launch_reduce2_finalize<A, ReduceColEpilogue<T, P>>(c.cols, c.split, false, part, e, stream);
   } else {
     const unsigned grid = static_cast<unsigned>(plan.n_out < 65536 ? plan.n_out : 65536);
     hipLaunchKernelGGL((reduce_gather<T, P>), dim3(grid), dim3(kReduceThreads), 0, stream,

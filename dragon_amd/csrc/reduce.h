@@ -180,6 +180,52 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_finalize(
   e(o, a, b);
 }
 
+// Stage two for the scratch layout of reduce2_columns when `split` is large:
+// a workgroup owns 64 adjacent outputs (one per lane, so every load is 64
+// adjacent pairs), its four wavefronts stride over k and are combined in
+// wavefront order through LDS. Fixed summation order, like reduce2_finalize.
+template <typename A, typename E>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_finalize_columns(
+    const uint32_t n_out, const uint32_t split, const A* __restrict__ partial, E e) {
+  __shared__ A lds[kReduceWaves][kWaveSize][2];
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t o = blockIdx.x * kWaveSize + lane;
+  A a = A(0), b = A(0);
+  if (o < n_out) {
+#pragma unroll 4
+    for (uint32_t k = wave; k < split; k += kReduceWaves) {
+      const size_t idx = static_cast<size_t>(k) * n_out + o;
+      a += partial[idx * 2];
+      b += partial[idx * 2 + 1];
+    }
+  }
+  lds[wave][lane][0] = a;
+  lds[wave][lane][1] = b;
+  __syncthreads();
+  if (wave == 0 && o < n_out) {
+#pragma unroll
+    for (int w = 1; w < kReduceWaves; ++w) {
+      a += lds[w][lane][0];
+      b += lds[w][lane][1];
+    }
+    e(o, a, b);
+  }
+}
+
+// Launches the stage-two kernel that suits the layout and the split.
+template <typename A, typename E>
+inline void launch_reduce2_finalize(uint32_t n_out, uint32_t split, bool segment_major,
+                                    const A* partial, E e, hipStream_t stream) {
+  if (!segment_major && split > 16) {
+    hipLaunchKernelGGL((reduce2_finalize_columns<A, E>), dim3((n_out + kWaveSize - 1) / kWaveSize),
+                       dim3(kReduceThreads), 0, stream, n_out, split, partial, e);
+  } else {
+    hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3((n_out + kReduceThreads - 1) / kReduceThreads),
+                       dim3(kReduceThreads), 0, stream, n_out, split, segment_major, partial, e);
+  }
+}
+
 // Flat element-wise map over `total` elements in packets of kVec. F provides
 //   void operator()(uint32_t i, A (&v0)[V], const A (&v1)[V])
 // which overwrites v0 (loaded from in0) with the result; v1 comes from in1
