@@ -26,6 +26,7 @@
 #include <cstdlib>
 
 #include "reduce.h"
+#include "row_loop.h"
 #include "row_tile.h"
 
 namespace dragon_hip {
@@ -479,6 +480,73 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
   }
 }
 
+// The same for any S and any alignment (S not a multiple of a packet, so
+// that a packet may straddle channels and groups start at element-aligned
+// addresses): ragged tiles, the channel of an element found from its column.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y) {
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), true>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const A inv_l = A(1) / A(L);
+  const int lane = Tile::lane();
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Tile t;
+    t.load(x + row * L, L, A(0));
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += t.v[i][e];
+    const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_l;
+    A q = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A d = t.v[i][e] - mean;
+        if (Tile::elem_active(i, e, L)) q += d * d;
+      }
+    const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_l;
+    const A rs = acc_rsqrt_exact(var + eps);
+    if (lane == 0) {
+      mu[row] = mean;
+      rsig[row] = rs;
+    }
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, L)) {
+        const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
+        const uint32_t first = col / S;
+        const uint32_t rem = col - first * S;
+        if (rem + kVec <= S) {  // the packet lies within one channel
+          const A gam = gamma[c0 + first] * rs, bet = beta[c0 + first];
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * gam + bet;
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            uint32_t k = rem + e, c = first;
+            while (k >= S) k -= S, ++c;
+            if (c >= D) c = D - 1;  // padding beyond the group: not stored
+            t.v[i][e] = (t.v[i][e] - mean) * (gamma[c0 + c] * rs) + beta[c0 + c];
+          }
+        }
+      }
+    }
+    t.store(y + row * L, L);
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
 // GroupNormGrad in one pass over x and dy: one workgroup per group keeps both
 // as raw packets. Requires S to be a multiple of 64 packets, so that every
 // (slot, wavefront) pair lies in one channel and the per-channel sums are a
@@ -577,6 +645,154 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
       o[1] = b;
     }
     __syncthreads();  // chan_part and slots are reused by the next group
+  }
+}
+
+// --------------------------------------------------------------------------
+// General NCHW backward, stage one: per (n, c) row of S contiguous elements,
+//   a = sum dy * (x - mu[n, g]),  b = sum dy      -> sums[(n*C + c)*2 + {0,1}]
+// One pass over x and dy feeds both the per-group sums (ds, db) and the
+// per-channel sums (dgamma, dbeta), which stage two forms from the N*C pairs.
+// --------------------------------------------------------------------------
+template <typename T, int kTPR, int kVPT, bool kRagged>
+__global__ __launch_bounds__(row_threads(kTPR)) void channel_pair_sums_rows(
+    const int64_t rows, const int S, const uint32_t D, const T* __restrict__ x,
+    const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ mu,
+    typename IO<T>::Acc* __restrict__ sums) {
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2 * Tile::kSlots];
+  const int extent = Tile::extent_of(S);
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    Tile tx, tg;
+    tx.load(x + row * S, extent, A(0));
+    tg.load(dy + row * S, extent, A(0));
+    const A m = mu[row / D];  // row = n*C + c, so row / D = n*G + g
+    A a = A(0), b = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        a += tg.v[i][e] * (tx.v[i][e] - m);  // padding holds dy = 0
+        b += tg.v[i][e];
+      }
+    Tile::reduce_sum_pair(a, b, slots);
+    if (Tile::lane() == 0) {
+      sums[row * 2] = a;
+      sums[row * 2 + 1] = b;
+    }
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// Rows longer than the tiles: a 1024-thread workgroup walks the row.
+template <typename T>
+__global__ __launch_bounds__(kLoopThreads) void channel_pair_sums_looped(
+    const int64_t rows, const int64_t S, const uint32_t D, const T* __restrict__ x,
+    const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ mu,
+    typename IO<T>::Acc* __restrict__ sums) {
+  using A = typename IO<T>::Acc;
+  using Loop = RowLoop<T>;
+  constexpr int kVec = Loop::kVec;
+  __shared__ A slots[2][kLoopWaves];
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const A m = mu[row / D];
+    A a = A(0), b = A(0);
+    Loop::visit2(x + row * S, dy + row * S, S, A(0),
+                 [&](int64_t, const A(&xv)[kVec], const A(&gv)[kVec], int n) {
+#pragma unroll
+                   for (int e = 0; e < kVec; ++e) {
+                     if (e < n) a += gv[e] * (xv[e] - m);
+                     b += gv[e];
+                   }
+                 });
+    a = block_allreduce<kLoopWaves>(a, SumOp(), slots[0]);
+    b = block_allreduce<kLoopWaves>(b, SumOp(), slots[1]);
+    if (threadIdx.x == 0) {
+      sums[row * 2] = a;
+      sums[row * 2 + 1] = b;
+    }
+    __syncthreads();
+  }
+}
+
+// Rows of a few elements (S < 16): one thread per row.
+template <typename T>
+__global__ __launch_bounds__(256) void channel_pair_sums_short(
+    const int64_t rows, const int S, const uint32_t D, const T* __restrict__ x,
+    const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ mu,
+    typename IO<T>::Acc* __restrict__ sums) {
+  using A = typename IO<T>::Acc;
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; row < rows;
+       row += static_cast<int64_t>(gridDim.x) * 256) {
+    const A m = mu[row / D];
+    A a = A(0), b = A(0);
+    for (int j = 0; j < S; ++j) {
+      const A g = IO<T>::load1(dy + row * S + j);
+      a += g * (IO<T>::load1(x + row * S + j) - m);
+      b += g;
+    }
+    sums[row * 2] = a;
+    sums[row * 2 + 1] = b;
+  }
+}
+
+// Stage two. Workgroups [0, group_blocks) form, one thread per (n, g),
+//   ds = sum_c gamma_c * (a_c + mu * b_c),  db = sum_c gamma_c * b_c   over the group's channels;
+// the others own 64 adjacent channels each (one per lane), their four
+// wavefronts stride over n and are combined in wavefront order:
+//   dgamma_c = sum_n a[n, c] * rsig[n, g],  dbeta_c = sum_n b[n, c].
+template <typename A>
+__global__ __launch_bounds__(256) void group_grad_from_channel_sums(
+    const uint32_t N, const uint32_t G, const uint32_t D, const uint32_t group_blocks,
+    const A* __restrict__ sums, const A* __restrict__ gamma, const A* __restrict__ mu,
+    const A* __restrict__ rsig, A* __restrict__ ds, A* __restrict__ db, A* __restrict__ dgamma,
+    A* __restrict__ dbeta) {
+  __shared__ A lds[4][kWaveSize][2];
+  const uint32_t C = G * D;
+  if (blockIdx.x < group_blocks) {
+    const uint32_t ng = blockIdx.x * 256 + threadIdx.x;
+    if (ng >= N * G) return;
+    const uint32_t g = ng % G;
+    const A m = mu[ng];
+    const A* row = sums + (static_cast<size_t>(ng / G) * C + g * D) * 2;
+    A s = A(0), b = A(0);
+    for (uint32_t d = 0; d < D; ++d) {
+      const A w = gamma[g * D + d];
+      s += w * (row[2 * d] + m * row[2 * d + 1]);
+      b += w * row[2 * d + 1];
+    }
+    ds[ng] = s;
+    db[ng] = b;
+    return;
+  }
+  if (dgamma == nullptr) return;
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t c = (blockIdx.x - group_blocks) * kWaveSize + lane;
+  A a = A(0), b = A(0);
+  if (c < C) {
+    const uint32_t g = c / D;
+#pragma unroll 4
+    for (uint32_t n = wave; n < N; n += 4) {
+      const size_t idx = (static_cast<size_t>(n) * C + c) * 2;
+      a += sums[idx] * rsig[n * G + g];
+      b += sums[idx + 1];
+    }
+  }
+  lds[wave][lane][0] = a;
+  lds[wave][lane][1] = b;
+  __syncthreads();
+  if (wave == 0 && c < C) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      a += lds[w][lane][0];
+      b += lds[w][lane][1];
+    }
+    dgamma[c] = a;
+    dbeta[c] = b;
   }
 }
 
@@ -680,8 +896,7 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
       : pick_split(ceil_div(C, kWaveSize), N * S * kWaveSize);
   const size_t wbytes = static_cast<size_t>(C) * split_c * 2 * sizeof(A);
   if (wbytes > bytes) bytes = wbytes;
-  RowConfig cfg;
-  if (plan_group_grad_rows<T>(G, D, S, layout, &cfg)) {
+  if (layout == DRAGON_HIP_NCHW) {  // per-(n, c) pairs of the fused and the general path
     const size_t fbytes = static_cast<size_t>(N) * C * 2 * sizeof(A);
     if (fbytes > bytes) bytes = fbytes;
   }
@@ -697,11 +912,23 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   constexpr int kVec = IO<T>::kVec;
   RowConfig cfg;
   const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
-  if (!sh.nchw || sh.S % kVec != 0 || !aligned16(x) || !aligned16(y) ||
-      !pick_row_config(L / kVec, 8, &cfg)) {
-    return false;
-  }
+  if (!sh.nchw || !pick_row_config(ceil_div(L, kVec), 8, &cfg)) return false;
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+  if (sh.S % kVec != 0 || !aligned16(x) || !aligned16(y)) {
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    using Tile = RowTile<T, TPR, VPT>;                                                          \
+    hipLaunchKernelGGL((group_norm_forward_rows_any<T, TPR, VPT>),                              \
+                       dim3(row_grid(rows, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,      \
+                       stream, rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),             \
+                       static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig), \
+                       static_cast<T*>(y));                                                     \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+    return true;
+  }
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
@@ -825,6 +1052,40 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 
   const uint32_t total = sh.N * sh.C * sh.S;
   const bool base_ok = aligned16(x) && aligned16(dy) && aligned16(dx);
+  if (sh.nchw) {
+    // 1+2. one pass over x and dy for the per-(n, c) pairs, then ds/db and dgamma/dbeta from them
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    RowConfig cfg;
+    if (sh.S < 16) {
+      hipLaunchKernelGGL((channel_pair_sums_short<T>), dim3(map_grid(static_cast<uint32_t>(rows))),
+                         dim3(256), 0, stream, rows, static_cast<int>(sh.S), sh.D, xp, dyp, mup,
+                         part);
+    } else if (pick_row_config(ceil_div(sh.S, kVec), 4, &cfg)) {
+      const bool regular = sh.S % kVec == 0 && aligned16(x) && aligned16(dy);
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    using Tile = RowTile<T, TPR, VPT>;                                                          \
+    const dim3 grid(row_grid(rows, Tile::kRowsPerBlock)), block(Tile::kThreads);                \
+    if (regular) {                                                                              \
+      hipLaunchKernelGGL((channel_pair_sums_rows<T, TPR, VPT, false>), grid, block, 0, stream,  \
+                         rows, static_cast<int>(sh.S), sh.D, xp, dyp, mup, part);               \
+    } else {                                                                                    \
+      hipLaunchKernelGGL((channel_pair_sums_rows<T, TPR, VPT, true>), grid, block, 0, stream,   \
+                         rows, static_cast<int>(sh.S), sh.D, xp, dyp, mup, part);               \
+    }                                                                                           \
+  }
+      DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
+    } else {
+      hipLaunchKernelGGL((channel_pair_sums_looped<T>), dim3(loop_grid(rows)), dim3(kLoopThreads),
+                         0, stream, rows, static_cast<int64_t>(sh.S), sh.D, xp, dyp, mup, part);
+    }
+    const uint32_t group_blocks = static_cast<uint32_t>(ceil_div(sh.N * sh.G, 256));
+    const uint32_t chan_blocks = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize));
+    hipLaunchKernelGGL((group_grad_from_channel_sums<A>), dim3(group_blocks + chan_blocks),
+                       dim3(256), 0, stream, sh.N, sh.G, sh.D, group_blocks, part, gp, mup, rsp,
+                       dsp, dbp, dgp, dbtp);
+  } else {
   // 1. ds, db per (n, g)
   {
     SegmentedReduce s;
@@ -877,6 +1138,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          stream, c, xp, dyp, f, part);
       launch_reduce2_finalize<A, StorePairEpilogue<A>>(sh.C, c.split, false, part, e, stream);
     }
+  }
   }
   // 3. dx
   {
