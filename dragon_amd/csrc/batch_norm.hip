@@ -33,13 +33,9 @@ inline SegmentedReduce channel_segments(const ChannelShape& sh) {
   s.split = pick_split(sh.C, static_cast<int64_t>(sh.N) * sh.S);
   return s;
 }
-inline ColumnReduce channel_columns(const ChannelShape& sh) {
-  ColumnReduce c{sh.N * sh.S, sh.C, 1};
-  c.split = pick_split(ceil_div(sh.C, kWaveSize), static_cast<int64_t>(sh.N) * sh.S * kWaveSize);
-  return c;
-}
 inline size_t channel_scratch_bytes(const ChannelShape& sh, size_t acc_bytes) {
-  const uint32_t split = sh.nchw ? channel_segments(sh).split : channel_columns(sh).split;
+  const uint32_t split = sh.nchw ? channel_segments(sh).split
+                                 : column_split_bound(static_cast<int64_t>(sh.N) * sh.S, sh.C);
   return static_cast<size_t>(sh.C) * split * 2 * acc_bytes;
 }
 
@@ -65,11 +61,9 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
     hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3(fin_grid), dim3(kReduceThreads), 0, stream,
                        sh.C, s.split, true, part, e);
   } else {
-    const ColumnReduce c = channel_columns(sh);
-    const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
-    hipLaunchKernelGGL((reduce2_columns<T, kIn, F>), grid, dim3(kReduceThreads), 0, stream, c, in0,
-                       in1, f, part);
-    launch_reduce2_finalize<A, E>(sh.C, c.split, false, part, e, stream);
+    const uint32_t split = launch_reduce2_columns<T, kIn, F>(sh.N * sh.S, sh.C, in0, in1, f, part,
+                                                             stream);
+    launch_reduce2_finalize<A, E>(sh.C, split, false, part, e, stream);
   }
 }
 
@@ -232,6 +226,16 @@ struct ChannelIndex {
   }
 };
 
+// kVec consecutive per-channel parameters starting at channel c (NHWC packets).
+template <int kVec, typename A>
+__device__ __forceinline__ void load_channel_params(const A* p, uint32_t c, A (&v)[kVec]) {
+  if constexpr (kVec == 1) {
+    v[0] = p[c];
+  } else {
+    load_params_ragged<kVec>(p + c, kVec, v);
+  }
+}
+
 template <typename T, int kVec>
 struct AffineApply {  // y = x*scale[c] + bias[c]
   using A = typename IO<T>::Acc;
@@ -245,8 +249,11 @@ struct AffineApply {  // y = x*scale[c] + bias[c]
 #pragma unroll
       for (int e = 0; e < kVec; ++e) v[e] = v[e] * s + b;
     } else {
+      A s[kVec], b[kVec];
+      load_channel_params<kVec>(scale, c, s);
+      load_channel_params<kVec>(bias, c, b);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = v[e] * scale[c + e] + bias[c + e];
+      for (int e = 0; e < kVec; ++e) v[e] = v[e] * s[e] + b[e];
     }
   }
 };
@@ -261,11 +268,6 @@ struct TrainingGradApply {
   const A* dgamma;
   const A* dbeta;
   A normalizer;
-  __device__ __forceinline__ A one(A x, A dy, uint32_t c) const {
-    const A r = rsig[c];
-    const A x_norm = (x - mu[c]) * r;
-    return gamma[c] * r * (dy - (x_norm * dgamma[c] + dbeta[c]) / normalizer);
-  }
   __device__ __forceinline__ void operator()(uint32_t i, A (&x)[kVec], const A (&dy)[kVec]) const {
     const uint32_t c = idx(i);
     if (idx.sh.nchw) {
@@ -275,8 +277,17 @@ struct TrainingGradApply {
         x[e] = g * (dy[e] - ((x[e] - m) * r * dg + db) / normalizer);
       }
     } else {
+      A r[kVec], m[kVec], g[kVec], dg[kVec], db[kVec];
+      load_channel_params<kVec>(rsig, c, r);
+      load_channel_params<kVec>(mu, c, m);
+      load_channel_params<kVec>(gamma, c, g);
+      load_channel_params<kVec>(dgamma, c, dg);
+      load_channel_params<kVec>(dbeta, c, db);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) x[e] = one(x[e], dy[e], c + e);
+      for (int e = 0; e < kVec; ++e) {
+        const A x_norm = (x[e] - m[e]) * r[e];
+        x[e] = g[e] * r[e] * (dy[e] - (x_norm * dg[e] + db[e]) / normalizer);
+      }
     }
   }
 };
@@ -294,8 +305,11 @@ struct InferenceGradApply {  // dx = dy * gamma[c] * rsig[c]
 #pragma unroll
       for (int e = 0; e < kVec; ++e) dy[e] = dy[e] * g;
     } else {
+      A g[kVec], r[kVec];
+      load_channel_params<kVec>(gamma, c, g);
+      load_channel_params<kVec>(rsig, c, r);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) dy[e] = dy[e] * (gamma[c + e] * rsig[c + e]);
+      for (int e = 0; e < kVec; ++e) dy[e] = dy[e] * (g[e] * r[e]);
     }
   }
 };
@@ -417,7 +431,9 @@ int make_shape(int64_t N, int64_t C, int64_t S, int layout, ChannelShape* sh) {
   if (layout != DRAGON_HIP_NCHW && layout != DRAGON_HIP_NHWC) return DRAGON_HIP_EINVAL;
   if (!fits_int32(N * C * S)) return DRAGON_HIP_EINVAL;
   sh->N = static_cast<uint32_t>(N), sh->C = static_cast<uint32_t>(C);
-  sh->S = static_cast<uint32_t>(S), sh->nchw = layout == DRAGON_HIP_NCHW;
+  // [N, C, 1] and [N, 1, C] are the same memory: with S == 1 a channel is a
+  // column of the [N, C] matrix, whatever the layout tag says.
+  sh->S = static_cast<uint32_t>(S), sh->nchw = layout == DRAGON_HIP_NCHW && S != 1;
   return DRAGON_HIP_OK;
 }
 

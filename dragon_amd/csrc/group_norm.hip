@@ -893,7 +893,7 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   size_t bytes = static_cast<size_t>(N) * G * split_g * 2 * sizeof(A);
   const uint32_t split_c = layout == DRAGON_HIP_NCHW
       ? pick_split(C, N * S)
-      : pick_split(ceil_div(C, kWaveSize), N * S * kWaveSize);
+      : column_split_bound(N * S, C);
   const size_t wbytes = static_cast<size_t>(C) * split_c * 2 * sizeof(A);
   if (wbytes > bytes) bytes = wbytes;
   if (layout == DRAGON_HIP_NCHW) {  // per-(n, c) pairs of the fused and the general path
@@ -1130,13 +1130,10 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          dim3(static_cast<unsigned>(ceil_div(sh.C, kReduceThreads))),
                          dim3(kReduceThreads), 0, stream, sh.C, s.split, true, part, e);
     } else {
-      ColumnReduce c{sh.N * sh.S, sh.C, 1};
-      c.split = pick_split(ceil_div(sh.C, kWaveSize), static_cast<int64_t>(sh.N) * sh.S * kWaveSize);
       WGradAccumNHWC<T> f{sh, mup, rsp, 0};
-      const dim3 grid(static_cast<unsigned>(ceil_div(sh.C, kWaveSize)) * c.split);
-      hipLaunchKernelGGL((reduce2_columns<T, 2, WGradAccumNHWC<T>>), grid, dim3(kReduceThreads), 0,
-                         stream, c, xp, dyp, f, part);
-      launch_reduce2_finalize<A, StorePairEpilogue<A>>(sh.C, c.split, false, part, e, stream);
+      const uint32_t split = launch_reduce2_columns<T, 2, WGradAccumNHWC<T>>(
+          sh.N * sh.S, sh.C, xp, dyp, f, part, stream);
+      launch_reduce2_finalize<A, StorePairEpilogue<A>>(sh.C, split, false, part, e, stream);
     }
   }
   }

@@ -218,7 +218,7 @@ int make_plan(int dtype, int num_dims, const int64_t* dims, int num_axes, const 
   } else if (pat == "RK") {
     plan->kind = kPlanColumns;
     plan->col = ColumnReduce{u32(ext[0]), u32(ext[1]), 1};
-    plan->col.split = pick_split(ceil_div(ext[1], kWaveSize), ext[0] * kWaveSize);
+    plan->col.split = column_split_bound(ext[0], ext[1]);  // upper bound: sizes the scratch
     plan->scratch_bytes = static_cast<size_t>(plan->col.split) * ext[1] * 2 * acc_bytes;
   } else {
     if (ext.size() > kMaxDims) return DRAGON_HIP_EINVAL;
@@ -270,11 +270,10 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
   } else if (plan.kind == kPlanColumns) {
     const ColumnReduce& c = plan.col;
     Accum f{xp, A(0)};
-    const dim3 grid(static_cast<unsigned>(ceil_div(c.cols, kWaveSize)) * c.split);
-    hipLaunchKernelGGL((reduce2_columns<T, 1, Accum>), grid, dim3(kReduceThreads), 0, stream, c, xp,
-                       xp, f, part);
+    const uint32_t split = launch_reduce2_columns<T, 1, Accum>(c.rows, c.cols, xp, xp, f, part,
+                                                               stream);
     ReduceColEpilogue<T, P> e{xp, inv_n, out};
-    launch_reduce2_finalize<A, ReduceColEpilogue<T, P>>(c.cols, c.split, false, part, e, stream);
+    launch_reduce2_finalize<A, ReduceColEpilogue<T, P>>(c.cols, split, false, part, e, stream);
   } else {
     const unsigned grid = static_cast<unsigned>(plan.n_out < 65536 ? plan.n_out : 65536);
     hipLaunchKernelGGL((reduce_gather<T, P>), dim3(grid), dim3(kReduceThreads), 0, stream,

@@ -160,6 +160,92 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_columns(
   }
 }
 
+// The same with a 16-byte packet of kVec adjacent columns per lane (cols a
+// multiple of kVec, 16-byte aligned base): a wavefront reads 1 KiB of a row at
+// a time. Each column keeps its own copy of the accumulator functor.
+template <typename T, int kIn, typename F>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_columns_packets(
+    const ColumnReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  __shared__ A lds[kReduceWaves][kWaveSize][2 * kVec];
+  const uint32_t tile_cols = kWaveSize * kVec;
+  const uint32_t tiles = (d.cols + tile_cols - 1) / tile_cols;
+  const uint32_t tile = blockIdx.x % tiles;
+  const uint32_t k = blockIdx.x / tiles;
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t c0 = tile * tile_cols + lane * kVec;
+  A a[kVec], b[kVec];
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) a[e] = b[e] = A(0);
+  if (c0 < d.cols) {
+    F fs[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      fs[e] = f;
+      fs[e].begin(c0 + e, c0 + e);
+    }
+#pragma unroll 4
+    for (uint32_t r = k * kReduceWaves + wave; r < d.rows; r += d.split * kReduceWaves) {
+      const uint32_t off = r * d.cols + c0;
+      A x0[kVec], x1[kVec];
+      load_unpack<T>(in0 + off, x0);
+      if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        fs[e].add(r, c0 + e, off + e, x0[e], kIn == 2 ? x1[e] : A(0), a[e], b[e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) {
+    lds[wave][lane][2 * e] = a[e];
+    lds[wave][lane][2 * e + 1] = b[e];
+  }
+  __syncthreads();
+  if (wave == 0 && c0 < d.cols) {
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+#pragma unroll
+      for (int w = 1; w < kReduceWaves; ++w) {
+        a[e] += lds[w][lane][2 * e];
+        b[e] += lds[w][lane][2 * e + 1];
+      }
+      partial[(static_cast<size_t>(k) * d.cols + c0 + e) * 2] = a[e];
+      partial[(static_cast<size_t>(k) * d.cols + c0 + e) * 2 + 1] = b[e];
+    }
+  }
+}
+
+// The largest split any column stage one chooses for a [rows, cols] reduction
+// (the packet kernel, with the fewest tiles, splits the rows finest): sizes the
+// scratch, split * cols pairs.
+inline uint32_t column_split_bound(int64_t rows, int64_t cols) {
+  return pick_split(ceil_div(cols, kWaveSize * 8), rows * kWaveSize * 8);
+}
+// Launches the column stage one that suits the shape and returns its split.
+template <typename T, int kIn, typename F>
+inline uint32_t launch_reduce2_columns(uint32_t rows, uint32_t cols, const T* in0, const T* in1,
+                                       F f, typename IO<T>::Acc* partial, hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  ColumnReduce d{rows, cols, 1};
+  const bool packets = cols % kVec == 0 && aligned16(in0) && (kIn == 1 || aligned16(in1));
+  if (packets) {
+    const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, kWaveSize * kVec));
+    d.split = pick_split(tiles, static_cast<int64_t>(rows) * kWaveSize * kVec);
+    hipLaunchKernelGGL((reduce2_columns_packets<T, kIn, F>), dim3(tiles * d.split),
+                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+  } else {
+    d.split = pick_split(ceil_div(cols, kWaveSize), static_cast<int64_t>(rows) * kWaveSize);
+    hipLaunchKernelGGL((reduce2_columns<T, kIn, F>),
+                       dim3(static_cast<unsigned>(ceil_div(cols, kWaveSize)) * d.split),
+                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+  }
+  return d.split;
+}
+
 // Stage two: one thread per output adds its `split` pairs in index order and
 // hands the totals to the epilogue E: void operator()(uint32_t o, A a, A b).
 // `segment_major` selects the scratch layout of reduce2_segments
