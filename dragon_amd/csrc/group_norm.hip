@@ -796,6 +796,195 @@ __global__ __launch_bounds__(256) void group_grad_from_channel_sums(
   }
 }
 
+// --------------------------------------------------------------------------
+// NHWC: x is [N, S, C] and a group is D adjacent columns of one sample's
+// [S, C] matrix. Stage one reduces every (n, c) column over s with full-width
+// row accesses (a lane owns kW adjacent channels: one 16-byte packet, or one
+// element for unaligned tensors); a sample's rows are split over `split`
+// workgroups. partial[((n*split + k)*C + c)*2 + {0,1}]. F provides
+//   void begin(uint32_t n, uint32_t c)
+//   void add(A x0, A x1, A& a, A& b)
+// --------------------------------------------------------------------------
+struct BatchedColumns {
+  uint32_t N, S, C, split;
+};
+
+template <typename T, int kIn, int kW, typename F>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
+    const BatchedColumns d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds[kReduceWaves][kWaveSize][2 * kW];
+  const uint32_t tile_cols = kWaveSize * kW;
+  const uint32_t tiles = (d.C + tile_cols - 1) / tile_cols;
+  const uint32_t tile = blockIdx.x % tiles;
+  const uint32_t k = (blockIdx.x / tiles) % d.split;
+  const uint32_t n = blockIdx.x / (tiles * d.split);
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const uint32_t c0 = tile * tile_cols + lane * kW;
+  A a[kW], b[kW];
+#pragma unroll
+  for (int e = 0; e < kW; ++e) a[e] = b[e] = A(0);
+  if (c0 < d.C) {
+    F fs[kW];
+#pragma unroll
+    for (int e = 0; e < kW; ++e) {
+      fs[e] = f;
+      fs[e].begin(n, c0 + e);
+    }
+    const uint32_t base = n * d.S * d.C + c0;
+#pragma unroll 4
+    for (uint32_t r = k * kReduceWaves + wave; r < d.S; r += d.split * kReduceWaves) {
+      const uint32_t off = base + r * d.C;
+      A x0[kW], x1[kW];
+      if constexpr (kW == 1) {
+        x0[0] = IO<T>::load1(in0 + off);
+        x1[0] = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
+      } else {
+        load_unpack<T>(in0 + off, x0);
+        if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
+      }
+#pragma unroll
+      for (int e = 0; e < kW; ++e) fs[e].add(x0[e], kIn == 2 ? x1[e] : A(0), a[e], b[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kW; ++e) {
+    lds[wave][lane][2 * e] = a[e];
+    lds[wave][lane][2 * e + 1] = b[e];
+  }
+  __syncthreads();
+  if (wave == 0 && c0 < d.C) {
+    A* out = partial + ((static_cast<size_t>(n) * d.split + k) * d.C + c0) * 2;
+#pragma unroll
+    for (int e = 0; e < kW; ++e) {
+#pragma unroll
+      for (int w = 1; w < kReduceWaves; ++w) {
+        a[e] += lds[w][lane][2 * e];
+        b[e] += lds[w][lane][2 * e + 1];
+      }
+      out[2 * e] = a[e];
+      out[2 * e + 1] = b[e];
+    }
+  }
+}
+
+// Rows of one sample per stage-one workgroup: enough workgroups to fill the
+// device, at least ~64 rows each.
+inline uint32_t batched_split(int64_t N, int64_t S, int64_t C, int kw) {
+  const int64_t tiles = ceil_div(C, kWaveSize * kw);
+  int64_t split = ceil_div(static_cast<int64_t>(kNumCUs) * 8, N * tiles);
+  const int64_t by_work = ceil_div(S, 64);
+  if (split > by_work) split = by_work;
+  if (split < 1) split = 1;
+  if (split > 256) split = 256;
+  return static_cast<uint32_t>(split);
+}
+// Largest scratch either variant (packet or scalar lanes) needs, in pairs.
+inline size_t batched_partial_pairs(int64_t N, int64_t S, int64_t C) {
+  uint32_t split = batched_split(N, S, C, 1);
+  const uint32_t split8 = batched_split(N, S, C, 8);
+  if (split8 > split) split = split8;
+  return static_cast<size_t>(N) * split * C;
+}
+
+template <typename T>
+struct ColumnStatsAccum {  // sums shifted by the column's first element
+  using A = typename IO<T>::Acc;
+  const T* x;
+  uint32_t S, C;
+  A shift;
+  __device__ __forceinline__ void begin(uint32_t n, uint32_t c) {
+    shift = IO<T>::load1(x + static_cast<size_t>(n) * S * C + c);
+  }
+  __device__ __forceinline__ void add(A x0, A, A& a, A& b) const {
+    const A d = x0 - shift;
+    a += d;
+    b += d * d;
+  }
+};
+
+template <typename T>
+struct ColumnPairAccum {  // a = sum dy * (x - mu[n, g]), b = sum dy
+  using A = typename IO<T>::Acc;
+  const A* mu;
+  uint32_t G, D;
+  A m;
+  __device__ __forceinline__ void begin(uint32_t n, uint32_t c) { m = mu[n * G + c / D]; }
+  __device__ __forceinline__ void add(A x0, A dy, A& a, A& b) const {
+    a += dy * (x0 - m);
+    b += dy;
+  }
+};
+
+// Last stage of the NHWC statistics, one thread per (n, g), from the per-(n, c)
+// pairs: per channel mean_c = shift_c + a_c/S and M2_c = b_c - a_c^2/S, combined
+// over the group's D channels as mean = avg(mean_c),
+// M2 = sum(M2_c + S*(mean_c - mean)^2).
+template <typename T>
+__global__ __launch_bounds__(256) void group_stats_from_column_sums(
+    const BatchedColumns d, const uint32_t G, const uint32_t D, const typename IO<T>::Acc eps,
+    const T* __restrict__ x, const typename IO<T>::Acc* __restrict__ sums,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig) {
+  using A = typename IO<T>::Acc;
+  const uint32_t ng = blockIdx.x * 256 + threadIdx.x;
+  if (ng >= d.N * G) return;
+  const uint32_t n = ng / G, g = ng - n * G;
+  const A inv_s = A(1) / A(d.S);
+  const T* first_row = x + static_cast<size_t>(n) * d.S * d.C + g * D;
+  const A* pairs = sums + (static_cast<size_t>(n) * d.C + g * D) * 2;
+  A mean = A(0);
+  for (uint32_t j = 0; j < D; ++j) mean += IO<T>::load1(first_row + j) + pairs[2 * j] * inv_s;
+  mean = mean / A(D);
+  A m2 = A(0);
+  for (uint32_t j = 0; j < D; ++j) {
+    const A a = pairs[2 * j], b = pairs[2 * j + 1];
+    const A dm = IO<T>::load1(first_row + j) + a * inv_s - mean;
+    m2 += (b - a * a * inv_s) + A(d.S) * dm * dm;
+  }
+  mu[ng] = mean;
+  rsig[ng] = acc_rsqrt_exact(m2 / (A(D) * A(d.S)) + eps);
+}
+
+// sums[(n*C + c)*2 + {0,1}] = sum over the `split` partial pairs of (n, c).
+template <typename A>
+__global__ __launch_bounds__(256) void sum_batched_partials(const BatchedColumns d,
+                                                            const A* __restrict__ partial,
+                                                            A* __restrict__ sums) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= d.N * d.C) return;
+  const uint32_t n = i / d.C, c = i - n * d.C;
+  A a = A(0), b = A(0);
+  for (uint32_t k = 0; k < d.split; ++k) {
+    const size_t idx = ((static_cast<size_t>(n) * d.split + k) * d.C + c) * 2;
+    a += partial[idx];
+    b += partial[idx + 1];
+  }
+  sums[static_cast<size_t>(i) * 2] = a;
+  sums[static_cast<size_t>(i) * 2 + 1] = b;
+}
+
+template <typename T, int kIn, typename F>
+BatchedColumns launch_batched_columns(const GroupShape& sh, const T* in0, const T* in1, F f,
+                                      typename IO<T>::Acc* partial, hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const bool packets = sh.C % kVec == 0 && aligned16(in0) && (kIn == 1 || aligned16(in1));
+  BatchedColumns d{sh.N, sh.S, sh.C, 1};
+  if (packets) {
+    d.split = batched_split(sh.N, sh.S, sh.C, kVec);
+    const uint32_t tiles = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize * kVec));
+    hipLaunchKernelGGL((reduce2_batched_columns<T, kIn, kVec, F>), dim3(sh.N * d.split * tiles),
+                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+  } else {
+    d.split = batched_split(sh.N, sh.S, sh.C, 1);
+    const uint32_t tiles = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize));
+    hipLaunchKernelGGL((reduce2_batched_columns<T, kIn, 1, F>), dim3(sh.N * d.split * tiles),
+                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+  }
+  return d;
+}
+
 // Sums P partial rows of 2*C interleaved (dgamma, dbeta) words. A workgroup of
 // 16 wavefronts owns 64 adjacent words; wavefront w adds rows w, w+16, ...
 template <typename A>
@@ -898,6 +1087,9 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   if (wbytes > bytes) bytes = wbytes;
   if (layout == DRAGON_HIP_NCHW) {  // per-(n, c) pairs of the fused and the general path
     const size_t fbytes = static_cast<size_t>(N) * C * 2 * sizeof(A);
+    if (fbytes > bytes) bytes = fbytes;
+  } else {  // stage-one partial pairs, then the per-(n, c) pairs
+    const size_t fbytes = (batched_partial_pairs(N, S, C) + static_cast<size_t>(N) * C) * 2 * sizeof(A);
     if (fbytes > bytes) bytes = fbytes;
   }
   return bytes;
@@ -1086,56 +1278,18 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                        dim3(256), 0, stream, sh.N, sh.G, sh.D, group_blocks, part, gp, mup, rsp,
                        dsp, dbp, dgp, dbtp);
   } else {
-  // 1. ds, db per (n, g)
-  {
-    SegmentedReduce s;
-    s.n_out = sh.N * sh.G;
-    if (sh.nchw) {
-      s = SegmentedReduce{sh.N * sh.G, 1, sh.D * sh.S, 0, 1, sh.D * sh.S, 0, 1};
-    } else {
-      s = SegmentedReduce{sh.N * sh.G, sh.G, sh.S * sh.C, sh.D, sh.S, sh.D, sh.C, 1};
-    }
-    s.split = pick_split(s.n_out, static_cast<int64_t>(sh.D) * sh.S);
-    InternalGradAccum<T> f{sh, gp, 0};
-    const bool vec_ok = base_ok && (sh.nchw ? sh.S % kVec == 0 : sh.D % kVec == 0);
-    const dim3 grid(s.n_out * s.split);
-    if (vec_ok) {
-      hipLaunchKernelGGL((reduce2_segments<T, 2, kVec, InternalGradAccum<T>>), grid,
-                         dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
-    } else {
-      hipLaunchKernelGGL((reduce2_segments<T, 2, 1, InternalGradAccum<T>>), grid,
-                         dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
-    }
-    StorePairEpilogue<A> e{dsp, dbp};
-    hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
-                       dim3(static_cast<unsigned>(ceil_div(s.n_out, kReduceThreads))),
-                       dim3(kReduceThreads), 0, stream, s.n_out, s.split, true, part, e);
-  }
-  // 2. dgamma, dbeta per channel (scratch is reused: stream order keeps step 1 finished)
-  {
-    StorePairEpilogue<A> e{dgp, dbtp};
-    if (sh.nchw) {
-      SegmentedReduce s{sh.C, sh.C, 0, sh.S, sh.N, sh.S, sh.C * sh.S, 1};
-      s.split = pick_split(sh.C, static_cast<int64_t>(sh.N) * sh.S);
-      WGradAccumNCHW<T> f{sh, mup, rsp, 0};
-      const dim3 grid(s.n_out * s.split);
-      if (base_ok && sh.S % kVec == 0) {
-        hipLaunchKernelGGL((reduce2_segments<T, 2, kVec, WGradAccumNCHW<T>>), grid,
-                           dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
-      } else {
-        hipLaunchKernelGGL((reduce2_segments<T, 2, 1, WGradAccumNCHW<T>>), grid,
-                           dim3(kReduceThreads), 0, stream, s, xp, dyp, f, part);
-      }
-      hipLaunchKernelGGL((reduce2_finalize<A, StorePairEpilogue<A>>),
-                         dim3(static_cast<unsigned>(ceil_div(sh.C, kReduceThreads))),
-                         dim3(kReduceThreads), 0, stream, sh.C, s.split, true, part, e);
-    } else {
-      WGradAccumNHWC<T> f{sh, mup, rsp, 0};
-      const uint32_t split = launch_reduce2_columns<T, 2, WGradAccumNHWC<T>>(
-          sh.N * sh.S, sh.C, xp, dyp, f, part, stream);
-      launch_reduce2_finalize<A, StorePairEpilogue<A>>(sh.C, split, false, part, e, stream);
-    }
-  }
+    // NHWC: the same per-(n, c) pairs from full-width column reductions of each sample
+    A* sums = part + batched_partial_pairs(sh.N, sh.S, sh.C) * 2;
+    const BatchedColumns d = launch_batched_columns<T, 2>(
+        sh, xp, dyp, ColumnPairAccum<T>{mup, sh.G, sh.D, A(0)}, part, stream);
+    hipLaunchKernelGGL((sum_batched_partials<A>),
+                       dim3(static_cast<unsigned>(ceil_div(sh.N * sh.C, 256))), dim3(256), 0,
+                       stream, d, part, sums);
+    const uint32_t group_blocks = static_cast<uint32_t>(ceil_div(sh.N * sh.G, 256));
+    const uint32_t chan_blocks = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize));
+    hipLaunchKernelGGL((group_grad_from_channel_sums<A>), dim3(group_blocks + chan_blocks),
+                       dim3(256), 0, stream, sh.N, sh.G, sh.D, group_blocks, sums, gp, mup, rsp,
+                       dsp, dbp, dgp, dbtp);
   }
   // 3. dx
   {
@@ -1154,9 +1308,36 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   return status_of_launch();
 }
 
+// NHWC statistics of the fused forward: column sums per sample, then mean and
+// rsig per group (InvStd folded into the second stage).
+template <typename T>
+int group_norm_stats_nhwc(const GroupShape& sh, float eps, const void* x, void* mu, void* rsig,
+                          void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  const T* xp = static_cast<const T*>(x);
+  A* part = static_cast<A*>(scratch);
+  A* sums = part + batched_partial_pairs(sh.N, sh.S, sh.C) * 2;
+  const BatchedColumns d = launch_batched_columns<T, 1>(
+      sh, xp, xp, ColumnStatsAccum<T>{xp, sh.S, sh.C, A(0)}, part, stream);
+  hipLaunchKernelGGL((sum_batched_partials<A>),
+                     dim3(static_cast<unsigned>(ceil_div(sh.N * sh.C, 256))), dim3(256), 0, stream,
+                     d, part, sums);
+  hipLaunchKernelGGL((group_stats_from_column_sums<T>),
+                     dim3(static_cast<unsigned>(ceil_div(sh.N * sh.G, 256))), dim3(256), 0, stream,
+                     d, sh.G, sh.D, A(eps), xp, sums, static_cast<A*>(mu), static_cast<A*>(rsig));
+  return status_of_launch();
+}
+
+// [N, G, D, 1] and [N, 1, G, D] are the same memory: with S == 1 a group is a
+// contiguous row of D elements whatever the layout tag says.
+inline int canonical_layout(int layout, int64_t S) {
+  return (layout == DRAGON_HIP_NHWC && S == 1) ? DRAGON_HIP_NCHW : layout;
+}
+
 int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShape* sh) {
   if (N < 0 || G <= 0 || D <= 0 || S < 0) return DRAGON_HIP_EINVAL;
   if (layout != DRAGON_HIP_NCHW && layout != DRAGON_HIP_NHWC) return DRAGON_HIP_EINVAL;
+  layout = canonical_layout(layout, S);
   if (!fits_int32(N * G * D * S)) return DRAGON_HIP_EINVAL;
   sh->N = static_cast<uint32_t>(N), sh->G = static_cast<uint32_t>(G);
   sh->D = static_cast<uint32_t>(D), sh->S = static_cast<uint32_t>(S);
@@ -1191,6 +1372,7 @@ size_t dragon_hip_group_norm_grad_scratch_bytes(int dtype, int64_t N, int64_t G,
                                                 int64_t S, int layout) {
   dragon_hip::GroupShape sh;
   if (dragon_hip::make_shape(N, G, D, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  layout = dragon_hip::canonical_layout(layout, S);
   switch (dtype) {
     case DRAGON_HIP_F16: return dragon_hip::grad_scratch_t<dragon_hip::f16_t>(N, G, D, S, layout);
     case DRAGON_HIP_BF16: return dragon_hip::grad_scratch_t<dragon_hip::bf16_t>(N, G, D, S, layout);
@@ -1251,8 +1433,15 @@ size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t
                                                    int64_t S, int layout) {
   dragon_hip::GroupShape sh;
   if (dragon_hip::make_shape(N, G, D, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  layout = dragon_hip::canonical_layout(layout, S);
   const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
-  return dragon_hip_moments_scratch_bytes(dtype, v.num_dims, v.dims, v.num_axes, v.axes);
+  size_t bytes = dragon_hip_moments_scratch_bytes(dtype, v.num_dims, v.dims, v.num_axes, v.axes);
+  if (layout == DRAGON_HIP_NHWC) {
+    const size_t nhwc = (dragon_hip::batched_partial_pairs(N, S, G * D) +
+                         static_cast<size_t>(N) * G * D) * 2 * (dtype == DRAGON_HIP_F64 ? 8 : 4);
+    if (nhwc > bytes) bytes = nhwc;
+  }
+  return bytes;
 }
 
 int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
@@ -1262,6 +1451,7 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
   dragon_hip::GroupShape sh;
   int st = dragon_hip::make_shape(N, G, D, S, layout, &sh);
   if (st != DRAGON_HIP_OK) return st;
+  layout = dragon_hip::canonical_layout(layout, S);
   if (N * S == 0) return DRAGON_HIP_OK;
   if (!x || !gamma || !beta || !mu || !rsig || !y) return DRAGON_HIP_EINVAL;
   hipStream_t hs = static_cast<hipStream_t>(stream);
@@ -1283,6 +1473,20 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
       return DRAGON_HIP_EDTYPE;
   }
   if (fused) return dragon_hip::status_of_launch();
+  if (!sh.nchw && S > 1) {
+    // NHWC: statistics from full-width column reductions of each sample
+    if (!scratch || scratch_bytes < dragon_hip_group_norm_forward_scratch_bytes(dtype, N, G, D, S, layout)) {
+      return DRAGON_HIP_ESCRATCH;
+    }
+    switch (dtype) {
+      case DRAGON_HIP_F16: st = dragon_hip::group_norm_stats_nhwc<dragon_hip::f16_t>(sh, eps, x, mu, rsig, scratch, hs); break;
+      case DRAGON_HIP_BF16: st = dragon_hip::group_norm_stats_nhwc<dragon_hip::bf16_t>(sh, eps, x, mu, rsig, scratch, hs); break;
+      case DRAGON_HIP_F32: st = dragon_hip::group_norm_stats_nhwc<float>(sh, eps, x, mu, rsig, scratch, hs); break;
+      default: st = dragon_hip::group_norm_stats_nhwc<double>(sh, eps, x, mu, rsig, scratch, hs); break;
+    }
+    if (st != DRAGON_HIP_OK) return st;
+    return dragon_hip_group_norm(dtype, N, G, D, S, layout, x, mu, rsig, gamma, beta, y, stream);
+  }
   const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
   st = dragon_hip_moments(dtype, v.num_dims, v.dims, v.num_axes, v.axes, x, mu, rsig, scratch,
                           scratch_bytes, stream);
