@@ -20,6 +20,10 @@
 // row's element count; for regular tiles it is the row's packet count.
 #pragma once
 
+#include <map>
+#include <mutex>
+#include <tuple>
+
 #include "common.h"
 
 namespace dragon_hip {
@@ -249,12 +253,36 @@ inline bool pick_row_config(int64_t npackets, int max_vpt, RowConfig* cfg) {
 // Workgroups of `kernel` (block size `threads`, `dynamic_lds` bytes of dynamic
 // LDS) that can be resident on the whole device at once: the grid of a
 // persistent kernel. Also raises the kernel's dynamic-LDS limit when needed.
+// The answer is cached per (device, kernel, LDS size): the queries cost
+// microseconds of host time, and a launch path that a caller captures into a
+// graph should not depend on them after its first use.
 template <typename Kernel>
 inline unsigned resident_grid(Kernel kernel, int threads, size_t dynamic_lds) {
-  if (dynamic_lds > 48 * 1024) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(dynamic_lds));
+  struct Key {
+    int device;
+    const void* fn;
+    size_t lds;
+    bool operator<(const Key& o) const {
+      return std::tie(device, fn, lds) < std::tie(o.device, o.fn, o.lds);
+    }
+  };
+  static std::mutex lock;
+  static std::map<Key, unsigned> cache;
+  static std::map<Key, size_t> lds_limit;  // per (device, kernel): the limit set so far
+  int device = 0;
+  (void)hipGetDevice(&device);
+  const void* fn = reinterpret_cast<const void*>(kernel);
+  const Key key{device, fn, dynamic_lds};
+  {
+    std::lock_guard<std::mutex> guard(lock);
+    const auto hit = cache.find(key);
+    if (hit != cache.end()) return hit->second;
+    size_t& limit = lds_limit[Key{device, fn, 0}];
+    if (dynamic_lds > 48 * 1024 && dynamic_lds > limit) {  // only ever raised
+      (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(dynamic_lds));
+      limit = dynamic_lds;
+    }
   }
   int per_cu = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) !=
@@ -263,7 +291,10 @@ inline unsigned resident_grid(Kernel kernel, int threads, size_t dynamic_lds) {
     (void)hipGetLastError();
     per_cu = 1;
   }
-  return static_cast<unsigned>(per_cu) * kNumCUs;
+  const unsigned grid = static_cast<unsigned>(per_cu) * kNumCUs;
+  std::lock_guard<std::mutex> guard(lock);
+  cache[key] = grid;
+  return grid;
 }
 
 // LDS a workgroup may use for staged parameters (of 160 KB per compute unit).
