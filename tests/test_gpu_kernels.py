@@ -162,21 +162,32 @@ def test_softmax_forward_backward(K, shape, axis, dtype, log):
     assert U.normwise(dxw[ok], np.asarray(dx_ref)[ok]) <= U.TIGHT[dtype]
 
 
+@pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (3, 10, 33)])
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
-def test_softmax_in_place(K, dtype):
-    shape = (64, 512)
+def test_softmax_in_place(K, dtype, shape):
     x, dy = _softmax_inputs(shape, dtype, 5)
     xo, od = oracle_dtype_inputs(x, dtype)
-    y_ref = R.op_softmax(od, xo)
+    axis = 1  # the last axis of the 2-d shapes, the strided middle axis of the 3-d one
+    N, C = shape[0], shape[1]
+    S = int(np.prod(shape[2:] or (1,)))
+    y_ref = R.op_softmax(od, xo, axis)
     buf = U.to_device(x, dtype)
-    K.softmax(64, 1, 512, buf, buf)  # Y aliases X (AllowInplace {0,0})
-    assert U.rowwise_normwise(U.widen(U.to_host(buf), dtype), y_ref) <= U.TIGHT[dtype]
+    K.softmax(N, S, C, buf, buf)  # Y aliases X (AllowInplace {0,0})
+    got = np.moveaxis(U.widen(U.to_host(buf), dtype).reshape(shape), axis, -1)
+    x64 = np.moveaxis(np.asarray(xo, np.float64), axis, -1)
+    e64 = np.exp(x64 - x64.max(-1, keepdims=True))
+    y64 = e64 / e64.sum(-1, keepdims=True)
+    yr = np.moveaxis(np.asarray(y_ref), axis, -1)
+    # rows of 66001 put the oracle's sequential fp32 sum itself off: three-way check
+    e_ge, e_go, e_oe = (U.rowwise_normwise(got, y64), U.rowwise_normwise(got, yr),
+                        U.rowwise_normwise(yr, y64))
+    assert e_ge <= U.TIGHT[dtype] and e_go <= U.TIGHT[dtype] + e_oe, (e_go, e_ge, e_oe)
     g = U.to_device(dy, dtype)
-    yo, _ = oracle_dtype_inputs(U.to_host(buf), dtype)
+    yo, _ = oracle_dtype_inputs(U.to_host(buf).reshape(shape), dtype)
     dyo, _ = oracle_dtype_inputs(dy, dtype)
-    dx_ref = R.op_softmax_grad(od, yo, dyo)
-    K.softmax_grad(64, 1, 512, g, buf, g)  # dX aliases dY (AllowInplace {1,0})
-    assert U.normwise(U.widen(U.to_host(g), dtype), dx_ref) <= U.TIGHT[dtype]
+    dx_ref = R.op_softmax_grad(od, yo, dyo, axis)
+    K.softmax_grad(N, S, C, g, buf, g)  # dX aliases dY (AllowInplace {1,0})
+    assert U.normwise(U.widen(U.to_host(g), dtype).reshape(shape), dx_ref) <= U.TIGHT[dtype]
 
 
 def test_softmax_masked_logits_are_exact_zero(K):
