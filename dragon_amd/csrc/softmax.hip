@@ -14,8 +14,8 @@
 // alignment (ragged tiles take widths that are not whole 16-byte packets). 16-bit I/O accumulates in fp32
 // and uses the hardware exp2 (relative error ~1e-7 near the row maximum,
 // below 3e-6 in the far tail, both far under one 16-bit ulp); fp32 / fp64 I/O
-// use the correctly-scaled library exp and a true division, which is what the
-// reference's CPU expression does.
+// use the library exp. fp32 multiplies by the reciprocal of the row sum (one
+// ulp from the reference's quotient), fp64 divides as the reference does.
 //
 // S > 1 keeps a [C, columns] tile in the registers of a workgroup (col_tile.h)
 // when C <= 1024: one read, one write. Longer strided
@@ -39,8 +39,11 @@ struct SoftmaxMath {
       return acc_exp(v);
     }
   }
+  // fp32 and 16-bit outputs multiply by the correctly rounded reciprocal of the
+  // sum (within one fp32 ulp of the quotient, a tenth of a microsecond-scale
+  // division sequence per element saved); fp64 divides.
   static __device__ __forceinline__ A normalise(A e, A sum, A inv_sum) {
-    if constexpr (kFast) {
+    if constexpr (sizeof(A) == 4) {
       return e * inv_sum;
     } else {
       return e / sum;
@@ -110,6 +113,71 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
   }
 }
 
+// Rows that take a whole 1024-thread workgroup (a compute unit holds one or
+// two of those): a persistent workgroup requests the next row's packets before
+// it reduces the current row, and issues the current row's stores after the
+// wait for them, so loads, arithmetic and stores of neighbouring rows overlap.
+template <typename T, int kKind, int kVPT>
+__global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const int C, const T* x,
+                                                          T* y) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const int npackets = C / kVec;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  Raw cur;
+  cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    const bool more = row + stride < N;
+    nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
+    Tile t;
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      cur.unpack(i, t.v[i]);
+      const bool on = Tile::active(i, npackets);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = on ? t.v[i][e] : acc_neg_inf<A>();  // raw padding is zero bits
+        m = MaxOp()(m, t.v[i][e]);
+      }
+    }
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (kKind == kSoftmax) {
+          t.v[i][e] = M::exp_of(t.v[i][e] - m);
+          s += t.v[i][e];
+        } else {
+          t.v[i][e] = t.v[i][e] - m;
+          s += M::exp_of(t.v[i][e]);
+        }
+      }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    const A inv = A(1) / s;
+    const A l = acc_log(s);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = kKind == kSoftmax ? M::normalise(t.v[i][e], s, inv) : t.v[i][e] - l;
+      }
+    nxt.wait_ready();
+    cur = nxt;
+    t.store(y + row * C, npackets);
+    __syncthreads();  // slots are reused by the next row
+  }
+}
+
 template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
     const int64_t N, const int C, const T* dy, const T* y, T* dx) {
@@ -151,6 +219,75 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
       }
     g.store(dx + row * C, npackets);
     if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// The gradient for 1024-thread rows: dy and y as raw packets, the next row
+// prefetched where two rows of packets fit the registers (kPrefetch).
+template <typename T, int kKind, int kVPT, bool kPrefetch>
+__global__ __launch_bounds__(1024) void softmax_grad_wide_rows(const int64_t N, const int C,
+                                                               const T* dy, const T* y, T* dx) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[Tile::kSlots];
+  const int npackets = C / kVec;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  Raw tg, to;
+  if (kPrefetch) {
+    tg.load(dy + (row < N ? row : 0) * C, npackets, row < N);
+    to.load(y + (row < N ? row : 0) * C, npackets, row < N);
+  }
+  for (; row < N; row += stride) {
+    Raw ng, no;
+    if (kPrefetch) {
+      const bool more = row + stride < N;
+      ng.load(dy + (more ? row + stride : 0) * C, npackets, more);
+      no.load(y + (more ? row + stride : 0) * C, npackets, more);
+    } else {
+      tg.load(dy + row * C, npackets);
+      to.load(y + row * C, npackets);
+    }
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A g[kVec], o[kVec];
+      tg.unpack(i, g);
+      to.unpack(i, o);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += kKind == kSoftmax ? g[e] * o[e] : g[e];  // padding: dy = 0
+    }
+    s = Tile::reduce(s, SumOp(), slots);
+    tg.refresh();
+    to.refresh();
+    u32x4 out[kVPT];
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A g[kVec], o[kVec];
+      tg.unpack(i, g);
+      to.unpack(i, o);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        g[e] = kKind == kSoftmax ? (g[e] - s) * o[e] : g[e] - M::exp_of(o[e]) * s;
+      }
+      out[i] = IO<T>::pack(g);
+    }
+    if (kPrefetch) {
+      ng.wait_ready();
+      no.wait_ready();
+    }
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        store_packet(dx + row * C + static_cast<int64_t>(i * kTPR + threadIdx.x) * kVec, out[i]);
+      }
+    }
+    if (kPrefetch) tg = ng, to = no;
+    __syncthreads();  // slots are reused by the next row
   }
 }
 
@@ -448,6 +585,19 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
     // rows that are whole, aligned packets take the regular tiles, any other
     // width or base address the ragged ones
     const bool regular = C % kVec == 0 && aligned16(x) && aligned16(y);
+    // 1024-thread tiles: persistent workgroups that prefetch the next row
+    if (regular && cfg.tpr == 1024) {
+#define LAUNCH_WIDE(VPT)                                                                     \
+  {                                                                                          \
+    auto kernel = softmax_wide_rows<T, kKind, VPT>;                                          \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), xp, yp); \
+  }
+      if (cfg.vpt == 2) LAUNCH_WIDE(2) else if (cfg.vpt == 4) LAUNCH_WIDE(4) else LAUNCH_WIDE(8)
+#undef LAUNCH_WIDE
+      return status_of_launch();
+    }
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
@@ -498,9 +648,25 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   const T* yp = static_cast<const T*>(y);
   T* dp = static_cast<T*>(dx);
   RowConfig cfg;
+  const bool regular = C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx);
+  // 1024-thread rows: raw packets, persistent workgroups; the next row is
+  // prefetched up to 4 packets per thread and tensor
+  if (S == 1 && regular && pick_row_config(C / kVec, 8, &cfg) && cfg.tpr == 1024) {
+#define LAUNCH_WIDE(VPT, PREFETCH)                                                           \
+  {                                                                                          \
+    auto kernel = softmax_grad_wide_rows<T, kKind, VPT, PREFETCH>;                           \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), gp, yp, \
+                       dp);                                                                  \
+  }
+    if (cfg.vpt == 2) LAUNCH_WIDE(2, true) else if (cfg.vpt == 4) LAUNCH_WIDE(4, true)
+    else LAUNCH_WIDE(8, false)
+#undef LAUNCH_WIDE
+    return status_of_launch();
+  }
   // Two tiles live at once: halve the packets a thread may hold.
   if (S == 1 && pick_row_config(ceil_div(C, kVec), 4, &cfg)) {
-    const bool regular = C % kVec == 0 && aligned16(dy) && aligned16(y) && aligned16(dx);
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
