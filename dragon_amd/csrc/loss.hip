@@ -292,11 +292,12 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_ce_rows(
     s = Tile::reduce(s, SumOp(), slots[1]);
     const bool valid = target_valid(tgt, ignore_index, C);
     const int col = valid ? static_cast<int>(tgt) : -1;
+    const A inv = A(1) / s;  // fp32 multiplies by the reciprocal, as the softmax kernels do
 #pragma unroll
     for (int i = 0; i < kVPT; ++i)
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        t.v[i][e] = t.v[i][e] / s;
+        t.v[i][e] = sizeof(A) == 4 ? t.v[i][e] * inv : t.v[i][e] / s;
         if ((i * kTPR + Tile::lane()) * kVec + e == col) {
           loss[row] = neg_log_clamped(t.v[i][e]);
           mask[row] = T(1);
@@ -305,6 +306,73 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_ce_rows(
     if (!valid && Tile::lane() == 0) loss[row] = mask[row] = T(0);
     t.store(prob + row * C, npackets);
     if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// The same for rows that take a whole 1024-thread workgroup: persistent
+// workgroups that request the next row's packets before reducing the current
+// one (see softmax_wide_rows).
+template <typename T, typename TargetT, int kVPT>
+__global__ __launch_bounds__(1024) void softmax_ce_wide_rows(
+    const int64_t N, const int C, const int64_t ignore_index, const T* __restrict__ x,
+    const TargetT* __restrict__ target, T* __restrict__ prob, T* __restrict__ loss,
+    T* __restrict__ mask) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const int npackets = C / kVec;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  Raw cur;
+  cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    const bool more = row + stride < N;
+    nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
+    const TargetT tgt = target[row];
+    Tile t;
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      cur.unpack(i, t.v[i]);
+      const bool on = Tile::active(i, npackets);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = on ? t.v[i][e] : acc_neg_inf<A>();  // raw padding is zero bits
+        m = MaxOp()(m, t.v[i][e]);
+      }
+    }
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = acc_exp(t.v[i][e] - m);
+        s += t.v[i][e];
+      }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    const bool valid = target_valid(tgt, ignore_index, C);
+    const int col = valid ? static_cast<int>(tgt) : -1;
+    const A inv = A(1) / s;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = sizeof(A) == 4 ? t.v[i][e] * inv : t.v[i][e] / s;
+        if ((i * kTPR + static_cast<int>(threadIdx.x)) * kVec + e == col) {
+          loss[row] = neg_log_clamped(t.v[i][e]);
+          mask[row] = T(1);
+        }
+      }
+    if (!valid && threadIdx.x == 0) loss[row] = mask[row] = T(0);
+    nxt.wait_ready();
+    cur = nxt;
+    t.store(prob + row * C, npackets);
+    __syncthreads();  // slots are reused by the next row
   }
 }
 
@@ -331,13 +399,25 @@ __global__ __launch_bounds__(kLossThreads) void softmax_ce_backward(
     }
     if constexpr (kAlongC) {
       const int64_t n = i / C, k0 = i - n * C;
-      const TargetT tgt = target[n];
-      const bool valid = target_valid(tgt, ignore_index, C);
-      const A w = valid ? (kPerPosition ? static_cast<A>(dl[n]) : alpha) : A(0);
+      if (k0 + kVec <= C) {  // the packet lies within one row
+        const TargetT tgt = target[n];
+        const bool valid = target_valid(tgt, ignore_index, C);
+        const A w = valid ? (kPerPosition ? static_cast<A>(dl[n]) : alpha) : A(0);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A hot = (valid && k0 + e == static_cast<int64_t>(tgt)) ? A(1) : A(0);
-        v[e] = (v[e] - hot) * w;
+        for (int e = 0; e < kVec; ++e) {
+          const A hot = (valid && k0 + e == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+          v[e] = (v[e] - hot) * w;
+        }
+      } else {  // C is not a multiple of the packet: this one straddles rows
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const int64_t ne = (i + e) / C, ke = (i + e) - ne * C;
+          const TargetT tgt = target[ne];
+          const bool valid = target_valid(tgt, ignore_index, C);
+          const A w = valid ? (kPerPosition ? static_cast<A>(dl[ne]) : alpha) : A(0);
+          const A hot = (valid && ke == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+          v[e] = (v[e] - hot) * w;
+        }
       }
     } else {
       const int64_t n = i / (C * S);
@@ -500,6 +580,18 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
   RowConfig cfg;
   if (S == 1 && pick_row_config(ceil_div(C, kVec), 8, &cfg)) {
     const bool regular = C % kVec == 0 && aligned16(x) && aligned16(prob);  // else ragged tiles
+    if (regular && cfg.tpr == 1024) {
+#define LAUNCH_WIDE(VPT)                                                                        \
+  {                                                                                             \
+    auto kernel = softmax_ce_wide_rows<T, TargetT, VPT>;                                        \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                   \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C),       \
+                       ignore_index, xp, tp, pp, loss, mask);                                   \
+  }
+      if (cfg.vpt == 2) LAUNCH_WIDE(2) else if (cfg.vpt == 4) LAUNCH_WIDE(4) else LAUNCH_WIDE(8)
+#undef LAUNCH_WIDE
+    } else {
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
@@ -514,6 +606,7 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
+    }
   } else {
     const int st = dragon_hip_softmax(sizeof(T) == 8 ? DRAGON_HIP_F64 : DRAGON_HIP_F32, N, S, C, x, prob, stream);
     if (st != DRAGON_HIP_OK) return st;
@@ -576,7 +669,7 @@ int launch_fused_backward(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
   hipLaunchKernelGGL((softmax_ce_backward<T, TargetT, VEC, ALONG_C, PER_POS>),                 \
                      dim3(loss_grid(total / VEC)), dim3(kLossThreads), 0, stream, total / VEC, \
                      S, C, ignore_index, pp, tp, dlp, scalar, dp)
-  if (S == 1 && C % kVec == 0 && aligned) {
+  if (S == 1 && total % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, true, true); else LAUNCH(kVec, true, false);
   } else if (S > 1 && S % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, false, true); else LAUNCH(kVec, false, false);

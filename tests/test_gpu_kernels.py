@@ -618,6 +618,8 @@ def test_sum_of_a_large_vector_and_empty_reduction(K):
 
 SCE_SHAPES = [((64, 512), -1), ((10, 1000), -1), ((5, 37), -1), ((6, 4096), -1), ((3, 7, 5), 1),
               ((2, 19, 8, 8), 1), ((4, 1), -1), ((3, 40000), -1), ((2, 6, 16), 1),
+              # 1024-thread rows (prefetching forward); packets that straddle rows in the backward
+              ((4, 20000), -1), ((3, 6000), -1), ((8, 1001), -1),
               # more than 16384 positions: the two-stage loss reductions
               ((70000, 8), -1), ((2, 5, 40000), 1)]
 
