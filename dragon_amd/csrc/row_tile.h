@@ -195,6 +195,26 @@ struct RawRowTile {
       p[s] = on ? t : z;
     }
   }
+  // Rows of any width at element-aligned addresses: whole packets with one
+  // unaligned access, the row's last partial packet element by element.
+  // Elements beyond the row hold zero bits.
+  __device__ __forceinline__ void load_any(const T* row, int ncols, bool valid = true) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int col = (s * kTPR + lane()) * kVec;
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      if (valid && col + kVec <= ncols) {
+        p[s] = load_packet_unaligned(row + col);
+      } else if (valid && col < ncols) {
+        A v[kVec];
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = col + e < ncols ? IO<T>::load1(row + col + e) : A(0);
+        p[s] = IO<T>::pack(v);
+      } else {
+        p[s] = z;
+      }
+    }
+  }
   __device__ __forceinline__ void unpack(int s, A (&v)[kVec]) const { IO<T>::unpack(p[s], v); }
   // Called between two passes over the tile: makes the compiler treat the
   // packets as new values, so it converts them again in the next pass instead

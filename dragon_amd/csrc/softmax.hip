@@ -222,6 +222,92 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
   }
 }
 
+// Rows of up to 16384 packets (a 128K-entry 16-bit or a 64K-entry fp32
+// vocabulary): sixteen raw packets per thread of a 1024-thread workgroup, any
+// width and alignment. One read of x; fp32 / fp64 packets keep the
+// exponentials in place, 16-bit packets evaluate them twice.
+template <typename T, int kKind, bool kRagged>
+__global__ __launch_bounds__(1024) void softmax_huge_rows(const int64_t N, const int C, const T* x,
+                                                          T* y) {
+  constexpr int kTPR = 1024, kVPT = 16;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Raw::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Raw::kVec;
+  constexpr bool kKeepExp = kKind == kSoftmax && sizeof(T) == sizeof(A);
+  __shared__ A slots[2][kTPR / kWaveSize];
+  const int lane = threadIdx.x;
+  for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
+    Raw t;
+    if (kRagged) {
+      t.load_any(x + row * C, C);
+    } else {
+      t.load(x + row * C, C / kVec);
+    }
+    // whether element e of slot i lies inside the row (regular rows: whole packets)
+    auto inside = [&](int i, int e) {
+      const int col = (i * kTPR + lane) * kVec;
+      return kRagged ? col + e < C : col < C;
+    };
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      t.unpack(i, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (inside(i, e)) m = MaxOp()(m, v[e]);
+      }
+    }
+    m = block_allreduce<kTPR / kWaveSize>(m, MaxOp(), slots[0]);
+    t.refresh();
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      t.unpack(i, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        v[e] = inside(i, e) ? M::exp_of(v[e] - m) : A(0);
+        s += v[e];
+      }
+      if (kKeepExp) t.p[i] = IO<T>::pack(v);
+    }
+    s = block_allreduce<kTPR / kWaveSize>(s, SumOp(), slots[1]);
+    t.refresh();
+    const A inv = A(1) / s;
+    const A l = acc_log(s);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int col = (i * kTPR + lane) * kVec;
+      if (col < C) {
+        A v[kVec];
+        t.unpack(i, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (kKeepExp) {
+            v[e] = M::normalise(v[e], s, inv);
+          } else {
+            const A d = v[e] - m;
+            v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), s, inv) : d - l;
+          }
+        }
+        if (!kRagged) {
+          store_packet(y + row * C + col, IO<T>::pack(v));
+        } else if (col + kVec <= C) {
+          store_packet_unaligned(y + row * C + col, IO<T>::pack(v));
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (col + e < C) IO<T>::store1(y + row * C + col + e, v[e]);
+          }
+        }
+      }
+    }
+    __syncthreads();  // slots are reused by the next row
+  }
+}
+
 // The gradient for 1024-thread rows: dy and y as raw packets, the next row
 // prefetched where two rows of packets fit the registers (kPrefetch).
 template <typename T, int kKind, int kVPT, bool kPrefetch>
@@ -612,6 +698,12 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
+  } else if (S == 1 && sizeof(T) <= 4 && ceil_div(C, kVec) <= 16 * 1024) {
+    const bool regular = C % kVec == 0 && aligned16(x) && aligned16(y);
+    auto kernel = regular ? softmax_huge_rows<T, kKind, false> : softmax_huge_rows<T, kKind, true>;
+    const unsigned resident = resident_grid(kernel, 1024, 0);
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), xp, yp);
   } else if (S == 1) {
     hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
                        stream, N, C, xp, yp);
