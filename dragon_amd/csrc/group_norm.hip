@@ -22,7 +22,13 @@
 //          accumulated per thread across the rows a workgroup visits, combined
 //          through LDS, written as one partial row per workgroup, and summed
 //          by a second small kernel (two-stage, no atomics).
-//   general  three split reductions / one flat map, any layout, any alignment.
+//   groups (NCHW, a group fits a register tile): fused forward for any S;
+//          fused backward when channels span whole wavefronts of packets.
+//   general  one pass over x and dy for the per-(n, c) pairs
+//          (sum dy*(x - mu), sum dy): rows of S elements (NCHW) or column
+//          reductions of each sample's [S, C] matrix (NHWC); ds/db and
+//          dgamma/dbeta from those N*C pairs; one flat map for dx. Any layout,
+//          any alignment.
 #include <cstdlib>
 
 #include "reduce.h"
@@ -84,83 +90,8 @@ struct GroupNormApply {
 };
 
 // --------------------------------------------------------------------------
-// General backward: ds/db per group, dgamma/dbeta per channel, then dx
+// General backward: the last step, dx from the per-group and per-row scalars
 // --------------------------------------------------------------------------
-template <typename T>
-struct InternalGradAccum {  // segments over one (n, g)
-  using A = typename IO<T>::Acc;
-  GroupShape sh;
-  const A* gamma;
-  uint32_t g;
-  __device__ __forceinline__ void begin(uint32_t o, uint32_t) { g = o % sh.G; }
-  template <int V>
-  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t p, uint32_t, const A (&x)[V],
-                                      const A (&dy)[V], A& a, A& b) const {
-    if (sh.nchw) {
-      const A w = gamma[g * sh.D + p / sh.S];  // packet within one channel
-#pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const A t = w * dy[e];
-        a += t * x[e];
-        b += t;
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const A t = gamma[g * sh.D + p + e] * dy[e];
-        a += t * x[e];
-        b += t;
-      }
-    }
-  }
-};
-
-template <typename A>
-struct StorePairEpilogue {
-  A* out_a;
-  A* out_b;
-  __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
-    out_a[o] = a;
-    out_b[o] = b;
-  }
-};
-
-template <typename T>
-struct WGradAccumNCHW {  // segments: output c, segment n
-  using A = typename IO<T>::Acc;
-  GroupShape sh;
-  const A* mu;
-  const A* rsig;
-  uint32_t g;
-  __device__ __forceinline__ void begin(uint32_t c, uint32_t) { g = c / sh.D; }
-  template <int V>
-  __device__ __forceinline__ void add(uint32_t, uint32_t n, uint32_t, uint32_t, const A (&x)[V],
-                                      const A (&dy)[V], A& a, A& b) const {
-    const uint32_t ng = n * sh.G + g;
-    const A m = mu[ng], r = rsig[ng];
-#pragma unroll
-    for (int e = 0; e < V; ++e) {
-      a += dy[e] * (x[e] - m) * r;
-      b += dy[e];
-    }
-  }
-};
-
-template <typename T>
-struct WGradAccumNHWC {  // columns: rows = N*S, cols = C
-  using A = typename IO<T>::Acc;
-  GroupShape sh;
-  const A* mu;
-  const A* rsig;
-  uint32_t g;
-  __device__ __forceinline__ void begin(uint32_t c, uint32_t) { g = c / sh.D; }
-  __device__ __forceinline__ void add(uint32_t r, uint32_t, uint32_t, A x, A dy, A& a, A& b) const {
-    const uint32_t ng = (r / sh.S) * sh.G + g;
-    a += dy * (x - mu[ng]) * rsig[ng];
-    b += dy;
-  }
-};
-
 template <typename T, int kVec>
 struct GroupNormGradApply {
   using A = typename IO<T>::Acc;
@@ -1078,21 +1009,10 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   const RowGradPlan rp = plan_row_grad<T>(N, G, D, S);
   if (rp.use_rows) return static_cast<size_t>(rp.grid) * D * 2 * sizeof(A);
   const int64_t C = G * D;
-  const uint32_t split_g = pick_split(N * G, D * S);
-  size_t bytes = static_cast<size_t>(N) * G * split_g * 2 * sizeof(A);
-  const uint32_t split_c = layout == DRAGON_HIP_NCHW
-      ? pick_split(C, N * S)
-      : column_split_bound(N * S, C);
-  const size_t wbytes = static_cast<size_t>(C) * split_c * 2 * sizeof(A);
-  if (wbytes > bytes) bytes = wbytes;
-  if (layout == DRAGON_HIP_NCHW) {  // per-(n, c) pairs of the fused and the general path
-    const size_t fbytes = static_cast<size_t>(N) * C * 2 * sizeof(A);
-    if (fbytes > bytes) bytes = fbytes;
-  } else {  // stage-one partial pairs, then the per-(n, c) pairs
-    const size_t fbytes = (batched_partial_pairs(N, S, C) + static_cast<size_t>(N) * C) * 2 * sizeof(A);
-    if (fbytes > bytes) bytes = fbytes;
-  }
-  return bytes;
+  // per-(n, c) pairs of the fused and the general path; NHWC adds the stage-one partial pairs
+  size_t pairs = static_cast<size_t>(N) * C;
+  if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
+  return pairs * 2 * sizeof(A);
 }
 
 // Fused forward: true when the register-resident kernel was launched.
