@@ -145,7 +145,8 @@ struct GroupNormGradApply {
 
 // Two 512-thread workgroups share a compute unit (128 registers per thread):
 // while one waits for its rows the other computes, which a single 1024-thread
-// workgroup with its barriers cannot do. gamma is staged in LDS once per
+// workgroup with its barriers cannot do. Rows of 1025 to 1536 packets take a
+// 768-thread workgroup (two packets per thread, no idle lanes, 168 registers). gamma is staged in LDS once per
 // (persistent) workgroup; x and dy of a row are kept as raw packets;
 // dgamma / dbeta are accumulated per thread across the rows the workgroup
 // visits, combined across its row groups through LDS, and written as one
@@ -155,7 +156,7 @@ struct GroupNormGradApply {
 //   xc = x - mu;  w = dy*rsig;  dgamma += w*xc;  dbeta += dy;
 //   dx = gamma*w + (a*xc + b)
 template <typename T, int kTPR, int kVPT, int kGradThreads>
-__global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
+__global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void layer_norm_grad_rows(
     const int64_t N, const int C, const T* __restrict__ x, const T* __restrict__ dy,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
     const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
@@ -170,6 +171,10 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
   // A round of the final cross-group combine moves kChunk (dgamma, dbeta) pairs per thread.
   constexpr int kChunk = kVec < 4 ? kVec : 4;
   constexpr int kRedWords = kGroups > 1 ? (kGroups - 1) * kTPR * kChunk * 2 : 1;
+  // Rows requested ahead of the current one: two where three rows of raw
+  // packets and the accumulators fit the register budget (128 per thread; 168
+  // for the 768-thread workgroup, which runs three wavefronts per SIMD).
+  constexpr int kDepth = (kVPT * kVec <= 8 || kGradThreads == 768) ? 2 : 1;
   extern __shared__ u32x4 staged[];  // gamma[C]
   __shared__ A slots[2 * Tile::kSlots];
   __shared__ A red[kRedWords];
@@ -190,9 +195,10 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
 #pragma unroll
     for (int e = 0; e < kVec; ++e) dg[i][e] = dbt[i][e] = A(0);
 
-  // The next row's packets are requested before the current row is reduced, so
-  // its HBM latency hides behind this row's arithmetic. Uniform trip count
-  // across the workgroup: the row reductions hold barriers.
+  // The packets of the next kDepth rows are requested before the current row
+  // is reduced, so their HBM latency hides behind this row's arithmetic and
+  // enough bytes stay in flight per compute unit. Uniform trip count across the
+  // workgroup: the row reductions hold barriers.
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
   int64_t row = static_cast<int64_t>(blockIdx.x) * kGroups + sub;
   // Rows past the end are clamped to row 0 for addressing and masked off.
@@ -201,15 +207,27 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
   tdy.load(dy + (row < N ? row : 0) * C, npackets, row < N);
   A m = mu[row < N ? row : 0];
   A r = rsig[row < N ? row : 0];
+  Raw px[kDepth], pdy[kDepth];  // rows row + stride .. row + kDepth * stride
+  A pm[kDepth], pr[kDepth];
+#pragma unroll
+  for (int k = 0; k + 1 < kDepth; ++k) {
+    const int64_t ahead = row + (k + 1) * stride;
+    const bool ok = ahead < N;
+    px[k].load(x + (ok ? ahead : 0) * C, npackets, ok);
+    pdy[k].load(dy + (ok ? ahead : 0) * C, npackets, ok);
+    pm[k] = mu[ok ? ahead : 0];
+    pr[k] = rsig[ok ? ahead : 0];
+  }
   for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N; base += stride) {
     const bool valid = row < N;
-    const int64_t next = row + stride;
-    const bool next_valid = next < N;
-    Raw nx, ndy;
-    nx.load(x + (next_valid ? next : 0) * C, npackets, next_valid);
-    ndy.load(dy + (next_valid ? next : 0) * C, npackets, next_valid);
-    const A nm = mu[next_valid ? next : 0];
-    const A nr = rsig[next_valid ? next : 0];
+    {
+      const int64_t far = row + kDepth * stride;
+      const bool ok = far < N;
+      px[kDepth - 1].load(x + (ok ? far : 0) * C, npackets, ok);
+      pdy[kDepth - 1].load(dy + (ok ? far : 0) * C, npackets, ok);
+      pm[kDepth - 1] = mu[ok ? far : 0];
+      pr[kDepth - 1] = rsig[ok ? far : 0];
+    }
 
     A s1 = A(0), s2 = A(0);
 #pragma unroll
@@ -259,9 +277,10 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
       }
       out[i] = IO<T>::pack(xv);
     }
-    // Wait for the prefetched row here, before this row's stores are issued.
-    nx.wait_ready();
-    ndy.wait_ready();
+    // Wait for the next row here, before this row's stores are issued (the
+    // rows requested after it stay in flight).
+    px[0].wait_ready();
+    pdy[0].wait_ready();
     T* dxr = dx + (valid ? row : 0) * C;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
@@ -270,7 +289,11 @@ __global__ __launch_bounds__(kGradThreads, 4) void layer_norm_grad_rows(
       }
     }
     if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
-    tx = nx, tdy = ndy, m = nm, r = nr, row = next;
+    tx = px[0], tdy = pdy[0], m = pm[0], r = pr[0], row += stride;
+#pragma unroll
+    for (int k = 0; k + 1 < kDepth; ++k) {
+      px[k] = px[k + 1], pdy[k] = pdy[k + 1], pm[k] = pm[k + 1], pr[k] = pr[k + 1];
+    }
   }
 
   // Combine the kGroups row groups of this workgroup, kChunk pairs at a time.
@@ -502,12 +525,24 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
   const uint32_t packets_per_chan = S / kVec;
   const A denom = A(1) / A(L);
   const int lane = threadIdx.x;
-  const int wave = threadIdx.x / kWaveSize;
+  // Uniform over the wavefront, so everything indexed by it (the channel of a
+  // slot, its gamma) stays in scalar registers.
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kWaveSize));
 
+  // A workgroup fills the compute unit's registers, so the next group cannot be
+  // held beside the current one: its packets are requested slot by slot into the
+  // registers the second pass has just finished with, and are in flight while
+  // the rest of this group is computed, stored and reduced.
+  Raw tx, tdy;
+  if (blockIdx.x < rows) {
+    tx.load(x + static_cast<int64_t>(blockIdx.x) * L, npackets);
+    tdy.load(dy + static_cast<int64_t>(blockIdx.x) * L, npackets);
+  }
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    Raw tx, tdy;
-    tx.load(x + row * L, npackets);
-    tdy.load(dy + row * L, npackets);
+    const int64_t next = row + gridDim.x;
+    const bool next_valid = next < rows;
+    const T* nx = x + (next_valid ? next : row) * L;
+    const T* ndy = dy + (next_valid ? next : row) * L;
     const A m = mu[row], r = rsig[row];
     const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
 
@@ -515,8 +550,10 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     A s1 = A(0), s2 = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      const uint32_t chan = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) / packets_per_chan;
-      gam[i] = Tile::active(i, npackets) ? gamma[c0 + chan] : A(0);
+      // Slots beyond the group hold dy = 0 and take the last channel's gamma.
+      uint32_t chan = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) / packets_per_chan;
+      chan = chan < D ? chan : D - 1;
+      gam[i] = gamma[c0 + chan];
       A xv[kVec], dv[kVec];
       tx.unpack(i, xv);
       tdy.unpack(i, dv);
@@ -550,6 +587,10 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
         xv[e] = gam[i] * dv[e] * r + (u0 * xc - v0) * denom;
       }
       if (Tile::active(i, npackets)) tx.store_slot(dx + row * L, i, xv);
+      if (next_valid) {
+        tx.load_slot(nx, i, npackets);
+        tdy.load_slot(ndy, i, npackets);
+      }
       t1 = wave_allreduce(t1, SumOp());
       t2 = wave_allreduce(t2, SumOp());
       if ((threadIdx.x & (kWaveSize - 1)) == 0) {
@@ -965,8 +1006,8 @@ RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
   if (D % kVec != 0 || static_cast<size_t>(D) * sizeof(typename IO<T>::Acc) > kMaxStagedParamBytes / 2) {
     return p;
   }
-  static const RowConfig table[] = {{64, 1},  {64, 2},  {256, 1},  {256, 2}, {512, 1},
-                                    {512, 2}, {1024, 1}, {1024, 2}, {1024, 4}};
+  static const RowConfig table[] = {{64, 1},  {64, 2},  {256, 1},  {256, 2},  {512, 1},
+                                    {512, 2}, {1024, 1}, {768, 2}, {1024, 2}, {1024, 4}};
   bool found = false;
   for (const RowConfig& c : table) {
     if (!found && c.vpt <= kMaxVpt && D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
@@ -975,7 +1016,7 @@ RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
     }
   }
   if (!found) return p;
-  p.threads = p.cfg.tpr == 1024 ? 1024 : 512;
+  p.threads = p.cfg.tpr >= 768 ? p.cfg.tpr : 512;
   const int per_cu = p.threads == 512 ? 2 : 1;
   const int64_t groups = p.threads / p.cfg.tpr;
   const int64_t want = ceil_div(N, groups);
@@ -1119,8 +1160,8 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 #define LAUNCH(TPR, VPT)                                                    \
   {                                                                         \
     if constexpr (VPT * IO<T>::kVec <= 16 || sizeof(A) == 8) {              \
-      if constexpr (TPR == 1024) {                                          \
-        LAUNCH_T(TPR, VPT, 1024)                                            \
+      if constexpr (TPR >= 768) {                                           \
+        LAUNCH_T(TPR, VPT, TPR)                                             \
       } else {                                                              \
         LAUNCH_T(TPR, VPT, 512)                                             \
       }                                                                     \
@@ -1133,6 +1174,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 1) LAUNCH(512, 1)
     else if (rp.cfg.tpr == 512 && rp.cfg.vpt == 2) LAUNCH(512, 2)
     else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 1) LAUNCH(1024, 1)
+    else if (rp.cfg.tpr == 768 && rp.cfg.vpt == 2) LAUNCH(768, 2)
     else if (rp.cfg.tpr == 1024 && rp.cfg.vpt == 2) LAUNCH(1024, 2)
     else LAUNCH(1024, 4)
 #undef LAUNCH_T

@@ -72,6 +72,15 @@ struct RowTile {
   // loads in flight is static, and the compiler can wait for exactly the ones a
   // computation needs instead of draining the queue. `row` must point to
   // readable memory even when `valid` is false.
+  // Rows that fill the tile exactly (npackets == kMaxPackets): no slot is masked,
+  // so no select is spent on the fill value.
+  __device__ __forceinline__ void load_full(const T* row) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      load_unpack<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
+    }
+  }
+
   __device__ __forceinline__ void load(const T* row, int npackets, A fill, bool valid = true) {
     if constexpr (kRagged) {
       load_ragged(row, npackets, fill, valid);
@@ -194,6 +203,14 @@ struct RawRowTile {
       const u32x4 z = {0u, 0u, 0u, 0u};
       p[s] = on ? t : z;
     }
+  }
+  // One slot of load().
+  __device__ __forceinline__ void load_slot(const T* row, int s, int npackets) {
+    const bool on = active(s, npackets);
+    const int packet = on ? s * kTPR + lane() : 0;
+    const u32x4 t = load_packet(row + static_cast<int64_t>(packet) * kVec);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    p[s] = on ? t : z;
   }
   // Rows of any width at element-aligned addresses: whole packets with one
   // unaligned access, the row's last partial packet element by element.

@@ -53,7 +53,7 @@ struct SoftmaxMath {
 
 enum SoftmaxKind { kSoftmax = 0, kLogSoftmax = 1 };
 
-template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
+template <typename T, int kKind, int kTPR, int kVPT, bool kRagged, bool kFull = false>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
     const int64_t N, const int C, const T* x, T* y) {
   using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
@@ -66,7 +66,11 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
     Tile t;
-    t.load(x + row * C, npackets, acc_neg_inf<A>());
+    if constexpr (kFull) {
+      t.load_full(x + row * C);  // the row fills the tile: nothing to mask
+    } else {
+      t.load(x + row * C, npackets, acc_neg_inf<A>());
+    }
 
     A m = acc_neg_inf<A>();
 #pragma unroll
@@ -688,7 +692,10 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, hipS
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
     const dim3 grid(row_grid(N, Tile::kRowsPerBlock)), block(Tile::kThreads);                \
-    if (regular) {                                                                           \
+    if (regular && C / kVec == TPR * VPT) {                                                  \
+      hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT, false, true>), grid, block, 0,    \
+                         stream, N, static_cast<int>(C), xp, yp);                            \
+    } else if (regular) {                                                                    \
       hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT, false>), grid, block, 0, stream, N, \
                          static_cast<int>(C), xp, yp);                                       \
     } else {                                                                                 \
