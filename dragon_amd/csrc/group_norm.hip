@@ -201,10 +201,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   // workgroup: the row reductions hold barriers.
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
   int64_t row = static_cast<int64_t>(blockIdx.x) * kGroups + sub;
-  // Rows past the end are clamped to row 0 for addressing and masked off.
+  // Rows past the end are clamped to row 0 for addressing; neither they nor the
+  // slots beyond the row are zero-filled (no selects on the loaded packets):
+  // such rows skip the second pass, and such slots only ever feed accumulators
+  // of columns that are not written out.
   Raw tx, tdy;
-  tx.load(x + (row < N ? row : 0) * C, npackets, row < N);
-  tdy.load(dy + (row < N ? row : 0) * C, npackets, row < N);
+  tx.load_unmasked(x + (row < N ? row : 0) * C, npackets);
+  tdy.load_unmasked(dy + (row < N ? row : 0) * C, npackets);
   A m = mu[row < N ? row : 0];
   A r = rsig[row < N ? row : 0];
   Raw px[kDepth], pdy[kDepth];  // rows row + stride .. row + kDepth * stride
@@ -213,8 +216,8 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   for (int k = 0; k + 1 < kDepth; ++k) {
     const int64_t ahead = row + (k + 1) * stride;
     const bool ok = ahead < N;
-    px[k].load(x + (ok ? ahead : 0) * C, npackets, ok);
-    pdy[k].load(dy + (ok ? ahead : 0) * C, npackets, ok);
+    px[k].load_unmasked(x + (ok ? ahead : 0) * C, npackets);
+    pdy[k].load_unmasked(dy + (ok ? ahead : 0) * C, npackets);
     pm[k] = mu[ok ? ahead : 0];
     pr[k] = rsig[ok ? ahead : 0];
   }
@@ -223,8 +226,8 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     {
       const int64_t far = row + kDepth * stride;
       const bool ok = far < N;
-      px[kDepth - 1].load(x + (ok ? far : 0) * C, npackets, ok);
-      pdy[kDepth - 1].load(dy + (ok ? far : 0) * C, npackets, ok);
+      px[kDepth - 1].load_unmasked(x + (ok ? far : 0) * C, npackets);
+      pdy[kDepth - 1].load_unmasked(dy + (ok ? far : 0) * C, npackets);
       pm[kDepth - 1] = mu[ok ? far : 0];
       pr[kDepth - 1] = rsig[ok ? far : 0];
     }
@@ -256,26 +259,25 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     tx.refresh();
     tdy.refresh();
     u32x4 out[kVPT];
+    if (valid) {  // uniform over the wavefront
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i) {
-      A xv[kVec], dv[kVec], g[kVec];
-      tx.unpack(i, xv);
-      tdy.unpack(i, dv);
-      if (Tile::active(i, npackets)) {
-        load_params<kVec>(lds_gamma + (i * kTPR + lane) * kVec, g);
-      } else {
+      for (int i = 0; i < kVPT; ++i) {
+        A xv[kVec], dv[kVec], g[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
+        // A slot beyond the row reads gamma of column 0 .. kVec - 1: its dx is not stored.
+        const int col = Tile::active(i, npackets) ? (i * kTPR + lane) * kVec : 0;
+        load_params<kVec>(lds_gamma + col, g);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) g[e] = A(0);
+        for (int e = 0; e < kVec; ++e) {
+          const A xc = xv[e] - m;
+          const A w = dv[e] * r;
+          dg[i][e] += w * xc;
+          dbt[i][e] += dv[e];
+          xv[e] = g[e] * w + (a * xc + b);
+        }
+        out[i] = IO<T>::pack(xv);
       }
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A xc = xv[e] - m;
-        const A w = dv[e] * r;
-        dg[i][e] += w * xc;  // masked slots hold dy = 0: they add nothing
-        dbt[i][e] += dv[e];
-        xv[e] = g[e] * w + (a * xc + b);
-      }
-      out[i] = IO<T>::pack(xv);
     }
     // Wait for the next row here, before this row's stores are issued (the
     // rows requested after it stay in flight).

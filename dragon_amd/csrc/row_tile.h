@@ -204,6 +204,15 @@ struct RawRowTile {
       p[s] = on ? t : z;
     }
   }
+  // load() without the zero fill: inactive slots (and every slot when `valid`
+  // is false) hold packet 0 of `row`, for kernels that mask at the point of use.
+  __device__ __forceinline__ void load_unmasked(const T* row, int npackets) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int packet = active(s, npackets) ? s * kTPR + lane() : 0;
+      p[s] = load_packet(row + static_cast<int64_t>(packet) * kVec);
+    }
+  }
   // One slot of load().
   __device__ __forceinline__ void load_slot(const T* row, int s, int npackets) {
     const bool on = active(s, npackets);
