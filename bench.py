@@ -220,8 +220,7 @@ def wl_batch_norm(shape, dtype_name, seed=2):
     nbytes = x.numel() * x.element_size()
 
     def backward():
-        K.batch_norm_wgrad(N, C, S, "NCHW", x, mu, rsig, dy, wg, wg)
-        K.batch_norm_training_grad(N, C, S, float(N * S), "NCHW", x, mu, rsig, g, wg, wg, dy, dx)
+        K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", x, mu, rsig, g, dy, wg, wg, dx)
 
     kernels = [
         ("batch_norm_training_forward",

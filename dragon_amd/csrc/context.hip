@@ -16,6 +16,8 @@ const char* dragon_hip_status_string(int status) {
     case DRAGON_HIP_EDTYPE: return "unsupported dtype";
     case DRAGON_HIP_ESCRATCH: return "scratch buffer missing or too small";
     case DRAGON_HIP_ENODEVICE: return "no HIP device";
+    case DRAGON_HIP_ETIMEOUT:
+      return "an earlier single-read BatchNorm launch gave up waiting for partial sums";
     default: break;
   }
   if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -178,6 +178,17 @@ namespace kernels {
     HIP_CHECK(dragon_hip_batch_norm_training_forward(                                             \
         Tag<T>(), N, C, S, layout, momentum, epsilon, x, gamma, beta, running_mean, running_var,  \
         mu, rsig, params, y, Scratch(ctx, bytes), bytes, ctx->hip_stream()));                     \
+  }                                                                                               \
+  template <>                                                                                     \
+  void BatchNormTrainingBackward<T, AccT, HIPContext>(                                            \
+      const int N, const int C, const int S, const float normalizer, const string& data_format,   \
+      const T* x, const AccT* mu, const AccT* rsig, const AccT* gamma, const T* dy, AccT* dgamma, \
+      AccT* dbeta, T* dx, HIPContext* ctx) {                                                      \
+    const int layout = LayoutTag(data_format);                                                    \
+    const size_t bytes = dragon_hip_batch_norm_reduce_scratch_bytes(Tag<T>(), N, C, S, layout);   \
+    HIP_CHECK(dragon_hip_batch_norm_training_backward(                                            \
+        Tag<T>(), N, C, S, normalizer, layout, x, mu, rsig, gamma, dy, dgamma, dbeta, dx,         \
+        Scratch(ctx, bytes), bytes, ctx->hip_stream()));                                          \
   }
 
 DEFINE_KERNEL_LAUNCHERS(float16, float);

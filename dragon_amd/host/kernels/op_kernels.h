@@ -5,10 +5,11 @@
 // specialised for HIPContext in kernels_hip.cc, where each specialisation is a
 // forward to the C-ABI entry point of the same name.
 //
-// Two additions have no counterpart among the reference's kernels:: functions:
-// GroupNormForward and BatchNormTrainingForward run a sequence an operator
-// body issues (Moments, InvStd, ... ) as one call, so that x is read once
-// where the device can keep the reduction unit on-die.
+// Three additions have no counterpart among the reference's kernels:: functions:
+// GroupNormForward, BatchNormTrainingForward and BatchNormTrainingBackward run
+// a sequence an operator body issues (Moments, InvStd, ... ; WGrad,
+// TrainingGrad) as one call, so that x (and dy) is read once where the device
+// can keep the reduction unit on-die.
 #pragma once
 
 #include "core/common.h"
@@ -171,6 +172,14 @@ void BatchNormTrainingForward(const int N, const int C, const int S, const strin
                               const AccT* gamma, const AccT* beta, AccT* running_mean,
                               AccT* running_var, AccT* mu, AccT* rsig, AccT* params, T* y,
                               Context* ctx);
+
+// BatchNormWGrad followed by BatchNormTrainingGrad (dgamma == dbeta means
+// dbeta = dgamma + C, as for the two kernels).
+template <typename T, typename AccT, class Context>
+void BatchNormTrainingBackward(const int N, const int C, const int S, const float normalizer,
+                               const string& data_format, const T* x, const AccT* mu,
+                               const AccT* rsig, const AccT* gamma, const T* dy, AccT* dgamma,
+                               AccT* dbeta, T* dx, Context* ctx);
 
 } // namespace kernels
 

@@ -95,7 +95,15 @@ void BatchNormGradientOp<Context>::RunTraining() {
   const int N = static_cast<int>(this->N_), C = static_cast<int>(this->C_), S = static_cast<int>(this->S_);
 
   // {dgamma, dbeta} packed in X_params, then copied out to the requested outputs.
-  kernels::BatchNormWGrad(N, C, S, data_format(), x, mu, rsig, dy, params, params, ctx());
+  // Without cross-rank statistics nothing separates the two kernels of the
+  // reference's body, so they run as one call that reads x and dy once.
+  if (dX->has_name()) {
+    kernels::BatchNormTrainingBackward(
+        N, C, S, static_cast<float>(this->N_ * this->S_), data_format(), x, mu, rsig, gamma, dy,
+        params, params, dX->template mutable_data<T, Context>(ctx()), ctx());
+  } else {
+    kernels::BatchNormWGrad(N, C, S, data_format(), x, mu, rsig, dy, params, params, ctx());
+  }
   if (dW->has_name()) {
     math::Copy(C, static_cast<const AccT*>(params),
                dW->Reshape({this->C_})->template mutable_data<AccT, Context>(ctx()), ctx());
@@ -103,12 +111,6 @@ void BatchNormGradientOp<Context>::RunTraining() {
   if (dB->has_name()) {
     math::Copy(C, static_cast<const AccT*>(params + C),
                dB->Reshape({this->C_})->template mutable_data<AccT, Context>(ctx()), ctx());
-  }
-  if (dX->has_name()) {
-    kernels::BatchNormTrainingGrad(
-        N, C, S, static_cast<float>(this->N_ * this->S_), data_format(), x, mu, rsig, gamma,
-        static_cast<const AccT*>(params), static_cast<const AccT*>(params), dy,
-        dX->template mutable_data<T, Context>(ctx()), ctx());
   }
 }
 

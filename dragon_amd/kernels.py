@@ -312,6 +312,27 @@ def batch_norm_training_forward(N, C, S, data_format, momentum, epsilon, x, gamm
           _ptr(params), _ptr(y), _ptr(ws), need, _stream())
 
 
+def batch_norm_training_backward(N, C, S, normalizer, data_format, x, mu, rsig, gamma, dy, dgamma,
+                                 dbeta, dx):
+    """BatchNormWGrad + BatchNormTrainingGrad in one call (x and dy read once where a
+    channel slice fits the registers)."""
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    ws, need = _bn_scratch(tag, N, C, S, lay, x.device)
+    _call("dragon_hip_batch_norm_training_backward", tag, N, C, S, normalizer, lay, _ptr(x),
+          _ptr(mu), _ptr(rsig), _ptr(gamma), _ptr(dy), _ptr(dgamma), _ptr(dbeta), _ptr(dx),
+          _ptr(ws), need, _stream())
+
+
+def exchange_timed_out():
+    """True when a single-read BatchNorm launch gave up waiting for its peers' partial sums."""
+    return bool(_lib.lib().dragon_hip_exchange_timed_out())
+
+
+def exchange_reset(patience=0):
+    """Clears the time-out state; ``patience`` polls per wait (0 = the default)."""
+    _lib.lib().dragon_hip_exchange_reset(int(patience))
+
+
 # ---------------------------------------------------------------- measurement
 
 def stream_probe(mode, src, dst, nbytes):

@@ -58,7 +58,9 @@ typedef enum {
   DRAGON_HIP_EINVAL = -1,   /* bad size, layout, null pointer or misalignment */
   DRAGON_HIP_EDTYPE = -2,   /* dtype not in dragon_hip_dtype                  */
   DRAGON_HIP_ESCRATCH = -3, /* scratch missing or too small                   */
-  DRAGON_HIP_ENODEVICE = -4 /* no gfx950 device visible                       */
+  DRAGON_HIP_ENODEVICE = -4, /* no gfx950 device visible                      */
+  DRAGON_HIP_ETIMEOUT = -5  /* an earlier single-read BatchNorm launch gave up
+                               waiting (dragon_hip_exchange_timed_out)         */
 } dragon_hip_status;
 
 /* Human-readable text for a status returned by any function below. */
@@ -353,6 +355,31 @@ int dragon_hip_batch_norm_training_forward(int dtype, int64_t N, int64_t C, int6
                                            void* running_mean, void* running_var, void* mu,
                                            void* rsig, void* params, void* y, void* scratch,
                                            size_t scratch_bytes, void* stream);
+
+/* BatchNormGradientOp::RunTraining body without sync,
+ * dragon/operators/normalization/batch_norm_op.cc:118-190: BatchNormWGrad ->
+ * BatchNormTrainingGrad in one call, so that x and dy are read once where a
+ * channel slice fits the registers. Writes dgamma, dbeta (AccT[C]; dgamma ==
+ * dbeta means dbeta = dgamma + C) and dx.
+ * Scratch size: dragon_hip_batch_norm_reduce_scratch_bytes. */
+int dragon_hip_batch_norm_training_backward(int dtype, int64_t N, int64_t C, int64_t S,
+                                            float normalizer, int layout, const void* x,
+                                            const void* mu, const void* rsig, const void* gamma,
+                                            const void* dy, void* dgamma, void* dbeta, void* dx,
+                                            void* scratch, size_t scratch_bytes, void* stream);
+
+/* The single-read path of the two training entry points above (NCHW, S a
+ * whole number of 16-byte packets) keeps the slices of a channel in the
+ * registers of several workgroups, which exchange partial sums inside one
+ * kernel and wait for each other, bounded. No counterpart in the reference.
+ * dragon_hip_exchange_timed_out: 1 when such a wait has given up since the
+ * last reset: the outputs of that launch are invalid, and the two entry points
+ * return DRAGON_HIP_ETIMEOUT until dragon_hip_exchange_reset is called.
+ * dragon_hip_exchange_reset: clears that state and sets how many polls (of
+ * about 0.2 us) a wait lasts; 0 = the default (about a second). The first use
+ * allocates four bytes of pinned host memory (do it before capturing a graph). */
+int dragon_hip_exchange_timed_out(void);
+void dragon_hip_exchange_reset(unsigned patience);
 
 /* ------------------------------------------------------------------------ */
 /* Measurement utility (no counterpart in the reference): a streaming read    */

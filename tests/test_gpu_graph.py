@@ -18,6 +18,13 @@ def _step(K, t):
     K.softmax_grad(N, 1, C, t["dy"], t["p"], t["dp"])
     K.batch_norm_training_forward(N, C, 1, "NCHW", 0.9, 1e-5, t["x32"], t["g"], t["b"], t["rm"],
                                   t["rv"], t["bmu"], t["brsig"], t["bparams"], t["by"])
+    # the same tensor as [8, 64, N*C/512]: the single-read path, several slices per channel
+    n, c = 8, 64
+    s = N * C // (n * c)
+    K.batch_norm_training_forward(n, c, s, "NCHW", 0.9, 1e-5, t["x32"], t["g64"], t["b64"], t["rm64"],
+                                  t["rv64"], t["cmu"], t["crsig"], t["cparams"], t["cy"])
+    K.batch_norm_training_backward(n, c, s, float(n * s), "NCHW", t["x32"], t["cmu"], t["crsig"],
+                                   t["g64"], t["cy"], t["cwg"], t["cwg"], t["cdx"])
 
 
 def _tensors(N, C):
@@ -31,6 +38,13 @@ def _tensors(N, C):
     t["g"].fill_(1.0)
     t["rv"].fill_(1.0)
     t["bparams"] = torch.empty(2 * C, device=dev)
+    for k in ("cy", "cdx"):
+        t[k] = torch.empty((N, C), device=dev)
+    for k in ("g64", "rv64"):
+        t[k] = torch.ones(64, device=dev)
+    for k in ("b64", "rm64", "cmu", "crsig"):
+        t[k] = torch.zeros(64, device=dev)
+    t["cparams"], t["cwg"] = torch.empty(128, device=dev), torch.empty(128, device=dev)
     t["mu"], t["rsig"] = torch.empty(N, device=dev), torch.empty(N, device=dev)
     t["params"] = torch.empty(2 * N, device=dev)
     return t
@@ -59,10 +73,11 @@ def test_entry_points_replay_from_a_captured_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         _step(K, t)
-    outs = ("y", "dx", "dg", "db", "p", "dp", "by", "bmu", "brsig")
+    outs = ("y", "dx", "dg", "db", "p", "dp", "by", "bmu", "brsig", "cy", "cmu", "crsig", "cdx", "cwg")
     for _ in range(3):
         refill()
         rm0, rv0 = t["rm"].clone(), t["rv"].clone()
+        rm1, rv1 = t["rm64"].clone(), t["rv64"].clone()
         graph.replay()
         torch.cuda.synchronize()
         got = {k: t[k].float().cpu().numpy().copy() for k in outs}
@@ -70,6 +85,8 @@ def test_entry_points_replay_from_a_captured_graph():
         # the same step eagerly from the same inputs and running statistics
         t["rm"].copy_(rm0)
         t["rv"].copy_(rv0)
+        t["rm64"].copy_(rm1)
+        t["rv64"].copy_(rv1)
         for k in outs:
             t[k].zero_()
         _step(K, t)

@@ -310,8 +310,12 @@ def test_group_norm_forward_backward(K, shape, axis, group, dtype, fused):
 
 # ---------------------------------------------------------------- BatchNorm
 
+# The NCHW shapes from (8, 40, 56, 56) on take the single-read path with several slices per
+# channel: 6 slices in one round of work items; 1100 single-slice channels over two rounds;
+# 5 slices per channel over two rounds, with channels that straddle the round boundary.
 BN_CASES = [((8, 16, 7, 7), 1), ((4, 3, 2), 1), ((16, 32), -1), ((4, 5, 5, 24), -1),
-            ((6, 64, 28, 28), 1), ((4, 2, 3), -1), ((3, 130, 4), 1), ((50, 70), -1)]
+            ((6, 64, 28, 28), 1), ((4, 2, 3), -1), ((3, 130, 4), 1), ((50, 70), -1),
+            ((8, 40, 56, 56), 1), ((2, 1100, 16, 16), 1), ((32, 350, 28, 28), 1)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16", "float16"])
@@ -380,6 +384,51 @@ def test_batch_norm_training(K, shape, axis, dtype):
     wref = U.to_device(np.concatenate([dg_ref, db_ref]).astype(U.acc_np(dtype)), an)
     K.batch_norm_training_grad(N, C, S, float(N * S), layout, xd, mud, rsd, gd, wref, wref, dyd, dx)
     assert U.normwise(U.widen(U.to_host(dx), dtype), dx_ref) <= U.TIGHT[dtype]
+
+    # the two as one call (x and dy read once where a channel slice fits the registers)
+    wg2, dx2 = empty((2 * C,), an), empty(shape, dtype)
+    K.batch_norm_training_backward(N, C, S, float(N * S), layout, xd, mud, rsd, gd, dyd, wg2, wg2, dx2)
+    w2 = U.to_host(wg2)
+    assert U.normwise(w2[:C], dg_ref) <= ptol and U.normwise(w2[C:], db_ref) <= ptol
+    assert U.normwise(U.widen(U.to_host(dx2), dtype), dx_ref) <= U.TIGHT[dtype]
+
+
+def test_batch_norm_exchange_timeout_is_reported(K):
+    """A wait of one poll gives up before the other slices of a channel have published their
+    sums: every kernel still runs to its end, the library says so, and refuses further
+    single-read launches until the state is cleared."""
+    import torch
+    from dragon_amd._lib import DragonHipError
+    N, C, S = 8, 40, 56 * 56  # six slices per channel
+    x = torch.randn((N, C, S), device="cuda")
+    g, b = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+    rm, rv = torch.zeros(C, device="cuda"), torch.ones(C, device="cuda")
+    mu, rsig, params = (torch.empty(n, device="cuda") for n in (C, C, 2 * C))
+    y = torch.empty_like(x)
+
+    def forward():
+        K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, x, g, b, rm, rv, mu, rsig, params, y)
+
+    forward()
+    torch.cuda.synchronize()
+    assert not K.exchange_timed_out()
+    try:
+        K.exchange_reset(1)
+        for _ in range(4):  # a peer that is late by one poll is all it takes
+            forward()
+            torch.cuda.synchronize()
+            if K.exchange_timed_out():
+                break
+        assert K.exchange_timed_out()
+        with pytest.raises(DragonHipError):
+            forward()
+    finally:
+        K.exchange_reset(0)
+    assert not K.exchange_timed_out()
+    forward()
+    torch.cuda.synchronize()
+    ref = (x - x.mean((0, 2), keepdim=True)) * torch.rsqrt(x.var((0, 2), unbiased=False, keepdim=True) + 1e-5)
+    assert float((y - ref).abs().max()) < 1e-4
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16"])
