@@ -273,8 +273,12 @@ def measure_workload(name, steps, warmup):
     for kname, fn, nbytes in kernels:
         ms = time_calls(fn, steps, warmup)
         gbs = nbytes / (ms * 1e-3) / 1e9
+        elems = 1
+        for d in meta.get("shape", (meta.get("rows", 1), meta.get("width", 1))):
+            elems *= d
         per_kernel.append({"workload": name, "kernel": kname, "us": round(ms * 1e3, 2),
                            "algorithmic_bytes": nbytes, "GB/s": round(gbs, 1),
+                           "Gelem/s": round(elems / (ms * 1e-3) / 1e9, 1),
                            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
 
     def step():
@@ -360,6 +364,8 @@ def main():
             if name != head:
                 all_kernels += measure_workload(name, max(10, args.steps // 2), args.warmup)[0]
     ceiling = streaming_ceiling(20, 5)
+    for k in all_kernels:  # the second denominator: an achieved 1:1 streaming copy on this device
+        k["frac_copy_probe"] = round(k["GB/s"] / ceiling["copy"], 3)
 
     cpu = None
     if not args.no_cpu and head == "softmax_f16_16x32x512x512":

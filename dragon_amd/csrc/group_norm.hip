@@ -34,6 +34,7 @@
 #include "reduce.h"
 #include "row_loop.h"
 #include "row_tile.h"
+#include "slices.h"
 
 namespace dragon_hip {
 namespace {
@@ -1055,7 +1056,227 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   // per-(n, c) pairs of the fused and the general path; NHWC adds the stage-one partial pairs
   size_t pairs = static_cast<size_t>(N) * C;
   if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
+  // the slice path: K pairs per group and one pair per wavefront block
+  if (layout == DRAGON_HIP_NCHW && S % (IO<T>::kVec * kWaveSize) == 0) {
+    const uint32_t L = static_cast<uint32_t>(D * S);
+    const SliceUnits u{static_cast<uint32_t>(N * G), 1u, L, L, L};
+    const CoopPlan p = plan_coop<T>(u, 2);
+    if (p.ok) {
+      const size_t slices = static_cast<size_t>(u.units) * p.K +
+          static_cast<size_t>(N) * C * (S / IO<T>::kVec / kWaveSize);
+      if (slices > pairs) pairs = slices;
+    }
+  }
   return pairs * 2 * sizeof(A);
+}
+
+// --------------------------------------------------------------------------
+// NCHW groups too large for one workgroup's registers: the slice kernel
+// (slices.h) with the group as the reduction unit, one run of D*S elements.
+// --------------------------------------------------------------------------
+inline SliceUnits group_units(const GroupShape& sh) {
+  const uint32_t L = sh.D * sh.S;
+  return SliceUnits{sh.N * sh.G, 1u, L, L, L};
+}
+
+// Moments -> InvStd -> GroupNorm with x read once.
+template <typename T>
+struct GroupSlicesForward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  A inv_l, eps;
+  const A* gamma;
+  const A* beta;
+  A* mu;
+  A* rsig;
+  uint32_t G, D, packets_per_chan;
+  A shift, mean, rs;
+  __device__ __forceinline__ void begin(uint32_t, uint32_t base, const T* x) {
+    shift = IO<T>::load1(x + base);  // one sample of the group
+  }
+  template <int V>
+  __device__ __forceinline__ void accumulate(uint32_t, uint32_t, const A (&x)[V], const A (&)[V],
+                                             A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const A t = x[e] - shift;
+      a += t;
+      b += t * t;
+    }
+  }
+  __device__ __forceinline__ void finish(uint32_t row, bool leader, A a, A b) {
+    const A dm = a * inv_l;
+    mean = shift + dm;
+    const A var = b * inv_l - dm * dm;
+    rs = acc_rsqrt_exact(var + eps);
+    if (leader) {
+      mu[row] = mean;
+      rsig[row] = rs;
+    }
+  }
+  template <int V>
+  __device__ __forceinline__ void transform(uint32_t row, uint32_t j, A (&x)[V], const A (&)[V]) const {
+    const uint32_t c = (row % G) * D + j / packets_per_chan;
+    const A gs = gamma[c] * rs, bc = beta[c];
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[e] = (x[e] - mean) * gs + bc;
+  }
+};
+
+// GroupNormGrad with x and dy read once. The sums exchanged between the slices
+// are the group's ds and db; a wavefront's 64 packets lie in one channel
+// (S / kVec is a multiple of 64), so its share of that channel's dgamma / dbeta
+// is one wave reduction, written to chan_part[(row * blocks + j / 64) * 2] and
+// summed per channel by a second, small kernel.
+template <typename T>
+struct GroupSlicesBackward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 2;
+  A denom;  // 1 / (D * S)
+  const A* mu;
+  const A* rsig;
+  const A* gamma;
+  A* ds;
+  A* db;
+  A* chan_part;
+  uint32_t G, D, packets_per_chan, blocks_per_row;
+  A m, r, u0, v0;
+  __device__ __forceinline__ void begin(uint32_t row, uint32_t, const T*) { m = mu[row], r = rsig[row]; }
+  template <int V>
+  __device__ __forceinline__ void accumulate(uint32_t row, uint32_t j, const A (&x)[V],
+                                             const A (&dy)[V], A& a, A& b) const {
+    const A g = gamma[(row % G) * D + j / packets_per_chan];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const A t = g * dy[e];
+      a += t * x[e];
+      b += t;
+    }
+  }
+  __device__ __forceinline__ void finish(uint32_t row, bool leader, A a, A b) {
+    if (leader) {
+      ds[row] = a;
+      db[row] = b;
+    }
+    u0 = (b * m - a) * (r * r * r) * denom;
+    v0 = b * r * denom;
+  }
+  template <int V>
+  __device__ __forceinline__ void transform(uint32_t row, uint32_t j, A (&x)[V],
+                                            const A (&dy)[V]) const {
+    const A gr = gamma[(row % G) * D + j / packets_per_chan] * r;
+    A t1 = A(0), t2 = A(0);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const A xc = x[e] - m;
+      t1 += dy[e] * xc * r;
+      t2 += dy[e];
+      x[e] = gr * dy[e] + (u0 * xc - v0);
+    }
+    t1 = wave_allreduce(t1, SumOp());
+    t2 = wave_allreduce(t2, SumOp());
+    if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+      A* o = chan_part + (static_cast<size_t>(row) * blocks_per_row + j / kWaveSize) * 2;
+      o[0] = t1;
+      o[1] = t2;
+    }
+  }
+};
+
+// dgamma[c], dbeta[c] = sum over n and over the wavefront blocks of channel (n, c).
+template <typename A>
+__global__ __launch_bounds__(kReduceThreads) void sum_channel_blocks(
+    const uint32_t N, const uint32_t C, const uint32_t blocks_per_chan, const A* __restrict__ part,
+    A* __restrict__ dgamma, A* __restrict__ dbeta) {
+  __shared__ A lds[2 * kReduceWaves];
+  const uint32_t c = blockIdx.x;
+  A a = A(0), b = A(0);
+  for (uint32_t i = threadIdx.x; i < N * blocks_per_chan; i += kReduceThreads) {
+    const uint32_t n = i / blocks_per_chan, e = i - n * blocks_per_chan;
+    const A* p = part + ((static_cast<size_t>(n) * C + c) * blocks_per_chan + e) * 2;
+    a += p[0];
+    b += p[1];
+  }
+  block_reduce_pair(a, b, lds);
+  if (threadIdx.x == 0) {
+    dgamma[c] = a;
+    dbeta[c] = b;
+  }
+}
+
+// Pairs of scratch the backward needs beyond the slices' own: one per wavefront block.
+template <typename T>
+size_t group_slices_block_pairs(const GroupShape& sh) {
+  return static_cast<size_t>(sh.N) * sh.C * (sh.S / IO<T>::kVec / kWaveSize);
+}
+
+template <typename T>
+int try_group_norm_grad_slices(const GroupShape& sh, const void* x, const void* mu, const void* rsig,
+                               const void* gamma, const void* dy, void* ds, void* db, void* dgamma,
+                               void* dbeta, void* dx, void* scratch, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  if (!sh.nchw || sh.S % (kVec * kWaveSize) != 0) return kNotApplicable;
+  const SliceUnits u = group_units(sh);
+  const CoopPlan p = plan_coop<T>(u, 2);
+  if (!p.ok) return kNotApplicable;
+  A* pairs = static_cast<A*>(scratch);
+  A* chan_part = pairs + static_cast<size_t>(u.units) * p.K * 2;
+  const uint32_t blocks_per_chan = sh.S / kVec / kWaveSize;
+  const GroupSlicesBackward<T> op{A(1) / A(static_cast<int64_t>(sh.D) * sh.S),
+                                  static_cast<const A*>(mu),
+                                  static_cast<const A*>(rsig),
+                                  static_cast<const A*>(gamma),
+                                  static_cast<A*>(ds),
+                                  static_cast<A*>(db),
+                                  chan_part,
+                                  sh.G,
+                                  sh.D,
+                                  sh.S / kVec,
+                                  sh.D * blocks_per_chan,
+                                  A(0), A(0), A(0), A(0)};
+  const int st = try_channel_slices<T>(u, op, static_cast<const T*>(x), static_cast<const T*>(dy),
+                                       static_cast<T*>(dx), pairs, stream);
+  if (st != DRAGON_HIP_OK) return st;
+  hipLaunchKernelGGL((sum_channel_blocks<A>), dim3(sh.C), dim3(kReduceThreads), 0, stream, sh.N, sh.C,
+                     blocks_per_chan, chan_part, static_cast<A*>(dgamma), static_cast<A*>(dbeta));
+  return status_of_launch();
+}
+
+template <typename T>
+int try_group_norm_forward_slices(const GroupShape& sh, float eps, const void* x, const void* gamma,
+                                  const void* beta, void* mu, void* rsig, void* y, void* scratch,
+                                  size_t scratch_bytes, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  if (!sh.nchw || sh.S % kVec != 0) return kNotApplicable;
+  const SliceUnits u = group_units(sh);
+  if (!plan_coop<T>(u, 1).ok) return kNotApplicable;
+  if (!scratch || scratch_bytes < coop_scratch_bytes<T>(u)) return DRAGON_HIP_ESCRATCH;
+  const GroupSlicesForward<T> op{A(1) / A(static_cast<int64_t>(sh.D) * sh.S),
+                                 A(eps),
+                                 static_cast<const A*>(gamma),
+                                 static_cast<const A*>(beta),
+                                 static_cast<A*>(mu),
+                                 static_cast<A*>(rsig),
+                                 sh.G,
+                                 sh.D,
+                                 sh.S / kVec,
+                                 A(0), A(0), A(0)};
+  const T* xp = static_cast<const T*>(x);
+  return try_channel_slices<T>(u, op, xp, xp, static_cast<T*>(y), static_cast<A*>(scratch), stream);
+}
+
+inline size_t group_slices_scratch_bytes(int dtype, const GroupShape& sh) {
+  if (!sh.nchw) return 0;
+  const SliceUnits u = group_units(sh);
+  switch (dtype) {
+    case DRAGON_HIP_F16: return sh.S % 8 == 0 ? coop_scratch_bytes<f16_t>(u) : 0;
+    case DRAGON_HIP_BF16: return sh.S % 8 == 0 ? coop_scratch_bytes<bf16_t>(u) : 0;
+    case DRAGON_HIP_F32: return sh.S % 4 == 0 ? coop_scratch_bytes<float>(u) : 0;
+    case DRAGON_HIP_F64: return sh.S % 2 == 0 ? coop_scratch_bytes<double>(u) : 0;
+    default: return 0;
+  }
 }
 
 // Fused forward: true when the register-resident kernel was launched.
@@ -1204,6 +1425,12 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.C, kWaveSize))),
                        dim3(1024), 0, stream, sh.N, sh.C, part, dgp, dbtp);
     return status_of_launch();
+  }
+
+  {
+    const int st = try_group_norm_grad_slices<T>(sh, x, mu, rsig, gamma, dy, ds, db, dgamma, dbeta,
+                                                 dx, scratch, stream);
+    if (st != kNotApplicable) return st;
   }
 
   const uint32_t total = sh.N * sh.C * sh.S;
@@ -1404,6 +1631,9 @@ size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t
     const size_t nhwc = (dragon_hip::batched_partial_pairs(N, S, G * D) +
                          static_cast<size_t>(N) * G * D) * 2 * (dtype == DRAGON_HIP_F64 ? 8 : 4);
     if (nhwc > bytes) bytes = nhwc;
+  } else {
+    const size_t slices = dragon_hip::group_slices_scratch_bytes(dtype, sh);
+    if (slices > bytes) bytes = slices;
   }
   return bytes;
 }
@@ -1437,6 +1667,13 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
       return DRAGON_HIP_EDTYPE;
   }
   if (fused) return dragon_hip::status_of_launch();
+  switch (dtype) {
+    case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_slices<dragon_hip::f16_t>(sh, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+    case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_slices<dragon_hip::bf16_t>(sh, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+    case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_slices<float>(sh, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+    default: st = dragon_hip::try_group_norm_forward_slices<double>(sh, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+  }
+  if (st != dragon_hip::kNotApplicable) return st;
   if (!sh.nchw && S > 1) {
     // NHWC: statistics from full-width column reductions of each sample
     if (!scratch || scratch_bytes < dragon_hip_group_norm_forward_scratch_bytes(dtype, N, G, D, S, layout)) {
