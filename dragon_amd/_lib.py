@@ -70,10 +70,11 @@ SIGNATURES = {
                                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dragon_hip_batch_norm_inference_grad": (_int, [_int, _i64, _i64, _i64, _int, _vp, _vp, _vp,
                                                     _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "dragon_hip_softmax": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp]),
-    "dragon_hip_log_softmax": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp]),
-    "dragon_hip_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
-    "dragon_hip_log_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "dragon_hip_softmax_scratch_bytes": (_sz, [_int, _i64, _i64, _i64]),
+    "dragon_hip_softmax": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_log_softmax": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dragon_hip_log_softmax_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dragon_hip_l1_norm": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp]),
     "dragon_hip_l2_norm": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp]),
     "dragon_hip_l1_norm_grad": (_int, [_int, _i64, _i64, _i64, _f32, _f32, _vp, _vp, _vp, _vp]),
@@ -87,7 +88,7 @@ SIGNATURES = {
     "dragon_hip_reduce_loss": (_int, [_int, _i64, _i64, _f32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dragon_hip_reduce_loss_grad": (_int, [_int, _i64, _i64, _f32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dragon_hip_broadcast_loss_grad": (_int, [_int, _i64, _i64, _i64, _vp, _vp, _vp]),
-    "dragon_hip_softmax_cross_entropy_loss_scratch_bytes": (_sz, [_int, _i64, _i64]),
+    "dragon_hip_softmax_cross_entropy_loss_scratch_bytes": (_sz, [_int, _i64, _i64, _i64]),
     "dragon_hip_softmax_cross_entropy_loss_forward": (_int, [_int, _int, _i64, _i64, _i64, _i64,
                                                              _int, _vp, _vp, _vp, _vp, _vp, _sz,
                                                              _vp]),

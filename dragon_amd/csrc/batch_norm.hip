@@ -352,6 +352,7 @@ template <typename T>
 struct CoopForward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 1;
+  using Merge = PairSum;
   A inv_n, momentum, one_minus_momentum, eps;
   const A* gamma;
   const A* beta;
@@ -401,6 +402,7 @@ template <typename T>
 struct CoopBackward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 2;
+  using Merge = PairSum;
   A normalizer;
   const A* mu;
   const A* rsig;

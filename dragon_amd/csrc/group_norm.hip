@@ -24,6 +24,10 @@
 //          by a second small kernel (two-stage, no atomics).
 //   groups (NCHW, a group fits a register tile): fused forward for any S;
 //          fused backward when channels span whole wavefronts of packets.
+//   slices (NCHW, a group larger than one workgroup's registers): the group's
+//          slices stay in the registers of several workgroups that exchange
+//          their partial sums inside one kernel (slices.h), so x and dy are
+//          still read once.
 //   general  one pass over x and dy for the per-(n, c) pairs
 //          (sum dy*(x - mu), sum dy): rows of S elements (NCHW) or column
 //          reductions of each sample's [S, C] matrix (NHWC); ds/db and
@@ -1084,6 +1088,7 @@ template <typename T>
 struct GroupSlicesForward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 1;
+  using Merge = PairSum;
   A inv_l, eps;
   const A* gamma;
   const A* beta;
@@ -1132,6 +1137,7 @@ template <typename T>
 struct GroupSlicesBackward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 2;
+  using Merge = PairSum;
   A denom;  // 1 / (D * S)
   const A* mu;
   const A* rsig;

@@ -457,6 +457,13 @@ inline int partial_blocks(int64_t n) {
 
 // Scratch of a loss reduction: the partial pairs plus one scalar.
 inline size_t reduce_loss_scratch(size_t elem) { return (2 * kMaxPartials + 1) * elem; }
+// Scratch of the fused loss forward: loss[NxS], mask[NxS], the reduction's
+// partial pairs and scalar, rounded up to 16 bytes; what the softmax of rows
+// beyond the fused row tiles asks for follows.
+inline size_t fused_loss_head_bytes(size_t elem, int64_t N, int64_t S) {
+  const size_t head = static_cast<size_t>(2 * N * S) * elem + reduce_loss_scratch(elem);
+  return (head + 15) / 16 * 16;
+}
 
 template <typename T>
 int launch_cross_entropy(int64_t N, const void* input, const void* target, void* loss,
@@ -608,7 +615,12 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
 #undef LAUNCH
     }
   } else {
-    const int st = dragon_hip_softmax(sizeof(T) == 8 ? DRAGON_HIP_F64 : DRAGON_HIP_F32, N, S, C, x, prob, stream);
+    // rows beyond the fused row tiles: Softmax (several workgroups per row where
+    // that pays), then the per-position loss
+    const int tag = sizeof(T) == 8 ? DRAGON_HIP_F64 : DRAGON_HIP_F32;
+    const int st = dragon_hip_softmax(tag, N, S, C, x, prob,
+                                      static_cast<char*>(scratch) + fused_loss_head_bytes(sizeof(T), N, S),
+                                      dragon_hip_softmax_scratch_bytes(tag, N, S, C), stream);
     if (st != DRAGON_HIP_OK) return st;
     hipLaunchKernelGGL((cross_entropy_sparse<T, TargetT>), dim3(loss_grid(NxS)),
                        dim3(kLossThreads), 0, stream, NxS, S, C, ignore_index, pp, tp, loss, mask);
@@ -778,10 +790,11 @@ int dragon_hip_broadcast_loss_grad(int dtype, int64_t N, int64_t S, int64_t C, c
   DRAGON_HIP_DISPATCH_LOSS_T(dtype, launch_broadcast_loss_grad, N, S, C, dl, dx, s);
 }
 
-size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S) {
-  if (!loss_dtype_ok(dtype) || N < 0 || S < 0) return 0;
-  // loss[NxS], mask[NxS], then the reduction's partial pairs and scalar
-  return (static_cast<size_t>(2 * N * S)) * loss_elem(dtype) + reduce_loss_scratch(loss_elem(dtype));
+size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S,
+                                                           int64_t C) {
+  if (!loss_dtype_ok(dtype) || N < 0 || S < 0 || C <= 0) return 0;
+  return dragon_hip::fused_loss_head_bytes(loss_elem(dtype), N, S) +
+      dragon_hip_softmax_scratch_bytes(dtype, N, S, C);
 }
 
 int dragon_hip_softmax_cross_entropy_loss_forward(int dtype, int target_dtype, int64_t N, int64_t S,
@@ -795,7 +808,7 @@ int dragon_hip_softmax_cross_entropy_loss_forward(int dtype, int target_dtype, i
   if (N * S > 0 && (!x || !target || !prob)) return DRAGON_HIP_EINVAL;
   if (N * S == 0 && reduction == kNone) return DRAGON_HIP_OK;
   if (!scratch ||
-      scratch_bytes < dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S)) {
+      scratch_bytes < dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S, C)) {
     return DRAGON_HIP_ESCRATCH;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -23,6 +23,8 @@
 //
 // The arithmetic is a policy Op:
 //   kIn                              tensors held (x; x and dy)
+//   Merge                            how two partial pairs combine (PairSum, or the
+//                                    Op's own merge / identity)
 //   begin(u, base, in0)              per-item setup (base = first element of the unit)
 //   accumulate(u, j, x, dy, a, b)    the terms of packet j of unit u in the two sums
 //   finish(u, leader, a, b)          coefficients from the unit's totals; the thread
@@ -214,11 +216,50 @@ __global__ __launch_bounds__(256) void fill_words(Bits* p, uint32_t n, Bits valu
 // per-XCD L2 caches without flushing or invalidating them; a slot is complete
 // as soon as it no longer holds the unset pattern, so no counter or fence
 // orders the exchange.
-template <typename A>
+// How two partial pairs combine: sums (the default policy of an Op), or an
+// Op's own associative, symmetric merge (with its identity), e.g. the running
+// (maximum, scaled sum) of a softmax.
+struct PairSum {
+  static constexpr bool kIsSum = true;
+  template <typename A>
+  static __device__ __forceinline__ void identity(A& a, A& b) {
+    a = A(0), b = A(0);
+  }
+  template <typename A>
+  static __device__ __forceinline__ void merge(A& a, A& b, A a2, A b2) {
+    a += a2, b += b2;
+  }
+};
+
+// All-reduce of a pair over the workgroup with Merge; every thread returns the
+// same bits (the per-wavefront results are merged in wavefront order).
+template <typename Merge, typename A>
+__device__ __forceinline__ void block_merge_pair(A& a, A& b, A* lds /*2*kReduceWaves*/) {
+  if constexpr (Merge::kIsSum) {
+    block_reduce_pair(a, b, lds);
+  } else {
+#pragma unroll
+    for (int o = 1; o < kWaveSize; o <<= 1) {
+      const A a2 = __shfl_xor(a, o, kWaveSize), b2 = __shfl_xor(b, o, kWaveSize);
+      Merge::merge(a, b, a2, b2);
+    }
+    const int wave = threadIdx.x / kWaveSize;
+    if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+      lds[2 * wave] = a;
+      lds[2 * wave + 1] = b;
+    }
+    __syncthreads();
+    a = lds[0], b = lds[1];
+#pragma unroll
+    for (int i = 1; i < kReduceWaves; ++i) Merge::merge(a, b, lds[2 * i], lds[2 * i + 1]);
+  }
+}
+
+template <typename Merge, typename A>
 __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t c, uint32_t w,
                                                     A& a, A& b, A* partial, A* lds_a, A* lds_b) {
   using Bits = typename Unset<A>::Bits;
-  block_reduce_pair(a, b, lds_a);
+  block_merge_pair<Merge>(a, b, lds_a);
   Bits* slots = reinterpret_cast<Bits*>(partial);
   if (threadIdx.x == 0) {
     __hip_atomic_store(slots + 2 * static_cast<size_t>(w), __builtin_bit_cast(Bits, a),
@@ -226,7 +267,8 @@ __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t
     __hip_atomic_store(slots + 2 * static_cast<size_t>(w) + 1, __builtin_bit_cast(Bits, b),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  A ta = A(0), tb = A(0);
+  A ta, tb;
+  Merge::identity(ta, tb);
   const Bits* pairs = slots + 2 * static_cast<size_t>(c) * d.K;
   for (uint32_t q = threadIdx.x; q < d.K; q += kCoopThreads) {
     Bits ua, ub;
@@ -243,10 +285,9 @@ __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t
       }
       __builtin_amdgcn_s_sleep(8);
     }
-    ta += __builtin_bit_cast(A, ua);
-    tb += __builtin_bit_cast(A, ub);
+    Merge::merge(ta, tb, __builtin_bit_cast(A, ua), __builtin_bit_cast(A, ub));
   }
-  block_reduce_pair(ta, tb, lds_b);
+  block_merge_pair<Merge>(ta, tb, lds_b);
   a = ta, b = tb;
 }
 
@@ -298,7 +339,8 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
   constexpr int kVec = IO<T>::kVec;
   const CoopItem it(d, w);
   op.begin(it.c, it.base, in0);
-  A a = A(0), b = A(0);
+  A a, b;
+  Op::Merge::identity(a, b);
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     if (it.has(i)) {
@@ -308,7 +350,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
       op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
     }
   }
-  coop_channel_totals(d, it.c, w, a, b, partial, lds_a, lds_b);
+  coop_channel_totals<typename Op::Merge>(d, it.c, w, a, b, partial, lds_a, lds_b);
   op.finish(it.c, it.k == 0 && threadIdx.x == 0, a, b);
   // convert the packets again instead of keeping every converted element
 #pragma unroll

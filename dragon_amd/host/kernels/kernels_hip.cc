@@ -201,22 +201,30 @@ DEFINE_KERNEL_LAUNCHERS(double, double);
   template <>                                                                                     \
   void Softmax<T, HIPContext>(const int N, const int S, const int C, const T* x, T* y,            \
                               HIPContext* ctx) {                                                  \
-    HIP_CHECK(dragon_hip_softmax(Tag<T>(), N, S, C, x, y, ctx->hip_stream()));                    \
+    const size_t bytes = dragon_hip_softmax_scratch_bytes(Tag<T>(), N, S, C);                     \
+    HIP_CHECK(dragon_hip_softmax(Tag<T>(), N, S, C, x, y, Scratch(ctx, bytes), bytes,             \
+                                 ctx->hip_stream()));                                             \
   }                                                                                               \
   template <>                                                                                     \
   void LogSoftmax<T, HIPContext>(const int N, const int S, const int C, const T* x, T* y,         \
                                  HIPContext* ctx) {                                               \
-    HIP_CHECK(dragon_hip_log_softmax(Tag<T>(), N, S, C, x, y, ctx->hip_stream()));                \
+    const size_t bytes = dragon_hip_softmax_scratch_bytes(Tag<T>(), N, S, C);                     \
+    HIP_CHECK(dragon_hip_log_softmax(Tag<T>(), N, S, C, x, y, Scratch(ctx, bytes), bytes,         \
+                                     ctx->hip_stream()));                                         \
   }                                                                                               \
   template <>                                                                                     \
   void SoftmaxGrad<T, HIPContext>(const int N, const int S, const int C, const T* dy, const T* y, \
                                   T* dx, HIPContext* ctx) {                                       \
-    HIP_CHECK(dragon_hip_softmax_grad(Tag<T>(), N, S, C, dy, y, dx, ctx->hip_stream()));          \
+    const size_t bytes = dragon_hip_softmax_scratch_bytes(Tag<T>(), N, S, C);                     \
+    HIP_CHECK(dragon_hip_softmax_grad(Tag<T>(), N, S, C, dy, y, dx, Scratch(ctx, bytes), bytes,   \
+                                      ctx->hip_stream()));                                        \
   }                                                                                               \
   template <>                                                                                     \
   void LogSoftmaxGrad<T, HIPContext>(const int N, const int S, const int C, const T* dy,          \
                                      const T* y, T* dx, HIPContext* ctx) {                        \
-    HIP_CHECK(dragon_hip_log_softmax_grad(Tag<T>(), N, S, C, dy, y, dx, ctx->hip_stream()));      \
+    const size_t bytes = dragon_hip_softmax_scratch_bytes(Tag<T>(), N, S, C);                     \
+    HIP_CHECK(dragon_hip_log_softmax_grad(Tag<T>(), N, S, C, dy, y, dx, Scratch(ctx, bytes),      \
+                                          bytes, ctx->hip_stream()));                             \
   }
 
 DEFINE_SOFTMAX_LAUNCHERS(float16);
@@ -327,7 +335,7 @@ DEFINE_LOSS_LAUNCHERS(double);
   void SoftmaxCrossEntropyLossForward<InputT, TargetT, HIPContext>(                               \
       const int N, const int S, const int C, const int ignore_index, const string& reduction,     \
       const InputT* x, const TargetT* target, InputT* prob, InputT* loss, HIPContext* ctx) {      \
-    const size_t bytes = dragon_hip_softmax_cross_entropy_loss_scratch_bytes(Tag<InputT>(), N, S); \
+    const size_t bytes = dragon_hip_softmax_cross_entropy_loss_scratch_bytes(Tag<InputT>(), N, S, C); \
     HIP_CHECK(dragon_hip_softmax_cross_entropy_loss_forward(                                      \
         Tag<InputT>(), TargetTag<TargetT>(), N, S, C, ignore_index, ReductionTag(reduction), x,   \
         target, prob, loss, Scratch(ctx, bytes), bytes, ctx->hip_stream()));                      \

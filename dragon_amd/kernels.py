@@ -199,21 +199,32 @@ def batch_norm_inference_grad(N, C, S, data_format, x, mu, rsig, gamma, dy, dgam
           _ptr(gamma), _ptr(dy), _ptr(dgamma), _ptr(dbeta), _ptr(dx), _ptr(ws), need, _stream())
 
 
+def _softmax_scratch(tag, N, S, C, device):
+    need = _lib.lib().dragon_hip_softmax_scratch_bytes(tag, N, S, C)
+    return workspace(need, device), need
+
+
 def softmax(N, S, C, x, y):
-    _call("dragon_hip_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _stream())
+    ws, need = _softmax_scratch(dtype_tag(x), N, S, C, x.device)
+    _call("dragon_hip_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _ptr(ws), need, _stream())
 
 
 def log_softmax(N, S, C, x, y):
-    _call("dragon_hip_log_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _stream())
+    ws, need = _softmax_scratch(dtype_tag(x), N, S, C, x.device)
+    _call("dragon_hip_log_softmax", dtype_tag(x), N, S, C, _ptr(x), _ptr(y), _ptr(ws), need,
+          _stream())
 
 
 def softmax_grad(N, S, C, dy, y, dx):
-    _call("dragon_hip_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx), _stream())
+    ws, need = _softmax_scratch(dtype_tag(y), N, S, C, y.device)
+    _call("dragon_hip_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx), _ptr(ws),
+          need, _stream())
 
 
 def log_softmax_grad(N, S, C, dy, y, dx):
+    ws, need = _softmax_scratch(dtype_tag(y), N, S, C, y.device)
     _call("dragon_hip_log_softmax_grad", dtype_tag(y), N, S, C, _ptr(dy), _ptr(y), _ptr(dx),
-          _stream())
+          _ptr(ws), need, _stream())
 
 
 def l1_norm(N, S, C, normalizer, epsilon, x, y):
@@ -280,7 +291,7 @@ def broadcast_loss_grad(N, S, C, dl, dx):
 
 def softmax_cross_entropy_loss_forward(N, S, C, ignore_index, reduction, x, target, prob, loss):
     tag = dtype_tag(x)
-    need = _lib.lib().dragon_hip_softmax_cross_entropy_loss_scratch_bytes(tag, N, S)
+    need = _lib.lib().dragon_hip_softmax_cross_entropy_loss_scratch_bytes(tag, N, S, C)
     ws = workspace(need, x.device)
     _call("dragon_hip_softmax_cross_entropy_loss_forward", tag, target_tag(target), N, S, C,
           ignore_index, REDUCTIONS[reduction.upper()], _ptr(x), _ptr(target), _ptr(prob),

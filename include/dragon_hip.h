@@ -232,15 +232,24 @@ int dragon_hip_batch_norm_inference_grad(int dtype, int64_t N, int64_t C, int64_
 /* Tensors are T[N, C, S]: the reduced axis has length C and element stride  */
 /* S. y may alias x; dx may alias dy (softmax_op.cc:46-60).                  */
 /* 16-bit I/O accumulates in fp32.                                           */
+/* scratch may be NULL. With dragon_hip_softmax_scratch_bytes(...) bytes of it  */
+/* (0 for shapes that need none) rows of many thousands of packets, e.g.      */
+/* vocabulary-sized rows, are processed by several workgroups per row that     */
+/* exchange their partial results through it; without it they take the         */
+/* one-workgroup-per-row kernels. The context's workspace is what the          */
+/* reference's launchers would pass (ctx->workspace()).                        */
 /* ------------------------------------------------------------------------ */
+size_t dragon_hip_softmax_scratch_bytes(int dtype, int64_t N, int64_t S, int64_t C);
 int dragon_hip_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
-                       void* stream);
+                       void* scratch, size_t scratch_bytes, void* stream);
 int dragon_hip_log_softmax(int dtype, int64_t N, int64_t S, int64_t C, const void* x, void* y,
-                           void* stream);
+                           void* scratch, size_t scratch_bytes, void* stream);
 int dragon_hip_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
-                            const void* y, void* dx, void* stream);
+                            const void* y, void* dx, void* scratch, size_t scratch_bytes,
+                            void* stream);
 int dragon_hip_log_softmax_grad(int dtype, int64_t N, int64_t S, int64_t C, const void* dy,
-                                const void* y, void* dx, void* stream);
+                                const void* y, void* dx, void* scratch, size_t scratch_bytes,
+                                void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* L1Norm / L2Norm, dragon/kernels/normalization/op_kernels.h:145-189        */
@@ -314,9 +323,10 @@ int dragon_hip_broadcast_loss_grad(int dtype, int64_t N, int64_t S, int64_t C, c
  *             else the reduced scalar T[1]
  *   backward  dx = (prob - onehot(target)) * w, w = 0 at ignored positions,
  *             dl[n, s] for NONE, else dl[0] / max(normalizer or valid count, 0.5)
- * Scratch: forward dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S),
+ * Scratch: forward dragon_hip_softmax_cross_entropy_loss_scratch_bytes(dtype, N, S, C),
  * backward dragon_hip_reduce_loss_scratch_bytes(dtype). */
-size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S);
+size_t dragon_hip_softmax_cross_entropy_loss_scratch_bytes(int dtype, int64_t N, int64_t S,
+                                                           int64_t C);
 int dragon_hip_softmax_cross_entropy_loss_forward(int dtype, int target_dtype, int64_t N, int64_t S,
                                                   int64_t C, int64_t ignore_index, int reduction,
                                                   const void* x, const void* target, void* prob,

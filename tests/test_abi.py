@@ -60,8 +60,8 @@ def test_argument_errors_need_no_device(handle):
     assert lib.dragon_hip_layer_norm(2, -1, 8, 1e-5, one, one, one, one, one, one, None) == -1
     assert lib.dragon_hip_layer_norm(2, 4, 0, 1e-5, one, one, one, one, one, one, None) == -1
     assert lib.dragon_hip_layer_norm(2, 0, 8, 1e-5, None, None, None, None, None, None, None) == 0
-    assert lib.dragon_hip_softmax(2, 0, 1, 8, None, None, None) == 0
-    assert lib.dragon_hip_softmax(2, 4, 1, 0, one, one, None) == -1
+    assert lib.dragon_hip_softmax(2, 0, 1, 8, None, None, None, 0, None) == 0
+    assert lib.dragon_hip_softmax(2, 4, 1, 0, one, one, None, 0, None) == -1
     assert lib.dragon_hip_group_norm(2, 2, 2, 2, 2, 7, one, one, one, one, one, one, None) == -1
     assert lib.dragon_hip_batch_norm_training_grad(2, 1 << 20, 1 << 10, 1 << 10, 1.0, 0, one, one,
                                                    one, one, one, one, one, one, None) == -1

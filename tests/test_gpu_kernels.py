@@ -99,7 +99,10 @@ def test_layer_norm_large_mean_stays_accurate(K):
 
 SM_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 100000), -1), ((5, 37), -1),
              ((6, 300), -1), ((3, 7, 5), 1), ((2, 3, 4, 6), 2), ((4, 1), -1), ((2, 16, 8, 8), -1),
-             ((3, 8200), -1)]
+             ((3, 8200), -1),
+             # rows beyond the one-workgroup tiles: several workgroups per row (with the
+             # scratch the wrapper passes); (3, 100000) above takes the same path
+             ((5, 131072), -1)]
 
 
 def _softmax_inputs(shape, dtype, seed):
@@ -162,7 +165,7 @@ def test_softmax_forward_backward(K, shape, axis, dtype, log):
     assert U.normwise(dxw[ok], np.asarray(dx_ref)[ok]) <= U.TIGHT[dtype]
 
 
-@pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (3, 10, 33)])
+@pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (2, 66000), (3, 10, 33)])
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_softmax_in_place(K, dtype, shape):
     x, dy = _softmax_inputs(shape, dtype, 5)
@@ -188,6 +191,45 @@ def test_softmax_in_place(K, dtype, shape):
     dx_ref = R.op_softmax_grad(od, yo, dyo, axis)
     K.softmax_grad(N, S, C, g, buf, g)  # dX aliases dY (AllowInplace {1,0})
     assert U.normwise(U.widen(U.to_host(g), dtype).reshape(shape), dx_ref) <= U.TIGHT[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_softmax_wide_rows_with_and_without_scratch(K, dtype):
+    """Scratch is optional: without it wide rows take the one-workgroup-per-row kernels,
+    with it the slice kernel; both must agree with the oracle."""
+    import ctypes
+    import torch
+    from dragon_amd import _lib
+    shape = (4, 81920)
+    N, C = shape
+    x, dy = _softmax_inputs(shape, dtype, 11)
+    # fp64 is the judge: the oracle's sequential fp32 sum over 81920 terms is itself ~1e-4 off
+    x64 = np.asarray(U.widen(x, dtype), np.float64).reshape(shape)
+    e64 = np.exp(x64 - x64.max(1, keepdims=True))
+    y_ref = e64 / e64.sum(1, keepdims=True)
+    xd = U.to_device(x, dtype)
+    lib, tag = _lib.lib(), K.dtype_tag(xd)
+    need = lib.dragon_hip_softmax_scratch_bytes(tag, N, 1, C)
+    assert need > 0
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for scratch in (None, torch.empty(need, dtype=torch.uint8, device="cuda")):
+        y = empty(shape, dtype)
+        ptr = ctypes.c_void_p(scratch.data_ptr()) if scratch is not None else None
+        st = lib.dragon_hip_softmax(tag, N, 1, C, ctypes.c_void_p(xd.data_ptr()),
+                                    ctypes.c_void_p(y.data_ptr()), ptr,
+                                    need if scratch is not None else 0, stream)
+        assert st == 0
+        yw = U.widen(U.to_host(y), dtype).reshape(shape)
+        assert U.rowwise_normwise(yw, y_ref) <= U.TIGHT[dtype]
+        outs.append(yw)
+    # too little scratch is the same as none
+    y = empty(shape, dtype)
+    small = torch.empty(16, dtype=torch.uint8, device="cuda")
+    assert lib.dragon_hip_softmax(tag, N, 1, C, ctypes.c_void_p(xd.data_ptr()),
+                                  ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(small.data_ptr()),
+                                  16, stream) == 0
+    assert np.array_equal(U.widen(U.to_host(y), dtype).reshape(shape), outs[0])
 
 
 def test_softmax_masked_logits_are_exact_zero(K):
