@@ -204,6 +204,20 @@ struct RawRowTile {
       p[s] = on ? t : z;
     }
   }
+  // Rows of any width at element-aligned addresses, read in whole (unaligned)
+  // packets: the row's last packet may reach up to kVec - 1 elements past the
+  // row, so the caller guarantees that those are readable (another row follows)
+  // and masks them itself.
+  __device__ __forceinline__ void load_over(const T* row, int ncols, bool valid = true) {
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int col = (s * kTPR + lane()) * kVec;
+      const bool on = valid && col < ncols;
+      const u32x4 t = load_packet_unaligned(row + (on ? col : 0));
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      p[s] = on ? t : z;
+    }
+  }
   // load() without the zero fill: inactive slots (and every slot when `valid`
   // is false) hold packet 0 of `row`, for kernels that mask at the point of use.
   __device__ __forceinline__ void load_unmasked(const T* row, int npackets) {

@@ -122,25 +122,40 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
 // two of those): a persistent workgroup requests the next row's packets before
 // it reduces the current row, and issues the current row's stores after the
 // wait for them, so loads, arithmetic and stores of neighbouring rows overlap.
-template <typename T, int kKind, int kVPT>
+// The ragged flavour takes rows of any width at element-aligned addresses and
+// reads whole packets, up to kVec - 1 elements past a row's end: the caller
+// gives it all rows but the tensor's last.
+template <typename T, int kKind, int kVPT, bool kRagged = false>
 __global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const int C, const T* x,
                                                           T* y) {
   constexpr int kTPR = 1024;
-  using Tile = RowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, kTPR, kRagged>;
   using Raw = RawRowTile<T, kTPR, kVPT>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
-  const int npackets = C / kVec;
+  const int npackets = Tile::extent_of(C);  // columns for the ragged flavour
+  // the row's last packet when it is partial: its slot, lane and element count
+  const int tail_valid = C % kVec;
+  const int tail_slot = tail_valid ? (C / kVec) / kTPR : -1;
+  const int tail_lane = (C / kVec) % kTPR;
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
   Raw cur;
-  cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
+  if constexpr (kRagged) {
+    cur.load_over(x + (row < N ? row : 0) * C, C, row < N);
+  } else {
+    cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
+  }
   for (; row < N; row += stride) {
     Raw nxt;
     const bool more = row + stride < N;
-    nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
+    if constexpr (kRagged) {
+      nxt.load_over(x + (more ? row + stride : 0) * C, C, more);
+    } else {
+      nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
+    }
     Tile t;
     A m = acc_neg_inf<A>();
 #pragma unroll
@@ -150,8 +165,18 @@ __global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
         t.v[i][e] = on ? t.v[i][e] : acc_neg_inf<A>();  // raw padding is zero bits
-        m = MaxOp()(m, t.v[i][e]);
       }
+      if constexpr (kRagged) {
+        // only the slot of the row's last, partial packet holds elements past the row
+        if (i == tail_slot) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (Tile::lane() == tail_lane && e >= tail_valid) t.v[i][e] = acc_neg_inf<A>();
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) m = MaxOp()(m, t.v[i][e]);
     }
     m = Tile::reduce(m, MaxOp(), slots[0]);
     A s = A(0);
@@ -178,7 +203,23 @@ __global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const
       }
     nxt.wait_ready();
     cur = nxt;
-    t.store(y + row * C, npackets);
+    if constexpr (kRagged) {
+      T* out = y + row * C;
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        const int col = (i * kTPR + Tile::lane()) * kVec;
+        if (i == tail_slot && Tile::lane() == tail_lane) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (e < tail_valid) IO<T>::store1(out + col + e, t.v[i][e]);
+          }
+        } else if (col < C) {
+          store_packet_unaligned(out + col, IO<T>::pack(t.v[i]));
+        }
+      }
+    } else {
+      t.store(y + row * C, npackets);
+    }
     __syncthreads();  // slots are reused by the next row
   }
 }
@@ -786,13 +827,24 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
     // width or base address the ragged ones
     const bool regular = C % kVec == 0 && aligned16(x) && aligned16(y);
     // 1024-thread tiles: persistent workgroups that prefetch the next row
-    if (regular && cfg.tpr == 1024) {
+    // (not the ragged flavour of eight 16-bit packets per thread: 64 converted
+    // elements beside the next row's packets do not fit 128 registers)
+    if (cfg.tpr == 1024 && (regular || (N > 1 && !(cfg.vpt == 8 && sizeof(T) == 2)))) {
+      // ragged rows: all but the last here (whole packets may read past a row's
+      // end), the last one through the element-exact tile below
+      const int64_t rows = regular ? N : N - 1;
 #define LAUNCH_WIDE(VPT)                                                                     \
   {                                                                                          \
-    auto kernel = softmax_wide_rows<T, kKind, VPT>;                                          \
+    auto kernel = regular ? softmax_wide_rows<T, kKind, VPT, false>                          \
+                          : softmax_wide_rows<T, kKind, VPT, true>;                          \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                \
-    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), xp, yp); \
+    const unsigned grid = rows < static_cast<int64_t>(resident) ? static_cast<unsigned>(rows) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, rows, static_cast<int>(C), xp, yp); \
+    if (!regular) {                                                                          \
+      hipLaunchKernelGGL((softmax_rows<T, kKind, 1024, VPT, true>), dim3(1), dim3(1024), 0,  \
+                         stream, static_cast<int64_t>(1), static_cast<int>(C), xp + rows * C, \
+                         yp + rows * C);                                                     \
+    }                                                                                        \
   }
       if (cfg.vpt == 2) LAUNCH_WIDE(2) else if (cfg.vpt == 4) LAUNCH_WIDE(4) else LAUNCH_WIDE(8)
 #undef LAUNCH_WIDE
