@@ -914,9 +914,11 @@ __global__ __launch_bounds__(256) void group_stats_from_column_sums(
   const T* first_row = x + static_cast<size_t>(n) * d.S * d.C + g * D;
   const A* pairs = sums + (static_cast<size_t>(n) * d.C + g * D) * 2;
   A mean = A(0);
+#pragma unroll 8
   for (uint32_t j = 0; j < D; ++j) mean += IO<T>::load1(first_row + j) + pairs[2 * j] * inv_s;
   mean = mean / A(D);
   A m2 = A(0);
+#pragma unroll 8
   for (uint32_t j = 0; j < D; ++j) {
     const A a = pairs[2 * j], b = pairs[2 * j + 1];
     const A dm = IO<T>::load1(first_row + j) + a * inv_s - mean;
@@ -935,7 +937,8 @@ __global__ __launch_bounds__(256) void sum_batched_partials(const BatchedColumns
   if (i >= d.N * d.C) return;
   const uint32_t n = i / d.C, c = i - n * d.C;
   A a = A(0), b = A(0);
-  for (uint32_t k = 0; k < d.split; ++k) {
+#pragma unroll 16
+  for (uint32_t k = 0; k < d.split; ++k) {  // independent loads: issued sixteen at a time
     const size_t idx = ((static_cast<size_t>(n) * d.split + k) * d.C + c) * 2;
     a += partial[idx];
     b += partial[idx + 1];

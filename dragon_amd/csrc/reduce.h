@@ -267,33 +267,47 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_finalize(
 }
 
 // Stage two for the scratch layout of reduce2_columns when `split` is large:
-// a workgroup owns 64 adjacent outputs (one per lane, so every load is 64
-// adjacent pairs), its four wavefronts stride over k and are combined in
-// wavefront order through LDS. Fixed summation order, like reduce2_finalize.
+// a 1024-thread workgroup owns 16 adjacent outputs; thread (ol, kl) sums the
+// pairs k = kl, kl + 64, ... of output ol (a wavefront reads four runs of 16
+// adjacent pairs), the four k-lanes of a wavefront are combined by shuffles
+// and the sixteen wavefronts in wavefront order through LDS. Fixed summation
+// order, like reduce2_finalize.
+constexpr int kFinalizeThreads = 1024;
+constexpr int kFinalizeOutputs = 16;
+constexpr int kFinalizeWaves = kFinalizeThreads / kWaveSize;
 template <typename A, typename E>
-__global__ __launch_bounds__(kReduceThreads) void reduce2_finalize_columns(
+__global__ __launch_bounds__(kFinalizeThreads) void reduce2_finalize_columns(
     const uint32_t n_out, const uint32_t split, const A* __restrict__ partial, E e) {
-  __shared__ A lds[kReduceWaves][kWaveSize][2];
-  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  __shared__ A lds[kFinalizeWaves][kFinalizeOutputs][2];
+  const uint32_t ol = threadIdx.x & (kFinalizeOutputs - 1);
+  const uint32_t kl = threadIdx.x / kFinalizeOutputs;
   const uint32_t wave = threadIdx.x / kWaveSize;
-  const uint32_t o = blockIdx.x * kWaveSize + lane;
+  const uint32_t o = blockIdx.x * kFinalizeOutputs + ol;
   A a = A(0), b = A(0);
   if (o < n_out) {
-#pragma unroll 4
-    for (uint32_t k = wave; k < split; k += kReduceWaves) {
+#pragma unroll 8
+    for (uint32_t k = kl; k < split; k += kFinalizeThreads / kFinalizeOutputs) {
       const size_t idx = static_cast<size_t>(k) * n_out + o;
       a += partial[idx * 2];
       b += partial[idx * 2 + 1];
     }
   }
-  lds[wave][lane][0] = a;
-  lds[wave][lane][1] = b;
-  __syncthreads();
-  if (wave == 0 && o < n_out) {
 #pragma unroll
-    for (int w = 1; w < kReduceWaves; ++w) {
-      a += lds[w][lane][0];
-      b += lds[w][lane][1];
+  for (int off = kFinalizeOutputs; off < kWaveSize; off <<= 1) {
+    a += __shfl_xor(a, off, kWaveSize);
+    b += __shfl_xor(b, off, kWaveSize);
+  }
+  if ((threadIdx.x & (kWaveSize - 1)) < kFinalizeOutputs) {
+    lds[wave][ol][0] = a;
+    lds[wave][ol][1] = b;
+  }
+  __syncthreads();
+  if (threadIdx.x < kFinalizeOutputs && o < n_out) {
+    a = lds[0][ol][0], b = lds[0][ol][1];
+#pragma unroll
+    for (int w = 1; w < kFinalizeWaves; ++w) {
+      a += lds[w][ol][0];
+      b += lds[w][ol][1];
     }
     e(o, a, b);
   }
@@ -304,8 +318,9 @@ template <typename A, typename E>
 inline void launch_reduce2_finalize(uint32_t n_out, uint32_t split, bool segment_major,
                                     const A* partial, E e, hipStream_t stream) {
   if (!segment_major && split > 16) {
-    hipLaunchKernelGGL((reduce2_finalize_columns<A, E>), dim3((n_out + kWaveSize - 1) / kWaveSize),
-                       dim3(kReduceThreads), 0, stream, n_out, split, partial, e);
+    hipLaunchKernelGGL((reduce2_finalize_columns<A, E>),
+                       dim3((n_out + kFinalizeOutputs - 1) / kFinalizeOutputs),
+                       dim3(kFinalizeThreads), 0, stream, n_out, split, partial, e);
   } else {
     hipLaunchKernelGGL((reduce2_finalize<A, E>), dim3((n_out + kReduceThreads - 1) / kReduceThreads),
                        dim3(kReduceThreads), 0, stream, n_out, split, segment_major, partial, e);
