@@ -102,7 +102,9 @@ SM_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 100000), 
              ((3, 8200), -1),
              # rows beyond the one-workgroup tiles: several workgroups per row (with the
              # scratch the wrapper passes); (3, 100000) above takes the same path
-             ((5, 131072), -1)]
+             ((5, 131072), -1),
+             # short rows staged through LDS, several rows per wavefront
+             ((64, 64), -1), ((33, 197), -1), ((9, 577), -1), ((100, 128), -1), ((300, 8), -1)]
 
 
 def _softmax_inputs(shape, dtype, seed):
@@ -230,6 +232,48 @@ def test_softmax_wide_rows_with_and_without_scratch(K, dtype):
                                   ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(small.data_ptr()),
                                   16, stream) == 0
     assert np.array_equal(U.widen(U.to_host(y), dtype).reshape(shape), outs[0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shift_x,shift_y", [(1, 1), (3, 3), (1, 0), (0, 5)])
+def test_softmax_short_rows_at_shifted_bases(K, dtype, shift_x, shift_y):
+    """Input and output that start a few elements past a 16-byte boundary: equal shifts take the
+    staged short-row kernels (whose first and last packet reach outside the tensors), unequal
+    shifts the register tiles."""
+    shape = (37, 197)
+    N, C = shape
+    x, dy = _softmax_inputs(shape, dtype, 21)
+    x64 = np.asarray(U.widen(x, dtype), np.float64).reshape(shape)
+    e64 = np.exp(x64 - x64.max(1, keepdims=True))
+    y_ref = e64 / e64.sum(1, keepdims=True)
+    guard = 8
+
+    def shifted(shift, bits=None):
+        buf = empty((N * C + shift + guard,), dtype)
+        buf.zero_()
+        view = buf[shift:shift + N * C].view(N, C)
+        if bits is not None:
+            view.copy_(U.to_device(bits, dtype))
+        return buf, view
+
+    _, xd = shifted(shift_x, x)
+    ybuf, y = shifted(shift_y)
+    K.softmax(N, 1, C, xd, y)
+    yw = U.widen(U.to_host(y.contiguous()), dtype).reshape(shape)
+    assert U.rowwise_normwise(yw, y_ref) <= U.TIGHT[dtype]
+    # nothing outside the output was written
+    flat = U.widen(U.to_host(ybuf), dtype).ravel()
+    assert np.all(flat[:shift_y] == 0) and np.all(flat[shift_y + N * C:] == 0)
+    _, dyd = shifted(shift_x, dy)
+    dxbuf, dx = shifted(shift_x)
+    _, yin = shifted(shift_x, U.to_host(y.contiguous()).reshape(shape))
+    K.softmax_grad(N, 1, C, dyd, yin, dx)
+    dy64 = np.asarray(U.widen(dy, dtype), np.float64).reshape(shape)
+    y64 = np.asarray(yw, np.float64)
+    dx_ref = (dy64 - (dy64 * y64).sum(1, keepdims=True)) * y64
+    assert U.normwise(U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape), dx_ref) <= U.TIGHT[dtype]
+    flat = U.widen(U.to_host(dxbuf), dtype).ravel()
+    assert np.all(flat[:shift_x] == 0) and np.all(flat[shift_x + N * C:] == 0)
 
 
 def test_softmax_masked_logits_are_exact_zero(K):
