@@ -38,6 +38,7 @@
 #include "reduce.h"
 #include "row_loop.h"
 #include "row_tile.h"
+#include "short_rows.h"
 #include "slices.h"
 
 namespace dragon_hip {
@@ -345,6 +346,115 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
       }
     }
   }
+}
+
+// --------------------------------------------------------------------------
+// LayerNorm backward of short rows (per-head normalisations, odd widths): a
+// policy of the LDS-staged kernel (short_rows.h). in0 = x (overwritten with
+// dx), in1 = dy. A thread keeps dgamma / dbeta of its elements across the rows
+// its workgroup visits; the workgroup's lane groups are combined through LDS
+// into one partial row per workgroup, summed by sum_partial_rows.
+// --------------------------------------------------------------------------
+constexpr int kShortGradMaxGrid = kNumCUs * 8;
+
+template <typename T, int kE>
+struct LayerNormShortBackward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = static_cast<size_t>(kShortThreads) * kE * 2 * sizeof(A);
+  static constexpr int kSideWords = 2;
+  A inv_c;
+  const A* mu;
+  const A* rsig;
+  const A* gamma;
+  A* ds;
+  A* db;
+  A* partial;  // [gridDim.x][C][2]
+  A g[kE], dg[kE], dbt[kE];
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int l, int C) {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      g[j] = l + j * kL < C ? gamma[l + j * kL] : A(0);
+      dg[j] = dbt[j] = A(0);
+    }
+  }
+  // mean and rsig of a row: requested with the range's packets, ahead of the
+  // row loop (where every row would otherwise wait for HBM)
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[2]) const {
+    w[0] = mu[row];
+    w[1] = rsig[row];
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t row, const A* side, int l, int, A (&x)[kE],
+                                      const A (&dy)[kE]) {
+    const A m = side[0], r = side[1];
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const A t = g[j] * dy[j];
+      s1 += t * x[j];
+      s2 += t;
+    }
+    s1 = group_allreduce<kL>(s1, SumOp());
+    s2 = group_allreduce<kL>(s2, SumOp());
+    if (l == 0) {
+      ds[row] = s1;
+      db[row] = s2;
+    }
+    const A a = (s2 * m - s1) * (r * r * r) * inv_c;
+    const A b = -(s2 * r) * inv_c;
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const A xc = x[j] - m;
+      const A w = dy[j] * r;  // lanes past the row hold dy = 0: they add nothing
+      dg[j] += w * xc;
+      dbt[j] += dy[j];
+      x[j] = g[j] * w + (a * xc + b);
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A* lds, int C) const {
+    constexpr int kGroups = kShortThreads / kL;
+    const int l = threadIdx.x % kL, sub = threadIdx.x / kL;
+    __syncthreads();  // the stage is free
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      lds[((sub * kE + j) * kL + l) * 2] = dg[j];
+      lds[((sub * kE + j) * kL + l) * 2 + 1] = dbt[j];
+    }
+    __syncthreads();
+    if (sub == 0) {
+      A* out = partial + static_cast<size_t>(blockIdx.x) * C * 2;
+#pragma unroll
+      for (int j = 0; j < kE; ++j) {
+        const int e = l + j * kL;
+        if (e < C) {
+          A a = A(0), b = A(0);
+          for (int q = 0; q < kGroups; ++q) {  // fixed order
+            a += lds[((q * kE + j) * kL + l) * 2];
+            b += lds[((q * kE + j) * kL + l) * 2 + 1];
+          }
+          out[2 * e] = a;
+          out[2 * e + 1] = b;
+        }
+      }
+    }
+  }
+};
+
+// LayerNorm backward rows that take the staged kernel: as for the forward.
+inline bool layer_norm_grad_short_rows(int64_t G, int64_t D, int64_t S, size_t elem_bytes,
+                                       const void* x, const void* dy, const void* dx) {
+  if (G != 1 || S != 1 || D > 1024 || !congruent16(x, dy) || !congruent16(x, dx)) return false;
+  const size_t row_bytes = static_cast<size_t>(D) * elem_bytes;
+  return row_bytes <= 512 || row_bytes % 16 != 0 || !aligned16(x);
+}
+inline unsigned short_grad_grid(int64_t N, uint32_t rows_per_chunk) {
+  const unsigned grid = short_grid(N, rows_per_chunk);
+  return grid < static_cast<unsigned>(kShortGradMaxGrid) ? grid : kShortGradMaxGrid;
 }
 
 // --------------------------------------------------------------------------
@@ -1058,10 +1168,18 @@ template <typename T>
 size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
   using A = typename IO<T>::Acc;
   const RowGradPlan rp = plan_row_grad<T>(N, G, D, S);
-  if (rp.use_rows) return static_cast<size_t>(rp.grid) * D * 2 * sizeof(A);
+  // LayerNorm backward: one partial (dgamma, dbeta) row per workgroup of the row
+  // kernels, or of the staged short-row kernel when the addresses select it
+  size_t row_paths = rp.use_rows ? static_cast<size_t>(rp.grid) * D * 2 * sizeof(A) : 0;
+  if (G == 1 && S == 1 && D <= 1024) {
+    const size_t staged = static_cast<size_t>(kShortGradMaxGrid) * D * 2 * sizeof(A);
+    if (staged > row_paths) row_paths = staged;
+  }
+  if (rp.use_rows) return row_paths;
   const int64_t C = G * D;
   // per-(n, c) pairs of the fused and the general path; NHWC adds the stage-one partial pairs
   size_t pairs = static_cast<size_t>(N) * C;
+  if (pairs * 2 * sizeof(A) < row_paths) pairs = row_paths / (2 * sizeof(A));
   if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
   // the slice path: K pairs per group and one pair per wavefront block
   if (layout == DRAGON_HIP_NCHW && S % (IO<T>::kVec * kWaveSize) == 0) {
@@ -1376,6 +1494,22 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   const int layout = sh.nchw ? DRAGON_HIP_NCHW : DRAGON_HIP_NHWC;
   if (scratch_bytes < group_norm_grad_scratch<T>(sh.N, sh.G, sh.D, sh.S, layout) || !scratch) {
     return DRAGON_HIP_ESCRATCH;
+  }
+
+  ShortPlan sp;
+  if (layer_norm_grad_short_rows(sh.G, sh.D, sh.S, sizeof(T), x, dy, dx) &&
+      plan_short_rows(sh.D, sizeof(T), 2, aligned16(x), &sp)) {
+    size_t lds = static_cast<size_t>(sp.stage_packets) * 32 + sp.rows_per_chunk * 2 * sizeof(A);
+    const size_t end_bytes = static_cast<size_t>(kShortThreads) * sp.per_lane * 2 * sizeof(A);
+    if (lds < end_bytes) lds = end_bytes;
+    const unsigned grid = short_grad_grid(sh.N, sp.rows_per_chunk);
+    const int64_t rows = sh.N;
+    DRAGON_HIP_SHORT_LAUNCH(T, LayerNormShortBackward, sp, lds, grid, stream, rows,
+                            static_cast<int>(sh.D), xp, dyp, dxp, A(1) / A(sh.D), mup, rsp, gp, dsp,
+                            dbp, part, {}, {}, {});
+    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
+                       dim3(1024), 0, stream, grid, sh.D, part, dgp, dbtp);
+    return status_of_launch();
   }
 
   const RowGradPlan rp = plan_row_grad<T>(sh.N, sh.G, sh.D, sh.S);

@@ -13,6 +13,7 @@
 // cancellation.
 #include "row_loop.h"
 #include "row_tile.h"
+#include "short_rows.h"
 
 namespace dragon_hip {
 namespace {
@@ -219,6 +220,64 @@ __global__ __launch_bounds__(kLoopThreads) void layer_norm_rows_looped(
   }
 }
 
+// Short rows (per-head normalisations, odd widths): a policy of the LDS-staged
+// kernel (short_rows.h). Mean, then the centred sum of squares, over the kL
+// lanes of a row; gamma / beta of a thread's elements live in registers.
+template <typename T, int kE>
+struct LayerNormShortForward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  A inv_c, eps;
+  const A* gamma;
+  const A* beta;
+  A* mu;
+  A* rsig;
+  A g[kE], b[kE];
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int l, int C) {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const int e = l + j * kL;
+      g[j] = e < C ? gamma[e] : A(0);
+      b[j] = e < C ? beta[e] : A(0);
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A*, int l, int C, A (&v)[kE], const A (&)[kE]) const {
+    A s = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) s += v[j];  // lanes past the row hold 0
+    const A mean = group_allreduce<kL>(s, SumOp()) * inv_c;
+    A q = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const A d = v[j] - mean;
+      q += l + j * kL < C ? d * d : A(0);
+    }
+    const A rs = acc_rsqrt_exact(group_allreduce<kL>(q, SumOp()) * inv_c + eps);
+    if (l == 0) {
+      mu[r] = mean;
+      rsig[r] = rs;
+    }
+#pragma unroll
+    for (int j = 0; j < kE; ++j) v[j] = (v[j] - mean) * rs * g[j] + b[j];
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
+// Rows of up to 512 bytes, and rows of up to 1024 elements that are not whole
+// aligned packets, take the staged kernel (as for softmax).
+inline bool layer_norm_short_rows(int64_t C, size_t elem_bytes, const void* x, const void* y) {
+  if (C > 1024 || !congruent16(x, y)) return false;
+  const size_t row_bytes = static_cast<size_t>(C) * elem_bytes;
+  return row_bytes <= 512 || row_bytes % 16 != 0 || !aligned16(x);
+}
+
 template <typename T>
 int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void* gamma,
                       const void* beta, void* mu, void* rsig, void* y, hipStream_t stream) {
@@ -230,6 +289,14 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
   const A* bp = static_cast<const A*>(beta);
   A* mp = static_cast<A*>(mu);
   A* rp = static_cast<A*>(rsig);
+  ShortPlan sp;
+  if (layer_norm_short_rows(C, sizeof(T), x, y) && plan_short_rows(C, sizeof(T), 4, aligned16(x), &sp)) {
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16;
+    DRAGON_HIP_SHORT_LAUNCH(T, LayerNormShortForward, sp, lds, short_grid(N, sp.rows_per_chunk),
+                            stream, N, static_cast<int>(C), xp, xp, yp, A(1) / A(C), A(eps), gp, bp,
+                            mp, rp, {}, {});
+    return status_of_launch();
+  }
   RowConfig cfg;
   const bool fits = pick_row_config(ceil_div(C, kVec), 8, &cfg);
   const bool packets_ok = fits && C % kVec == 0 && aligned16(x) && aligned16(y) &&

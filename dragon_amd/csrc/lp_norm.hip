@@ -24,6 +24,7 @@
 #include "col_tile.h"
 #include "row_loop.h"
 #include "row_tile.h"
+#include "short_rows.h"
 
 namespace dragon_hip {
 namespace {
@@ -325,6 +326,85 @@ inline unsigned flat_grid(int64_t threads_needed) {
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 
+// Short rows (embedding-sized, odd widths): policies of the LDS-staged kernel
+// (short_rows.h).
+template <typename T, int kP, int kE>
+struct LpNormShortForwardOp {
+  using A = typename IO<T>::Acc;
+  using M = LpMath<T, kP>;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  A normalizer, eps;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A*, int, int, A (&v)[kE], const A (&)[kE]) const {
+    A acc = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) acc += M::term(v[j]);
+    const A norm = M::norm_of(group_allreduce<kL>(acc, SumOp()), normalizer, eps);
+    const A inv = A(1) / norm;
+#pragma unroll
+    for (int j = 0; j < kE; ++j) v[j] = M::forward(v[j], norm, inv);
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename T, int kE>
+using L1NormShortForward = LpNormShortForwardOp<T, 1, kE>;
+template <typename T, int kE>
+using L2NormShortForward = LpNormShortForwardOp<T, 2, kE>;
+
+// in0 = dy (overwritten with dx), in1 = x.
+template <typename T, int kP, int kE>
+struct LpNormShortBackwardOp {
+  using A = typename IO<T>::Acc;
+  using M = LpMath<T, kP>;
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  A normalizer, eps;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A*, int, int, A (&g)[kE], const A (&x)[kE]) const {
+    A acc = A(0), dot = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      acc += M::term(x[j]);
+      dot += g[j] * x[j];
+    }
+    acc = group_allreduce<kL>(acc, SumOp());
+    dot = group_allreduce<kL>(dot, SumOp());
+    const A norm = M::norm_of(acc, normalizer, eps);
+    const A inv = A(1) / norm;
+    const A coef = M::coef_of(dot, normalizer, norm);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) g[j] = M::backward(g[j], x[j], norm, inv, coef);
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename T, int kE>
+using L1NormShortBackward = LpNormShortBackwardOp<T, 1, kE>;
+template <typename T, int kE>
+using L2NormShortBackward = LpNormShortBackwardOp<T, 2, kE>;
+
+// Rows of up to 512 bytes in both directions; longer rows (up to 1024 elements)
+// that are not whole aligned packets forward only, as for softmax.
+inline bool lp_norm_short_rows(int64_t C, size_t elem_bytes, bool grad, const void* a,
+                               const void* b, const void* out) {
+  if (C > 1024 || !congruent16(a, out) || (grad && !congruent16(a, b))) return false;
+  const size_t row_bytes = static_cast<size_t>(C) * elem_bytes;
+  if (row_bytes <= 512) return true;
+  return !grad && (row_bytes % 16 != 0 || !aligned16(a));
+}
+
 template <typename T, int kP, bool kGrad>
 int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsilon,
                    const void* dy, const void* x, void* out, hipStream_t stream) {
@@ -335,6 +415,26 @@ int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsi
   T* op = static_cast<T*>(out);
   const A nrm = static_cast<A>(normalizer), eps = static_cast<A>(epsilon);
   const bool packets_ok = aligned16(x) && aligned16(out) && (!kGrad || aligned16(dy));
+  ShortPlan sp;
+  if (S == 1 && lp_norm_short_rows(C, sizeof(T), kGrad, x, dy, out) &&
+      plan_short_rows(C, sizeof(T), kGrad ? 1 : 4, aligned16(x), &sp)) {
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * (kGrad ? 32 : 16);
+    const unsigned grid = short_grid(N, sp.rows_per_chunk);
+    if constexpr (kGrad && kP == 1) {
+      DRAGON_HIP_SHORT_LAUNCH(T, L1NormShortBackward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), gp, xp, op, nrm, eps);
+    } else if constexpr (kGrad) {
+      DRAGON_HIP_SHORT_LAUNCH(T, L2NormShortBackward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), gp, xp, op, nrm, eps);
+    } else if constexpr (kP == 1) {
+      DRAGON_HIP_SHORT_LAUNCH(T, L1NormShortForward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), xp, xp, op, nrm, eps);
+    } else {
+      DRAGON_HIP_SHORT_LAUNCH(T, L2NormShortForward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), xp, xp, op, nrm, eps);
+    }
+    return status_of_launch();
+  }
   RowConfig cfg;
   // The gradient holds two tiles at once: halve the packets a thread may hold.
   if (S == 1 && pick_row_config(ceil_div(C, kVec), kGrad ? 4 : 8, &cfg)) {

@@ -24,6 +24,7 @@
 #include "col_tile.h"
 #include "row_loop.h"
 #include "row_tile.h"
+#include "short_rows.h"
 #include "slices.h"
 
 namespace dragon_hip {
@@ -801,233 +802,81 @@ size_t softmax_slices_scratch(int64_t N, int64_t S, int64_t C) {
 }
 
 // --------------------------------------------------------------------------
-// Short rows (up to 1024 elements) of any width and alignment, e.g. the
-// 197-key attention rows of a vision transformer. A workgroup takes a run of
-// consecutive rows, i.e. one contiguous byte range: it copies the aligned
-// 16-byte packets that cover the range into LDS, works on the rows there with
-// kL lanes per row (kE elements per lane, so short rows do not idle most of a
-// wavefront), and writes the range back in aligned packets; only the first
-// and last packet of a range are touched element by element. HBM therefore
-// sees aligned, fully coalesced 128-bit accesses whatever the row length.
+// Short rows: policies of the LDS-staged kernel (short_rows.h).
 // --------------------------------------------------------------------------
-constexpr int kShortThreads = 256;
-
-// All-reduce over groups of kL adjacent lanes (kL a power of two, 4 .. 64).
-template <int kL, typename Op>
-__device__ __forceinline__ float group_allreduce(float v, Op op) {
-  v = dpp_step<0xB1>(v, op);                              // quad_perm [1,0,3,2]
-  v = dpp_step<0x4E>(v, op);                              // quad_perm [2,3,0,1]
-  if constexpr (kL >= 8) v = dpp_step<0x141>(v, op);      // row_half_mirror
-  if constexpr (kL >= 16) v = dpp_step<0x140>(v, op);     // row_mirror
-  if constexpr (kL >= 32) v = op(v, __shfl_xor(v, 16, kWaveSize));
-  if constexpr (kL >= 64) v = op(v, __shfl_xor(v, 32, kWaveSize));
-  return v;
-}
-template <int kL, typename Op>
-__device__ __forceinline__ double group_allreduce(double v, Op op) {
-#pragma unroll
-  for (int o = kL / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, kWaveSize));
-  return v;
-}
-
-// The byte range [a0, a1) of a tensor that starts at `base` and has `total`
-// bytes, staged in LDS from the aligned packet that contains a0 on.
-struct StagedRange {
-  uintptr_t base, total;  // the whole tensor
-  uintptr_t a0, a1;       // this range (absolute addresses)
-  uintptr_t first;        // a0 rounded down to 16 bytes
-  uint32_t packets;       // aligned packets covering the range
-  __device__ __forceinline__ StagedRange(const void* tensor, size_t total_bytes, size_t b0,
-                                         size_t b1) {
-    base = reinterpret_cast<uintptr_t>(tensor), total = total_bytes;
-    a0 = base + b0, a1 = base + b1;
-    first = a0 & ~static_cast<uintptr_t>(15);
-    packets = static_cast<uint32_t>((a1 - first + 15) / 16);
-  }
-  __device__ __forceinline__ uint32_t lead() const { return static_cast<uint32_t>(a0 - first); }
-};
-
-// Copies the packets of `r` into stage[0 .. r.packets). A packet that reaches
-// outside the tensor (only the tensor's first or last can) is read element by
-// element; what lies outside reads as zero.
-template <typename T>
-__device__ __forceinline__ void stage_in(const StagedRange& r, u32x4* stage) {
-  for (uint32_t p = threadIdx.x; p < r.packets; p += kShortThreads) {
-    const uintptr_t addr = r.first + 16u * p;
-    if (addr >= r.base && addr + 16 <= r.base + r.total) {
-      stage[p] = *reinterpret_cast<const u32x4*>(addr);
-    } else {
-      T* out = reinterpret_cast<T*>(stage + p);
-#pragma unroll
-      for (uint32_t i = 0; i < 16 / sizeof(T); ++i) {
-        const uintptr_t ea = addr + i * sizeof(T);
-        T zero{};
-        out[i] = (ea >= r.base && ea + sizeof(T) <= r.base + r.total)
-                     ? *reinterpret_cast<const T*>(ea) : zero;
-      }
-    }
-  }
-}
-
-// Writes stage[0 .. r.packets) back to the range `r` of the output: packets
-// inside the range whole, the range's first and last packet element by element
-// (their other elements belong to neighbouring rows of other workgroups).
-template <typename T>
-__device__ __forceinline__ void stage_out(const StagedRange& r, const u32x4* stage) {
-  for (uint32_t p = threadIdx.x; p < r.packets; p += kShortThreads) {
-    const uintptr_t addr = r.first + 16u * p;
-    if (addr >= r.a0 && addr + 16 <= r.a1) {
-      store_packet(reinterpret_cast<T*>(addr), stage[p]);
-    } else {
-      const T* in = reinterpret_cast<const T*>(stage + p);
-#pragma unroll
-      for (uint32_t i = 0; i < 16 / sizeof(T); ++i) {
-        const uintptr_t ea = addr + i * sizeof(T);
-        if (ea >= r.a0 && ea + sizeof(T) <= r.a1) *reinterpret_cast<T*>(ea) = in[i];
-      }
-    }
-  }
-}
-
-// x and y must be congruent modulo 16 bytes (they usually are: allocations are
-// aligned far beyond that), so that the staged packets map one to one.
-template <typename T, int kKind, int kL, int kE>
-__global__ __launch_bounds__(kShortThreads) void softmax_short_rows(
-    const int64_t N, const int C, const uint32_t rows_per_chunk, const T* x, T* y) {
+template <typename T, int kKind, int kE>
+struct SoftmaxShortForwardOp {
   using A = typename IO<T>::Acc;
   using M = SoftmaxMath<T>;
-  extern __shared__ u32x4 stage[];
-  const size_t row_bytes = static_cast<size_t>(C) * sizeof(T);
-  const size_t total = static_cast<size_t>(N) * row_bytes;
-  const int l = threadIdx.x % kL;
-  const int sub = threadIdx.x / kL;
-  constexpr int kRowsPerPass = kShortThreads / kL;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rows_per_chunk; row0 < N;
-       row0 += static_cast<int64_t>(gridDim.x) * rows_per_chunk) {
-    const int rows = static_cast<int>(N - row0 < rows_per_chunk ? N - row0 : rows_per_chunk);
-    const StagedRange in(x, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    stage_in<T>(in, stage);
-    __syncthreads();
-    T* tile = reinterpret_cast<T*>(reinterpret_cast<char*>(stage) + in.lead());
-    for (int r = sub; r < rows; r += kRowsPerPass) {
-      T* row = tile + static_cast<size_t>(r) * C;
-      A v[kE];
-      A m = acc_neg_inf<A>();
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  __device__ __forceinline__ A fill0() const { return acc_neg_inf<A>(); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A*, int, int, A (&v)[kE], const A (&)[kE]) const {
+    A m = acc_neg_inf<A>();
 #pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
-        v[j] = e < C ? IO<T>::load1(row + e) : acc_neg_inf<A>();
-        m = MaxOp()(m, v[j]);
-      }
-      m = group_allreduce<kL>(m, MaxOp());
-      A s = A(0);
+    for (int j = 0; j < kE; ++j) m = MaxOp()(m, v[j]);
+    m = group_allreduce<kL>(m, MaxOp());
+    A s = A(0);
 #pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        if (kKind == kSoftmax) {
-          v[j] = M::exp_of(v[j] - m);  // lanes past the row: exp(-inf) = 0
-          s += v[j];
-        } else {
-          v[j] = v[j] - m;
-          s += M::exp_of(v[j]);
-        }
-      }
-      s = group_allreduce<kL>(s, SumOp());
-      const A inv = A(1) / s;
-      const A lg = acc_log(s);
-#pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
-        if (e < C) IO<T>::store1(row + e, kKind == kSoftmax ? M::normalise(v[j], s, inv) : v[j] - lg);
+    for (int j = 0; j < kE; ++j) {
+      if (kKind == kSoftmax) {
+        v[j] = M::exp_of(v[j] - m);  // lanes past the row: exp(-inf) = 0
+        s += v[j];
+      } else {
+        v[j] = v[j] - m;
+        s += M::exp_of(v[j]);
       }
     }
-    __syncthreads();
-    const StagedRange out(y, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    stage_out<T>(out, stage);
-    __syncthreads();  // the stage is refilled by the next range
+    s = group_allreduce<kL>(s, SumOp());
+    const A inv = A(1) / s;
+    const A lg = acc_log(s);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) v[j] = kKind == kSoftmax ? M::normalise(v[j], s, inv) : v[j] - lg;
   }
-}
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename T, int kE>
+using SoftmaxShortForward = SoftmaxShortForwardOp<T, kSoftmax, kE>;
+template <typename T, int kE>
+using LogSoftmaxShortForward = SoftmaxShortForwardOp<T, kLogSoftmax, kE>;
 
-// dx from dy and y; the three tensors congruent modulo 16 bytes.
-template <typename T, int kKind, int kL, int kE>
-__global__ __launch_bounds__(kShortThreads) void softmax_grad_short_rows(
-    const int64_t N, const int C, const uint32_t rows_per_chunk, const uint32_t stage_packets,
-    const T* dy, const T* y, T* dx) {
+// in0 = dy (overwritten with dx), in1 = y.
+template <typename T, int kKind, int kE>
+struct SoftmaxShortBackwardOp {
   using A = typename IO<T>::Acc;
   using M = SoftmaxMath<T>;
-  extern __shared__ u32x4 stage[];
-  u32x4* stage_y = stage + stage_packets;
-  const size_t row_bytes = static_cast<size_t>(C) * sizeof(T);
-  const size_t total = static_cast<size_t>(N) * row_bytes;
-  const int l = threadIdx.x % kL;
-  const int sub = threadIdx.x / kL;
-  constexpr int kRowsPerPass = kShortThreads / kL;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rows_per_chunk; row0 < N;
-       row0 += static_cast<int64_t>(gridDim.x) * rows_per_chunk) {
-    const int rows = static_cast<int>(N - row0 < rows_per_chunk ? N - row0 : rows_per_chunk);
-    const StagedRange in_g(dy, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    const StagedRange in_y(y, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    stage_in<T>(in_g, stage);
-    stage_in<T>(in_y, stage_y);
-    __syncthreads();
-    T* tile_g = reinterpret_cast<T*>(reinterpret_cast<char*>(stage) + in_g.lead());
-    const T* tile_y = reinterpret_cast<const T*>(reinterpret_cast<const char*>(stage_y) + in_y.lead());
-    for (int r = sub; r < rows; r += kRowsPerPass) {
-      T* row_g = tile_g + static_cast<size_t>(r) * C;
-      const T* row_y = tile_y + static_cast<size_t>(r) * C;
-      A g[kE], o[kE];
-      A s = A(0);
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return kKind == kSoftmax ? A(0) : acc_neg_inf<A>(); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A*, int, int, A (&g)[kE], const A (&o)[kE]) const {
+    A s = A(0);
 #pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
-        g[j] = e < C ? IO<T>::load1(row_g + e) : A(0);
-        o[j] = e < C ? IO<T>::load1(row_y + e) : (kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
-        s += kKind == kSoftmax ? g[j] * o[j] : g[j];
-      }
-      s = group_allreduce<kL>(s, SumOp());
+    for (int j = 0; j < kE; ++j) s += kKind == kSoftmax ? g[j] * o[j] : g[j];
+    s = group_allreduce<kL>(s, SumOp());
 #pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
-        if (e < C) {
-          IO<T>::store1(row_g + e, kKind == kSoftmax ? (g[j] - s) * o[j] : g[j] - M::exp_of(o[j]) * s);
-        }
-      }
+    for (int j = 0; j < kE; ++j) {
+      g[j] = kKind == kSoftmax ? (g[j] - s) * o[j] : g[j] - M::exp_of(o[j]) * s;
     }
-    __syncthreads();
-    const StagedRange out(dx, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    stage_out<T>(out, stage);
-    __syncthreads();
   }
-}
-
-// Lanes per row and elements per lane for rows of C elements, the rows a
-// workgroup stages at a time (about 16 KB) and the LDS that takes.
-struct ShortPlan {
-  int lanes, per_lane;
-  uint32_t rows_per_chunk, stage_packets;
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
 };
-inline bool plan_short_rows(int64_t C, size_t elem_bytes, size_t stage_bytes, ShortPlan* p) {
-  if (C > 1024) return false;
-  int lanes = 4;
-  while (lanes < 64 && C > lanes * 8) lanes <<= 1;
-  p->lanes = lanes;
-  p->per_lane = C <= lanes * 8 ? 8 : 16;
-  const size_t row_bytes = static_cast<size_t>(C) * elem_bytes;
-  const uint32_t per_pass = kShortThreads / lanes;
-  uint32_t rows = static_cast<uint32_t>(stage_bytes / row_bytes);
-  rows = rows / per_pass * per_pass;
-  if (rows < per_pass) rows = per_pass;
-  p->rows_per_chunk = rows;
-  p->stage_packets = static_cast<uint32_t>((rows * row_bytes + 15) / 16 + 2);
-  return true;
-}
-inline unsigned short_grid(int64_t N, uint32_t rows_per_chunk) {
-  const int64_t chunks = ceil_div(N, rows_per_chunk);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 16;
-  return static_cast<unsigned>(chunks < cap ? chunks : cap);
-}
-inline bool congruent16(const void* a, const void* b) {
-  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
-}
+template <typename T, int kE>
+using SoftmaxShortBackward = SoftmaxShortBackwardOp<T, kSoftmax, kE>;
+template <typename T, int kE>
+using LogSoftmaxShortBackward = SoftmaxShortBackwardOp<T, kLogSoftmax, kE>;
+
 // Which rows take the staged path. Measured on MI355X (fraction of the HBM peak,
 // staged against the register tiles): rows of up to 512 bytes gain in both
 // directions (bf16 [1M,64] 0.68 / 0.77 against 0.18 / 0.38, bf16 [605184,197]
@@ -1043,16 +892,6 @@ inline bool use_short_rows(int64_t C, size_t elem_bytes, bool forward, const voi
   const bool regular = row_bytes % 16 == 0 && aligned16(a);
   return forward && !regular;
 }
-#define DRAGON_HIP_SHORT_SWITCH(sp, LAUNCH)                        \
-  if (sp.per_lane == 8) {                                          \
-    if (sp.lanes == 4) LAUNCH(4, 8)                                \
-    else if (sp.lanes == 8) LAUNCH(8, 8)                           \
-    else if (sp.lanes == 16) LAUNCH(16, 8)                         \
-    else if (sp.lanes == 32) LAUNCH(32, 8)                         \
-    else LAUNCH(64, 8)                                             \
-  } else {                                                         \
-    LAUNCH(64, 16)                                                 \
-  }
 
 inline unsigned flat_grid(int64_t threads_needed) {
   const int64_t want = ceil_div(threads_needed, 256);
@@ -1076,14 +915,17 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
     }
   }
   ShortPlan sp;
-  if (S == 1 && use_short_rows(C, sizeof(T), true, x, y) && plan_short_rows(C, sizeof(T), 16384, &sp)) {
+  if (S == 1 && use_short_rows(C, sizeof(T), true, x, y) &&
+      plan_short_rows(C, sizeof(T), 4, aligned16(x), &sp)) {
     const size_t lds = static_cast<size_t>(sp.stage_packets) * 16;
-    const dim3 grid(short_grid(N, sp.rows_per_chunk)), block(kShortThreads);
-#define LAUNCH(L, E)                                                                          \
-  hipLaunchKernelGGL((softmax_short_rows<T, kKind, L, E>), grid, block, lds, stream, N,       \
-                     static_cast<int>(C), sp.rows_per_chunk, xp, yp);
-    DRAGON_HIP_SHORT_SWITCH(sp, LAUNCH);
-#undef LAUNCH
+    const unsigned grid = short_grid(N, sp.rows_per_chunk);
+    if (kKind == kSoftmax) {
+      DRAGON_HIP_SHORT_LAUNCH(T, SoftmaxShortForward, sp, lds, grid, stream, N, static_cast<int>(C),
+                              xp, xp, yp, );
+    } else {
+      DRAGON_HIP_SHORT_LAUNCH(T, LogSoftmaxShortForward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), xp, xp, yp, );
+    }
     return status_of_launch();
   }
   RowConfig cfg;
@@ -1184,15 +1026,18 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
     }
   }
   ShortPlan sp;
+  // two staged tensors: 4 KB each keeps eight workgroups per compute unit
   if (S == 1 && use_short_rows(C, sizeof(T), false, dy, y) && congruent16(dy, dx) &&
-      plan_short_rows(C, sizeof(T), 4096, &sp)) {  // two staged tensors: 4 KB each keeps eight workgroups per CU
+      plan_short_rows(C, sizeof(T), 1, aligned16(dy), &sp)) {
     const size_t lds = static_cast<size_t>(sp.stage_packets) * 32;
-    const dim3 grid(short_grid(N, sp.rows_per_chunk)), block(kShortThreads);
-#define LAUNCH(L, E)                                                                          \
-  hipLaunchKernelGGL((softmax_grad_short_rows<T, kKind, L, E>), grid, block, lds, stream, N,  \
-                     static_cast<int>(C), sp.rows_per_chunk, sp.stage_packets, gp, yp, dp);
-    DRAGON_HIP_SHORT_SWITCH(sp, LAUNCH);
-#undef LAUNCH
+    const unsigned grid = short_grid(N, sp.rows_per_chunk);
+    if (kKind == kSoftmax) {
+      DRAGON_HIP_SHORT_LAUNCH(T, SoftmaxShortBackward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), gp, yp, dp, );
+    } else {
+      DRAGON_HIP_SHORT_LAUNCH(T, LogSoftmaxShortBackward, sp, lds, grid, stream, N,
+                              static_cast<int>(C), gp, yp, dp, );
+    }
     return status_of_launch();
   }
   RowConfig cfg;

@@ -43,7 +43,9 @@ def oracle_dtype_inputs(bits, dtype):
 # ---------------------------------------------------------------- LayerNorm forward
 
 LN_SHAPES = [(64, 1024), (33, 1000), (7, 12288), (5, 4096), (300, 48), (3, 37), (9, 8),
-             (2, 70000), (1, 1), (513, 256)]
+             (2, 70000), (1, 1), (513, 256),
+             # short and odd rows staged through LDS (several ranges per workgroup)
+             (5000, 64), (700, 197), (130, 577), (9000, 16)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
@@ -290,7 +292,10 @@ def test_softmax_masked_logits_are_exact_zero(K):
 # ---------------------------------------------------------------- LayerNorm backward
 
 LNB_SHAPES = [(64, 1024), (33, 1000), (16, 12288), (300, 48), (5, 37), (1100, 256), (40, 4096),
-              (3, 20000), (2, 8)]
+              (3, 20000), (2, 8),
+              # short and odd rows staged through LDS: several ranges per workgroup, 8 to 64
+              # lanes per row, a last range that is not full
+              (5000, 64), (700, 197), (130, 577), (9000, 16)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
@@ -626,7 +631,9 @@ def test_math_helpers_bitwise(K):
 
 LP_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 70000), -1), ((5, 37), -1),
              ((6, 300), -1), ((3, 7, 5), 1), ((2, 3, 4, 16), 2), ((4, 1), -1), ((2, 16, 8, 8), 1),
-             ((3, 8200), -1), ((2, 40, 24), 1)]
+             ((3, 8200), -1), ((2, 40, 24), 1),
+             # short and odd rows staged through LDS
+             ((5000, 64), -1), ((700, 197), -1), ((130, 577), -1)]
 
 
 def _lp_fp64(x, dy, ax, p, normalizer, eps):
