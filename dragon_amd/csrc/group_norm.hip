@@ -161,7 +161,10 @@ struct GroupNormGradApply {
 // Per element, with the row scalars a = (db*mu - ds)*rsig^3/C, b = -db*rsig/C:
 //   xc = x - mu;  w = dy*rsig;  dgamma += w*xc;  dbeta += dy;
 //   dx = gamma*w + (a*xc + b)
-template <typename T, int kTPR, int kVPT, int kGradThreads>
+// The ragged flavour takes rows of any width at element-aligned addresses:
+// exact (branching) loads that zero what lies past a row, element-wise stores
+// for a row's partial last packet; gamma is staged element by element.
+template <typename T, int kTPR, int kVPT, int kGradThreads, bool kRagged = false>
 __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void layer_norm_grad_rows(
     const int64_t N, const int C, const T* __restrict__ x, const T* __restrict__ dy,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
@@ -185,12 +188,19 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   __shared__ A slots[2 * Tile::kSlots];
   __shared__ A red[kRedWords];
   const A* lds_gamma = reinterpret_cast<const A*>(staged);
-  for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
-    staged[i] = load_packet(gamma + i * kPerPacket);
+  const int npackets = (C + kVec - 1) / kVec;
+  if constexpr (kRagged) {
+    A* stage_gamma = reinterpret_cast<A*>(staged);
+    for (int i = threadIdx.x; i < npackets * kVec; i += kGradThreads) {
+      stage_gamma[i] = i < C ? gamma[i] : A(0);
+    }
+  } else {
+    for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
+      staged[i] = load_packet(gamma + i * kPerPacket);
+    }
   }
   __syncthreads();
 
-  const int npackets = C / kVec;
   const int lane = Tile::lane();
   const int sub = Tile::sub_row();
   const A inv_c = A(1) / A(C);
@@ -212,8 +222,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   // such rows skip the second pass, and such slots only ever feed accumulators
   // of columns that are not written out.
   Raw tx, tdy;
-  tx.load_unmasked(x + (row < N ? row : 0) * C, npackets);
-  tdy.load_unmasked(dy + (row < N ? row : 0) * C, npackets);
+  if constexpr (kRagged) {
+    tx.load_any(x + (row < N ? row : 0) * C, C);
+    tdy.load_any(dy + (row < N ? row : 0) * C, C);
+  } else {
+    tx.load_unmasked(x + (row < N ? row : 0) * C, npackets);
+    tdy.load_unmasked(dy + (row < N ? row : 0) * C, npackets);
+  }
   A m = mu[row < N ? row : 0];
   A r = rsig[row < N ? row : 0];
   Raw px[kDepth], pdy[kDepth];  // rows row + stride .. row + kDepth * stride
@@ -222,8 +237,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   for (int k = 0; k + 1 < kDepth; ++k) {
     const int64_t ahead = row + (k + 1) * stride;
     const bool ok = ahead < N;
-    px[k].load_unmasked(x + (ok ? ahead : 0) * C, npackets);
-    pdy[k].load_unmasked(dy + (ok ? ahead : 0) * C, npackets);
+    if constexpr (kRagged) {
+      px[k].load_any(x + (ok ? ahead : 0) * C, C);
+      pdy[k].load_any(dy + (ok ? ahead : 0) * C, C);
+    } else {
+      px[k].load_unmasked(x + (ok ? ahead : 0) * C, npackets);
+      pdy[k].load_unmasked(dy + (ok ? ahead : 0) * C, npackets);
+    }
     pm[k] = mu[ok ? ahead : 0];
     pr[k] = rsig[ok ? ahead : 0];
   }
@@ -232,8 +252,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     {
       const int64_t far = row + kDepth * stride;
       const bool ok = far < N;
-      px[kDepth - 1].load_unmasked(x + (ok ? far : 0) * C, npackets);
-      pdy[kDepth - 1].load_unmasked(dy + (ok ? far : 0) * C, npackets);
+      if constexpr (kRagged) {
+        px[kDepth - 1].load_any(x + (ok ? far : 0) * C, C);
+        pdy[kDepth - 1].load_any(dy + (ok ? far : 0) * C, C);
+      } else {
+        px[kDepth - 1].load_unmasked(x + (ok ? far : 0) * C, npackets);
+        pdy[kDepth - 1].load_unmasked(dy + (ok ? far : 0) * C, npackets);
+      }
       pm[kDepth - 1] = mu[ok ? far : 0];
       pr[kDepth - 1] = rsig[ok ? far : 0];
     }
@@ -293,7 +318,19 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (valid && Tile::active(i, npackets)) {
-        store_packet(dxr + static_cast<int64_t>(i * kTPR + lane) * kVec, out[i]);
+        const int col = (i * kTPR + lane) * kVec;
+        if constexpr (!kRagged) {
+          store_packet(dxr + col, out[i]);
+        } else if (col + kVec <= C) {
+          store_packet_unaligned(dxr + col, out[i]);
+        } else {
+          A last[kVec];
+          IO<T>::unpack(out[i], last);
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (col + e < C) IO<T>::store1(dxr + col + e, last[e]);
+          }
+        }
       }
     }
     if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
@@ -337,11 +374,14 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
             pb[e] += w[2 * e + 1];
           }
         }
-        A* o = out + (static_cast<size_t>(i * kTPR + lane) * kVec + h * kChunk) * 2;
+        const int col = (i * kTPR + lane) * kVec + h * kChunk;
+        A* o = out + static_cast<size_t>(col) * 2;
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
-          o[2 * e] = pg[e];
-          o[2 * e + 1] = pb[e];
+          if (!kRagged || col + e < C) {
+            o[2 * e] = pg[e];
+            o[2 * e + 1] = pb[e];
+          }
         }
       }
     }
@@ -1112,6 +1152,7 @@ struct RowGradPlan {
   RowConfig cfg;
   int threads;  // workgroup size: 512 (two per compute unit) or 1024 (one)
   unsigned grid;
+  bool ragged;  // rows that are not whole packets
 };
 
 // Tiles of the fused row path: the fewest threads per row that hold it with at
@@ -1119,18 +1160,21 @@ struct RowGradPlan {
 // prefetched one and two accumulator sets must fit 128 registers).
 template <typename T>
 RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
-  RowGradPlan p = {false, {0, 0}, 512, 0};
+  RowGradPlan p = {false, {0, 0}, 512, 0, false};
   if (G != 1 || S != 1) return p;
   constexpr int kVec = IO<T>::kVec;
   constexpr int kMaxVpt = kVec == 8 ? 2 : 4;
-  if (D % kVec != 0 || static_cast<size_t>(D) * sizeof(typename IO<T>::Acc) > kMaxStagedParamBytes / 2) {
+  // staged gamma, padded to whole packets of the row
+  if (static_cast<size_t>(ceil_div(D, kVec) * kVec) * sizeof(typename IO<T>::Acc) >
+      kMaxStagedParamBytes / 2) {
     return p;
   }
+  p.ragged = D % kVec != 0;
   static const RowConfig table[] = {{64, 1},  {64, 2},  {256, 1},  {256, 2},  {512, 1},
                                     {512, 2}, {1024, 1}, {768, 2}, {1024, 2}, {1024, 4}};
   bool found = false;
   for (const RowConfig& c : table) {
-    if (!found && c.vpt <= kMaxVpt && D / kVec <= static_cast<int64_t>(c.tpr) * c.vpt) {
+    if (!found && c.vpt <= kMaxVpt && ceil_div(D, kVec) <= static_cast<int64_t>(c.tpr) * c.vpt) {
       p.cfg = c;
       found = true;
     }
@@ -1513,11 +1557,15 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   }
 
   const RowGradPlan rp = plan_row_grad<T>(sh.N, sh.G, sh.D, sh.S);
-  if (rp.use_rows && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma)) {
-    const size_t staged_bytes = static_cast<size_t>(sh.D) * sizeof(A);
+  if (rp.use_rows) {
+    // rows of whole aligned packets, or the ragged flavour for any width and alignment
+    const bool ragged =
+        rp.ragged || !(aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma));
+    const size_t staged_bytes = static_cast<size_t>(ceil_div(sh.D, kVec) * kVec) * sizeof(A);
 #define LAUNCH_T(TPR, VPT, THREADS)                                                           \
   {                                                                                           \
-    auto kernel = layer_norm_grad_rows<T, TPR, VPT, THREADS>;                                 \
+    auto kernel = ragged ? layer_norm_grad_rows<T, TPR, VPT, THREADS, true>                   \
+                         : layer_norm_grad_rows<T, TPR, VPT, THREADS, false>;                 \
     if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, THREADS, staged_bytes);         \
     hipLaunchKernelGGL(kernel, dim3(rp.grid), dim3(THREADS), staged_bytes, stream,            \
                        static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp, mup,  \

@@ -295,7 +295,9 @@ LNB_SHAPES = [(64, 1024), (33, 1000), (16, 12288), (300, 48), (5, 37), (1100, 25
               (3, 20000), (2, 8),
               # short and odd rows staged through LDS: several ranges per workgroup, 8 to 64
               # lanes per row, a last range that is not full
-              (5000, 64), (700, 197), (130, 577), (9000, 16)]
+              (5000, 64), (700, 197), (130, 577), (9000, 16),
+              # wider rows that are not whole packets: the ragged flavour of the fused kernel
+              (70, 1030), (300, 4097), (33, 12289)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
