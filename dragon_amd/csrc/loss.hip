@@ -22,6 +22,7 @@
 #include <cfloat>
 
 #include "row_tile.h"
+#include "short_rows.h"
 
 namespace dragon_hip {
 namespace {
@@ -309,6 +310,62 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_ce_rows(
   }
 }
 
+// The same for short rows (a handful to a few hundred classes): a policy of the
+// LDS-staged kernel (short_rows.h), several rows per wavefront. The row's target
+// travels as the per-row scalar: its column, or -1 when ignored.
+template <typename T, typename TargetT, int kE>
+struct SoftmaxCeShortOp {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 1;
+  int64_t ignore_index;
+  int classes;
+  const TargetT* target;
+  T* loss;
+  T* mask;
+  __device__ __forceinline__ A fill0() const { return acc_neg_inf<A>(); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[1]) const {
+    const TargetT tgt = target[row];
+    w[0] = target_valid(tgt, ignore_index, classes) ? static_cast<A>(tgt) : A(-1);  // < 1024: exact
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A* side, int l, int, A (&v)[kE],
+                                      const A (&)[kE]) const {
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int j = 0; j < kE; ++j) m = MaxOp()(m, v[j]);
+    m = group_allreduce<kL>(m, MaxOp());
+    A s = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      v[j] = acc_exp(v[j] - m);  // lanes past the row: exp(-inf) = 0
+      s += v[j];
+    }
+    s = group_allreduce<kL>(s, SumOp());
+    const int col = static_cast<int>(side[0]);
+    const A inv = A(1) / s;
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      v[j] = sizeof(A) == 4 ? v[j] * inv : v[j] / s;
+      if (l + j * kL == col) {
+        loss[r] = neg_log_clamped(v[j]);
+        mask[r] = T(1);
+      }
+    }
+    if (col < 0 && l == 0) loss[r] = mask[r] = T(0);
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename T, int kE>
+using SoftmaxCeShortI32 = SoftmaxCeShortOp<T, int32_t, kE>;
+template <typename T, int kE>
+using SoftmaxCeShortI64 = SoftmaxCeShortOp<T, int64_t, kE>;
+
 // The same for rows that take a whole 1024-thread workgroup: persistent
 // workgroups that request the next row's packets before reducing the current
 // one (see softmax_wide_rows).
@@ -584,8 +641,24 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
   T* loss = reduction == kNone ? static_cast<T*>(out) : static_cast<T*>(scratch);
   T* mask = static_cast<T*>(scratch) + NxS;
   T* part = mask + NxS;
-  RowConfig cfg;
-  if (S == 1 && pick_row_config(ceil_div(C, kVec), 8, &cfg)) {
+  ShortPlan sp;
+  // rows of up to 512 bytes, and longer rows that are not whole aligned packets
+  if (S == 1 && C <= 1024 && congruent16(x, prob) &&
+      (C * sizeof(T) <= 512 || (C * sizeof(T)) % 16 != 0 || !aligned16(x)) &&
+      plan_short_rows(C, sizeof(T), 4, aligned16(x), &sp)) {
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 + sp.rows_per_chunk * sizeof(T);
+    const unsigned grid = short_grid(N, sp.rows_per_chunk);
+    if constexpr (sizeof(TargetT) == 4) {
+      DRAGON_HIP_SHORT_LAUNCH(T, SoftmaxCeShortI32, sp, lds, grid, stream, N, static_cast<int>(C),
+                              xp, xp, pp, ignore_index, static_cast<int>(C),
+                              reinterpret_cast<const int32_t*>(tp), loss, mask);
+    } else {
+      DRAGON_HIP_SHORT_LAUNCH(T, SoftmaxCeShortI64, sp, lds, grid, stream, N, static_cast<int>(C),
+                              xp, xp, pp, ignore_index, static_cast<int>(C),
+                              reinterpret_cast<const int64_t*>(tp), loss, mask);
+    }
+  } else
+  if (RowConfig cfg; S == 1 && pick_row_config(ceil_div(C, kVec), 8, &cfg)) {
     const bool regular = C % kVec == 0 && aligned16(x) && aligned16(prob);  // else ragged tiles
     if (regular && cfg.tpr == 1024) {
 #define LAUNCH_WIDE(VPT)                                                                        \
