@@ -248,6 +248,11 @@ WORKLOADS = {
     "softmax_cross_entropy_f32_8192x4096": lambda: wl_softmax_cross_entropy(8192, 4096),
     "l2_norm_bf16_8192x4096": lambda: wl_lp_norm(8192, 4096, "bfloat16", 2),
     "l2_norm_f32_8192x4096": lambda: wl_lp_norm(8192, 4096, "float32", 2),
+    # shapes at the ends of the row-length range: attention rows of a vision transformer,
+    # per-head normalisation, vocabulary-sized logits
+    "softmax_bf16_605184x197": lambda: wl_softmax((605184, 197), "bfloat16", 1),
+    "layer_norm_bf16_1048576x64": lambda: wl_layer_norm(1048576, 64, "bfloat16", 4),
+    "softmax_f32_2048x128256": lambda: wl_softmax((2048, 128256), "float32", 1),
 }
 
 
