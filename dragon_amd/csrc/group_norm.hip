@@ -498,6 +498,188 @@ inline unsigned short_grad_grid(int64_t N, uint32_t rows_per_chunk) {
 }
 
 // --------------------------------------------------------------------------
+// LayerNorm backward of rows wider than the register tiles (flattened feature
+// maps, vocabulary-sized rows): two passes over x and dy.
+//   1. row sums: a row is cut into `splits` column ranges, one workgroup each,
+//      which writes the range's (sum gamma*dy*x, sum gamma*dy) pair;
+//   2. a workgroup owns 256*kW adjacent columns of a chunk of rows: a thread
+//      keeps gamma, dgamma and dbeta of its kW columns in registers, walks the
+//      chunk's rows (adding up the row's pairs in fixed order), writes dx and
+//      leaves one partial (dgamma, dbeta) row per chunk for sum_partial_rows.
+// kW is a whole packet for rows of aligned packets and 1 otherwise.
+// --------------------------------------------------------------------------
+constexpr int kWideRowsAhead = 4;  // rows whose loads are in flight per thread
+
+struct WideGradPlan {
+  uint32_t col_blocks;      // workgroups across a row in the second pass
+  uint32_t row_chunks;      // partial (dgamma, dbeta) rows
+  uint32_t rows_per_chunk;
+  uint32_t splits;          // workgroups per row in the first pass
+  uint32_t split_cols;      // columns per split, whole workgroup tiles
+};
+
+inline WideGradPlan plan_wide_grad(int64_t N, int64_t D, int kw) {
+  WideGradPlan p;
+  const int64_t tile = static_cast<int64_t>(kReduceThreads) * kw;
+  const int64_t col_blocks = ceil_div(D, tile);
+  // first pass: enough workgroups for the chip, at least four tiles each
+  int64_t splits = ceil_div(static_cast<int64_t>(kNumCUs) * 4, N);
+  const int64_t max_splits = col_blocks / 4 > 1 ? col_blocks / 4 : 1;
+  if (splits > max_splits) splits = max_splits;
+  const int64_t tiles_per_split = ceil_div(col_blocks, splits);
+  splits = ceil_div(col_blocks, tiles_per_split);
+  // second pass: about eight workgroups per compute unit, eight rows or more per chunk
+  int64_t chunks = ceil_div(static_cast<int64_t>(kNumCUs) * 8, col_blocks);
+  const int64_t max_chunks = N / 8 > 1 ? N / 8 : 1;
+  if (chunks > max_chunks) chunks = max_chunks;
+  const int64_t rows_per_chunk = ceil_div(N, chunks);
+  chunks = ceil_div(N, rows_per_chunk);
+  p.col_blocks = static_cast<uint32_t>(col_blocks);
+  p.row_chunks = static_cast<uint32_t>(chunks);
+  p.rows_per_chunk = static_cast<uint32_t>(rows_per_chunk);
+  p.splits = static_cast<uint32_t>(splits);
+  p.split_cols = static_cast<uint32_t>(tiles_per_split * tile);
+  return p;
+}
+
+// Words of scratch: the row pairs (rounded to whole packets), then the partial rows.
+inline size_t wide_grad_pair_words(int64_t N, const WideGradPlan& p) {
+  return (static_cast<size_t>(N) * p.splits * 2 + 3) / 4 * 4;
+}
+inline size_t wide_grad_words(int64_t N, int64_t D, int kw) {
+  const WideGradPlan p = plan_wide_grad(N, D, kw);
+  return wide_grad_pair_words(N, p) + static_cast<size_t>(p.row_chunks) * D * 2;
+}
+
+template <typename T, int kW>
+__device__ __forceinline__ void load_run(const T* p, typename IO<T>::Acc (&v)[kW]) {
+  if constexpr (kW == 1) {
+    v[0] = IO<T>::load1(p);
+  } else {
+    IO<T>::unpack(load_packet(p), v);
+  }
+}
+template <int kW, typename A>
+__device__ __forceinline__ void load_param_run(const A* p, A (&v)[kW]) {
+  if constexpr (kW == 1) {
+    v[0] = *p;
+  } else {
+    load_params<kW>(p, v);
+  }
+}
+
+template <typename T, int kW>
+__global__ __launch_bounds__(kReduceThreads) void layer_norm_wide_row_sums(
+    const int D, const WideGradPlan p, const T* __restrict__ x, const T* __restrict__ dy,
+    const typename IO<T>::Acc* __restrict__ gamma, typename IO<T>::Acc* __restrict__ pairs) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds[2 * kReduceWaves];
+  const int64_t row = blockIdx.x / p.splits;
+  const uint32_t split = blockIdx.x % p.splits;
+  const int c0 = static_cast<int>(split * p.split_cols);
+  const int c1 = D - c0 < static_cast<int>(p.split_cols) ? D : c0 + static_cast<int>(p.split_cols);
+  const T* xr = x + row * D;
+  const T* dyr = dy + row * D;
+  A s1 = A(0), s2 = A(0);
+#pragma unroll 4
+  for (int c = c0 + static_cast<int>(threadIdx.x) * kW; c < c1; c += kReduceThreads * kW) {
+    A xv[kW], dv[kW], g[kW];
+    load_run<T, kW>(xr + c, xv);
+    load_run<T, kW>(dyr + c, dv);
+    load_param_run<kW>(gamma + c, g);
+#pragma unroll
+    for (int e = 0; e < kW; ++e) {
+      const A t = g[e] * dv[e];
+      s1 += t * xv[e];
+      s2 += t;
+    }
+  }
+  block_reduce_pair(s1, s2, lds);
+  if (threadIdx.x == 0) {
+    pairs[static_cast<size_t>(blockIdx.x) * 2] = s1;
+    pairs[static_cast<size_t>(blockIdx.x) * 2 + 1] = s2;
+  }
+}
+
+template <typename T, int kW>
+__global__ __launch_bounds__(kReduceThreads) void layer_norm_wide_grad(
+    const int64_t N, const int D, const WideGradPlan p, const T* __restrict__ x,
+    const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
+    const typename IO<T>::Acc* __restrict__ mu, const typename IO<T>::Acc* __restrict__ rsig,
+    const typename IO<T>::Acc* __restrict__ pairs, typename IO<T>::Acc* __restrict__ ds,
+    typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  const uint32_t block = blockIdx.x % p.col_blocks;  // neighbours share rows
+  const uint32_t chunk = blockIdx.x / p.col_blocks;
+  const int col = static_cast<int>(block * kReduceThreads + threadIdx.x) * kW;
+  const bool active = col < D;
+  const int at = active ? col : 0;  // threads past the row address its start and store nothing
+  const bool reports = block == 0 && threadIdx.x == 0;
+  const A inv_d = A(1) / A(D);
+  A g[kW], dg[kW], dbt[kW];
+  load_param_run<kW>(gamma + at, g);
+#pragma unroll
+  for (int e = 0; e < kW; ++e) dg[e] = dbt[e] = A(0);
+
+  const int64_t r0 = static_cast<int64_t>(chunk) * p.rows_per_chunk;
+  const int64_t r1 = N - r0 < static_cast<int64_t>(p.rows_per_chunk) ? N : r0 + p.rows_per_chunk;
+  for (int64_t r = r0; r < r1; r += kWideRowsAhead) {
+    A xv[kWideRowsAhead][kW], dv[kWideRowsAhead][kW];
+    A m[kWideRowsAhead], rs[kWideRowsAhead], s1[kWideRowsAhead], s2[kWideRowsAhead];
+#pragma unroll
+    for (int u = 0; u < kWideRowsAhead; ++u) {
+      const int64_t rr = r + u < r1 ? r + u : r1 - 1;  // uniform over the workgroup
+      load_run<T, kW>(x + rr * D + at, xv[u]);
+      load_run<T, kW>(dy + rr * D + at, dv[u]);
+      m[u] = mu[rr];
+      rs[u] = rsig[rr];
+      s1[u] = s2[u] = A(0);
+      const A* pr = pairs + static_cast<size_t>(rr) * p.splits * 2;
+      for (uint32_t s = 0; s < p.splits; ++s) {
+        s1[u] += pr[2 * s];
+        s2[u] += pr[2 * s + 1];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kWideRowsAhead; ++u) {
+      if (r + u < r1) {
+        if (reports) {
+          ds[r + u] = s1[u];
+          db[r + u] = s2[u];
+        }
+        const A a = (s2[u] * m[u] - s1[u]) * (rs[u] * rs[u] * rs[u]) * inv_d;
+        const A b = -(s2[u] * rs[u]) * inv_d;
+        if (active) {
+#pragma unroll
+          for (int e = 0; e < kW; ++e) {
+            const A xc = xv[u][e] - m[u];
+            const A w = dv[u][e] * rs[u];
+            dg[e] += w * xc;
+            dbt[e] += dv[u][e];
+            xv[u][e] = g[e] * w + (a * xc + b);
+          }
+          T* out = dx + (r + u) * D + col;
+          if constexpr (kW == 1) {
+            IO<T>::store1(out, xv[u][0]);
+          } else {
+            store_packet(out, IO<T>::pack(xv[u]));
+          }
+        }
+      }
+    }
+  }
+  if (active) {
+    A* out = partial + (static_cast<size_t>(chunk) * D + col) * 2;
+#pragma unroll
+    for (int e = 0; e < kW; ++e) {
+      out[2 * e] = dg[e];
+      out[2 * e + 1] = dbt[e];
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
 // Fused group paths (NCHW): a group's D*S elements are contiguous, so a group
 // is a row of width L = D*S whose affine parameters change every S elements.
 // --------------------------------------------------------------------------
@@ -1220,6 +1402,11 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
     if (staged > row_paths) row_paths = staged;
   }
   if (rp.use_rows) return row_paths;
+  if (G == 1 && S == 1) {
+    // wide rows: the packet or the element flavour, by the addresses
+    const size_t packets = wide_grad_words(N, D, IO<T>::kVec), elems = wide_grad_words(N, D, 1);
+    return (packets > elems ? packets : elems) * sizeof(A);
+  }
   const int64_t C = G * D;
   // per-(n, c) pairs of the fused and the general path; NHWC adds the stage-one partial pairs
   size_t pairs = static_cast<size_t>(N) * C;
@@ -1595,6 +1782,33 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 #undef LAUNCH
     hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
                        dim3(1024), 0, stream, rp.grid, sh.D, part, dgp, dbtp);
+    return status_of_launch();
+  }
+
+  if (sh.G == 1 && sh.S == 1) {
+    // rows beyond the register tiles: row sums, then dx with column partials
+    const bool packets = sh.D % kVec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) &&
+        aligned16(gamma);
+    const WideGradPlan wp = plan_wide_grad(sh.N, sh.D, packets ? kVec : 1);
+    A* pairs = part;
+    A* rows = part + wide_grad_pair_words(sh.N, wp);
+    const dim3 first(sh.N * wp.splits), second(wp.col_blocks * wp.row_chunks);
+    const int D = static_cast<int>(sh.D);
+    if (packets) {
+      hipLaunchKernelGGL((layer_norm_wide_row_sums<T, kVec>), first, dim3(kReduceThreads), 0,
+                         stream, D, wp, xp, dyp, gp, pairs);
+      hipLaunchKernelGGL((layer_norm_wide_grad<T, kVec>), second, dim3(kReduceThreads), 0, stream,
+                         static_cast<int64_t>(sh.N), D, wp, xp, dyp, gp, mup, rsp, pairs, dsp, dbp,
+                         dxp, rows);
+    } else {
+      hipLaunchKernelGGL((layer_norm_wide_row_sums<T, 1>), first, dim3(kReduceThreads), 0, stream,
+                         D, wp, xp, dyp, gp, pairs);
+      hipLaunchKernelGGL((layer_norm_wide_grad<T, 1>), second, dim3(kReduceThreads), 0, stream,
+                         static_cast<int64_t>(sh.N), D, wp, xp, dyp, gp, mup, rsp, pairs, dsp, dbp,
+                         dxp, rows);
+    }
+    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
+                       dim3(1024), 0, stream, wp.row_chunks, sh.D, rows, dgp, dbtp);
     return status_of_launch();
   }
 

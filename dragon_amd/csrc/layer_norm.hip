@@ -298,7 +298,11 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
     return status_of_launch();
   }
   RowConfig cfg;
-  const bool fits = pick_row_config(ceil_div(C, kVec), 8, &cfg);
+  // Eight 16-bit packets per thread of a 1024-thread tile (64 fp32 values and
+  // as many parameters) do not fit the 128 registers of such a workgroup:
+  // those rows take the looped kernel.
+  const bool fits = pick_row_config(ceil_div(C, kVec), 8, &cfg) &&
+      !(sizeof(T) == 2 && cfg.tpr == 1024 && cfg.vpt == 8);
   const bool packets_ok = fits && C % kVec == 0 && aligned16(x) && aligned16(y) &&
       aligned16(gamma) && aligned16(beta);
   const size_t staged_bytes = 2 * static_cast<size_t>(C) * sizeof(A);

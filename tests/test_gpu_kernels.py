@@ -43,7 +43,7 @@ def oracle_dtype_inputs(bits, dtype):
 # ---------------------------------------------------------------- LayerNorm forward
 
 LN_SHAPES = [(64, 1024), (33, 1000), (7, 12288), (5, 4096), (300, 48), (3, 37), (9, 8),
-             (2, 70000), (1, 1), (513, 256),
+             (2, 70000), (3, 40000), (1, 1), (513, 256),
              # short and odd rows staged through LDS (several ranges per workgroup)
              (5000, 64), (700, 197), (130, 577), (9000, 16)]
 
@@ -297,7 +297,10 @@ LNB_SHAPES = [(64, 1024), (33, 1000), (16, 12288), (300, 48), (5, 37), (1100, 25
               # lanes per row, a last range that is not full
               (5000, 64), (700, 197), (130, 577), (9000, 16),
               # wider rows that are not whole packets: the ragged flavour of the fused kernel
-              (70, 1030), (300, 4097), (33, 12289)]
+              (70, 1030), (300, 4097), (33, 12289),
+              # rows beyond the register tiles: row sums, then dx with column partials
+              # (packets; elements for the odd width; a row cut over several workgroups)
+              (40, 33000), (19, 40001), (2, 300000)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
