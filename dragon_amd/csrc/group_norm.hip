@@ -213,56 +213,38 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
 
   // The packets of the next kDepth rows are requested before the current row
   // is reduced, so their HBM latency hides behind this row's arithmetic and
-  // enough bytes stay in flight per compute unit. Uniform trip count across the
+  // enough bytes stay in flight per compute unit. The rows in flight live in a
+  // ring of kDepth + 1 register tiles and the row loop is unrolled over the
+  // ring, so that a tile never moves between registers: copying a tile whose
+  // loads are in flight would wait for them. Uniform trip count across the
   // workgroup: the row reductions hold barriers.
+  constexpr int kRing = kDepth + 1;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
   int64_t row = static_cast<int64_t>(blockIdx.x) * kGroups + sub;
   // Rows past the end are clamped to row 0 for addressing; neither they nor the
   // slots beyond the row are zero-filled (no selects on the loaded packets):
   // such rows skip the second pass, and such slots only ever feed accumulators
   // of columns that are not written out.
-  Raw tx, tdy;
-  if constexpr (kRagged) {
-    tx.load_any(x + (row < N ? row : 0) * C, C);
-    tdy.load_any(dy + (row < N ? row : 0) * C, C);
-  } else {
-    tx.load_unmasked(x + (row < N ? row : 0) * C, npackets);
-    tdy.load_unmasked(dy + (row < N ? row : 0) * C, npackets);
-  }
-  A m = mu[row < N ? row : 0];
-  A r = rsig[row < N ? row : 0];
-  Raw px[kDepth], pdy[kDepth];  // rows row + stride .. row + kDepth * stride
-  A pm[kDepth], pr[kDepth];
-#pragma unroll
-  for (int k = 0; k + 1 < kDepth; ++k) {
-    const int64_t ahead = row + (k + 1) * stride;
-    const bool ok = ahead < N;
+  Raw rx[kRing], rdy[kRing];  // phase k: rx[k] is the current row, the others follow it
+  A rm[kRing], rr[kRing];
+  auto request = [&](Raw& tx, Raw& tdy, A& m, A& r, const int64_t at) {
+    const int64_t from = at < N ? at : 0;
     if constexpr (kRagged) {
-      px[k].load_any(x + (ok ? ahead : 0) * C, C);
-      pdy[k].load_any(dy + (ok ? ahead : 0) * C, C);
+      tx.load_any(x + from * C, C);
+      tdy.load_any(dy + from * C, C);
     } else {
-      px[k].load_unmasked(x + (ok ? ahead : 0) * C, npackets);
-      pdy[k].load_unmasked(dy + (ok ? ahead : 0) * C, npackets);
+      tx.load_unmasked(x + from * C, npackets);
+      tdy.load_unmasked(dy + from * C, npackets);
     }
-    pm[k] = mu[ok ? ahead : 0];
-    pr[k] = rsig[ok ? ahead : 0];
-  }
-  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N; base += stride) {
-    const bool valid = row < N;
-    {
-      const int64_t far = row + kDepth * stride;
-      const bool ok = far < N;
-      if constexpr (kRagged) {
-        px[kDepth - 1].load_any(x + (ok ? far : 0) * C, C);
-        pdy[kDepth - 1].load_any(dy + (ok ? far : 0) * C, C);
-      } else {
-        px[kDepth - 1].load_unmasked(x + (ok ? far : 0) * C, npackets);
-        pdy[kDepth - 1].load_unmasked(dy + (ok ? far : 0) * C, npackets);
-      }
-      pm[kDepth - 1] = mu[ok ? far : 0];
-      pr[kDepth - 1] = rsig[ok ? far : 0];
-    }
+    m = mu[from];
+    r = rsig[from];
+  };
+#pragma unroll
+  for (int k = 0; k < kDepth; ++k) request(rx[k], rdy[k], rm[k], rr[k], row + k * stride);
 
+  // One row: tx / tdy hold it, nx / ndy the row after it.
+  auto step = [&](Raw& tx, Raw& tdy, const A m, const A r, Raw& nx, Raw& ndy) {
+    const bool valid = row < N;
     A s1 = A(0), s2 = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
@@ -312,8 +294,10 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     }
     // Wait for the next row here, before this row's stores are issued (the
     // rows requested after it stay in flight).
-    px[0].wait_ready();
-    pdy[0].wait_ready();
+    if (kDepth == 1) {
+      nx.wait_ready();
+      ndy.wait_ready();
+    }
     T* dxr = dx + (valid ? row : 0) * C;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
@@ -334,10 +318,20 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
       }
     }
     if (Tile::kWavesPerRow > 1) __syncthreads();  // slots reused by the next row
-    tx = px[0], tdy = pdy[0], m = pm[0], r = pr[0], row += stride;
+  };
+
+  int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups;
+  while (base < N) {
 #pragma unroll
-    for (int k = 0; k + 1 < kDepth; ++k) {
-      px[k] = px[k + 1], pdy[k] = pdy[k + 1], pm[k] = pm[k + 1], pr[k] = pr[k + 1];
+    for (int k = 0; k < kRing; ++k) {
+      if (base < N) {  // uniform over the workgroup
+        const int kFar = (k + kDepth) % kRing;  // the tile the previous row has left
+        const int kNext = (k + 1) % kRing;
+        request(rx[kFar], rdy[kFar], rm[kFar], rr[kFar], row + kDepth * stride);
+        step(rx[k], rdy[k], rm[k], rr[k], rx[kNext], rdy[kNext]);
+        row += stride;
+        base += stride;
+      }
     }
   }
 

@@ -86,26 +86,28 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
 // Rows spanning several wavefronts: gamma and beta no longer fit the 32 KB L1
 // next to the streamed rows, and re-reading them from L2 for every row would
 // move more bytes than the row itself (fp32 parameters against 16-bit data).
-// A persistent workgroup stages both in LDS once and then walks its rows; the
-// 1024-thread tile, of which a compute unit holds few, also requests the next
-// row's packets before it reduces the current row.
-template <typename T, int kTPR, int kVPT>
-__global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
+// A persistent workgroup stages both in LDS once and then walks its rows.
+// A workgroup of kThreads threads holds kThreads / kTPR rows at a time; the
+// 1024-thread workgroups, of which a compute unit holds two at most, also
+// request their next rows' packets before they reduce the current ones.
+template <typename T, int kTPR, int kVPT, int kThreads = kTPR>
+__global__ __launch_bounds__(kThreads) void layer_norm_wide_rows(
     const int64_t N, const int C, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
     T* __restrict__ y) {
-  using Tile = RowTile<T, kTPR, kVPT>;
-  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using Tile = RowTile<T, kTPR, kVPT, kThreads>;
+  using Raw = RawRowTile<T, kTPR, kVPT, kThreads>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
+  constexpr int kGroups = Tile::kRowsPerBlock;
   constexpr int kPerPacket = 16 / sizeof(A);  // parameters per 16-byte LDS word
-  constexpr bool kPrefetch = kTPR == 1024;
+  constexpr bool kPrefetch = kThreads == 1024;
   extern __shared__ u32x4 staged[];  // gamma[C] then beta[C]
   __shared__ A slots[2][Tile::kSlots];
   A* lds_gamma = reinterpret_cast<A*>(staged);
   A* lds_beta = lds_gamma + C;
-  for (int i = threadIdx.x; i < C / kPerPacket; i += kTPR) {
+  for (int i = threadIdx.x; i < C / kPerPacket; i += kThreads) {
     staged[i] = load_packet(gamma + i * kPerPacket);
     staged[C / kPerPacket + i] = load_packet(beta + i * kPerPacket);
   }
@@ -113,18 +115,20 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
 
   const int npackets = C / kVec;
   const A inv_c = A(1) / A(C);
-  const int lane = threadIdx.x;
-  const int64_t stride = gridDim.x;
-  int64_t row = blockIdx.x;
+  const int lane = Tile::lane();
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
+  int64_t row = static_cast<int64_t>(blockIdx.x) * kGroups + Tile::sub_row();
   Raw cur;
   if (kPrefetch) cur.load(x + (row < N ? row : 0) * C, npackets, row < N);
-  for (; row < N; row += stride) {
+  // Uniform trip count over the workgroup: the row reductions hold barriers.
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kGroups; base < N; base += stride) {
+    const bool valid = row < N;
     Raw nxt;
     if (kPrefetch) {
       const bool more = row + stride < N;
       nxt.load(x + (more ? row + stride : 0) * C, npackets, more);
     } else {
-      cur.load(x + row * C, npackets);
+      cur.load(x + (valid ? row : 0) * C, npackets, valid);
     }
     Tile t;
     A s = A(0);
@@ -148,7 +152,7 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
     }
     const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_c;
     const A rs = acc_rsqrt_exact(var + eps);
-    if (lane == 0) {
+    if (lane == 0 && valid) {
       mu[row] = mean;
       rsig[row] = rs;
     }
@@ -167,7 +171,8 @@ __global__ __launch_bounds__(kTPR) void layer_norm_wide_rows(
       nxt.wait_ready();
       cur = nxt;
     }
-    t.store(y + row * C, npackets);
+    if (valid) t.store(y + row * C, npackets);
+    row += stride;
   }
 }
 
@@ -310,26 +315,35 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
     // 256-thread tiles need several workgroups per compute unit to hide HBM
     // latency; when the staged parameters leave room for fewer than four, use
     // the 1024-thread tile (which prefetches instead).
+    // the same with 16-bit rows of up to 1024 packets: four rows at a time on
+    // 256 threads each, so that a 1024-thread workgroup is not mostly idle
+    bool four_rows = false;
     if (cfg.tpr == 256 && staged_bytes * 4 > kMaxStagedParamBytes) {
       const int64_t need = ceil_div(C / kVec, 1024);
+      four_rows = sizeof(T) == 2 && need == 1;
       cfg.tpr = 1024;
       cfg.vpt = need <= 2 ? 2 : (need <= 4 ? 4 : 8);
     }
-#define LAUNCH(TPR, VPT)                                                                     \
+#define LAUNCH_T(TPR, VPT, THREADS)                                                          \
   {                                                                                          \
-    auto kernel = layer_norm_wide_rows<T, TPR, VPT>;                                         \
-    const unsigned resident = resident_grid(kernel, TPR, staged_bytes);                      \
-    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), staged_bytes, stream, N,               \
+    auto kernel = layer_norm_wide_rows<T, TPR, VPT, THREADS>;                                \
+    const int64_t groups = ceil_div(N, static_cast<int64_t>(THREADS / TPR));                 \
+    const unsigned resident = resident_grid(kernel, THREADS, staged_bytes);                  \
+    const unsigned grid =                                                                    \
+        groups < static_cast<int64_t>(resident) ? static_cast<unsigned>(groups) : resident;  \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), staged_bytes, stream, N,           \
                        static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);                 \
   }
-    if (cfg.tpr == 256 && cfg.vpt == 2) LAUNCH(256, 2)
+#define LAUNCH(TPR, VPT) LAUNCH_T(TPR, VPT, TPR)
+    if (four_rows) LAUNCH_T(256, 4, 1024)
+    else if (cfg.tpr == 256 && cfg.vpt == 2) LAUNCH(256, 2)
     else if (cfg.tpr == 256 && cfg.vpt == 4) LAUNCH(256, 4)
     else if (cfg.tpr == 256 && cfg.vpt == 8) LAUNCH(256, 8)
     else if (cfg.tpr == 1024 && cfg.vpt == 2) LAUNCH(1024, 2)
     else if (cfg.tpr == 1024 && cfg.vpt == 4) LAUNCH(1024, 4)
     else LAUNCH(1024, 8)
 #undef LAUNCH
+#undef LAUNCH_T
   } else if (packets_ok) {
 #define LAUNCH(TPR, VPT)                                                                   \
   {                                                                                        \
