@@ -36,6 +36,8 @@
 // by whole wavefronts and may reduce across the wavefront.
 #pragma once
 
+#include <type_traits>
+
 #include "reduce.h"
 #include "row_tile.h"
 
@@ -291,6 +293,21 @@ __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t
   a = ta, b = tb;
 }
 
+// Optional parts of an Op, both off unless it declares them:
+//   kScanFirst  op.scan(x) sees every packet of the item before the first
+//               accumulate (a thread-wide maximum, say);
+//   kRewrites   op.accumulate_rewrite(x, a, b) replaces the elements it is
+//               given, and the second pass reads those instead of the input
+//               (exact only where a packet holds accumulator-typed elements).
+template <typename Op, typename = void>
+struct OpScansFirst : std::false_type {};
+template <typename Op>
+struct OpScansFirst<Op, std::void_t<decltype(Op::kScanFirst)>> : std::bool_constant<Op::kScanFirst> {};
+template <typename Op, typename = void>
+struct OpRewrites : std::false_type {};
+template <typename Op>
+struct OpRewrites<Op, std::void_t<decltype(Op::kRewrites)>> : std::bool_constant<Op::kRewrites> {};
+
 template <typename T, int kR, int kIn>
 struct CoopSlice {  // the raw packets of one item
   u32x4 p0[kR];
@@ -341,13 +358,32 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
   op.begin(it.c, it.base, in0);
   A a, b;
   Op::Merge::identity(a, b);
+  if constexpr (OpScansFirst<Op>::value) {
+#pragma unroll
+    for (int i = 0; i < kR; ++i) {
+      if (it.has(i)) {
+        A xv[kVec];
+        IO<T>::unpack(s.p0[i], xv);
+        op.scan(xv);
+      }
+    }
+    // convert the packets again instead of keeping every converted element
+#pragma unroll
+    for (int i = 0; i < kR; ++i) asm volatile("" : "+v"(s.p0[i]));
+  }
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     if (it.has(i)) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
-      op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
+      if constexpr (OpRewrites<Op>::value) {
+        static_assert(sizeof(T) == sizeof(A), "rewritten elements must survive the packet");
+        op.accumulate_rewrite(xv, a, b);
+        s.p0[i] = IO<T>::pack(xv);
+      } else {
+        op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
+      }
     }
   }
   coop_channel_totals<typename Op::Merge>(d, it.c, w, a, b, partial, lds_a, lds_b);

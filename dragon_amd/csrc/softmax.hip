@@ -723,38 +723,62 @@ struct OnlineSoftmaxMerge {
   }
 };
 
+// A thread first takes the maximum of all its packets, then adds exp(x - that
+// maximum): one exp per element instead of a rescaled running sum per packet.
+// Softmax of accumulator-typed elements keeps those exponentials in the
+// packets, and the second pass only scales them by exp(thread maximum - row
+// maximum) / sum (fp32 exp is a dozen instructions: recomputing it made the
+// kernel arithmetic-bound).
 template <typename T, int kKind>
 struct SoftmaxSlicesForward {
   using A = typename IO<T>::Acc;
   using M = SoftmaxMath<T>;
   using Merge = OnlineSoftmaxMerge<T>;
   static constexpr int kIn = 1;
-  A m, s, inv;  // inv = 1/s (softmax) or log(s) (log-softmax)
-  __device__ __forceinline__ void begin(uint32_t, uint32_t, const T*) {}
+  static constexpr bool kScanFirst = true;
+  static constexpr bool kRewrites = kKind == kSoftmax && sizeof(T) == sizeof(A);
+  A top;         // maximum of this thread's elements
+  A m, s, inv;   // of the row; inv = 1/s (softmax) or log(s) (log-softmax)
+  A scale;       // exp(top - m)
+  __device__ __forceinline__ void begin(uint32_t, uint32_t, const T*) { top = acc_neg_inf<A>(); }
+  template <int V>
+  __device__ __forceinline__ void scan(const A (&x)[V]) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) top = MaxOp()(top, x[e]);
+  }
   template <int V>
   __device__ __forceinline__ void accumulate(uint32_t, uint32_t, const A (&x)[V], const A (&)[V],
                                              A& a, A& b) const {
-    A top = a;
-#pragma unroll
-    for (int e = 0; e < V; ++e) top = MaxOp()(top, x[e]);
-    if (top > acc_neg_inf<A>()) {
-      A t = b * M::exp_of(a - top);
-#pragma unroll
-      for (int e = 0; e < V; ++e) t += M::exp_of(x[e] - top);
-      b = t;
-    }
     a = top;
+    if (top > acc_neg_inf<A>()) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) b += M::exp_of(x[e] - top);
+    }
+  }
+  template <int V>
+  __device__ __forceinline__ void accumulate_rewrite(A (&x)[V], A& a, A& b) const {
+    a = top;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      x[e] = top > acc_neg_inf<A>() ? M::exp_of(x[e] - top) : A(0);
+      b += x[e];
+    }
   }
   __device__ __forceinline__ void finish(uint32_t, bool, A a, A b) {
     m = a, s = b;
     inv = kKind == kSoftmax ? A(1) / b : acc_log(b);
+    scale = top > acc_neg_inf<A>() ? M::exp_of(top - a) : A(0);
   }
   template <int V>
   __device__ __forceinline__ void transform(uint32_t, uint32_t, A (&x)[V], const A (&)[V]) const {
 #pragma unroll
     for (int e = 0; e < V; ++e) {
-      const A d = x[e] - m;
-      x[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), s, inv) : d - inv;
+      if constexpr (kRewrites) {
+        x[e] = M::normalise(x[e] * scale, s, inv);
+      } else {
+        const A d = x[e] - m;
+        x[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), s, inv) : d - inv;
+      }
     }
   }
 };
