@@ -701,23 +701,28 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
   constexpr bool kPrefetch = kTPR == 1024;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock;
   int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+  // The loaded packets are not masked (a select on them would wait for each
+  // load where it stands): slots beyond the group repeat its first packet and
+  // are skipped by the sums and the stores.
   Raw t;
-  if (kPrefetch) t.load(x + (row < rows ? row : 0) * L, npackets, row < rows);
+  if (kPrefetch) t.load_unmasked(x + (row < rows ? row : 0) * L, npackets);
   for (; row < rows; row += stride) {
     Raw nxt;
     if (kPrefetch) {
       const bool more = row + stride < rows;
-      nxt.load(x + (more ? row + stride : 0) * L, npackets, more);
+      nxt.load_unmasked(x + (more ? row + stride : 0) * L, npackets);
     } else {
-      t.load(x + row * L, npackets);
+      t.load_unmasked(x + row * L, npackets);
     }
     A s = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      A v[kVec];
-      t.unpack(i, v);
+      if (Tile::active(i, npackets)) {
+        A v[kVec];
+        t.unpack(i, v);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) s += v[e];
+        for (int e = 0; e < kVec; ++e) s += v[e];
+      }
     }
     const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_l;
     t.refresh();
@@ -835,11 +840,19 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
 }
 
 // GroupNormGrad in one pass over x and dy: one workgroup per group keeps both
-// as raw packets. Requires S to be a multiple of 64 packets, so that every
-// (slot, wavefront) pair lies in one channel and the per-channel sums are a
-// wave reduction plus a fixed-order sum over LDS entries.
+// as raw packets. A (slot, wavefront) pair covers 64 adjacent packets of the
+// group. Where S is a multiple of 64 packets these lie in one channel, and the
+// per-channel sums are a wave reduction plus a fixed-order sum over LDS
+// entries (kChannelWaves). kChannelStraddles takes any S of at least 64 whole
+// packets: the 64 packets then lie in at most two channels, split at a lane
+// known per wavefront, so gamma is one of two scalars and a pair contributes a
+// sum to each of them. kChannelLanes takes channels of 1, 2, 4 .. 32 packets:
+// a channel is a group of adjacent lanes of one (slot, wavefront) pair, reduced
+// with shuffles and written by its first lane; gamma is read per lane.
 // partial[(n*C + c)*2 + {0,1}] receives this group's share of dgamma / dbeta.
-template <typename T, int kTPR, int kVPT>
+enum ChannelMode { kChannelWaves = 0, kChannelStraddles = 1, kChannelLanes = 2 };
+
+template <typename T, int kTPR, int kVPT, int kMode>
 __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const T* __restrict__ x, const T* __restrict__ dy,
@@ -852,24 +865,39 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   constexpr int kWaves = kTPR / kWaveSize;
+  constexpr bool kStraddle = kMode == kChannelStraddles;
+  constexpr bool kLanes = kMode == kChannelLanes;
+  constexpr int kParts = kStraddle ? 4 : 2;  // per entry: (dgamma, dbeta) of one or two channels
   __shared__ A slots[2 * Tile::kSlots];
-  __shared__ A chan_part[kVPT][kWaves][2];
+  __shared__ A chan_part[kVPT][kWaves][kParts];
   const int npackets = L / kVec;
   const uint32_t packets_per_chan = S / kVec;
   const A denom = A(1) / A(L);
   const int lane = threadIdx.x;
+  const int wave_lane = lane & (kWaveSize - 1);
   // Uniform over the wavefront, so everything indexed by it (the channel of a
   // slot, its gamma) stays in scalar registers.
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kWaveSize));
+
+  // The first channel of the 64 packets of (slot i, this wavefront), and how
+  // many of them lie in it (64 or more: all). Packets beyond the group take
+  // the last channel.
+  auto first_channel = [&](int i, uint32_t& chan, uint32_t& in_first) {
+    const uint32_t p0 = static_cast<uint32_t>(i * kTPR + wave * kWaveSize);
+    chan = p0 / packets_per_chan;
+    in_first = (chan + 1) * packets_per_chan - p0;
+    if (chan >= D) chan = D - 1, in_first = kWaveSize;
+  };
 
   // A workgroup fills the compute unit's registers, so the next group cannot be
   // held beside the current one: its packets are requested slot by slot into the
   // registers the second pass has just finished with, and are in flight while
   // the rest of this group is computed, stored and reduced.
+  // The loaded packets are not masked: packets beyond the group skip the sums.
   Raw tx, tdy;
   if (blockIdx.x < rows) {
-    tx.load(x + static_cast<int64_t>(blockIdx.x) * L, npackets);
-    tdy.load(dy + static_cast<int64_t>(blockIdx.x) * L, npackets);
+    tx.load_unmasked(x + static_cast<int64_t>(blockIdx.x) * L, npackets);
+    tdy.load_unmasked(dy + static_cast<int64_t>(blockIdx.x) * L, npackets);
   }
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const int64_t next = row + gridDim.x;
@@ -883,18 +911,28 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     A s1 = A(0), s2 = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      // Slots beyond the group hold dy = 0 and take the last channel's gamma.
-      uint32_t chan = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) / packets_per_chan;
-      chan = chan < D ? chan : D - 1;
-      gam[i] = gamma[c0 + chan];
-      A xv[kVec], dv[kVec];
-      tx.unpack(i, xv);
-      tdy.unpack(i, dv);
+      if constexpr (kLanes) {
+        const uint32_t chan = static_cast<uint32_t>(i * kTPR + lane) / packets_per_chan;
+        gam[i] = gamma[c0 + (chan < D ? chan : D - 1)];
+      } else {
+        uint32_t chan, in_first;
+        first_channel(i, chan, in_first);
+        gam[i] = gamma[c0 + chan];
+        if constexpr (kStraddle) {
+          const A second = gamma[c0 + (chan + 1 < D ? chan + 1 : chan)];
+          gam[i] = static_cast<uint32_t>(wave_lane) < in_first ? gam[i] : second;
+        }
+      }
+      if (Tile::active(i, npackets)) {
+        A xv[kVec], dv[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A t = gam[i] * dv[e];
-        s1 += t * xv[e];
-        s2 += t;
+        for (int e = 0; e < kVec; ++e) {
+          const A t = gam[i] * dv[e];
+          s1 += t * xv[e];
+          s2 += t;
+        }
       }
     }
     Tile::reduce_sum_pair(s1, s2, slots);
@@ -908,41 +946,87 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     tdy.refresh();
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      A xv[kVec], dv[kVec];
-      tx.unpack(i, xv);
-      tdy.unpack(i, dv);
       A t1 = A(0), t2 = A(0);
+      if (Tile::active(i, npackets)) {
+        A xv[kVec], dv[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) {
-        const A xc = xv[e] - m;
-        t1 += dv[e] * xc * r;
-        t2 += dv[e];
-        xv[e] = gam[i] * dv[e] * r + (u0 * xc - v0) * denom;
+        for (int e = 0; e < kVec; ++e) {
+          const A xc = xv[e] - m;
+          t1 += dv[e] * xc * r;
+          t2 += dv[e];
+          xv[e] = gam[i] * dv[e] * r + (u0 * xc - v0) * denom;
+        }
+        tx.store_slot(dx + row * L, i, xv);
       }
-      if (Tile::active(i, npackets)) tx.store_slot(dx + row * L, i, xv);
       if (next_valid) {
-        tx.load_slot(nx, i, npackets);
-        tdy.load_slot(ndy, i, npackets);
+        tx.load_slot_unmasked(nx, i, npackets);
+        tdy.load_slot_unmasked(ndy, i, npackets);
       }
-      t1 = wave_allreduce(t1, SumOp());
-      t2 = wave_allreduce(t2, SumOp());
-      if ((threadIdx.x & (kWaveSize - 1)) == 0) {
-        chan_part[i][wave][0] = t1;
-        chan_part[i][wave][1] = t2;
+      if constexpr (kLanes) {
+        // packets_per_chan is a power of two below 64: xor-shuffles within the channel's lanes
+        for (uint32_t o = 1; o < packets_per_chan; o <<= 1) {
+          t1 += __shfl_xor(t1, static_cast<int>(o), kWaveSize);
+          t2 += __shfl_xor(t2, static_cast<int>(o), kWaveSize);
+        }
+        const uint32_t packet = static_cast<uint32_t>(i * kTPR + lane);
+        if ((packet & (packets_per_chan - 1)) == 0 && Tile::active(i, npackets)) {
+          const size_t n = static_cast<size_t>(row / G);
+          A* o = partial + (n * G * D + c0 + packet / packets_per_chan) * 2;
+          o[0] = t1;
+          o[1] = t2;
+        }
+      } else if constexpr (kStraddle) {
+        uint32_t chan, in_first;
+        first_channel(i, chan, in_first);
+        const bool head = static_cast<uint32_t>(wave_lane) < in_first;
+        const A a1 = wave_allreduce(head ? t1 : A(0), SumOp());
+        const A a2 = wave_allreduce(head ? t2 : A(0), SumOp());
+        A b1 = A(0), b2 = A(0);
+        if (in_first < static_cast<uint32_t>(kWaveSize)) {  // uniform over the wavefront
+          b1 = wave_allreduce(head ? A(0) : t1, SumOp());
+          b2 = wave_allreduce(head ? A(0) : t2, SumOp());
+        }
+        if (wave_lane == 0) {
+          chan_part[i][wave][0] = a1;
+          chan_part[i][wave][1] = a2;
+          chan_part[i][wave][2] = b1;
+          chan_part[i][wave][3] = b2;
+        }
+      } else {
+        t1 = wave_allreduce(t1, SumOp());
+        t2 = wave_allreduce(t2, SumOp());
+        if (wave_lane == 0) {
+          chan_part[i][wave][0] = t1;
+          chan_part[i][wave][1] = t2;
+        }
       }
     }
     __syncthreads();
-    if (static_cast<uint32_t>(lane) < D) {
+    if (!kLanes && static_cast<uint32_t>(lane) < D) {
       // Entry q = (slot, wavefront) covers packets [64 q, 64 q + 64); channel
-      // `lane` owns the entries [lane * waves_per_chan, (lane + 1) * waves_per_chan).
+      // `lane` owns the packets [lane * packets_per_chan, (lane + 1) * packets_per_chan).
       A a = A(0), b = A(0);
       const A* entries = &chan_part[0][0][0];
-      const uint32_t waves_per_chan = packets_per_chan / kWaveSize;
-      const uint32_t q0 = static_cast<uint32_t>(lane) * waves_per_chan;
+      if constexpr (kStraddle) {
+        const uint32_t lo = static_cast<uint32_t>(lane) * packets_per_chan;
+        const uint32_t q0 = lo / kWaveSize, q1 = (lo + packets_per_chan - 1) / kWaveSize;
 #pragma nounroll
-      for (uint32_t q = q0; q < q0 + waves_per_chan; ++q) {
-        a += entries[2 * q];
-        b += entries[2 * q + 1];
+        for (uint32_t q = q0; q <= q1; ++q) {
+          // the entry's first packet lies in this channel or in the one before it
+          const uint32_t part = q * kWaveSize >= lo ? 0u : 2u;
+          a += entries[4 * q + part];
+          b += entries[4 * q + part + 1];
+        }
+      } else {
+        const uint32_t waves_per_chan = packets_per_chan / kWaveSize;
+        const uint32_t q0 = static_cast<uint32_t>(lane) * waves_per_chan;
+#pragma nounroll
+        for (uint32_t q = q0; q < q0 + waves_per_chan; ++q) {
+          a += entries[2 * q];
+          b += entries[2 * q + 1];
+        }
       }
       const size_t n = static_cast<size_t>(row / G);
       A* o = partial + (n * G * D + c0 + lane) * 2;
@@ -1367,14 +1451,24 @@ RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
 }
 
 // Fused group backward applies to NCHW groups that fit a multi-wave register
-// tile and whose channels span whole wavefronts of packets.
+// tile and whose channels are whole packets: 64 or more of them (`mode` tells
+// whether they are whole wavefronts of packets), or a power of two below 64.
 template <typename T>
-bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig* cfg) {
+bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig* cfg, int* mode) {
   constexpr int kVec = IO<T>::kVec;
   if (layout != DRAGON_HIP_NCHW || G * D == 1) return false;
-  if (S % (kWaveSize * kVec) != 0) return false;
+  if (S % kVec != 0) return false;
+  const int64_t per_chan = S / kVec;
+  if (per_chan >= kWaveSize) {
+    *mode = per_chan % kWaveSize == 0 ? kChannelWaves : kChannelStraddles;
+  } else if ((per_chan & (per_chan - 1)) == 0) {
+    *mode = kChannelLanes;
+  } else {
+    return false;
+  }
   static const RowConfig table[] = {{256, 2}, {256, 4}, {256, 8}, {1024, 4}, {1024, 8}};
-  const int64_t npackets = D * S / kVec;
+  const int64_t npackets = D * per_chan;
+  if (npackets <= kWaveSize * 2) return false;  // a wavefront or two: the general path
   for (const RowConfig& c : table) {
     if (npackets <= static_cast<int64_t>(c.tpr) * c.vpt) {
       *cfg = c;
@@ -1807,14 +1901,20 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   }
 
   RowConfig gcfg;
-  if (plan_group_grad_rows<T>(sh.G, sh.D, sh.S, layout, &gcfg) && aligned16(x) && aligned16(dy) &&
-      aligned16(dx)) {
+  int mode = kChannelWaves;
+  if (plan_group_grad_rows<T>(sh.G, sh.D, sh.S, layout, &gcfg, &mode) && aligned16(x) &&
+      aligned16(dy) && aligned16(dx)) {
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
     const int L = static_cast<int>(sh.D * sh.S);
     const unsigned grid = static_cast<unsigned>(rows < (1 << 20) ? rows : (1 << 20));
-#define LAUNCH(TPR, VPT)                                                                       \
-  hipLaunchKernelGGL((group_norm_grad_rows<T, TPR, VPT>), dim3(grid), dim3(TPR), 0, stream, rows, \
-                     L, sh.G, sh.D, sh.S, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    auto kernel = mode == kChannelStraddles ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddles> \
+        : mode == kChannelLanes             ? group_norm_grad_rows<T, TPR, VPT, kChannelLanes>     \
+                                            : group_norm_grad_rows<T, TPR, VPT, kChannelWaves>;    \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), 0, stream, rows, L, sh.G, sh.D, sh.S, xp, \
+                       dyp, gp, mup, rsp, dsp, dbp, dxp, part);                                 \
+  }
     if (gcfg.tpr == 256 && gcfg.vpt == 2) LAUNCH(256, 2)
     else if (gcfg.tpr == 256 && gcfg.vpt == 4) LAUNCH(256, 4)
     else if (gcfg.tpr == 256 && gcfg.vpt == 8) LAUNCH(256, 8)

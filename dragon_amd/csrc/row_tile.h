@@ -227,13 +227,12 @@ struct RawRowTile {
       p[s] = load_packet(row + static_cast<int64_t>(packet) * kVec);
     }
   }
-  // One slot of load().
-  __device__ __forceinline__ void load_slot(const T* row, int s, int npackets) {
-    const bool on = active(s, npackets);
-    const int packet = on ? s * kTPR + lane() : 0;
-    const u32x4 t = load_packet(row + static_cast<int64_t>(packet) * kVec);
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    p[s] = on ? t : z;
+  // One slot of load_unmasked(): a slot beyond the row holds the row's first
+  // packet, and no select touches the loaded registers (a select would wait
+  // for the load where it stands, which defeats a request made ahead of use).
+  __device__ __forceinline__ void load_slot_unmasked(const T* row, int s, int npackets) {
+    const int packet = active(s, npackets) ? s * kTPR + lane() : 0;
+    p[s] = load_packet(row + static_cast<int64_t>(packet) * kVec);
   }
   // Rows of any width at element-aligned addresses: whole packets with one
   // unaligned access, the row's last partial packet element by element.

@@ -345,7 +345,12 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             ((1, 2, 300, 301), 1, 2),
             # groups beyond one workgroup's registers: slices of a group held by several
             # workgroups that exchange their partial sums (12 and 16+ slices per group)
-            ((2, 6, 128, 128), 1, 2), ((2, 8, 256, 256), 1, 2)]
+            ((2, 6, 128, 128), 1, 2), ((2, 8, 256, 256), 1, 2),
+            # channels of 64 or more packets that are not whole wavefronts of packets: the
+            # fused backward splits a wavefront's packets between two channels
+            ((2, 16, 28, 28), 1, 4), ((2, 64, 56, 56), 1, 8), ((1, 6, 24, 24), 1, 2),
+            # channels of a few packets: several channels per wavefront in the fused backward
+            ((2, 64, 16, 16), 1, 4), ((3, 48, 8, 8), 1, 2)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
