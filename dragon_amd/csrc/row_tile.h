@@ -86,11 +86,18 @@ struct RowTile {
       load_ragged(row, npackets, fill, valid);
       return;
     }
+    // every packet is requested before the first one is converted and masked
+    u32x4 raw[kVPT];
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       const bool on = valid && active(s, npackets);
       const int packet = on ? s * kTPR + lane() : 0;
-      load_unpack<T>(row + static_cast<int64_t>(packet) * kVec, v[s]);
+      raw[s] = load_packet(row + static_cast<int64_t>(packet) * kVec);
+    }
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const bool on = valid && active(s, npackets);
+      IO<T>::unpack(raw[s], v[s]);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) v[s][e] = on ? v[s][e] : fill;
     }
@@ -195,13 +202,18 @@ struct RawRowTile {
   // itself is unconditional (see RowTile::load); `row` must be readable even
   // when `valid` is false.
   __device__ __forceinline__ void load(const T* row, int npackets, bool valid = true) {
+    // every packet is requested before the first one is masked
 #pragma unroll
     for (int s = 0; s < kVPT; ++s) {
       const bool on = valid && active(s, npackets);
       const int packet = on ? s * kTPR + lane() : 0;
-      const u32x4 t = load_packet(row + static_cast<int64_t>(packet) * kVec);
+      p[s] = load_packet(row + static_cast<int64_t>(packet) * kVec);
+    }
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const bool on = valid && active(s, npackets);
       const u32x4 z = {0u, 0u, 0u, 0u};
-      p[s] = on ? t : z;
+      p[s] = on ? p[s] : z;
     }
   }
   // Rows of any width at element-aligned addresses, read in whole (unaligned)
