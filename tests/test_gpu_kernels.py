@@ -962,3 +962,69 @@ def test_rows_at_element_aligned_addresses(K, dtype, shape):
     K.l2_norm_grad(N, 1, C, 1.0, 1e-12, dyd, xd, dx)
     dxw = U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape)
     assert np.max(np.abs(dxw - dx64n)) / term <= tol
+
+
+# ---------------------------------------------------------------- more than 2^31 elements
+
+def _rows_to_bits(t, rows, dtype):
+    """Rows `rows` of device tensor t as the oracle's storage (bits for 16-bit types)."""
+    import torch
+    sel = t[torch.as_tensor(rows, device=t.device)].contiguous()
+    return U.to_host(sel)
+
+
+def test_softmax_rows_beyond_int32_elements(K):
+    """[2^20 + 7, 2304] fp16: element offsets pass 2^31. Sampled rows against the oracle,
+    every row through the size-independent properties (sums to one; dx sums to zero)."""
+    import torch
+    dtype = "float16"
+    N, C = (1 << 20) + 7, 2304
+    assert N * C > 2 ** 31
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.empty((N, C), dtype=torch.float16, device="cuda").normal_(0.0, 2.0, generator=gen)
+    y = torch.empty_like(x)
+    K.softmax(N, 1, C, x, y)
+    sums = y.sum(1, dtype=torch.float32)
+    assert float((sums - 1).abs().max()) < 2e-2
+    rows = [0, 1, N // 2, (2 ** 31) // C, (2 ** 31) // C + 1, N - 2, N - 1]
+    xs = _rows_to_bits(x, rows, dtype)
+    xo, od = oracle_dtype_inputs(xs, dtype)
+    y_ref = R.op_softmax(od, xo, 1)
+    got = U.widen(_rows_to_bits(y, rows, dtype), dtype)
+    assert U.normwise(got, y_ref) <= U.TIGHT[dtype]
+    dy = torch.empty_like(x).normal_(0.0, 1.0, generator=gen)
+    dx = torch.empty_like(x)
+    K.softmax_grad(N, 1, C, dy, y, dx)
+    # sum_j dx_j = sum_j y_j (dy_j - s) = s - s sum_j y_j ~ 0 (fp16 outputs: 2304 roundings)
+    assert float(dx.sum(1, dtype=torch.float32).abs().max()) < 5e-2
+    yo, _ = oracle_dtype_inputs(_rows_to_bits(y, rows, dtype), dtype)
+    dyo, _ = oracle_dtype_inputs(_rows_to_bits(dy, rows, dtype), dtype)
+    dx_ref = R.op_softmax_grad(od, yo, dyo, 1)
+    assert U.normwise(U.widen(_rows_to_bits(dx, rows, dtype), dtype), dx_ref) <= U.TIGHT[dtype]
+
+
+def test_layer_norm_rows_beyond_int32_elements(K):
+    """[2^20 + 7, 2304] bf16 LayerNorm forward: sampled rows against the oracle, every row
+    through mean(y) ~ 0 and mean(y^2) ~ 1 (gamma = 1, beta = 0)."""
+    import torch
+    dtype = "bfloat16"
+    N, C = (1 << 20) + 7, 2304
+    gen = torch.Generator(device="cuda").manual_seed(32)
+    x = torch.empty((N, C), dtype=torch.bfloat16, device="cuda").normal_(0.5, 2.0, generator=gen)
+    y = torch.empty_like(x)
+    g = torch.ones(C, device="cuda")
+    b = torch.zeros(C, device="cuda")
+    mu, rsig = torch.empty(N, device="cuda"), torch.empty(N, device="cuda")
+    K.layer_norm(N, C, 1e-5, x, g, b, mu, rsig, y)
+    yf = y.float()
+    assert float(yf.mean(1).abs().max()) < 1e-2
+    assert float(((yf * yf).mean(1) - 1).abs().max()) < 2e-2
+    del yf
+    rows = [0, N // 2, (2 ** 31) // C, (2 ** 31) // C + 1, N - 1]
+    xs = _rows_to_bits(x, rows, dtype)
+    y_ref, mu_ref, rsig_ref = R.layer_norm(dtype, xs, np.ones(C, np.float32), np.zeros(C, np.float32), 1e-5)
+    got = U.widen(_rows_to_bits(y, rows, dtype), dtype)
+    assert U.normwise(got, U.widen(y_ref, dtype)) <= U.TIGHT[dtype]
+    idx = torch.as_tensor(rows, device="cuda")
+    assert np.max(np.abs(U.to_host(mu[idx]) - mu_ref)) <= 1e-4
+    assert np.max(np.abs(U.to_host(rsig[idx]) / rsig_ref - 1)) <= 1e-4
