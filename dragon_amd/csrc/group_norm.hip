@@ -2024,11 +2024,18 @@ inline int canonical_layout(int layout, int64_t S) {
   return (layout == DRAGON_HIP_NHWC && S == 1) ? DRAGON_HIP_NCHW : layout;
 }
 
-int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShape* sh) {
+// `rows_only`: the caller's kernels address a [N, D] matrix (G = S = 1) by row
+// with 64-bit offsets, so only N and D have to fit 32 bits, not their product.
+int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShape* sh,
+               bool rows_only = false) {
   if (N < 0 || G <= 0 || D <= 0 || S < 0) return DRAGON_HIP_EINVAL;
   if (layout != DRAGON_HIP_NCHW && layout != DRAGON_HIP_NHWC) return DRAGON_HIP_EINVAL;
   layout = canonical_layout(layout, S);
-  if (!fits_int32(N * G * D * S)) return DRAGON_HIP_EINVAL;
+  if (rows_only && G == 1 && S == 1) {
+    if (!fits_int32(N) || !fits_int32(D)) return DRAGON_HIP_EINVAL;
+  } else if (!fits_int32(N * G * D * S)) {
+    return DRAGON_HIP_EINVAL;
+  }
   sh->N = static_cast<uint32_t>(N), sh->G = static_cast<uint32_t>(G);
   sh->D = static_cast<uint32_t>(D), sh->S = static_cast<uint32_t>(S);
   sh->C = static_cast<uint32_t>(G * D);
@@ -2061,7 +2068,7 @@ int dragon_hip_group_norm(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
 size_t dragon_hip_group_norm_grad_scratch_bytes(int dtype, int64_t N, int64_t G, int64_t D,
                                                 int64_t S, int layout) {
   dragon_hip::GroupShape sh;
-  if (dragon_hip::make_shape(N, G, D, S, layout, &sh) != DRAGON_HIP_OK || N * S == 0) return 0;
+  if (dragon_hip::make_shape(N, G, D, S, layout, &sh, true) != DRAGON_HIP_OK || N * S == 0) return 0;
   layout = dragon_hip::canonical_layout(layout, S);
   switch (dtype) {
     case DRAGON_HIP_F16: return dragon_hip::grad_scratch_t<dragon_hip::f16_t>(N, G, D, S, layout);
@@ -2078,7 +2085,8 @@ int dragon_hip_group_norm_grad(int dtype, int64_t N, int64_t G, int64_t D, int64
                                void* dgamma, void* dbeta, void* dx, void* scratch,
                                size_t scratch_bytes, void* stream) {
   dragon_hip::GroupShape sh;
-  const int st = dragon_hip::make_shape(N, G, D, S, layout, &sh);
+  // LayerNorm backward (G = S = 1) takes matrices of more than 2^31 elements
+  const int st = dragon_hip::make_shape(N, G, D, S, layout, &sh, true);
   if (st != DRAGON_HIP_OK) return st;
   if (!dgamma || !dbeta) return DRAGON_HIP_EINVAL;
   const size_t acc = dtype == DRAGON_HIP_F64 ? 8 : 4;

@@ -1028,3 +1028,46 @@ def test_layer_norm_rows_beyond_int32_elements(K):
     idx = torch.as_tensor(rows, device="cuda")
     assert np.max(np.abs(U.to_host(mu[idx]) - mu_ref)) <= 1e-4
     assert np.max(np.abs(U.to_host(rsig[idx]) / rsig_ref - 1)) <= 1e-4
+
+
+def test_layer_norm_backward_beyond_int32_elements(K):
+    """[2^20 + 7, 2304] bf16 LayerNorm backward: sampled rows of dx, ds, db against the oracle;
+    dgamma / dbeta against fp64 sums of the same products on the device."""
+    import torch
+    dtype = "bfloat16"
+    N, C = (1 << 20) + 7, 2304
+    gen = torch.Generator(device="cuda").manual_seed(33)
+    x = torch.empty((N, C), dtype=torch.bfloat16, device="cuda").normal_(0.5, 2.0, generator=gen)
+    dy = torch.empty_like(x).normal_(0.0, 1.0, generator=gen)
+    g = torch.empty(C, device="cuda").uniform_(0.5, 1.5, generator=gen)
+    b = torch.zeros(C, device="cuda")
+    mu, rsig = torch.empty(N, device="cuda"), torch.empty(N, device="cuda")
+    y = torch.empty_like(x)
+    K.layer_norm(N, C, 1e-5, x, g, b, mu, rsig, y)
+    del y
+    params = torch.empty(2 * N, device="cuda")
+    dg, db, dx = torch.empty(C, device="cuda"), torch.empty(C, device="cuda"), torch.empty_like(x)
+    K.group_norm_grad(N, 1, C, 1, "NHWC", x, mu, rsig, g, dy, params, params, dg, db, dx)
+    rows = [0, N // 2, (2 ** 31) // C, (2 ** 31) // C + 1, N - 1]
+    idx = torch.as_tensor(rows, device="cuda")
+    xs = R.from_bits(_rows_to_bits(x, rows, dtype), dtype)
+    dys = R.from_bits(_rows_to_bits(dy, rows, dtype), dtype)
+    dx_ref, _, _, ds_ref, db_ref = R.group_norm_grad(
+        "float32", len(rows), 1, C, 1, "NHWC", xs, U.to_host(mu[idx]), U.to_host(rsig[idx]),
+        U.to_host(g), dys)
+    assert U.normwise(U.widen(_rows_to_bits(dx, rows, dtype), dtype), dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(U.to_host(params[:N][idx]), ds_ref) <= 2e-5
+    assert U.normwise(U.to_host(params[N:][idx]), db_ref) <= 2e-5
+    # column sums over a million rows, in chunks to bound the fp64 temporaries
+    dg64 = torch.zeros(C, dtype=torch.float64, device="cuda")
+    db64 = torch.zeros(C, dtype=torch.float64, device="cuda")
+    step = 1 << 17
+    for r0 in range(0, N, step):
+        xc = x[r0:r0 + step].double()
+        dc = dy[r0:r0 + step].double()
+        m = mu[r0:r0 + step].double()[:, None]
+        r = rsig[r0:r0 + step].double()[:, None]
+        dg64 += (dc * (xc - m) * r).sum(0)
+        db64 += dc.sum(0)
+    assert U.normwise(U.to_host(dg), dg64.cpu().numpy()) <= 2e-5
+    assert U.normwise(U.to_host(db), db64.cpu().numpy()) <= 2e-5
