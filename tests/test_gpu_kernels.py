@@ -1071,3 +1071,36 @@ def test_layer_norm_backward_beyond_int32_elements(K):
         db64 += dc.sum(0)
     assert U.normwise(U.to_host(dg), dg64.cpu().numpy()) <= 2e-5
     assert U.normwise(U.to_host(db), db64.cpu().numpy()) <= 2e-5
+
+
+def test_l2_norm_and_cross_entropy_beyond_int32_elements(K):
+    """The same for the sibling row kernels: L2 norm of a bf16 and fused softmax
+    cross-entropy of an fp32 [2^20 + 7, 2304] matrix; sampled rows against the oracle,
+    every row through |y| = 1 and loss = -log prob[target]."""
+    import torch
+    N, C = (1 << 20) + 7, 2304
+    rows = [0, N // 2, (2 ** 31) // C, (2 ** 31) // C + 1, N - 1]
+    idx = torch.as_tensor(rows, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(34)
+    x = torch.empty((N, C), dtype=torch.bfloat16, device="cuda").normal_(0.0, 2.0, generator=gen)
+    y = torch.empty_like(x)
+    K.l2_norm(N, 1, C, 1.0, 1e-12, x, y)
+    norms = (y.float() ** 2).sum(1)
+    assert float((norms - 1).abs().max()) < 2e-2
+    y_ref = R.lp_norm("float32", 2, len(rows), 1, C, 1.0, 1e-12,
+                      R.from_bits(_rows_to_bits(x, rows, "bfloat16"), "bfloat16"))
+    assert U.normwise(U.widen(_rows_to_bits(y, rows, "bfloat16"), "bfloat16"), y_ref) <= U.TIGHT["bfloat16"]
+    del x, y, norms
+
+    logits = torch.empty((N, C), dtype=torch.float32, device="cuda").normal_(0.0, 2.0, generator=gen)
+    target = torch.randint(0, C, (N,), generator=gen, device="cuda", dtype=torch.int64)
+    prob = torch.empty_like(logits)
+    loss = torch.empty(N, device="cuda")
+    K.softmax_cross_entropy_loss_forward(N, 1, C, -1, "none", logits, target, prob, loss)
+    picked = prob.gather(1, target[:, None])[:, 0]
+    assert float((loss + picked.log()).abs().max()) < 1e-5
+    assert float((prob.sum(1) - 1).abs().max()) < 1e-4
+    loss_ref, prob_ref = R.op_softmax_cross_entropy_loss(
+        "float32", U.to_host(logits[idx]), U.to_host(target[idx]), reduction="none")
+    assert U.normwise(U.to_host(prob[idx]), prob_ref) <= U.TIGHT["float32"]
+    assert U.normwise(U.to_host(loss[idx]), loss_ref) <= U.TIGHT["float32"]
