@@ -71,7 +71,7 @@ inline ExchangeState& exchange_state() {
   }();
   return st;
 }
-constexpr uint32_t kCoopPatience = 1u << 20;  // polls of about 0.2 us each
+constexpr uint32_t kCoopPatience = 1u << 20;  // polls of about 1 us each (s_sleep 32 between them)
 
 struct CoopPlan {
   bool ok;
@@ -285,7 +285,7 @@ __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t
         }
         break;
       }
-      __builtin_amdgcn_s_sleep(8);
+      __builtin_amdgcn_s_sleep(32);
     }
     Merge::merge(ta, tb, __builtin_bit_cast(A, ua), __builtin_bit_cast(A, ub));
   }

@@ -386,7 +386,7 @@ int dragon_hip_batch_norm_training_backward(int dtype, int64_t N, int64_t C, int
  * last reset: the outputs of that launch are invalid, and the two entry points
  * return DRAGON_HIP_ETIMEOUT until dragon_hip_exchange_reset is called.
  * dragon_hip_exchange_reset: clears that state and sets how many polls (of
- * about 0.2 us) a wait lasts; 0 = the default (about a second). The first use
+ * about a microsecond) a wait lasts; 0 = the default (about a second). The first use
  * allocates four bytes of pinned host memory (do it before capturing a graph). */
 int dragon_hip_exchange_timed_out(void);
 void dragon_hip_exchange_reset(unsigned patience);
