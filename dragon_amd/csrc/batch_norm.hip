@@ -26,6 +26,7 @@
 //     (and dy) is read once: 2 tensor passes forward and 3 backward instead of
 //     3 and 5.
 #include "reduce.h"
+#include "short_rows.h"
 #include "slices.h"
 
 namespace dragon_hip {
@@ -44,8 +45,102 @@ inline SegmentedReduce channel_segments(const ChannelShape& sh) {
 inline size_t channel_scratch_bytes(const ChannelShape& sh, size_t acc_bytes) {
   const uint32_t split = sh.nchw ? channel_segments(sh).split
                                  : column_split_bound(static_cast<int64_t>(sh.N) * sh.S, sh.C);
-  return static_cast<size_t>(sh.C) * split * 2 * acc_bytes;
+  size_t pairs = static_cast<size_t>(sh.C) * split;
+  // one pair per (n, c) row where the rows may take the short-row kernel
+  if (sh.nchw && sh.S <= 1024 && pairs < static_cast<size_t>(sh.N) * sh.C) {
+    pairs = static_cast<size_t>(sh.N) * sh.C;
+  }
+  return pairs * 2 * acc_bytes;
 }
+
+// NCHW tensors whose (n, c) rows of S elements are not whole aligned packets
+// (14x14 and 7x7 feature maps in 16-bit types): the rows go through the
+// LDS-staged short-row kernel (short_rows.h), which reads and writes aligned
+// packets whatever S is. A reduction leaves one pair per (n, c) row, summed
+// over n by the column finalize; a map fetches its channel's parameters once
+// per row.
+inline bool short_channel_rows(const ChannelShape& sh, size_t elem_bytes, const void* a,
+                               const void* b, const void* c) {
+  const int vec = static_cast<int>(16 / elem_bytes);
+  const bool packets = sh.S % vec == 0 && aligned16(a) && aligned16(b) && aligned16(c);
+  return sh.nchw && !packets && sh.S <= 1024 && congruent16(a, b) && congruent16(a, c);
+}
+
+template <typename T, int kE, typename F, int kInputs>
+struct ChannelRowSumsOp {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = kInputs;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 1;
+  static constexpr bool kReadOnly = true;
+  F f;
+  uint32_t C, S;
+  A* partial;  // [N][C] pairs
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[1]) const {
+    const uint32_t c = static_cast<uint32_t>(row % C);
+    F g = f;
+    g.begin(c, c * S);
+    w[0] = g.state();
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A* side, int l, int width, A (&v0)[kE],
+                                      const A (&v1)[kE]) const {
+    F g = f;
+    g.set_state(side[0]);
+    A a = A(0), b = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      if (l + j * kL < width) g.add(0u, 0u, 0u, v0[j], v1[j], a, b);
+    }
+    a = group_allreduce<kL>(a, SumOp());
+    b = group_allreduce<kL>(b, SumOp());
+    if (l == 0) {
+      partial[2 * r] = a;
+      partial[2 * r + 1] = b;
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename F, int kInputs>
+struct RowSumsOf {
+  template <typename T, int kE>
+  using Op = ChannelRowSumsOp<T, kE, F, kInputs>;
+};
+
+template <typename T, int kE, typename F, int kInputs>
+struct ChannelRowMapOp {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = kInputs;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = F::kParams;
+  F f;
+  uint32_t C;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[F::kParams]) const {
+    f.params(static_cast<uint32_t>(row % C), w);
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A* side, int, int, A (&v0)[kE],
+                                      const A (&v1)[kE]) const {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) v0[j] = f.apply(side, v0[j], v1[j]);
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename F, int kInputs>
+struct RowMapOf {
+  template <typename T, int kE>
+  using Op = ChannelRowMapOp<T, kE, F, kInputs>;
+};
 
 // Runs the split reduction of accumulator F (one or two inputs) over every
 // channel and hands the per-channel totals to epilogue E.
@@ -55,6 +150,19 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
   const unsigned fin_grid = static_cast<unsigned>(ceil_div(sh.C, kReduceThreads));
+  ShortPlan sp;
+  if (short_channel_rows(sh, sizeof(T), in0, in1, in0) &&
+      plan_short_rows(sh.S, sizeof(T), kIn == 1 ? 4 : 2, false, &sp)) {
+    using Holder = RowSumsOf<F, kIn>;
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 * kIn + sp.rows_per_chunk * sizeof(A);
+    T* none = nullptr;
+    DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
+                            short_grid(rows, sp.rows_per_chunk), stream, rows,
+                            static_cast<int>(sh.S), in0, in1, none, f, sh.C, sh.S, part);
+    launch_reduce2_finalize<A, E>(sh.C, sh.N, false, part, e, stream);
+    return;
+  }
   if (sh.nchw) {
     const SegmentedReduce s = channel_segments(sh);
     const dim3 grid(s.n_out * s.split);
@@ -81,6 +189,9 @@ template <typename T>
 struct SumSqAccum {  // a = sum x, b = sum x^2
   using A = typename IO<T>::Acc;
   __device__ __forceinline__ void begin(uint32_t, uint32_t) {}
+  // the per-output scalar that begin() fetched (none here)
+  __device__ __forceinline__ A state() const { return A(0); }
+  __device__ __forceinline__ void set_state(A) {}
   template <int V>
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x)[V],
                                       const A (&)[V], A& a, A& b) const {
@@ -104,6 +215,8 @@ struct ShiftedSumSqAccum {  // a = sum (x-s), b = sum (x-s)^2, s = first value o
   __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
     shift = IO<T>::load1(x + first_off);
   }
+  __device__ __forceinline__ A state() const { return shift; }
+  __device__ __forceinline__ void set_state(A v) { shift = v; }
   template <int V>
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&v)[V],
                                       const A (&)[V], A& a, A& b) const {
@@ -127,6 +240,8 @@ struct WGradAccum {  // a = sum dy*(x-mu[c]), b = sum dy
   const A* mu;
   A m;
   __device__ __forceinline__ void begin(uint32_t c, uint32_t) { m = mu[c]; }
+  __device__ __forceinline__ A state() const { return m; }
+  __device__ __forceinline__ void set_state(A v) { m = v; }
   template <int V>
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x)[V],
                                       const A (&dy)[V], A& a, A& b) const {
@@ -250,6 +365,12 @@ struct AffineApply {  // y = x*scale[c] + bias[c]
   ChannelIndex idx;
   const A* scale;
   const A* bias;
+  // The same map with the channel's parameters fetched once per row (NCHW).
+  static constexpr int kParams = 2;
+  __device__ __forceinline__ void params(uint32_t c, A (&w)[kParams]) const {
+    w[0] = scale[c], w[1] = bias[c];
+  }
+  __device__ __forceinline__ A apply(const A* w, A x, A) const { return x * w[0] + w[1]; }
   __device__ __forceinline__ void operator()(uint32_t i, A (&v)[kVec], const A (&)[kVec]) const {
     const uint32_t c = idx(i);
     if (idx.sh.nchw) {
@@ -276,6 +397,13 @@ struct TrainingGradApply {
   const A* dgamma;
   const A* dbeta;
   A normalizer;
+  static constexpr int kParams = 5;
+  __device__ __forceinline__ void params(uint32_t c, A (&w)[kParams]) const {
+    w[0] = rsig[c], w[1] = mu[c], w[2] = gamma[c] * w[0], w[3] = dgamma[c], w[4] = dbeta[c];
+  }
+  __device__ __forceinline__ A apply(const A* w, A x, A dy) const {
+    return w[2] * (dy - ((x - w[1]) * w[0] * w[3] + w[4]) / normalizer);
+  }
   __device__ __forceinline__ void operator()(uint32_t i, A (&x)[kVec], const A (&dy)[kVec]) const {
     const uint32_t c = idx(i);
     if (idx.sh.nchw) {
@@ -306,6 +434,11 @@ struct InferenceGradApply {  // dx = dy * gamma[c] * rsig[c]
   ChannelIndex idx;
   const A* rsig;
   const A* gamma;
+  static constexpr int kParams = 1;
+  __device__ __forceinline__ void params(uint32_t c, A (&w)[kParams]) const {
+    w[0] = gamma[c] * rsig[c];
+  }
+  __device__ __forceinline__ A apply(const A* w, A dy, A) const { return dy * w[0]; }
   __device__ __forceinline__ void operator()(uint32_t i, A (&dy)[kVec], const A (&)[kVec]) const {
     const uint32_t c = idx(i);
     if (idx.sh.nchw) {
@@ -326,9 +459,24 @@ template <typename T, int kIn, template <typename, int> class F, typename... Arg
 void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hipStream_t stream,
                   Args... args) {
   constexpr int kVec = IO<T>::kVec;
+  using A = typename IO<T>::Acc;
   const uint32_t total = sh.N * sh.C * sh.S;
   const bool vec_ok = aligned16(in0) && aligned16(in1) && aligned16(out) &&
       (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
+  ShortPlan sp;
+  if (short_channel_rows(sh, sizeof(T), in0, in1, out) &&
+      plan_short_rows(sh.S, sizeof(T), kIn == 1 ? 4 : 2, false, &sp)) {
+    using Fn = F<T, 1>;
+    using Holder = RowMapOf<Fn, kIn>;
+    const Fn fn{ChannelIndex{sh}, args...};
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 * kIn +
+        static_cast<size_t>(sp.rows_per_chunk) * Fn::kParams * sizeof(A);
+    DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
+                            short_grid(rows, sp.rows_per_chunk), stream, rows,
+                            static_cast<int>(sh.S), in0, in1, out, fn, sh.C);
+    return;
+  }
   if (vec_ok) {
     F<T, kVec> f{ChannelIndex{sh}, args...};
     hipLaunchKernelGGL((map_flat<T, kIn, kVec, F<T, kVec>>), dim3(map_grid(total / kVec)), dim3(256),

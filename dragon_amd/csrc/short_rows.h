@@ -24,6 +24,8 @@
 //                          (e.g. column sums kept per thread); kEndBytes of LDS
 #pragma once
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace dragon_hip {
@@ -107,6 +109,13 @@ __device__ __forceinline__ void stage_out(const StagedRange& r, const u32x4* sta
   }
 }
 
+// An Op that declares `static constexpr bool kReadOnly = true` only reads its
+// rows (a reduction per row): nothing is written back and `out` is not used.
+template <typename Op, typename = void>
+struct OpReadOnly : std::false_type {};
+template <typename Op>
+struct OpReadOnly<Op, std::void_t<decltype(Op::kReadOnly)>> : std::bool_constant<Op::kReadOnly> {};
+
 // in0, in1 (when kIn == 2) and out must be congruent modulo 16 bytes (they
 // usually are: allocations are aligned far beyond that), so that the staged
 // packets map one to one. Several workgroups share a compute unit and overlap
@@ -160,16 +169,20 @@ __global__ __launch_bounds__(kShortThreads) void short_rows(
         if constexpr (Op::kIn == 2) v1[j] = e < C ? IO<T>::load1(p1 + e) : op.fill1();
       }
       op.template row<kL>(row0 + r, side + r * kSide, l, C, v0, v1);
+      if constexpr (!OpReadOnly<Op>::value) {
 #pragma unroll
-      for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
-        if (e < C) IO<T>::store1(p0 + e, v0[j]);
+        for (int j = 0; j < kE; ++j) {
+          const int e = l + j * kL;
+          if (e < C) IO<T>::store1(p0 + e, v0[j]);
+        }
       }
     }
     __syncthreads();
-    const StagedRange ro(out, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-    stage_out<T>(ro, stage);
-    __syncthreads();  // the stage is refilled by the next range
+    if constexpr (!OpReadOnly<Op>::value) {
+      const StagedRange ro(out, total, row0 * row_bytes, (row0 + rows) * row_bytes);
+      stage_out<T>(ro, stage);
+      __syncthreads();  // the stage is refilled by the next range
+    }
   }
   op.template end<kL>(reinterpret_cast<A*>(stage), C);
 }

@@ -428,7 +428,10 @@ def test_group_norm_forward_backward(K, shape, axis, group, dtype, fused):
 # 5 slices per channel over two rounds, with channels that straddle the round boundary.
 BN_CASES = [((8, 16, 7, 7), 1), ((4, 3, 2), 1), ((16, 32), -1), ((4, 5, 5, 24), -1),
             ((6, 64, 28, 28), 1), ((4, 2, 3), -1), ((3, 130, 4), 1), ((50, 70), -1),
-            ((8, 40, 56, 56), 1), ((2, 1100, 16, 16), 1), ((32, 350, 28, 28), 1)]
+            ((8, 40, 56, 56), 1), ((2, 1100, 16, 16), 1), ((32, 350, 28, 28), 1),
+            # feature maps that are not whole packets: (n, c) rows staged through LDS, several
+            # ranges per workgroup ((8, 16, 7, 7) and (4, 3, 2) above take the same path)
+            ((16, 96, 14, 14), 1), ((12, 200, 7, 7), 1), ((3, 33, 30, 30), 1)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16", "float16"])
