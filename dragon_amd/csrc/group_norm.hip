@@ -1128,6 +1128,93 @@ __global__ __launch_bounds__(256) void channel_pair_sums_short(
   }
 }
 
+// The same pairs, and the last step of the general backward, for (n, c) rows of
+// up to 1024 elements that are not whole aligned packets (14x14, 7x7 feature
+// maps): policies of the LDS-staged short-row kernel (short_rows.h), which
+// moves aligned packets whatever S is. The row's scalars are fetched once per
+// row with the range's packets.
+template <typename T, int kE>
+struct GroupRowPairSums {  // in0 = x, in1 = dy; reads only
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 1;
+  static constexpr bool kReadOnly = true;
+  const A* mu;
+  uint32_t D;
+  A* sums;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[1]) const { w[0] = mu[row / D]; }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A* side, int, int, A (&x)[kE],
+                                      const A (&dy)[kE]) const {
+    const A m = side[0];
+    A a = A(0), b = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {  // lanes past the row hold dy = 0
+      a += dy[j] * (x[j] - m);
+      b += dy[j];
+    }
+    a = group_allreduce<kL>(a, SumOp());
+    b = group_allreduce<kL>(b, SumOp());
+    if (threadIdx.x % kL == 0) {
+      sums[2 * r] = a;
+      sums[2 * r + 1] = b;
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
+template <typename T, int kE>
+struct GroupRowGradMap {  // in0 = x (overwritten with dx), in1 = dy
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 6;
+  GroupNormGradApply<T, 1> f;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  // the terms of GroupNormGradApply::one that depend on the row only
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[6]) const {
+    const uint32_t ng = static_cast<uint32_t>(row / f.sh.D);
+    const A m = f.mu[ng], r = f.rsig[ng], s = f.ds[ng], b = f.db[ng];
+    w[0] = m, w[1] = r, w[2] = b * m - s, w[3] = r * r * r, w[4] = b * r;
+    w[5] = f.gamma[row % f.sh.C];
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A* w, int, int, A (&x)[kE],
+                                      const A (&dy)[kE]) const {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const A u = w[2] * (x[j] - w[0]) * w[3];
+      x[j] = w[5] * dy[j] * w[1] + (u - w[4]) * f.denom;
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
+// Workgroups of group_grad_from_channel_sums that form ds / db: a group takes
+// D rounded up to a power of two (at most 64) of a workgroup's 256 threads.
+inline uint32_t group_sum_blocks(const GroupShape& sh) {
+  uint32_t span = 1;
+  while (span < sh.D && span < static_cast<uint32_t>(kWaveSize)) span <<= 1;
+  return static_cast<uint32_t>(ceil_div(static_cast<int64_t>(sh.N) * sh.G, 256 / span));
+}
+
+inline bool short_group_rows(const GroupShape& sh, size_t elem_bytes, const void* x,
+                             const void* dy, const void* dx) {
+  const uint32_t vec = static_cast<uint32_t>(16 / elem_bytes);
+  const bool packets = sh.S % vec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
+  return sh.nchw && !packets && sh.S <= 1024 && congruent16(x, dy) && congruent16(x, dx);
+}
+
 // Stage two. Workgroups [0, group_blocks) form, one thread per (n, g),
 //   ds = sum_c gamma_c * (a_c + mu * b_c),  db = sum_c gamma_c * b_c   over the group's channels;
 // the others own 64 adjacent channels each (one per lane), their four
@@ -1142,19 +1229,31 @@ __global__ __launch_bounds__(256) void group_grad_from_channel_sums(
   __shared__ A lds[4][kWaveSize][2];
   const uint32_t C = G * D;
   if (blockIdx.x < group_blocks) {
-    const uint32_t ng = blockIdx.x * 256 + threadIdx.x;
-    if (ng >= N * G) return;
-    const uint32_t g = ng % G;
-    const A m = mu[ng];
-    const A* row = sums + (static_cast<size_t>(ng / G) * C + g * D) * 2;
+    // `span` adjacent lanes (a power of two, D rounded up, at most 64) share a
+    // group: adjacent lanes read adjacent channel pairs.
+    uint32_t span = 1;
+    while (span < D && span < kWaveSize) span <<= 1;
+    const uint32_t per_block = 256 / span;
+    const uint32_t ng = blockIdx.x * per_block + threadIdx.x / span;
+    const uint32_t l = threadIdx.x % span;
+    const bool on = ng < N * G;
+    const uint32_t g = on ? ng % G : 0;
+    const A m = on ? mu[ng] : A(0);
+    const A* row = sums + (static_cast<size_t>(on ? ng / G : 0) * C + g * D) * 2;
     A s = A(0), b = A(0);
-    for (uint32_t d = 0; d < D; ++d) {
+    for (uint32_t d = l; d < D; d += span) {
       const A w = gamma[g * D + d];
       s += w * (row[2 * d] + m * row[2 * d + 1]);
       b += w * row[2 * d + 1];
     }
-    ds[ng] = s;
-    db[ng] = b;
+    for (uint32_t o = 1; o < span; o <<= 1) {
+      s += __shfl_xor(s, static_cast<int>(o), kWaveSize);
+      b += __shfl_xor(b, static_cast<int>(o), kWaveSize);
+    }
+    if (on && l == 0) {
+      ds[ng] = s;
+      db[ng] = b;
+    }
     return;
   }
   if (dgamma == nullptr) return;
@@ -1164,7 +1263,7 @@ __global__ __launch_bounds__(256) void group_grad_from_channel_sums(
   A a = A(0), b = A(0);
   if (c < C) {
     const uint32_t g = c / D;
-#pragma unroll 4
+#pragma unroll 8
     for (uint32_t n = wave; n < N; n += 4) {
       const size_t idx = (static_cast<size_t>(n) * C + c) * 2;
       a += sums[idx] * rsig[n * G + g];
@@ -1938,7 +2037,14 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     // 1+2. one pass over x and dy for the per-(n, c) pairs, then ds/db and dgamma/dbeta from them
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
     RowConfig cfg;
-    if (sh.S < 16) {
+    ShortPlan sp;
+    if (short_group_rows(sh, sizeof(T), x, dy, dx) &&
+        plan_short_rows(sh.S, sizeof(T), 2, false, &sp)) {
+      const size_t lds = static_cast<size_t>(sp.stage_packets) * 32 + sp.rows_per_chunk * sizeof(A);
+      T* none = nullptr;
+      DRAGON_HIP_SHORT_LAUNCH(T, GroupRowPairSums, sp, lds, short_grid(rows, sp.rows_per_chunk),
+                              stream, rows, static_cast<int>(sh.S), xp, dyp, none, mup, sh.D, part);
+    } else if (sh.S < 16) {
       hipLaunchKernelGGL((channel_pair_sums_short<T>), dim3(map_grid(static_cast<uint32_t>(rows))),
                          dim3(256), 0, stream, rows, static_cast<int>(sh.S), sh.D, xp, dyp, mup,
                          part);
@@ -1962,7 +2068,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       hipLaunchKernelGGL((channel_pair_sums_looped<T>), dim3(loop_grid(rows)), dim3(kLoopThreads),
                          0, stream, rows, static_cast<int64_t>(sh.S), sh.D, xp, dyp, mup, part);
     }
-    const uint32_t group_blocks = static_cast<uint32_t>(ceil_div(sh.N * sh.G, 256));
+    const uint32_t group_blocks = group_sum_blocks(sh);
     const uint32_t chan_blocks = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize));
     hipLaunchKernelGGL((group_grad_from_channel_sums<A>), dim3(group_blocks + chan_blocks),
                        dim3(256), 0, stream, sh.N, sh.G, sh.D, group_blocks, part, gp, mup, rsp,
@@ -1975,7 +2081,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     hipLaunchKernelGGL((sum_batched_partials<A>),
                        dim3(static_cast<unsigned>(ceil_div(sh.N * sh.C, 256))), dim3(256), 0,
                        stream, d, part, sums);
-    const uint32_t group_blocks = static_cast<uint32_t>(ceil_div(sh.N * sh.G, 256));
+    const uint32_t group_blocks = group_sum_blocks(sh);
     const uint32_t chan_blocks = static_cast<uint32_t>(ceil_div(sh.C, kWaveSize));
     hipLaunchKernelGGL((group_grad_from_channel_sums<A>), dim3(group_blocks + chan_blocks),
                        dim3(256), 0, stream, sh.N, sh.G, sh.D, group_blocks, sums, gp, mup, rsp,
@@ -1985,7 +2091,16 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   {
     const A denom = A(1) / A(static_cast<int64_t>(sh.D) * sh.S);
     const bool vec_ok = base_ok && (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
-    if (vec_ok) {
+    ShortPlan sp;
+    if (short_group_rows(sh, sizeof(T), x, dy, dx) &&
+        plan_short_rows(sh.S, sizeof(T), 2, false, &sp)) {
+      const GroupNormGradApply<T, 1> f{sh, mup, rsp, gp, dsp, dbp, denom};
+      const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+      const size_t lds =
+          static_cast<size_t>(sp.stage_packets) * 32 + sp.rows_per_chunk * 6 * sizeof(A);
+      DRAGON_HIP_SHORT_LAUNCH(T, GroupRowGradMap, sp, lds, short_grid(rows, sp.rows_per_chunk),
+                              stream, rows, static_cast<int>(sh.S), xp, dyp, dxp, f);
+    } else if (vec_ok) {
       GroupNormGradApply<T, kVec> f{sh, mup, rsp, gp, dsp, dbp, denom};
       hipLaunchKernelGGL((map_flat<T, 2, kVec, GroupNormGradApply<T, kVec>>),
                          dim3(map_grid(total / kVec)), dim3(256), 0, stream, total, xp, dyp, dxp, f);
