@@ -680,7 +680,9 @@ __global__ __launch_bounds__(kReduceThreads) void layer_norm_wide_grad(
 
 // Moments -> InvStd -> GroupNorm in one pass over x: the group stays in
 // registers between the statistics and the normalisation.
-template <typename T, int kTPR, int kVPT>
+// kAnyS: a channel is not whole packets (the group still is), so the elements
+// of a packet may belong to different channels.
+template <typename T, int kTPR, int kVPT, bool kAnyS = false>
 __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const typename IO<T>::Acc eps, const T* __restrict__ x,
@@ -752,12 +754,24 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
-      const uint32_t c = c0 + (Tile::active(i, npackets) ? col / S : 0u);  // kVec divides S
-      const A gam = gamma[c] * rs, bet = beta[c];
+      const uint32_t first = Tile::active(i, npackets) ? col / S : 0u;
       A v[kVec];
       t.unpack(i, v);
+      if constexpr (kAnyS) {
+        const uint32_t rem = Tile::active(i, npackets) ? col - first * S : 0u;
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+        for (int e = 0; e < kVec; ++e) {
+          uint32_t k = rem + e, c = first;
+          while (k >= S) k -= S, ++c;
+          c = c0 + (c < D ? c : D - 1);
+          v[e] = (v[e] - mean) * (gamma[c] * rs) + beta[c];
+        }
+      } else {
+        const uint32_t c = c0 + first;  // kVec divides S
+        const A gam = gamma[c] * rs, bet = beta[c];
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+      }
       t.p[i] = IO<T>::pack(v);
     }
     if (kPrefetch) nxt.wait_ready();
@@ -1835,7 +1849,7 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
   if (!sh.nchw || !pick_row_config(ceil_div(L, kVec), 8, &cfg)) return false;
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
-  if (sh.S % kVec != 0 || !aligned16(x) || !aligned16(y)) {
+  if (L % kVec != 0 || !aligned16(x) || !aligned16(y)) {
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
@@ -1854,9 +1868,10 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
     const unsigned one_shot = row_grid(rows, Tile::kRowsPerBlock);                              \
-    const unsigned resident =                                                                   \
-        TPR == 1024 ? resident_grid(group_norm_forward_rows<T, TPR, VPT>, TPR, 0) : one_shot;   \
-    hipLaunchKernelGGL((group_norm_forward_rows<T, TPR, VPT>),                                  \
+    auto kernel = sh.S % kVec != 0 ? group_norm_forward_rows<T, TPR, VPT, true>                 \
+                                   : group_norm_forward_rows<T, TPR, VPT, false>;               \
+    const unsigned resident = TPR == 1024 ? resident_grid(kernel, TPR, 0) : one_shot;           \
+    hipLaunchKernelGGL(kernel,                                                                  \
                        dim3(one_shot < resident ? one_shot : resident), dim3(Tile::kThreads), 0, stream, \
                        rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),                     \
                        static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
