@@ -25,6 +25,7 @@
 //     which exchange their partial sums through HBM inside one kernel, so x
 //     (and dy) is read once: 2 tensor passes forward and 3 backward instead of
 //     3 and 5.
+#include "long_rows.h"
 #include "reduce.h"
 #include "short_rows.h"
 #include "slices.h"
@@ -46,8 +47,8 @@ inline size_t channel_scratch_bytes(const ChannelShape& sh, size_t acc_bytes) {
   const uint32_t split = sh.nchw ? channel_segments(sh).split
                                  : column_split_bound(static_cast<int64_t>(sh.N) * sh.S, sh.C);
   size_t pairs = static_cast<size_t>(sh.C) * split;
-  // one pair per (n, c) row where the rows may take the short-row kernel
-  if (sh.nchw && sh.S <= 1024 && pairs < static_cast<size_t>(sh.N) * sh.C) {
+  // one pair per (n, c) row where the rows may take the short- or long-row kernels
+  if (sh.nchw && pairs < static_cast<size_t>(sh.N) * sh.C) {
     pairs = static_cast<size_t>(sh.N) * sh.C;
   }
   return pairs * 2 * acc_bytes;
@@ -59,11 +60,20 @@ inline size_t channel_scratch_bytes(const ChannelShape& sh, size_t acc_bytes) {
 // packets whatever S is. A reduction leaves one pair per (n, c) row, summed
 // over n by the column finalize; a map fetches its channel's parameters once
 // per row.
-inline bool short_channel_rows(const ChannelShape& sh, size_t elem_bytes, const void* a,
-                               const void* b, const void* c) {
+inline bool ragged_channel_rows(const ChannelShape& sh, size_t elem_bytes, const void* a,
+                                const void* b, const void* c) {
   const int vec = static_cast<int>(16 / elem_bytes);
   const bool packets = sh.S % vec == 0 && aligned16(a) && aligned16(b) && aligned16(c);
-  return sh.nchw && !packets && sh.S <= 1024 && congruent16(a, b) && congruent16(a, c);
+  return sh.nchw && !packets && congruent16(a, b) && congruent16(a, c);
+}
+inline bool short_channel_rows(const ChannelShape& sh, size_t elem_bytes, const void* a,
+                               const void* b, const void* c) {
+  return sh.S <= 1024 && ragged_channel_rows(sh, elem_bytes, a, b, c);
+}
+// Longer rows of that kind (35x35, 71x71 maps): one wavefront per row (long_rows.h).
+inline bool long_channel_rows(const ChannelShape& sh, size_t elem_bytes, const void* a,
+                              const void* b, const void* c) {
+  return sh.S > 1024 && ragged_channel_rows(sh, elem_bytes, a, b, c);
 }
 
 template <typename T, int kE, typename F, int kInputs>
@@ -85,6 +95,14 @@ struct ChannelRowSumsOp {
     F g = f;
     g.begin(c, c * S);
     w[0] = g.state();
+  }
+  // the same for the one-wavefront-per-row kernel (long_rows.h)
+  static constexpr int kParams = 1;
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[1]) const { fetch_side(row, w); }
+  __device__ __forceinline__ void add(const A* w, A x0, A x1, A& a, A& b) const {
+    F g = f;
+    g.set_state(w[0]);
+    g.add(0u, 0u, 0u, x0, x1, a, b);
   }
   template <int kL>
   __device__ __forceinline__ void row(int64_t r, const A* side, int l, int width, A (&v0)[kE],
@@ -127,6 +145,11 @@ struct ChannelRowMapOp {
   __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[F::kParams]) const {
     f.params(static_cast<uint32_t>(row % C), w);
   }
+  static constexpr int kParams = F::kParams;
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[F::kParams]) const {
+    fetch_side(row, w);
+  }
+  __device__ __forceinline__ A apply(const A* w, A x0, A x1) const { return f.apply(w, x0, x1); }
   template <int kL>
   __device__ __forceinline__ void row(int64_t, const A* side, int, int, A (&v0)[kE],
                                       const A (&v1)[kE]) const {
@@ -160,6 +183,15 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
     DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
                             short_grid(rows, sp.rows_per_chunk), stream, rows,
                             static_cast<int>(sh.S), in0, in1, none, f, sh.C, sh.S, part);
+    launch_reduce2_finalize<A, E>(sh.C, sh.N, false, part, e, stream);
+    return;
+  }
+  if (long_channel_rows(sh, sizeof(T), in0, in1, in0)) {
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    const ChannelRowSumsOp<T, 8, F, kIn> op{f, sh.C, sh.S, part};
+    hipLaunchKernelGGL((long_rows_sums<T, kIn, ChannelRowSumsOp<T, 8, F, kIn>>),
+                       dim3(long_rows_grid(rows)), dim3(kLongThreads), 0, stream, rows,
+                       static_cast<int>(sh.S), in0, in1, op, part);
     launch_reduce2_finalize<A, E>(sh.C, sh.N, false, part, e, stream);
     return;
   }
@@ -475,6 +507,15 @@ void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hi
     DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
                             short_grid(rows, sp.rows_per_chunk), stream, rows,
                             static_cast<int>(sh.S), in0, in1, out, fn, sh.C);
+    return;
+  }
+  if (long_channel_rows(sh, sizeof(T), in0, in1, out)) {
+    using Fn = F<T, 1>;
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    const ChannelRowMapOp<T, 8, Fn, kIn> op{Fn{ChannelIndex{sh}, args...}, sh.C};
+    hipLaunchKernelGGL((long_rows_map<T, kIn, ChannelRowMapOp<T, 8, Fn, kIn>>),
+                       dim3(long_rows_grid(rows)), dim3(kLongThreads), 0, stream, rows,
+                       static_cast<int>(sh.S), in0, in1, out, op);
     return;
   }
   if (vec_ok) {

@@ -35,6 +35,7 @@
 //          any alignment.
 #include <cstdlib>
 
+#include "long_rows.h"
 #include "reduce.h"
 #include "row_loop.h"
 #include "row_tile.h"
@@ -1162,6 +1163,13 @@ struct GroupRowPairSums {  // in0 = x, in1 = dy; reads only
   template <int kL>
   __device__ __forceinline__ void begin(int, int) {}
   __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[1]) const { w[0] = mu[row / D]; }
+  // the same for the one-wavefront-per-row kernel (long_rows.h)
+  static constexpr int kParams = 1;
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[1]) const { fetch_side(row, w); }
+  __device__ __forceinline__ void add(const A* w, A x, A dy, A& a, A& b) const {
+    a += dy * (x - w[0]);
+    b += dy;
+  }
   template <int kL>
   __device__ __forceinline__ void row(int64_t r, const A* side, int, int, A (&x)[kE],
                                       const A (&dy)[kE]) const {
@@ -1201,14 +1209,17 @@ struct GroupRowGradMap {  // in0 = x (overwritten with dx), in1 = dy
     w[0] = m, w[1] = r, w[2] = b * m - s, w[3] = r * r * r, w[4] = b * r;
     w[5] = f.gamma[row % f.sh.C];
   }
+  static constexpr int kParams = 6;
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[6]) const { fetch_side(row, w); }
+  __device__ __forceinline__ A apply(const A* w, A x, A dy) const {
+    const A u = w[2] * (x - w[0]) * w[3];
+    return w[5] * dy * w[1] + (u - w[4]) * f.denom;
+  }
   template <int kL>
   __device__ __forceinline__ void row(int64_t, const A* w, int, int, A (&x)[kE],
                                       const A (&dy)[kE]) const {
 #pragma unroll
-    for (int j = 0; j < kE; ++j) {
-      const A u = w[2] * (x[j] - w[0]) * w[3];
-      x[j] = w[5] * dy[j] * w[1] + (u - w[4]) * f.denom;
-    }
+    for (int j = 0; j < kE; ++j) x[j] = apply(w, x[j], dy[j]);
   }
   template <int kL>
   __device__ __forceinline__ void end(A*, int) const {}
@@ -1222,11 +1233,83 @@ inline uint32_t group_sum_blocks(const GroupShape& sh) {
   return static_cast<uint32_t>(ceil_div(static_cast<int64_t>(sh.N) * sh.G, 256 / span));
 }
 
-inline bool short_group_rows(const GroupShape& sh, size_t elem_bytes, const void* x,
-                             const void* dy, const void* dx) {
+// Forward of such rows. The map: y = (x - mu) * rsig * gamma + beta with the four
+// scalars of the (n, c) row. The statistics: a group is one row of D*S
+// elements; sums are shifted by the row's first element.
+template <typename T, int kE>
+struct GroupRowApply {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 4;
+  static constexpr int kParams = 4;
+  GroupNormApply<T, 1> f;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  __device__ __forceinline__ void fetch_side(int64_t row, A (&w)[4]) const {
+    const uint32_t ng = static_cast<uint32_t>(row / f.sh.D);
+    const uint32_t c = static_cast<uint32_t>(row % f.sh.C);
+    w[0] = f.mu[ng], w[1] = f.rsig[ng], w[2] = f.gamma[c], w[3] = f.beta[c];
+  }
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[4]) const { fetch_side(row, w); }
+  __device__ __forceinline__ A apply(const A* w, A x, A) const {
+    return (x - w[0]) * w[1] * w[2] + w[3];
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t, const A* w, int, int, A (&x)[kE],
+                                      const A (&)[kE]) const {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) x[j] = apply(w, x[j], A(0));
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
+template <typename T>
+struct GroupRowMoments {  // a = sum (x - first), b = sum (x - first)^2 over a group's row
+  using A = typename IO<T>::Acc;
+  static constexpr int kParams = 1;
+  const T* x;
+  int64_t L;
+  __device__ __forceinline__ void row_params(int64_t row, A (&w)[1]) const {
+    w[0] = IO<T>::load1(x + row * L);
+  }
+  __device__ __forceinline__ void add(const A* w, A v, A, A& a, A& b) const {
+    const A d = v - w[0];
+    a += d;
+    b += d * d;
+  }
+};
+template <typename T>
+__global__ __launch_bounds__(256) void group_stats_from_row_sums(
+    const int64_t rows, const int64_t L, const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ pairs, typename IO<T>::Acc* __restrict__ mu,
+    typename IO<T>::Acc* __restrict__ rsig) {
+  using A = typename IO<T>::Acc;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (row >= rows) return;
+  const A inv = A(1) / A(L);
+  const A d = pairs[2 * row] * inv;
+  mu[row] = IO<T>::load1(x + row * L) + d;
+  rsig[row] = acc_rsqrt_exact((pairs[2 * row + 1] * inv - d * d) + eps);
+}
+
+inline bool ragged_group_rows(const GroupShape& sh, size_t elem_bytes, const void* x,
+                              const void* dy, const void* dx) {
   const uint32_t vec = static_cast<uint32_t>(16 / elem_bytes);
   const bool packets = sh.S % vec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
-  return sh.nchw && !packets && sh.S <= 1024 && congruent16(x, dy) && congruent16(x, dx);
+  return sh.nchw && !packets && congruent16(x, dy) && congruent16(x, dx);
+}
+inline bool short_group_rows(const GroupShape& sh, size_t elem_bytes, const void* x,
+                             const void* dy, const void* dx) {
+  return sh.S <= 1024 && ragged_group_rows(sh, elem_bytes, x, dy, dx);
+}
+// Longer rows of that kind: one wavefront per (n, c) row (long_rows.h).
+inline bool long_group_rows(const GroupShape& sh, size_t elem_bytes, const void* x, const void* dy,
+                            const void* dx) {
+  return sh.S > 1024 && ragged_group_rows(sh, elem_bytes, x, dy, dx);
 }
 
 // Stage two. Workgroups [0, group_blocks) form, one thread per (n, g),
@@ -1892,7 +1975,24 @@ int launch_group_norm(const GroupShape& sh, const void* x, const void* mu, const
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   const bool vec_ok = aligned16(x) && aligned16(y) && (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
-  if (vec_ok) {
+  ShortPlan sp;
+  if (short_group_rows(sh, sizeof(T), x, x, y) && plan_short_rows(sh.S, sizeof(T), 4, false, &sp)) {
+    // (n, c) rows that are not whole aligned packets: staged through LDS
+    const GroupNormApply<T, 1> f{sh, static_cast<const A*>(mu), static_cast<const A*>(rsig),
+                                 static_cast<const A*>(gamma), static_cast<const A*>(beta)};
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 + sp.rows_per_chunk * 4 * sizeof(A);
+    DRAGON_HIP_SHORT_LAUNCH(T, GroupRowApply, sp, lds, short_grid(rows, sp.rows_per_chunk), stream,
+                            rows, static_cast<int>(sh.S), xp, xp, yp, f);
+  } else if (long_group_rows(sh, sizeof(T), x, x, y)) {
+    // longer rows of that kind: one wavefront per row
+    const GroupRowApply<T, 8> op{GroupNormApply<T, 1>{
+        sh, static_cast<const A*>(mu), static_cast<const A*>(rsig), static_cast<const A*>(gamma),
+        static_cast<const A*>(beta)}};
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+    hipLaunchKernelGGL((long_rows_map<T, 1, GroupRowApply<T, 8>>), dim3(long_rows_grid(rows)),
+                       dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, xp, yp, op);
+  } else if (vec_ok) {
     GroupNormApply<T, kVec> f{sh, static_cast<const A*>(mu), static_cast<const A*>(rsig),
                               static_cast<const A*>(gamma), static_cast<const A*>(beta)};
     hipLaunchKernelGGL((map_flat<T, 1, kVec, GroupNormApply<T, kVec>>), dim3(map_grid(total / kVec)),
@@ -2059,6 +2159,11 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       T* none = nullptr;
       DRAGON_HIP_SHORT_LAUNCH(T, GroupRowPairSums, sp, lds, short_grid(rows, sp.rows_per_chunk),
                               stream, rows, static_cast<int>(sh.S), xp, dyp, none, mup, sh.D, part);
+    } else if (long_group_rows(sh, sizeof(T), x, dy, dx)) {
+      const GroupRowPairSums<T, 8> op{mup, sh.D, part};
+      hipLaunchKernelGGL((long_rows_sums<T, 2, GroupRowPairSums<T, 8>>), dim3(long_rows_grid(rows)),
+                         dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, dyp, op,
+                         part);
     } else if (sh.S < 16) {
       hipLaunchKernelGGL((channel_pair_sums_short<T>), dim3(map_grid(static_cast<uint32_t>(rows))),
                          dim3(256), 0, stream, rows, static_cast<int>(sh.S), sh.D, xp, dyp, mup,
@@ -2115,6 +2220,12 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
           static_cast<size_t>(sp.stage_packets) * 32 + sp.rows_per_chunk * 6 * sizeof(A);
       DRAGON_HIP_SHORT_LAUNCH(T, GroupRowGradMap, sp, lds, short_grid(rows, sp.rows_per_chunk),
                               stream, rows, static_cast<int>(sh.S), xp, dyp, dxp, f);
+    } else if (long_group_rows(sh, sizeof(T), x, dy, dx)) {
+      const GroupRowGradMap<T, 8> op{GroupNormGradApply<T, 1>{sh, mup, rsp, gp, dsp, dbp, denom}};
+      const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
+      hipLaunchKernelGGL((long_rows_map<T, 2, GroupRowGradMap<T, 8>>), dim3(long_rows_grid(rows)),
+                         dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, dyp, dxp,
+                         op);
     } else if (vec_ok) {
       GroupNormGradApply<T, kVec> f{sh, mup, rsp, gp, dsp, dbp, denom};
       hipLaunchKernelGGL((map_flat<T, 2, kVec, GroupNormGradApply<T, kVec>>),
@@ -2130,6 +2241,30 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 
 // NHWC statistics of the fused forward: column sums per sample, then mean and
 // rsig per group (InvStd folded into the second stage).
+// Statistics of NCHW groups whose rows of D*S elements are not whole aligned
+// packets and exceed the register tiles: one wavefront per group row, then
+// mean and rsig from the shifted sums. kNotApplicable leaves the call to Moments.
+template <typename T>
+int try_group_norm_stats_rows(const GroupShape& sh, float eps, const void* x, void* mu, void* rsig,
+                              void* scratch, size_t scratch_bytes, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
+  const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+  const bool packets = L % kVec == 0 && aligned16(x);
+  if (!sh.nchw || packets || L <= 1024 || !fits_int32(L)) return kNotApplicable;
+  if (!scratch || scratch_bytes < static_cast<size_t>(rows) * 2 * sizeof(A)) return kNotApplicable;
+  const T* xp = static_cast<const T*>(x);
+  A* pairs = static_cast<A*>(scratch);
+  const GroupRowMoments<T> op{xp, L};
+  hipLaunchKernelGGL((long_rows_sums<T, 1, GroupRowMoments<T>>), dim3(long_rows_grid(rows)),
+                     dim3(kLongThreads), 0, stream, rows, static_cast<int>(L), xp, xp, op, pairs);
+  hipLaunchKernelGGL((group_stats_from_row_sums<T>), dim3(static_cast<unsigned>(ceil_div(rows, 256))),
+                     dim3(256), 0, stream, rows, L, A(eps), xp, pairs, static_cast<A*>(mu),
+                     static_cast<A*>(rsig));
+  return status_of_launch();
+}
+
 template <typename T>
 int group_norm_stats_nhwc(const GroupShape& sh, float eps, const void* x, void* mu, void* rsig,
                           void* scratch, hipStream_t stream) {
@@ -2271,6 +2406,9 @@ size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t
   } else {
     const size_t slices = dragon_hip::group_slices_scratch_bytes(dtype, sh);
     if (slices > bytes) bytes = slices;
+    // one pair per group row for the one-wavefront-per-row statistics
+    const size_t rows = static_cast<size_t>(N) * G * 2 * (dtype == DRAGON_HIP_F64 ? 8 : 4);
+    if (rows > bytes) bytes = rows;
   }
   return bytes;
 }
@@ -2325,6 +2463,16 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
     if (st != DRAGON_HIP_OK) return st;
     return dragon_hip_group_norm(dtype, N, G, D, S, layout, x, mu, rsig, gamma, beta, y, stream);
   }
+  switch (dtype) {
+    case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_stats_rows<dragon_hip::f16_t>(sh, eps, x, mu, rsig, scratch, scratch_bytes, hs); break;
+    case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_stats_rows<dragon_hip::bf16_t>(sh, eps, x, mu, rsig, scratch, scratch_bytes, hs); break;
+    case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_stats_rows<float>(sh, eps, x, mu, rsig, scratch, scratch_bytes, hs); break;
+    default: st = dragon_hip::try_group_norm_stats_rows<double>(sh, eps, x, mu, rsig, scratch, scratch_bytes, hs); break;
+  }
+  if (st == DRAGON_HIP_OK) {
+    return dragon_hip_group_norm(dtype, N, G, D, S, layout, x, mu, rsig, gamma, beta, y, stream);
+  }
+  if (st != dragon_hip::kNotApplicable) return st;
   const GroupMomentsView v = group_moments_view(N, G, D, S, layout);
   st = dragon_hip_moments(dtype, v.num_dims, v.dims, v.num_axes, v.axes, x, mu, rsig, scratch,
                           scratch_bytes, stream);

@@ -431,7 +431,10 @@ BN_CASES = [((8, 16, 7, 7), 1), ((4, 3, 2), 1), ((16, 32), -1), ((4, 5, 5, 24), 
             ((8, 40, 56, 56), 1), ((2, 1100, 16, 16), 1), ((32, 350, 28, 28), 1),
             # feature maps that are not whole packets: (n, c) rows staged through LDS, several
             # ranges per workgroup ((8, 16, 7, 7) and (4, 3, 2) above take the same path)
-            ((16, 96, 14, 14), 1), ((12, 200, 7, 7), 1), ((3, 33, 30, 30), 1)]
+            ((16, 96, 14, 14), 1), ((12, 200, 7, 7), 1), ((3, 33, 30, 30), 1),
+            # longer rows of that kind: one wavefront per (n, c) row, leading and trailing
+            # elements of a row moved one by one around its aligned packets
+            ((5, 24, 35, 35), 1), ((3, 10, 71, 71), 1)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float64", "bfloat16", "float16"])
