@@ -53,6 +53,17 @@ struct GroupShape {
 // --------------------------------------------------------------------------
 // Forward map
 // --------------------------------------------------------------------------
+// kVec consecutive per-channel parameters at p (16-byte aligned when kVec > 1:
+// the packet's first channel is a multiple of kVec).
+template <int kVec, typename A>
+__device__ __forceinline__ void load_channel_run(const A* p, A (&v)[kVec]) {
+  if constexpr (kVec == 1) {
+    v[0] = p[0];
+  } else {
+    load_params_ragged<kVec>(p, kVec, v);
+  }
+}
+
 template <typename T, int kVec>
 struct GroupNormApply {
   using A = typename IO<T>::Acc;
@@ -86,11 +97,33 @@ struct GroupNormApply {
         for (int e = 0; e < kVec; ++e) v[e] = (v[e] - m) * r * g[e] + b[e];
         return;
       }
+      if (kVec > 1 && sh.D == 1) {
+        // a group per channel: the statistics are packets as well
+        A m[kVec], r[kVec], gam[kVec], bet[kVec];
+        load_channel_run<kVec>(mu + n * sh.G + c, m);
+        load_channel_run<kVec>(rsig + n * sh.G + c, r);
+        load_channel_run<kVec>(gamma + c, gam);
+        load_channel_run<kVec>(beta + c, bet);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - m[e]) * r[e] * gam[e] + bet[e];
+        return;
+      }
+      // The packet spans several groups (D is not a multiple of kVec): one
+      // division per packet, then the group advances with the channel.
+      uint32_t g = sh.G == 1 ? 0u : c / sh.D;
+      uint32_t k = c - g * sh.D;
+      A m = mu[n * sh.G + g], r = rsig[n * sh.G + g];
+      A gam[kVec], bet[kVec];
+      load_channel_run<kVec>(gamma + c, gam);
+      load_channel_run<kVec>(beta + c, bet);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        const uint32_t ce = c + e;
-        const uint32_t ng = n * sh.G + (sh.G == 1 ? 0u : ce / sh.D);
-        v[e] = (v[e] - mu[ng]) * rsig[ng] * gamma[ce] + beta[ce];
+        if (k == sh.D) {
+          k = 0, ++g;
+          m = mu[n * sh.G + g], r = rsig[n * sh.G + g];
+        }
+        v[e] = (v[e] - m) * r * gam[e] + bet[e];
+        ++k;
       }
     }
   }
@@ -137,10 +170,39 @@ struct GroupNormGradApply {
         for (int e = 0; e < kVec; ++e) x[e] = g[e] * dy[e] * r + (ku * (x[e] - m) - kv);
         return;
       }
+      if (kVec > 1 && sh.D == 1) {
+        // a group per channel: the per-group scalars are packets as well
+        A m[kVec], r[kVec], s[kVec], b[kVec], gam[kVec];
+        load_channel_run<kVec>(mu + n * sh.G + c, m);
+        load_channel_run<kVec>(rsig + n * sh.G + c, r);
+        load_channel_run<kVec>(ds + n * sh.G + c, s);
+        load_channel_run<kVec>(db + n * sh.G + c, b);
+        load_channel_run<kVec>(gamma + c, gam);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A u = (b[e] * m[e] - s[e]) * (x[e] - m[e]) * (r[e] * r[e] * r[e]);
+          const A v = b[e] * r[e];
+          x[e] = gam[e] * dy[e] * r[e] + (u - v) * denom;
+        }
+        return;
+      }
+      // several groups per packet: as GroupNormApply
+      uint32_t g = sh.G == 1 ? 0u : c / sh.D;
+      uint32_t k = c - g * sh.D;
+      uint32_t ng = n * sh.G + g;
+      A m = mu[ng], r = rsig[ng], s = ds[ng], b = db[ng];
+      A gam[kVec];
+      load_channel_run<kVec>(gamma + c, gam);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        const uint32_t ce = c + e;
-        x[e] = one(x[e], dy[e], n * sh.G + (sh.G == 1 ? 0u : ce / sh.D), ce);
+        if (k == sh.D) {
+          k = 0, ++ng;
+          m = mu[ng], r = rsig[ng], s = ds[ng], b = db[ng];
+        }
+        const A u = (b * m - s) * (x[e] - m) * (r * r * r);
+        const A v = b * r;
+        x[e] = gam[e] * dy[e] * r + (u - v) * denom;
+        ++k;
       }
     }
   }
@@ -1400,14 +1462,20 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
     typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   __shared__ A lds[kReduceWaves][kWaveSize][2 * kW];
-  const uint32_t tile_cols = kWaveSize * kW;
+  // Lanes along a row: the whole wavefront, or for fewer than 64 * kW columns
+  // the power of two that covers a row, the other lane bits taking adjacent rows.
+  uint32_t along_lanes = 1;
+  while (along_lanes < kWaveSize && along_lanes * kW < d.C) along_lanes <<= 1;
+  const uint32_t rows_per_wave = kWaveSize / along_lanes;
+  const uint32_t tile_cols = along_lanes * kW;
   const uint32_t tiles = (d.C + tile_cols - 1) / tile_cols;
   const uint32_t tile = blockIdx.x % tiles;
   const uint32_t k = (blockIdx.x / tiles) % d.split;
   const uint32_t n = blockIdx.x / (tiles * d.split);
   const uint32_t lane = threadIdx.x & (kWaveSize - 1);
   const uint32_t wave = threadIdx.x / kWaveSize;
-  const uint32_t c0 = tile * tile_cols + lane * kW;
+  const uint32_t across = lane / along_lanes;
+  const uint32_t c0 = tile * tile_cols + (lane % along_lanes) * kW;
   A a[kW], b[kW];
 #pragma unroll
   for (int e = 0; e < kW; ++e) a[e] = b[e] = A(0);
@@ -1420,7 +1488,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
     }
     const uint32_t base = n * d.S * d.C + c0;
 #pragma unroll 4
-    for (uint32_t r = k * kReduceWaves + wave; r < d.S; r += d.split * kReduceWaves) {
+    for (uint32_t r = (k * kReduceWaves + wave) * rows_per_wave + across; r < d.S;
+         r += d.split * kReduceWaves * rows_per_wave) {
       const uint32_t off = base + r * d.C;
       A x0[kW], x1[kW];
       if constexpr (kW == 1) {
@@ -1434,13 +1503,20 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
       for (int e = 0; e < kW; ++e) fs[e].add(x0[e], kIn == 2 ? x1[e] : A(0), a[e], b[e]);
     }
   }
+  for (uint32_t o = along_lanes; o < kWaveSize; o <<= 1) {  // the lanes that share a column
+#pragma unroll
+    for (int e = 0; e < kW; ++e) {
+      a[e] += __shfl_xor(a[e], static_cast<int>(o), kWaveSize);
+      b[e] += __shfl_xor(b[e], static_cast<int>(o), kWaveSize);
+    }
+  }
 #pragma unroll
   for (int e = 0; e < kW; ++e) {
     lds[wave][lane][2 * e] = a[e];
     lds[wave][lane][2 * e + 1] = b[e];
   }
   __syncthreads();
-  if (wave == 0 && c0 < d.C) {
+  if (wave == 0 && across == 0 && c0 < d.C) {
     A* out = partial + ((static_cast<size_t>(n) * d.split + k) * d.C + c0) * 2;
 #pragma unroll
     for (int e = 0; e < kW; ++e) {

@@ -161,22 +161,28 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_columns(
 }
 
 // The same with a 16-byte packet of kVec adjacent columns per lane (cols a
-// multiple of kVec, 16-byte aligned base): a wavefront reads 1 KiB of a row at
-// a time. Each column keeps its own copy of the accumulator functor.
+// multiple of kVec, 16-byte aligned base): a wavefront reads 1 KiB at a time.
+// `lanes_per_row` lanes lie along a row: the whole wavefront, or, for a matrix
+// of fewer than 64 packets per row, the power of two that covers a row, the
+// remaining lane bits taking adjacent rows (so that 32 sixteen-bit channels do
+// not leave 60 of 64 lanes idle). Each column keeps its own copy of the
+// accumulator functor.
 template <typename T, int kIn, typename F>
 __global__ __launch_bounds__(kReduceThreads) void reduce2_columns_packets(
-    const ColumnReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
-    typename IO<T>::Acc* __restrict__ partial) {
+    const ColumnReduce d, const uint32_t lanes_per_row, const T* __restrict__ in0,
+    const T* __restrict__ in1, F f, typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
   __shared__ A lds[kReduceWaves][kWaveSize][2 * kVec];
-  const uint32_t tile_cols = kWaveSize * kVec;
+  const uint32_t rows_per_wave = kWaveSize / lanes_per_row;
+  const uint32_t tile_cols = lanes_per_row * kVec;
   const uint32_t tiles = (d.cols + tile_cols - 1) / tile_cols;
   const uint32_t tile = blockIdx.x % tiles;
   const uint32_t k = blockIdx.x / tiles;
   const uint32_t lane = threadIdx.x & (kWaveSize - 1);
   const uint32_t wave = threadIdx.x / kWaveSize;
-  const uint32_t c0 = tile * tile_cols + lane * kVec;
+  const uint32_t along = lane % lanes_per_row, across = lane / lanes_per_row;
+  const uint32_t c0 = tile * tile_cols + along * kVec;
   A a[kVec], b[kVec];
 #pragma unroll
   for (int e = 0; e < kVec; ++e) a[e] = b[e] = A(0);
@@ -188,7 +194,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_columns_packets(
       fs[e].begin(c0 + e, c0 + e);
     }
 #pragma unroll 4
-    for (uint32_t r = k * kReduceWaves + wave; r < d.rows; r += d.split * kReduceWaves) {
+    for (uint32_t r = (k * kReduceWaves + wave) * rows_per_wave + across; r < d.rows;
+         r += d.split * kReduceWaves * rows_per_wave) {
       const uint32_t off = r * d.cols + c0;
       A x0[kVec], x1[kVec];
       load_unpack<T>(in0 + off, x0);
@@ -199,13 +206,21 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_columns_packets(
       }
     }
   }
+  // the lanes that share a column (uniform trip count: every lane takes part)
+  for (uint32_t o = lanes_per_row; o < kWaveSize; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      a[e] += __shfl_xor(a[e], static_cast<int>(o), kWaveSize);
+      b[e] += __shfl_xor(b[e], static_cast<int>(o), kWaveSize);
+    }
+  }
 #pragma unroll
   for (int e = 0; e < kVec; ++e) {
     lds[wave][lane][2 * e] = a[e];
     lds[wave][lane][2 * e + 1] = b[e];
   }
   __syncthreads();
-  if (wave == 0 && c0 < d.cols) {
+  if (wave == 0 && across == 0 && c0 < d.cols) {
 #pragma unroll
     for (int e = 0; e < kVec; ++e) {
 #pragma unroll
@@ -233,10 +248,12 @@ inline uint32_t launch_reduce2_columns(uint32_t rows, uint32_t cols, const T* in
   ColumnReduce d{rows, cols, 1};
   const bool packets = cols % kVec == 0 && aligned16(in0) && (kIn == 1 || aligned16(in1));
   if (packets) {
-    const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, kWaveSize * kVec));
+    uint32_t lanes_per_row = 1;
+    while (lanes_per_row < kWaveSize && lanes_per_row * kVec < cols) lanes_per_row <<= 1;
+    const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, lanes_per_row * kVec));
     d.split = pick_split(tiles, static_cast<int64_t>(rows) * kWaveSize * kVec);
     hipLaunchKernelGGL((reduce2_columns_packets<T, kIn, F>), dim3(tiles * d.split),
-                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+                       dim3(kReduceThreads), 0, stream, d, lanes_per_row, in0, in1, f, partial);
   } else {
     d.split = pick_split(ceil_div(cols, kWaveSize), static_cast<int64_t>(rows) * kWaveSize);
     hipLaunchKernelGGL((reduce2_columns<T, kIn, F>),
