@@ -350,7 +350,11 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # fused backward splits a wavefront's packets between two channels
             ((2, 16, 28, 28), 1, 4), ((2, 64, 56, 56), 1, 8), ((1, 6, 24, 24), 1, 2),
             # channels of a few packets: several channels per wavefront in the fused backward
-            ((2, 64, 16, 16), 1, 4), ((3, 48, 8, 8), 1, 2)]
+            ((2, 64, 16, 16), 1, 4), ((3, 48, 8, 8), 1, 2),
+            # odd feature maps of more than 1024 elements in every dtype: one wavefront per
+            # (n, c) row in the backward and the map; per group row in the forward statistics
+            # of groups beyond the register tiles
+            ((2, 6, 33, 35), 1, 2), ((1, 2, 301, 303), 1, 2)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
