@@ -1114,3 +1114,85 @@ def test_l2_norm_and_cross_entropy_beyond_int32_elements(K):
         "float32", U.to_host(logits[idx]), U.to_host(target[idx]), reduction="none")
     assert U.normwise(U.to_host(prob[idx]), prob_ref) <= U.TIGHT["float32"]
     assert U.normwise(U.to_host(loss[idx]), loss_ref) <= U.TIGHT["float32"]
+
+
+# ---------------------------------------------------------------- channel ops at shifted bases
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(4, 12, 9, 9), (2, 6, 40, 41)])
+@pytest.mark.parametrize("shift", [1, 3])
+def test_channel_ops_at_shifted_bases(K, dtype, shape, shift):
+    """NCHW tensors that start `shift` elements past a 16-byte boundary (views into a larger
+    buffer): BatchNorm and GroupNorm forward and backward take the staged short-row kernels
+    ((n, c) rows of 81 elements) or one wavefront per row (1640 elements), whose first and
+    last packets reach outside the tensors. Nothing outside the outputs may be written."""
+    rng = U.rng_for(900 + shift)
+    N, C = shape[0], shape[1]
+    S = shape[2] * shape[3]
+    total = N * C * S
+    an = acc_name(dtype)
+    guard = 8
+    x = R.to_bits((2 * rng.standard_normal(shape) + 0.5).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+
+    def shifted(bits=None):
+        buf = empty((total + shift + guard,), dtype)
+        buf.zero_()
+        view = buf[shift:shift + total].view(shape)
+        if bits is not None:
+            view.copy_(U.to_device(bits, dtype).view(shape))
+        return buf, view
+
+    def untouched(buf):
+        flat = U.widen(U.to_host(buf), dtype).ravel()
+        return np.all(flat[:shift] == 0) and np.all(flat[shift + total:] == 0)
+
+    _, xd = shifted(x)
+    _, dyd = shifted(dy)
+    gd, bd = U.to_device(g, an), U.to_device(b, an)
+
+    # BatchNorm
+    rm_ref = np.zeros(C, U.acc_np(dtype))
+    rv_ref = np.ones(C, U.acc_np(dtype))
+    y_ref, mu_ref, rsig_ref, _ = R.op_batch_norm_train(
+        od, np.asarray(xo).reshape(shape), g, b, rm_ref, rv_ref, 1, 0.9, 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_train_grad(
+        od, np.asarray(xo).reshape(shape), g, np.asarray(dyo).reshape(shape), mu_ref, rsig_ref, 1)
+    mu, rsig, params = empty((C,), an), empty((C,), an), empty((2 * C,), an)
+    rm, rv = U.to_device(np.zeros(C, U.acc_np(dtype)), an), U.to_device(np.ones(C, U.acc_np(dtype)), an)
+    ybuf, y = shifted()
+    K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, xd, gd, bd, rm, rv, mu, rsig, params, y)
+    assert U.normwise(U.to_host(mu), mu_ref) <= 1e-5
+    assert U.normwise(U.widen(U.to_host(y.contiguous()), dtype).reshape(shape), y_ref) <= U.TIGHT[dtype]
+    assert untouched(ybuf)
+    dxbuf, dx = shifted()
+    dg, db = empty((C,), an), empty((C,), an)
+    K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", xd, U.to_device(mu_ref, an),
+                                   U.to_device(rsig_ref, an), gd, dyd, dg, db, dx)
+    assert U.normwise(U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape), dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(U.to_host(dg), dg_ref) <= 2e-5 and U.normwise(U.to_host(db), db_ref) <= 2e-5
+    assert untouched(dxbuf)
+
+    # GroupNorm, 3 groups
+    G = 3
+    D = C // G
+    y_ref, mu_ref, rsig_ref = R.op_group_norm(dtype, x, g, b, 1, G, 1e-5)
+    mu, rsig = empty((N * G,), an), empty((N * G,), an)
+    ybuf, y = shifted()
+    K.group_norm_forward(N, G, D, S, "NCHW", 1e-5, xd, gd, bd, mu, rsig, y)
+    assert U.normwise(U.to_host(mu), mu_ref) <= 1e-5
+    assert U.normwise(U.widen(U.to_host(y.contiguous()), dtype).reshape(shape),
+                      U.widen(y_ref, dtype).reshape(shape)) <= U.TIGHT[dtype]
+    assert untouched(ybuf)
+    dx_ref, dg_ref, db_ref, _, _ = R.group_norm_grad(od, N, G, D, S, "NCHW", xo, mu_ref, rsig_ref, g, dyo)
+    dxbuf, dx = shifted()
+    pr = empty((2 * N * G,), an)
+    K.group_norm_grad(N, G, D, S, "NCHW", xd, U.to_device(mu_ref, an), U.to_device(rsig_ref, an), gd,
+                      dyd, pr, pr, dg, db, dx)
+    assert U.normwise(U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape),
+                      np.asarray(dx_ref).reshape(shape)) <= U.TIGHT[dtype]
+    assert U.normwise(U.to_host(dg), dg_ref) <= 2e-5 and U.normwise(U.to_host(db), db_ref) <= 2e-5
+    assert untouched(dxbuf)
