@@ -21,6 +21,7 @@
 // (loss 0, mask 0, zero gradient); the reference would read out of bounds.
 #include <cfloat>
 
+#include "loss_math.h"
 #include "row_tile.h"
 #include "short_rows.h"
 
@@ -30,12 +31,6 @@ namespace {
 constexpr int kLossThreads = 256;
 constexpr int kLossWaves = kLossThreads / kWaveSize;
 constexpr int kMaxPartials = 1024;  // stage-one workgroups of a loss reduction
-
-template <typename A>
-__device__ __forceinline__ A neg_log_clamped(A p) {
-  const A lo = static_cast<A>(FLT_MIN);
-  return -acc_log(p > lo ? p : lo);
-}
 
 // ------------------------------------------------------------------ CrossEntropy
 
@@ -47,12 +42,6 @@ __global__ __launch_bounds__(kLossThreads) void cross_entropy_dense(
        i += static_cast<int64_t>(gridDim.x) * kLossThreads) {
     loss[i] = target[i] * neg_log_clamped(input[i]);
   }
-}
-
-template <typename TargetT>
-__device__ __forceinline__ bool target_valid(TargetT tgt, int64_t ignore_index, int64_t C) {
-  const int64_t t = static_cast<int64_t>(tgt);
-  return t != ignore_index && t >= 0 && t < C;
 }
 
 template <typename T, typename TargetT>
@@ -687,6 +676,11 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
     }
+  } else if (S > 1 && launch_softmax_cols_with_loss<T, TargetT>(N, S, C, ignore_index, xp, tp, pp,
+                                                                loss, mask, stream) ==
+                          DRAGON_HIP_OK) {
+    // class axis in the middle (segmentation logits): the column-tile softmax
+    // writes the per-position loss itself
   } else {
     // rows beyond the fused row tiles: Softmax (several workgroups per row where
     // that pays), then the per-position loss

@@ -22,6 +22,7 @@
 // axes assign one thread to each (n, s) column and walk it three times (max,
 // sum, write), the re-reads coming from L2.
 #include "col_tile.h"
+#include "loss_math.h"
 #include "row_loop.h"
 #include "row_tile.h"
 #include "short_rows.h"
@@ -427,9 +428,23 @@ __global__ __launch_bounds__(1024) void softmax_grad_wide_rows(const int64_t N, 
 // S > 1 with the whole reduced axis in one register tile (col_tile.h): every
 // tensor is read once. 16-bit types evaluate the exponential twice (statistics
 // and output) instead of keeping fp32 copies of the tile.
-template <typename T, int kKind, int kTW, int kR>
-__global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g, const T* x,
-                                                                 T* y) {
+// With a Gather, the thread that holds the class a position's target names
+// also writes that position's loss and mask (SparseCrossEntropy folded in).
+struct NoGather {
+  static constexpr bool kOn = false;
+};
+template <typename T, typename TargetT>
+struct LossGather {
+  static constexpr bool kOn = true;
+  int64_t ignore_index;
+  const TargetT* target;  // [N, S]
+  T* loss;                // [N, S]
+  T* mask;
+};
+
+template <typename T, int kKind, int kTW, int kR, typename Gather = NoGather>
+__global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g, const T* x, T* y,
+                                                                 const Gather gather = Gather()) {
   using Tile = ColTile<T, kTW, kR>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
@@ -442,6 +457,8 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
   // packets evaluate them again for the output.
   constexpr bool kKeepExp = kKind == kSoftmax && (kHold || sizeof(T) == sizeof(A));
   __shared__ A lds[Tile::kLdsWords];
+  __shared__ int wanted_lds[Gather::kOn ? kTW * kVec : 1];
+  __shared__ A picked_lds[Gather::kOn ? kTW * kVec : 1];
   const int nr = Tile::rows_used(g.C);  // uniform: later packets are padding
   for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
     const int64_t n = tile / g.strips;
@@ -451,6 +468,22 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
     const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
     Tile t;
     t.load(x + base, g.S, g.C, nvalid, acc_neg_inf<A>());
+    // Gather: the class whose probability is a column's loss (-1: none). The
+    // threads of the first row group read the targets and pass them to the
+    // others of their columns through LDS, so that a target is requested once.
+    int wanted[kVec];
+    if constexpr (Gather::kOn) {
+      if (Tile::tc() == 0) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          wanted[e] = -1;
+          if (e < nvalid) {
+            const auto tgt = gather.target[n * g.S + s0 + e];
+            if (target_valid(tgt, gather.ignore_index, g.C)) wanted[e] = static_cast<int>(tgt);
+          }
+        }
+      }
+    }
     A held[kHold ? kR : 1][kVec];
     if constexpr (kHold) {
 #pragma unroll
@@ -485,6 +518,14 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
       }
     }
     Tile::reduce_rows(m, MaxOp(), lds);
+    if constexpr (Gather::kOn) {
+      // after that reduction's barriers (every thread is done with the previous
+      // tile's values), read after the next reduction's
+      if (Tile::tc() == 0) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) wanted_lds[Tile::tw() * kVec + e] = wanted[e];
+      }
+    }
     if (!kHold) t.refresh();
 #pragma unroll
     for (int r = 0; r < kR; ++r) {
@@ -504,6 +545,13 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
     A inv[kVec], l[kVec];
 #pragma unroll
     for (int e = 0; e < kVec; ++e) inv[e] = A(1) / sum[e], l[e] = acc_log(sum[e]);
+    A picked[kVec];      // Gather: the target class's probability where this thread holds it
+    unsigned found = 0;  // one bit per column
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      picked[e] = A(0);
+      if constexpr (Gather::kOn) wanted[e] = wanted_lds[Tile::tw() * kVec + e];
+    }
 #pragma unroll
     for (int r = 0; r < kR; ++r) {
       if (r < nr) {
@@ -521,6 +569,46 @@ __global__ __launch_bounds__(kColThreads) void softmax_col_tiles(const ColGrid g
           }
         }
         Tile::store(y + base, g.S, g.C, nvalid, r, v);
+        if constexpr (Gather::kOn) {
+          // kept in registers until the tile is done: a store per row and column
+          // would be a vector-memory instruction with a lane or two active
+          const int c = r * Tile::kTC + Tile::tc();
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (c == wanted[e]) picked[e] = v[e], found |= 1u << e;  // wanted < C: never padding
+          }
+        }
+      }
+    }
+    if constexpr (Gather::kOn) {
+      // The probabilities go back to the first row group, which writes loss and
+      // mask as whole packets (a store from wherever the class was held would
+      // touch every cache line of the two arrays four times, a few bytes each).
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (found & (1u << e)) picked_lds[Tile::tw() * kVec + e] = picked[e];
+      }
+      __syncthreads();
+      if (Tile::tc() == 0 && nvalid > 0) {
+        A lv[kVec], mv[kVec];
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const bool on = wanted[e] >= 0;
+          lv[e] = on ? neg_log_clamped(picked_lds[Tile::tw() * kVec + e]) : A(0);
+          mv[e] = on ? A(1) : A(0);
+        }
+        T* lp = gather.loss + n * g.S + s0;
+        T* mp = gather.mask + n * g.S + s0;
+        const bool whole = ((reinterpret_cast<uintptr_t>(lp) | reinterpret_cast<uintptr_t>(mp)) & 15u) == 0;
+        if (nvalid == kVec && whole) {
+          store_packet(lp, IO<T>::pack(lv));
+          store_packet(mp, IO<T>::pack(mv));
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (e < nvalid) lp[e] = lv[e], mp[e] = mv[e];
+          }
+        }
       }
     }
   }
@@ -1159,6 +1247,44 @@ inline int check_softmax_args(int64_t N, int64_t S, int64_t C, const void* a, co
 }
 
 } // namespace
+
+template <typename T, typename TargetT>
+int launch_softmax_cols_with_loss(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
+                                  const T* x, const TargetT* target, T* prob, T* loss, T* mask,
+                                  hipStream_t stream) {
+  constexpr int kVec = IO<T>::kVec;
+  const int tw = pick_col_tw(C, S, kVec, 16);
+  if (tw == 0) return 1;
+  const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
+  const LossGather<T, TargetT> gather{ignore_index, target, loss, mask};
+#define LAUNCH(TW)                                                                              \
+  {                                                                                             \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                        \
+    const dim3 grid(col_launch_grid(g.tiles)), block(kColThreads);                              \
+    if (small) {                                                                                \
+      hipLaunchKernelGGL((softmax_col_tiles<T, kSoftmax, TW, 8, LossGather<T, TargetT>>), grid, \
+                         block, 0, stream, g, x, prob, gather);                                 \
+    } else {                                                                                    \
+      hipLaunchKernelGGL((softmax_col_tiles<T, kSoftmax, TW, 16, LossGather<T, TargetT>>), grid, \
+                         block, 0, stream, g, x, prob, gather);                                 \
+    }                                                                                           \
+  }
+  if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
+  return status_of_launch();
+}
+template int launch_softmax_cols_with_loss<float, int32_t>(int64_t, int64_t, int64_t, int64_t,
+                                                           const float*, const int32_t*, float*,
+                                                           float*, float*, hipStream_t);
+template int launch_softmax_cols_with_loss<float, int64_t>(int64_t, int64_t, int64_t, int64_t,
+                                                           const float*, const int64_t*, float*,
+                                                           float*, float*, hipStream_t);
+template int launch_softmax_cols_with_loss<double, int32_t>(int64_t, int64_t, int64_t, int64_t,
+                                                            const double*, const int32_t*, double*,
+                                                            double*, double*, hipStream_t);
+template int launch_softmax_cols_with_loss<double, int64_t>(int64_t, int64_t, int64_t, int64_t,
+                                                            const double*, const int64_t*, double*,
+                                                            double*, double*, hipStream_t);
 } // namespace dragon_hip
 
 extern "C" {
