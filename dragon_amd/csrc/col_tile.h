@@ -131,7 +131,14 @@ inline ColGrid make_col_grid(int64_t N, int64_t S, int64_t C, int cols_per_tile)
 // Threads along the columns for a strided reduction over C rows of S columns
 // with at most `max_r` packets per thread: the widest tile that still holds C
 // rows, not wider than the columns there are. 0 when no tile can hold C rows.
-inline int pick_col_tw(int64_t C, int64_t S, int vec, int max_r) {
+inline int pick_col_tw(int64_t N, int64_t C, int64_t S, int vec, int max_r) {
+  // A tile never spans two n: where one n holds a few hundred elements at most
+  // (a handful of classes over a handful of positions), a workgroup per n is
+  // mostly idle and a thread per column does better. The same where S is less
+  // than a packet (most of a tile's lanes along S have no column) and there are
+  // enough columns in all to fill the device with a thread each.
+  if (C * S <= 512) return 0;
+  if (S < vec && C <= 256 && N * S >= 16384) return 0;
   const int64_t packets = ceil_div(S, vec);
   const int tw_cap = packets > 16 ? 64 : (packets > 4 ? 16 : 4);
   for (int tw : {64, 16, 4}) {

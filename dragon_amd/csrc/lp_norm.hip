@@ -463,7 +463,7 @@ int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsi
   } else if (S == 1) {
     hipLaunchKernelGGL((lp_norm_rows_looped<T, kP, kGrad>), dim3(loop_grid(N)), dim3(kLoopThreads),
                        0, stream, N, C, nrm, eps, gp, xp, op);
-  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+  } else if (const int tw = pick_col_tw(N, C, S, kVec, 16)) {
     // the gradient holds two tiles: 8 packets per thread each where that holds C rows
     const bool small = kGrad && C <= static_cast<int64_t>(kColThreads / tw) * 8;
 #define LAUNCH(TW)                                                                            \

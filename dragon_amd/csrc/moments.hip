@@ -19,10 +19,12 @@
 // which equals the reference's E[x^2]-E[x]^2 in exact arithmetic and keeps
 // Welford-class accuracy in fp32 when |mean| >> stddev, while partial sums
 // still combine by plain addition.
+#include <algorithm>
 #include <string>
 #include <vector>
 
 #include "reduce.h"
+#include "short_rows.h"
 
 namespace dragon_hip {
 namespace {
@@ -156,7 +158,68 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_gather(
   }
 }
 
-enum PlanKind { kPlanSegments, kPlanColumns, kPlanGather };
+// Rows of up to 1024 contiguous elements (a trailing axis of a few or a few
+// hundred elements, millions of outputs): a policy of the LDS-staged short-row
+// kernel (short_rows.h), several rows per wavefront, the epilogue applied by
+// the row's first lane. A workgroup per output would need more workgroups
+// than a launch can hold.
+template <typename T, int kE, typename P>
+struct ReduceRowOp {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  static constexpr bool kReadOnly = true;
+  typename P::Out out;
+  A inv_n;
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int, int) {}
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A*, int l, int width, A (&v)[kE],
+                                      const A (&)[kE]) const {
+    // the row's first element, which lane 0 holds as v[0]
+    const A shift = P::kShift ? __shfl(v[0], (threadIdx.x & (kWaveSize - 1)) / kL * kL, kWaveSize) : A(0);
+    A a = A(0), b = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      if (l + j * kL < width) P::term(v[j] - shift, a, b);
+    }
+    a = group_allreduce<kL>(a, SumOp());
+    b = group_allreduce<kL>(b, SumOp());
+    if (l == 0) P::finish(out, static_cast<uint32_t>(r), shift, a, b, inv_n);
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+template <typename P>
+struct ReduceRowsOf {
+  template <typename T, int kE>
+  using Op = ReduceRowOp<T, kE, P>;
+};
+
+// One reduced axis between kept ones ([N, C, S] over C): a thread per output
+// walks its C elements S apart; adjacent threads read adjacent addresses.
+template <typename T, typename P>
+__global__ __launch_bounds__(kReduceThreads) void reduce_strided_columns(
+    const uint32_t N, const uint32_t C, const uint32_t S, const T* __restrict__ x,
+    const typename P::Out out) {
+  using A = typename IO<T>::Acc;
+  const uint32_t total = N * S;
+  for (uint32_t o = blockIdx.x * kReduceThreads + threadIdx.x; o < total;
+       o += gridDim.x * kReduceThreads) {
+    const uint32_t n = o / S;
+    const T* col = x + static_cast<size_t>(n) * C * S + (o - n * S);
+    const A shift = P::kShift ? IO<T>::load1(col) : A(0);
+    A a = A(0), b = A(0);
+#pragma unroll 8
+    for (uint32_t k = 0; k < C; ++k) P::term(IO<T>::load1(col + static_cast<size_t>(k) * S) - shift, a, b);
+    P::finish(out, o, shift, a, b, A(1) / A(C));
+  }
+}
+
+enum PlanKind { kPlanSegments, kPlanColumns, kPlanGather, kPlanShortRows, kPlanStrided };
 struct MomentsPlan {
   PlanKind kind;
   SegmentedReduce seg;
@@ -204,7 +267,13 @@ int make_plan(int dtype, int num_dims, const int64_t* dims, int num_axes, const 
   SegmentedReduce& s = plan->seg;
   s = SegmentedReduce{static_cast<uint32_t>(plan->n_out), 1, 0, 0, 1, 0, 0, 1};
   auto u32 = [](int64_t v) { return static_cast<uint32_t>(v); };
-  if (pat == "R" || pat == "KR") {
+  if (pat == "KR" && plan->n_red <= 1024 && plan->n_out >= 4096) {
+    plan->kind = kPlanShortRows;
+  } else if (pat == "KRK" && plan->n_out >= 16384) {
+    // enough outputs to fill the device with a thread each
+    plan->kind = kPlanStrided;
+    s.nseg = u32(ext[0]), s.seglen = u32(ext[1]), s.seg_stride = u32(ext[2]);  // N, C, S
+  } else if (pat == "R" || pat == "KR") {
     plan->kind = kPlanSegments;
     s.stride1 = u32(plan->n_red), s.seglen = u32(plan->n_red);
   } else if (pat == "RKR") {
@@ -251,7 +320,22 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
   const A inv_n = A(1) / A(plan.n_red);
   const unsigned fin_grid = static_cast<unsigned>(ceil_div(plan.n_out, kReduceThreads));
   using Accum = ReduceAccum<T, P>;
-  if (plan.kind == kPlanSegments) {
+  if (plan.kind == kPlanShortRows) {
+    ShortPlan sp;
+    if (!plan_short_rows(plan.n_red, sizeof(T), 4, aligned16(x), &sp)) return DRAGON_HIP_EINVAL;
+    using Holder = ReduceRowsOf<P>;
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16;
+    T* none = nullptr;
+    DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
+                            short_grid(plan.n_out, sp.rows_per_chunk), stream, plan.n_out,
+                            static_cast<int>(plan.n_red), xp, xp, none, out, inv_n);
+  } else if (plan.kind == kPlanStrided) {
+    const SegmentedReduce& s = plan.seg;
+    const unsigned grid = static_cast<unsigned>(
+        std::min<int64_t>(ceil_div(plan.n_out, kReduceThreads), static_cast<int64_t>(kNumCUs) * 32));
+    hipLaunchKernelGGL((reduce_strided_columns<T, P>), dim3(grid), dim3(kReduceThreads), 0, stream,
+                       s.nseg, s.seglen, s.seg_stride, xp, out);
+  } else if (plan.kind == kPlanSegments) {
     const SegmentedReduce& s = plan.seg;
     const bool vec_ok = aligned16(x) && s.seglen % kVec == 0 && s.stride1 % kVec == 0 &&
         s.stride2 % kVec == 0 && s.seg_stride % kVec == 0;

@@ -125,31 +125,40 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_segments(
 // partial[(k * cols + c) * 2 + {0,1}].
 template <typename T, int kIn, typename F>
 __global__ __launch_bounds__(kReduceThreads) void reduce2_columns(
-    const ColumnReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
-    typename IO<T>::Acc* __restrict__ partial) {
+    const ColumnReduce d, const uint32_t lanes_per_row, const T* __restrict__ in0,
+    const T* __restrict__ in1, F f, typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   __shared__ A lds[kReduceWaves][kWaveSize][2];
-  const uint32_t tiles = (d.cols + kWaveSize - 1) / kWaveSize;
+  // fewer than 64 columns: the lanes a row does not need take adjacent rows
+  // (as reduce2_columns_packets below)
+  const uint32_t rows_per_wave = kWaveSize / lanes_per_row;
+  const uint32_t tiles = (d.cols + lanes_per_row - 1) / lanes_per_row;
   const uint32_t tile = blockIdx.x % tiles;
   const uint32_t k = blockIdx.x / tiles;
   const uint32_t lane = threadIdx.x & (kWaveSize - 1);
   const uint32_t wave = threadIdx.x / kWaveSize;
-  const uint32_t c = tile * kWaveSize + lane;
+  const uint32_t across = lane / lanes_per_row;
+  const uint32_t c = tile * lanes_per_row + lane % lanes_per_row;
   A a = A(0), b = A(0);
   if (c < d.cols) {
     f.begin(c, c);
 #pragma unroll 4
-    for (uint32_t r = k * kReduceWaves + wave; r < d.rows; r += d.split * kReduceWaves) {
+    for (uint32_t r = (k * kReduceWaves + wave) * rows_per_wave + across; r < d.rows;
+         r += d.split * kReduceWaves * rows_per_wave) {
       const uint32_t off = r * d.cols + c;
       const A x0 = IO<T>::load1(in0 + off);
       const A x1 = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
       f.add(r, c, off, x0, x1, a, b);
     }
   }
+  for (uint32_t o = lanes_per_row; o < kWaveSize; o <<= 1) {
+    a += __shfl_xor(a, static_cast<int>(o), kWaveSize);
+    b += __shfl_xor(b, static_cast<int>(o), kWaveSize);
+  }
   lds[wave][lane][0] = a;
   lds[wave][lane][1] = b;
   __syncthreads();
-  if (wave == 0 && c < d.cols) {
+  if (wave == 0 && across == 0 && c < d.cols) {
 #pragma unroll
     for (int w = 1; w < kReduceWaves; ++w) {
       a += lds[w][lane][0];
@@ -255,10 +264,12 @@ inline uint32_t launch_reduce2_columns(uint32_t rows, uint32_t cols, const T* in
     hipLaunchKernelGGL((reduce2_columns_packets<T, kIn, F>), dim3(tiles * d.split),
                        dim3(kReduceThreads), 0, stream, d, lanes_per_row, in0, in1, f, partial);
   } else {
-    d.split = pick_split(ceil_div(cols, kWaveSize), static_cast<int64_t>(rows) * kWaveSize);
-    hipLaunchKernelGGL((reduce2_columns<T, kIn, F>),
-                       dim3(static_cast<unsigned>(ceil_div(cols, kWaveSize)) * d.split),
-                       dim3(kReduceThreads), 0, stream, d, in0, in1, f, partial);
+    uint32_t lanes_per_row = 1;
+    while (lanes_per_row < kWaveSize && lanes_per_row < cols) lanes_per_row <<= 1;
+    const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, lanes_per_row));
+    d.split = pick_split(tiles, static_cast<int64_t>(rows) * kWaveSize);
+    hipLaunchKernelGGL((reduce2_columns<T, kIn, F>), dim3(tiles * d.split), dim3(kReduceThreads), 0,
+                       stream, d, lanes_per_row, in0, in1, f, partial);
   }
   return d.split;
 }

@@ -1095,7 +1095,7 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
   } else if (S == 1) {
     hipLaunchKernelGGL((softmax_rows_looped<T, kKind>), dim3(loop_grid(N)), dim3(kLoopThreads), 0,
                        stream, N, C, xp, yp);
-  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+  } else if (const int tw = pick_col_tw(N, C, S, kVec, 16)) {
     // the widest tile wins (narrow row segments cost more than a second
     // exponential); within it, up to 8 packets per thread are held converted
     const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
@@ -1189,7 +1189,7 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   } else if (S == 1) {
     hipLaunchKernelGGL((softmax_grad_rows_looped<T, kKind>), dim3(loop_grid(N)),
                        dim3(kLoopThreads), 0, stream, N, C, gp, yp, dp);
-  } else if (const int tw = pick_col_tw(C, S, kVec, 16)) {
+  } else if (const int tw = pick_col_tw(N, C, S, kVec, 16)) {
     // two tiles live at once: 8 packets per thread each where that holds C rows
     const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
 #define LAUNCH(TW)                                                                        \
@@ -1253,7 +1253,7 @@ int launch_softmax_cols_with_loss(int64_t N, int64_t S, int64_t C, int64_t ignor
                                   const T* x, const TargetT* target, T* prob, T* loss, T* mask,
                                   hipStream_t stream) {
   constexpr int kVec = IO<T>::kVec;
-  const int tw = pick_col_tw(C, S, kVec, 16);
+  const int tw = pick_col_tw(N, C, S, kVec, 16);
   if (tw == 0) return 1;
   const bool small = C <= static_cast<int64_t>(kColThreads / tw) * 8;
   const LossGather<T, TargetT> gather{ignore_index, target, loss, mask};
