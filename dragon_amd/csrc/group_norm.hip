@@ -927,7 +927,10 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
 // a channel is a group of adjacent lanes of one (slot, wavefront) pair, reduced
 // with shuffles and written by its first lane; gamma is read per lane.
 // partial[(n*C + c)*2 + {0,1}] receives this group's share of dgamma / dbeta.
-enum ChannelMode { kChannelWaves = 0, kChannelStraddles = 1, kChannelLanes = 2 };
+enum ChannelMode { kChannelWaves = 0, kChannelStraddles = 1, kChannelLanes = 2, kChannelPackets = 3 };
+// kChannelPackets (group_norm_grad_rows_any): at most this many packets per
+// group, 4 accumulator words of LDS each.
+constexpr int kMaxEntryPackets = 4096;
 
 template <typename T, int kTPR, int kVPT, int kMode>
 __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
@@ -1111,6 +1114,129 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
       o[1] = b;
     }
     __syncthreads();  // chan_part and slots are reused by the next group
+  }
+}
+
+// The same for groups of whole aligned packets whose channels are not (S is
+// not a multiple of a packet but at least one: 14x14 and 7x7 maps): a packet
+// holds elements of at most two channels. gamma is one of two values per
+// packet, picked per element; a thread leaves the (dgamma, dbeta) shares of
+// its packet's first and second channel in LDS, one entry per packet, and the
+// thread that owns a channel adds the entries of that channel's packets in
+// order. Dynamic LDS: 4 accumulator words per packet of the group.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const T* __restrict__ x, const T* __restrict__ dy,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
+    const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
+    typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2 * Tile::kSlots];
+  extern __shared__ u32x4 dynamic_lds[];
+  A* entries = reinterpret_cast<A*>(dynamic_lds);  // [npackets][4]
+  const int npackets = L / kVec;
+  const A denom = A(1) / A(L);
+  const int lane = threadIdx.x;
+
+  Raw tx, tdy;
+  if (blockIdx.x < rows) {
+    tx.load_unmasked(x + static_cast<int64_t>(blockIdx.x) * L, npackets);
+    tdy.load_unmasked(dy + static_cast<int64_t>(blockIdx.x) * L, npackets);
+  }
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int64_t next = row + gridDim.x;
+    const bool next_valid = next < rows;
+    const T* nx = x + (next_valid ? next : row) * L;
+    const T* ndy = dy + (next_valid ? next : row) * L;
+    const A m = mu[row], r = rsig[row];
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+
+    // per slot: the channel of the packet's first element, that element's
+    // position in the channel, and gamma of that channel and of the next
+    uint32_t first[kVPT], rem[kVPT];
+    A g0[kVPT], g1[kVPT];
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const bool on = Tile::active(i, npackets);
+      const uint32_t col = on ? static_cast<uint32_t>(i * kTPR + lane) * kVec : 0u;
+      first[i] = col / S;
+      rem[i] = col - first[i] * S;
+      g0[i] = gamma[c0 + first[i]];
+      g1[i] = gamma[c0 + (first[i] + 1 < D ? first[i] + 1 : first[i])];
+      if (on) {
+        A xv[kVec], dv[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A t = (rem[i] + e >= S ? g1[i] : g0[i]) * dv[e];
+          s1 += t * xv[e];
+          s2 += t;
+        }
+      }
+    }
+    Tile::reduce_sum_pair(s1, s2, slots);
+    if (lane == 0) {
+      ds[row] = s1;
+      db[row] = s2;
+    }
+    const A u0 = (s2 * m - s1) * (r * r * r);
+    const A v0 = s2 * r;
+    tx.refresh();
+    tdy.refresh();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        A xv[kVec], dv[kVec];
+        tx.unpack(i, xv);
+        tdy.unpack(i, dv);
+        A h1 = A(0), h2 = A(0), t1 = A(0), t2 = A(0);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const bool second = rem[i] + e >= S;
+          const A xc = xv[e] - m;
+          const A w = dv[e] * xc * r;
+          h1 += second ? A(0) : w;
+          h2 += second ? A(0) : dv[e];
+          t1 += second ? w : A(0);
+          t2 += second ? dv[e] : A(0);
+          xv[e] = (second ? g1[i] : g0[i]) * dv[e] * r + (u0 * xc - v0) * denom;
+        }
+        tx.store_slot(dx + row * L, i, xv);
+        A* entry = entries + static_cast<size_t>(i * kTPR + lane) * 4;
+        entry[0] = h1, entry[1] = h2, entry[2] = t1, entry[3] = t2;
+      }
+      if (next_valid) {
+        tx.load_slot_unmasked(nx, i, npackets);
+        tdy.load_slot_unmasked(ndy, i, npackets);
+      }
+    }
+    __syncthreads();
+    for (uint32_t c = lane; c < D; c += kTPR) {
+      // channel c owns elements [c S, (c + 1) S): the first-channel share of the
+      // packets that start in it, the second-channel share of the one that
+      // starts before it and reaches in
+      const uint32_t lo = c * S;
+      const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+      A a = A(0), b = A(0);
+#pragma nounroll
+      for (uint32_t p = p0; p <= p1; ++p) {
+        const uint32_t part = p * kVec >= lo ? 0u : 2u;
+        a += entries[4 * p + part];
+        b += entries[4 * p + part + 1];
+      }
+      const size_t n = static_cast<size_t>(row / G);
+      A* o = partial + (n * G * D + c0 + c) * 2;
+      o[0] = a;
+      o[1] = b;
+    }
+    __syncthreads();  // entries and slots are reused by the next group
   }
 }
 
@@ -1729,17 +1855,20 @@ template <typename T>
 bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig* cfg, int* mode) {
   constexpr int kVec = IO<T>::kVec;
   if (layout != DRAGON_HIP_NCHW || G * D == 1) return false;
-  if (S % kVec != 0) return false;
+  static const RowConfig table[] = {{256, 2}, {256, 4}, {256, 8}, {1024, 4}, {1024, 8}};
   const int64_t per_chan = S / kVec;
-  if (per_chan >= kWaveSize) {
+  if (S % kVec == 0 && per_chan >= kWaveSize) {
     *mode = per_chan % kWaveSize == 0 ? kChannelWaves : kChannelStraddles;
-  } else if ((per_chan & (per_chan - 1)) == 0) {
+  } else if (S % kVec == 0 && (per_chan & (per_chan - 1)) == 0) {
     *mode = kChannelLanes;
+  } else if (S >= kVec && (D * S) % kVec == 0 && D * S / kVec <= kMaxEntryPackets) {
+    // channels that are not whole packets (or a number of packets the lane
+    // flavour does not take): one LDS entry per packet
+    *mode = kChannelPackets;
   } else {
     return false;
   }
-  static const RowConfig table[] = {{256, 2}, {256, 4}, {256, 8}, {1024, 4}, {1024, 8}};
-  const int64_t npackets = D * per_chan;
+  const int64_t npackets = D * S / kVec;
   if (npackets <= kWaveSize * 2) return false;  // a wavefront or two: the general path
   for (const RowConfig& c : table) {
     if (npackets <= static_cast<int64_t>(c.tpr) * c.vpt) {
@@ -2199,11 +2328,21 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     const unsigned grid = static_cast<unsigned>(rows < (1 << 20) ? rows : (1 << 20));
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
+  if (mode == kChannelPackets) {                                                                \
+    if constexpr (TPR * VPT <= kMaxEntryPackets) {                                              \
+      auto kernel = group_norm_grad_rows_any<T, TPR, VPT>;                                      \
+      const size_t lds = static_cast<size_t>(L / kVec) * 4 * sizeof(A);                         \
+      if (lds > 32 * 1024) (void)resident_grid(kernel, TPR, lds);                               \
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), lds, stream, rows, L, sh.G, sh.D, sh.S, \
+                         xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                           \
+    }                                                                                           \
+  } else {                                                                                      \
     auto kernel = mode == kChannelStraddles ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddles> \
         : mode == kChannelLanes             ? group_norm_grad_rows<T, TPR, VPT, kChannelLanes>     \
                                             : group_norm_grad_rows<T, TPR, VPT, kChannelWaves>;    \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), 0, stream, rows, L, sh.G, sh.D, sh.S, xp, \
                        dyp, gp, mup, rsp, dsp, dbp, dxp, part);                                 \
+  }                                                                                             \
   }
     if (gcfg.tpr == 256 && gcfg.vpt == 2) LAUNCH(256, 2)
     else if (gcfg.tpr == 256 && gcfg.vpt == 4) LAUNCH(256, 4)

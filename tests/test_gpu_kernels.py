@@ -354,7 +354,10 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # odd feature maps of more than 1024 elements in every dtype: one wavefront per
             # (n, c) row in the backward and the map; per group row in the forward statistics
             # of groups beyond the register tiles
-            ((2, 6, 33, 35), 1, 2), ((1, 2, 301, 303), 1, 2)]
+            ((2, 6, 33, 35), 1, 2), ((1, 2, 301, 303), 1, 2),
+            # 14x14 and 7x7 maps in groups of whole packets: the fused backward with one LDS
+            # entry per packet (up to 100 KB of dynamic LDS in fp64)
+            ((2, 64, 14, 14), 1, 2), ((3, 128, 7, 7), 1, 4)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
