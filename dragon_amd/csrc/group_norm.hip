@@ -822,12 +822,23 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
       t.unpack(i, v);
       if constexpr (kAnyS) {
         const uint32_t rem = Tile::active(i, npackets) ? col - first * S : 0u;
+        if (S >= static_cast<uint32_t>(kVec)) {
+          // at most two channels per packet: their parameters once, picked per element
+          const uint32_t ca = c0 + first, cb = c0 + (first + 1 < D ? first + 1 : first);
+          const A ga = gamma[ca] * rs, gb = gamma[cb] * rs, ba = beta[ca], bb = beta[cb];
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) {
-          uint32_t k = rem + e, c = first;
-          while (k >= S) k -= S, ++c;
-          c = c0 + (c < D ? c : D - 1);
-          v[e] = (v[e] - mean) * (gamma[c] * rs) + beta[c];
+          for (int e = 0; e < kVec; ++e) {
+            const bool second = rem + e >= S;
+            v[e] = (v[e] - mean) * (second ? gb : ga) + (second ? bb : ba);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            uint32_t k = rem + e, c = first;
+            while (k >= S) k -= S, ++c;
+            c = c0 + (c < D ? c : D - 1);
+            v[e] = (v[e] - mean) * (gamma[c] * rs) + beta[c];
+          }
         }
       } else {
         const uint32_t c = c0 + first;  // kVec divides S
@@ -1156,26 +1167,30 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
     const A m = mu[row], r = rsig[row];
     const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
 
-    // per slot: the channel of the packet's first element, that element's
-    // position in the channel, and gamma of that channel and of the next
-    uint32_t first[kVPT], rem[kVPT];
-    A g0[kVPT], g1[kVPT];
+    // Of slot i's packet: the position of its first element in that element's
+    // channel, and gamma of that channel and of the next. Found again in the
+    // second pass rather than kept: four more registers per slot cost occupancy.
+    auto channels_of = [&](int i, uint32_t& rem, A& g0, A& g1) {
+      const uint32_t col =
+          Tile::active(i, npackets) ? static_cast<uint32_t>(i * kTPR + lane) * kVec : 0u;
+      const uint32_t first = col / S;
+      rem = col - first * S;
+      g0 = gamma[c0 + first];
+      g1 = gamma[c0 + (first + 1 < D ? first + 1 : first)];
+    };
     A s1 = A(0), s2 = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      const bool on = Tile::active(i, npackets);
-      const uint32_t col = on ? static_cast<uint32_t>(i * kTPR + lane) * kVec : 0u;
-      first[i] = col / S;
-      rem[i] = col - first[i] * S;
-      g0[i] = gamma[c0 + first[i]];
-      g1[i] = gamma[c0 + (first[i] + 1 < D ? first[i] + 1 : first[i])];
-      if (on) {
+      if (Tile::active(i, npackets)) {
+        uint32_t rem;
+        A g0, g1;
+        channels_of(i, rem, g0, g1);
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const A t = (rem[i] + e >= S ? g1[i] : g0[i]) * dv[e];
+          const A t = (rem + e >= S ? g1 : g0) * dv[e];
           s1 += t * xv[e];
           s2 += t;
         }
@@ -1193,20 +1208,23 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (Tile::active(i, npackets)) {
+        uint32_t rem;
+        A g0, g1;
+        channels_of(i, rem, g0, g1);
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
         A h1 = A(0), h2 = A(0), t1 = A(0), t2 = A(0);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const bool second = rem[i] + e >= S;
+          const bool second = rem + e >= S;
           const A xc = xv[e] - m;
           const A w = dv[e] * xc * r;
           h1 += second ? A(0) : w;
           h2 += second ? A(0) : dv[e];
           t1 += second ? w : A(0);
           t2 += second ? dv[e] : A(0);
-          xv[e] = (second ? g1[i] : g0[i]) * dv[e] * r + (u0 * xc - v0) * denom;
+          xv[e] = (second ? g1 : g0) * dv[e] * r + (u0 * xc - v0) * denom;
         }
         tx.store_slot(dx + row * L, i, xv);
         A* entry = entries + static_cast<size_t>(i * kTPR + lane) * 4;
@@ -1218,23 +1236,47 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
       }
     }
     __syncthreads();
-    for (uint32_t c = lane; c < D; c += kTPR) {
-      // channel c owns elements [c S, (c + 1) S): the first-channel share of the
-      // packets that start in it, the second-channel share of the one that
-      // starts before it and reaches in
-      const uint32_t lo = c * S;
-      const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
-      A a = A(0), b = A(0);
+    // Channel c owns elements [c S, (c + 1) S), that is the first-channel share
+    // of the packets that start in it and the second-channel share of the one
+    // that starts before it and reaches in: a thread per channel where a channel
+    // is a few dozen packets, a wavefront per channel where it is more.
+    const size_t n = static_cast<size_t>(row / G);
+    if (S / kVec <= 32) {
+      for (uint32_t c = lane; c < D; c += kTPR) {
+        const uint32_t lo = c * S;
+        const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+        A a = A(0), b = A(0);
 #pragma nounroll
-      for (uint32_t p = p0; p <= p1; ++p) {
-        const uint32_t part = p * kVec >= lo ? 0u : 2u;
-        a += entries[4 * p + part];
-        b += entries[4 * p + part + 1];
+        for (uint32_t p = p0; p <= p1; ++p) {
+          const uint32_t part = p * kVec >= lo ? 0u : 2u;
+          a += entries[4 * p + part];
+          b += entries[4 * p + part + 1];
+        }
+        A* o = partial + (n * G * D + c0 + c) * 2;
+        o[0] = a;
+        o[1] = b;
       }
-      const size_t n = static_cast<size_t>(row / G);
-      A* o = partial + (n * G * D + c0 + c) * 2;
-      o[0] = a;
-      o[1] = b;
+    } else {
+      constexpr int kWaves = kTPR / kWaveSize;
+      const uint32_t wave = static_cast<uint32_t>(lane) / kWaveSize;
+      const uint32_t wave_lane = static_cast<uint32_t>(lane) & (kWaveSize - 1);
+      for (uint32_t c = wave; c < D; c += kWaves) {
+        const uint32_t lo = c * S;
+        const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+        A a = A(0), b = A(0);
+        for (uint32_t p = p0 + wave_lane; p <= p1; p += kWaveSize) {
+          const uint32_t part = p * kVec >= lo ? 0u : 2u;
+          a += entries[4 * p + part];
+          b += entries[4 * p + part + 1];
+        }
+        a = wave_allreduce(a, SumOp());
+        b = wave_allreduce(b, SumOp());
+        if (wave_lane == 0) {
+          A* o = partial + (n * G * D + c0 + c) * 2;
+          o[0] = a;
+          o[1] = b;
+        }
+      }
     }
     __syncthreads();  // entries and slots are reused by the next group
   }
