@@ -245,7 +245,7 @@ struct ShiftedSumSqAccum {  // a = sum (x-s), b = sum (x-s)^2, s = first value o
   const T* x;
   A shift;
   __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
-    shift = IO<T>::load1(x + first_off);
+    shift = load_shift(x + first_off);
   }
   __device__ __forceinline__ A state() const { return shift; }
   __device__ __forceinline__ void set_state(A v) { shift = v; }
@@ -349,7 +349,7 @@ struct TrainingStatsEpilogue {
   A* scale;
   A* bias;
   __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
-    const A shift = IO<T>::load1(x + c * chan_stride);
+    const A shift = load_shift(x + c * chan_stride);
     const A d = a * inv_n;
     const A mean = shift + d;
     const A var = b * inv_n - d * d;
@@ -553,7 +553,7 @@ struct CoopForward {
   A* bias;
   A shift, sc, bi;
   __device__ __forceinline__ void begin(uint32_t, uint32_t base, const T* x) {
-    shift = IO<T>::load1(x + base);  // one sample of the channel
+    shift = load_shift(x + base);  // one sample of the channel
   }
   template <int V>
   __device__ __forceinline__ void accumulate(uint32_t, uint32_t, const A (&x)[V], const A (&)[V],

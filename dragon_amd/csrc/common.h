@@ -138,6 +138,19 @@ struct IO<bf16_t> {
   }
 };
 
+// The sample that shifted sums are taken relative to (sum(x - s), sum((x - s)^2):
+// no cancellation against a large mean). A sample that is not finite would turn
+// every difference into inf or nan, so zero takes its place: the plain sums then
+// carry inf and nan into the mean and the variance as the CPU kernels' sums do.
+template <typename A>
+__device__ __forceinline__ A finite_or_zero(const A v) {
+  return __builtin_isfinite(v) ? v : A(0);
+}
+template <typename T>
+__device__ __forceinline__ typename IO<T>::Acc load_shift(const T* p) {
+  return finite_or_zero(IO<T>::load1(p));
+}
+
 // One aligned 16-byte packet to and from HBM. Outputs are written once and not
 // read again by the same kernel, so stores carry the non-temporal hint. Loads
 // do not: measured on MI355X, non-temporal loads slow every forward kernel

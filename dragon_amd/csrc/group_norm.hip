@@ -1504,7 +1504,7 @@ struct GroupRowMoments {  // a = sum (x - first), b = sum (x - first)^2 over a g
   const T* x;
   int64_t L;
   __device__ __forceinline__ void row_params(int64_t row, A (&w)[1]) const {
-    w[0] = IO<T>::load1(x + row * L);
+    w[0] = load_shift(x + row * L);
   }
   __device__ __forceinline__ void add(const A* w, A v, A, A& a, A& b) const {
     const A d = v - w[0];
@@ -1522,7 +1522,7 @@ __global__ __launch_bounds__(256) void group_stats_from_row_sums(
   if (row >= rows) return;
   const A inv = A(1) / A(L);
   const A d = pairs[2 * row] * inv;
-  mu[row] = IO<T>::load1(x + row * L) + d;
+  mu[row] = load_shift(x + row * L) + d;
   rsig[row] = acc_rsqrt_exact((pairs[2 * row + 1] * inv - d * d) + eps);
 }
 
@@ -1725,7 +1725,7 @@ struct ColumnStatsAccum {  // sums shifted by the column's first element
   uint32_t S, C;
   A shift;
   __device__ __forceinline__ void begin(uint32_t n, uint32_t c) {
-    shift = IO<T>::load1(x + static_cast<size_t>(n) * S * C + c);
+    shift = load_shift(x + static_cast<size_t>(n) * S * C + c);
   }
   __device__ __forceinline__ void add(A x0, A, A& a, A& b) const {
     const A d = x0 - shift;
@@ -1980,7 +1980,7 @@ struct GroupSlicesForward {
   uint32_t G, D, packets_per_chan;
   A shift, mean, rs;
   __device__ __forceinline__ void begin(uint32_t, uint32_t base, const T* x) {
-    shift = IO<T>::load1(x + base);  // one sample of the group
+    shift = load_shift(x + base);  // one sample of the group
   }
   template <int V>
   __device__ __forceinline__ void accumulate(uint32_t, uint32_t, const A (&x)[V], const A (&)[V],

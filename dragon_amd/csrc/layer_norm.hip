@@ -194,7 +194,7 @@ __global__ __launch_bounds__(kLoopThreads) void layer_norm_rows_looped(
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const T* xr = x + row * C;
     T* yr = y + row * C;
-    const A shift = IO<T>::load1(xr);
+    const A shift = load_shift(xr);
     A s = A(0), q = A(0);
     Loop::visit(xr, C, shift, [&](int64_t, const A(&v)[kVec], int) {
 #pragma unroll

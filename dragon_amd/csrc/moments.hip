@@ -81,7 +81,7 @@ struct ReduceAccum {
   const T* x;
   A shift;
   __device__ __forceinline__ void begin(uint32_t, uint32_t first_off) {
-    shift = P::kShift ? IO<T>::load1(x + first_off) : A(0);
+    shift = P::kShift ? load_shift(x + first_off) : A(0);
   }
   template <int V>
   __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x0)[V],
@@ -104,7 +104,7 @@ struct ReduceSegEpilogue {
   __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
     const uint32_t o1 = o / d.outer2;
     const uint32_t o2 = o - o1 * d.outer2;
-    const A shift = P::kShift ? IO<T>::load1(x + o1 * d.stride1 + o2 * d.stride2) : A(0);
+    const A shift = P::kShift ? load_shift(x + o1 * d.stride1 + o2 * d.stride2) : A(0);
     P::finish(out, o, shift, a, b, inv_n);
   }
 };
@@ -116,7 +116,7 @@ struct ReduceColEpilogue {
   A inv_n;
   typename P::Out out;
   __device__ __forceinline__ void operator()(uint32_t c, A a, A b) const {
-    const A shift = P::kShift ? IO<T>::load1(x + c) : A(0);
+    const A shift = P::kShift ? load_shift(x + c) : A(0);
     P::finish(out, c, shift, a, b, inv_n);
   }
 };
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_gather(
       base += (r % g.keep_dim[d]) * g.keep_stride[d];
       r /= g.keep_dim[d];
     }
-    const A shift = P::kShift ? IO<T>::load1(x + base) : A(0);
+    const A shift = P::kShift ? load_shift(x + base) : A(0);
     A a = A(0), b = A(0);
     for (uint32_t j = threadIdx.x; j < g.n_red_elems; j += kReduceThreads) {
       uint32_t off = base, q = j;
@@ -180,7 +180,7 @@ struct ReduceRowOp {
   __device__ __forceinline__ void row(int64_t r, const A*, int l, int width, A (&v)[kE],
                                       const A (&)[kE]) const {
     // the row's first element, which lane 0 holds as v[0]
-    const A shift = P::kShift ? __shfl(v[0], (threadIdx.x & (kWaveSize - 1)) / kL * kL, kWaveSize) : A(0);
+    const A shift = P::kShift ? finite_or_zero(__shfl(v[0], (threadIdx.x & (kWaveSize - 1)) / kL * kL, kWaveSize)) : A(0);
     A a = A(0), b = A(0);
 #pragma unroll
     for (int j = 0; j < kE; ++j) {
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_strided_columns(
        o += gridDim.x * kReduceThreads) {
     const uint32_t n = o / S;
     const T* col = x + static_cast<size_t>(n) * C * S + (o - n * S);
-    const A shift = P::kShift ? IO<T>::load1(col) : A(0);
+    const A shift = P::kShift ? load_shift(col) : A(0);
     A a = A(0), b = A(0);
 #pragma unroll 8
     for (uint32_t k = 0; k < C; ++k) P::term(IO<T>::load1(col + static_cast<size_t>(k) * S) - shift, a, b);

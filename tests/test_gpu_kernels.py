@@ -83,6 +83,32 @@ def test_layer_norm_empty_and_errors(K):
         K.layer_norm(1, 1, 1e-5, z.to(torch.int32), z, z, z, z, z)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
+@pytest.mark.parametrize("C", [37, 64, 1000, 4096, 12288, 40000, 70000])
+def test_layer_norm_special_values_follow_the_reference(K, C, dtype):
+    """A row holding one nan or one inf comes out all nan, statistics included, as the CPU
+    kernel's sums make it (layer_norm_kernel.cc:10-39); its neighbours are untouched."""
+    N = 6
+    rng = U.rng_for(C)
+    xf = rng.standard_normal((N, C)).astype(np.float32)
+    xf[1, C // 3] = np.nan
+    xf[3, C - 1] = np.inf
+    xf[4, 0] = -np.inf
+    x = R.to_bits(xf, dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    y_ref, mu_ref, rsig_ref = R.layer_norm(dtype, x, g, b, 1e-5)
+    y, mu, rsig = empty((N, C), dtype), empty((N,), "float32"), empty((N,), "float32")
+    K.layer_norm(N, C, 1e-5, U.to_device(x, dtype), U.to_device(g, "float32"),
+                 U.to_device(b, "float32"), mu, rsig, y)
+    yw, yr = U.widen(U.to_host(y), dtype), U.widen(y_ref, dtype)
+    assert np.array_equal(np.isnan(yw), np.isnan(yr))
+    assert np.array_equal(np.isnan(U.to_host(rsig)), np.isnan(rsig_ref))
+    assert np.array_equal(np.isnan(U.to_host(mu)), np.isnan(mu_ref))
+    assert np.array_equal(U.to_host(mu)[np.isinf(mu_ref)], mu_ref[np.isinf(mu_ref)])
+    clean = [0, 2, 5]
+    assert U.normwise(yw[clean], yr[clean]) <= U.TIGHT[dtype]
+
+
 def test_layer_norm_large_mean_stays_accurate(K):
     """|mean| >> stddev: the centred variance must not cancel (fp64 is the judge)."""
     rng = U.rng_for(7)
@@ -287,6 +313,76 @@ def test_softmax_masked_logits_are_exact_zero(K):
     yw = U.widen(U.to_host(y), "float16")
     assert np.all(yw[:, ::2] == 0)
     assert np.allclose(yw[:, 1::2], 1 / 256, rtol=1e-3)
+
+
+# one shape per kernel family: short rows in LDS, one wavefront, a workgroup, 1024-thread
+# rows, several workgroups per row, column tiles and long columns (S > 1)
+SPECIAL_SHAPES = [(8, 1, 37), (8, 1, 64), (8, 1, 512), (8, 1, 1000), (8, 1, 4096), (8, 1, 8200),
+                  (8, 1, 40000), (8, 1, 131072), (8, 5, 21), (8, 3, 2000)]
+
+
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("N,S,C", SPECIAL_SHAPES)
+def test_softmax_special_values_follow_the_reference(K, N, S, C, dtype, log):
+    """Rows holding -inf everywhere, one +inf, one nan, a finite mask everywhere, -inf in one
+    half, and one huge logit: nan and inf must appear exactly where the CPU kernels put them
+    (max-subtraction turns inf - inf into nan: softmax_kernel.cc's row maximum then exp), in
+    the forward and in the backward that consumes such an output."""
+    rng = U.rng_for(C)
+    x = (rng.standard_normal((N, C, S)) * 3).astype(np.float32)
+    x[0, :, 0] = -np.inf
+    x[1, C // 2, 0] = np.inf
+    x[2, C - 1, 0] = np.nan
+    x[3, :, 0] = -1e4
+    x[4, : C // 2, 0] = -np.inf
+    x[5, 0, 0] = 6e4
+    xb = R.to_bits(x, dtype)
+    xo, od = oracle_dtype_inputs(xb, dtype)
+
+    def stored(a):
+        """An fp32 oracle result as the I/O type stores it."""
+        a = np.asarray(a, np.float32).reshape(N, C, S)
+        return U.widen(R.to_bits(a, dtype), dtype) if dtype != "float32" else a.astype(np.float64)
+
+    def same_specials(got, want):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.isinf(got), np.isinf(want))
+        assert np.array_equal(got[np.isinf(got)], want[np.isinf(want)])
+
+    want = stored((R.log_softmax if log else R.softmax)(od, N, S, C, np.asarray(xo, np.float32)))
+    y = empty((N, C, S), dtype)
+    (K.log_softmax if log else K.softmax)(N, S, C, U.to_device(xb, dtype), y)
+    got = U.widen(U.to_host(y), dtype)
+    same_specials(got, want)
+    # finite values to the usual bar, per slice relative to its maximum, against fp64 and
+    # against the oracle (whose sequential fp32 sum of a long row is itself 1e-5 to 1e-4 off)
+    x64 = np.asarray(xo, np.float64).reshape(N, C, S)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        z = x64 - x64.max(1, keepdims=True)
+        y64 = z - np.log(np.exp(z).sum(1, keepdims=True)) if log else \
+            np.exp(z) / np.exp(z).sum(1, keepdims=True)
+    for n in range(N):
+        for s in range(S):
+            w, g, e = want[n, :, s], got[n, :, s], y64[n, :, s]
+            fin = np.isfinite(w) & np.isfinite(e)
+            if fin.any():
+                scale = max(np.max(np.abs(w[fin])), 1e-30)
+                e_go = np.max(np.abs(g[fin] - w[fin])) / scale
+                e_ge = np.max(np.abs(g[fin] - e[fin])) / scale
+                e_oe = np.max(np.abs(w[fin] - e[fin])) / scale
+                assert e_ge <= U.TIGHT[dtype] and e_go <= U.TIGHT[dtype] + e_oe, (n, s)
+
+    yb = R.to_bits(want.astype(np.float32), dtype)
+    dyb = R.to_bits(rng.standard_normal((N, C, S)).astype(np.float32), dtype)
+    yo, _ = oracle_dtype_inputs(yb, dtype)
+    dyo, _ = oracle_dtype_inputs(dyb, dtype)
+    want_dx = stored((R.log_softmax_grad if log else R.softmax_grad)(
+        od, N, S, C, np.asarray(dyo, np.float32), np.asarray(yo, np.float32)))
+    dx = empty((N, C, S), dtype)
+    (K.log_softmax_grad if log else K.softmax_grad)(N, S, C, U.to_device(dyb, dtype),
+                                                   U.to_device(yb, dtype), dx)
+    same_specials(U.widen(U.to_host(dx), dtype), want_dx)
 
 
 # ---------------------------------------------------------------- LayerNorm backward
@@ -636,6 +732,38 @@ def test_moments(K, shape, axes, dtype):
     assert ok, errs
     ok, *errs = U.close3(U.to_host(var), var_ref, x64.var(tuple(axes)).reshape(var_ref.shape), tol * 2)
     assert ok, errs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape,axes", [((6, 35), (1,)), ((16, 8192), (1,)), ((6, 70000), (1,)),
+                                        ((1000, 72), (0,)), ((64, 40, 49), (0, 2)),
+                                        ((5000, 7), (1,)), ((70, 9, 300), (1,)),
+                                        ((20000, 2), (0,)), ((2, 3, 4), (0, 1, 2))])
+def test_moments_special_values_follow_the_reference(K, shape, axes, dtype):
+    """inf and nan among the reduced elements, the first one included (the sample the
+    shifted sums are taken from): the mean is the infinity or nan that the CPU kernel's
+    plain sums give, the variance nan (moments.cc:10-120: E[x^2] - E[x]^2)."""
+    rng = U.rng_for(720 + len(shape))
+    xf = (rng.standard_normal(shape) + 0.5).astype(np.float32)
+    flat = xf.reshape(-1)
+    flat[0] = -np.inf                      # first sample of the first output
+    flat[flat.size // 2] = np.inf
+    flat[flat.size - 1] = np.nan
+    x = R.to_bits(xf, dtype)
+    mean_ref, var_ref = R.moments(dtype, x, list(axes))
+    an = acc_name(dtype)
+    mean, var = empty(mean_ref.shape, an), empty(var_ref.shape, an)
+    K.moments(list(shape), list(axes), U.to_device(x, dtype), mean, var)
+    m, v = U.to_host(mean), U.to_host(var)
+    assert np.array_equal(np.isnan(m), np.isnan(mean_ref))
+    assert np.array_equal(np.isinf(m), np.isinf(mean_ref))
+    assert np.array_equal(m[np.isinf(m)], mean_ref[np.isinf(mean_ref)])
+    assert np.array_equal(np.isnan(v), np.isnan(var_ref))
+    ok = np.isfinite(mean_ref)
+    with np.errstate(invalid="ignore"):
+        m64 = np.asarray(U.widen(x, dtype), np.float64).reshape(shape).mean(tuple(axes))
+    good, *errs = U.close3(m[ok], mean_ref[ok], m64.reshape(mean_ref.shape)[ok], 1e-5)
+    assert good, errs
 
 
 def test_math_helpers_bitwise(K):
