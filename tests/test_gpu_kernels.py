@@ -615,6 +615,89 @@ def test_batch_norm_training(K, shape, axis, dtype):
     assert U.normwise(U.widen(U.to_host(dx2), dtype), dx_ref) <= U.TIGHT[dtype]
 
 
+def _same_specials(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    assert np.array_equal(got[np.isinf(got)], want[np.isinf(want)])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape,axis", [((4, 6, 8, 8), 1), ((3, 5, 7, 7), 1), ((2, 4, 150, 150), 1),
+                                        ((4, 8, 8, 6), -1), ((64, 6, 56, 56), 1), ((9, 40), 1)])
+def test_batch_norm_special_values_follow_the_reference(K, shape, axis, dtype):
+    """A channel whose first sample is -inf, one holding +inf and one holding nan: batch and
+    running statistics, fused parameters and y carry inf / nan exactly where the CPU operator's
+    do (batch_norm_op.cc:49-82); the clean channels stay within the usual bar."""
+    rng = U.rng_for(520 + len(shape))
+    ax = axis % len(shape)
+    N, C = shape[0], shape[ax]
+    S = int(np.prod(shape)) // N // C
+    layout = "NHWC" if ax + 1 == len(shape) and len(shape) > 2 else "NCHW"
+    xf = (2 * rng.standard_normal(shape) + 0.5).astype(np.float32)
+    xc = np.moveaxis(xf, ax, 0)           # [C, ...] view
+    xc[0].reshape(-1)[0] = -np.inf         # the sample the shifted sums start from
+    xc[2].reshape(-1)[xc[2].size // 2] = np.inf
+    xc[3].reshape(-1)[-1] = np.nan
+    x = R.to_bits(xf, dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    rm0 = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    rv0 = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    rm_ref, rv_ref = rm0.copy(), rv0.copy()
+    y_ref, mu_ref, rsig_ref, params_ref = R.op_batch_norm_train(
+        od, np.asarray(xo).reshape(shape), g, b, rm_ref, rv_ref, axis, 0.9, 1e-5)
+    mu, rsig, params = empty((C,), "float32"), empty((C,), "float32"), empty((2 * C,), "float32")
+    rm, rv, y = U.to_device(rm0, "float32"), U.to_device(rv0, "float32"), empty(shape, dtype)
+    K.batch_norm_training_forward(N, C, S, layout, 0.9, 1e-5, U.to_device(x, dtype),
+                                  U.to_device(g, "float32"), U.to_device(b, "float32"), rm, rv, mu,
+                                  rsig, params, y)
+    _same_specials(U.to_host(mu), mu_ref)
+    _same_specials(U.to_host(rsig), rsig_ref)
+    _same_specials(U.to_host(rm), rm_ref)
+    _same_specials(U.to_host(rv), rv_ref)
+    _same_specials(U.to_host(params), params_ref)
+    yw = U.widen(U.to_host(y), dtype).reshape(shape)
+    yr = np.asarray(R.to_bits(np.asarray(y_ref, np.float32), dtype) if dtype != "float32" else y_ref)
+    yr = U.widen(yr, dtype).reshape(shape) if dtype != "float32" else np.asarray(y_ref, np.float64).reshape(shape)
+    _same_specials(yw, yr)
+    clean = [c for c in range(C) if c not in (0, 2, 3)]
+    # the oracle's sequential fp32 sum over a 200704-element channel is itself 2-6e-5 off
+    assert U.normwise(np.moveaxis(yw, ax, 0)[clean], np.moveaxis(yr, ax, 0)[clean]) <= max(
+        U.TIGHT[dtype], 6e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape,axis,group", [((4, 8, 8, 8), 1, 4), ((3, 6, 7, 7), 1, 3),
+                                              ((5, 4, 150, 150), 1, 2), ((4, 8, 8, 8), -1, 4),
+                                              ((5, 32, 64, 64), 1, 4), ((5, 6, 14, 14), 1, 0)])
+def test_group_norm_special_values_follow_the_reference(K, shape, axis, group, dtype):
+    """Groups that start with -inf, hold +inf or hold nan (group_norm_op.cc's Moments -> InvStd
+    -> GroupNorm sequence on the CPU): mu, rsig and y carry inf / nan in the same places."""
+    rng = U.rng_for(530 + len(shape) + group)
+    ax = axis % len(shape)
+    N, C = shape[0], shape[ax]
+    S = int(np.prod(shape)) // N // C
+    G = group if group > 0 else C
+    D = C // G
+    layout = "NHWC" if ax + 1 == len(shape) else "NCHW"
+    xf = (rng.standard_normal(shape) + 0.3).astype(np.float32)
+    xf[0].reshape(-1)[0] = -np.inf         # first element of sample 0, group 0
+    xf[1].reshape(-1)[xf[1].size // 2] = np.inf
+    xf[2].reshape(-1)[-1] = np.nan
+    x = R.to_bits(xf, dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    y_ref, mu_ref, rsig_ref = R.op_group_norm(dtype, x, g, b, axis, group, 1e-5)
+    mu, rsig, y = empty((N * G,), "float32"), empty((N * G,), "float32"), empty(shape, dtype)
+    K.group_norm_forward(N, G, D, S, layout, 1e-5, U.to_device(x, dtype), U.to_device(g, "float32"),
+                         U.to_device(b, "float32"), mu, rsig, y)
+    _same_specials(U.to_host(mu), mu_ref)
+    _same_specials(U.to_host(rsig), rsig_ref)
+    yw, yr = U.widen(U.to_host(y), dtype).reshape(shape), U.widen(y_ref, dtype).reshape(shape)
+    _same_specials(yw, yr)
+    assert U.normwise(yw[3:], yr[3:]) <= U.TIGHT[dtype]
+
+
 def test_batch_norm_exchange_timeout_is_reported(K):
     """A wait of one poll gives up before the other slices of a channel have published their
     sums: every kernel still runs to its end, the library says so, and refuses further
