@@ -469,13 +469,22 @@ struct LayerNormShortBackward {
   A* db;
   A* partial;  // [gridDim.x][C][2]
   A g[kE], dg[kE], dbt[kE];
+  bool packed = false;  // lane l owns elements l * kE + j instead of l + j * kL
+  __device__ __forceinline__ void set_packed(bool on) { packed = on; }
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
+  template <int kL>
+  __device__ __forceinline__ int element(int l, int j) const {
+    return packed ? l * kE + j : l + j * kL;
+  }
   __device__ __forceinline__ A fill0() const { return A(0); }
   __device__ __forceinline__ A fill1() const { return A(0); }
   template <int kL>
   __device__ __forceinline__ void begin(int l, int C) {
 #pragma unroll
     for (int j = 0; j < kE; ++j) {
-      g[j] = l + j * kL < C ? gamma[l + j * kL] : A(0);
+      const int e = element<kL>(l, j);
+      g[j] = e < C ? gamma[e] : A(0);
       dg[j] = dbt[j] = A(0);
     }
   }
@@ -528,7 +537,7 @@ struct LayerNormShortBackward {
       A* out = partial + static_cast<size_t>(blockIdx.x) * C * 2;
 #pragma unroll
       for (int j = 0; j < kE; ++j) {
-        const int e = l + j * kL;
+        const int e = element<kL>(l, j);
         if (e < C) {
           A a = A(0), b = A(0);
           for (int q = 0; q < kGroups; ++q) {  // fixed order

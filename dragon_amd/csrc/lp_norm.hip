@@ -336,6 +336,9 @@ struct LpNormShortForwardOp {
   static constexpr size_t kEndBytes = 0;
   static constexpr int kSideWords = 0;
   A normalizer, eps;
+  __device__ __forceinline__ void set_packed(bool) {}  // no per-element state: any order
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
   __device__ __forceinline__ A fill0() const { return A(0); }
   __device__ __forceinline__ A fill1() const { return A(0); }
   template <int kL>
@@ -367,6 +370,9 @@ struct LpNormShortBackwardOp {
   static constexpr size_t kEndBytes = 0;
   static constexpr int kSideWords = 0;
   A normalizer, eps;
+  __device__ __forceinline__ void set_packed(bool) {}  // no per-element state: any order
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
   __device__ __forceinline__ A fill0() const { return A(0); }
   __device__ __forceinline__ A fill1() const { return A(0); }
   template <int kL>

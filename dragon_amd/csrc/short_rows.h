@@ -116,6 +116,22 @@ struct OpReadOnly : std::false_type {};
 template <typename Op>
 struct OpReadOnly<Op, std::void_t<decltype(Op::kReadOnly)>> : std::bool_constant<Op::kReadOnly> {};
 
+// An Op with a member `set_packed(bool)` accepts the packed element order: when
+// a row is exactly kL * kE elements and the tensors are 16-byte aligned, lane l
+// owns the contiguous elements l * kE + j instead of l + j * kL and moves them
+// with 128-bit LDS accesses. A wavefront then touches one contiguous stretch of
+// LDS per access, free of bank conflicts; in the interleaved order its narrow
+// accesses hit rows a power of two apart (four- to eight-way conflicts for rows
+// of 64 elements). The kernel tells the Op which order is in force before
+// begin(); Ops that index per-element parameters must follow it.
+// Such an Op also says for which lane counts it wants the order:
+// `template <int kL> static constexpr bool packed_ok()`.
+template <typename Op, int kL, typename = void>
+struct OpPacked : std::false_type {};
+template <typename Op, int kL>
+struct OpPacked<Op, kL, std::void_t<decltype(Op::template packed_ok<kL>())>>
+    : std::bool_constant<Op::template packed_ok<kL>()> {};
+
 // in0, in1 (when kIn == 2) and out must be congruent modulo 16 bytes (they
 // usually are: allocations are aligned far beyond that), so that the staged
 // packets map one to one. Several workgroups share a compute unit and overlap
@@ -136,6 +152,14 @@ __global__ __launch_bounds__(kShortThreads) void short_rows(
   const int sub = threadIdx.x / kL;
   constexpr int kRowsPerPass = kShortThreads / kL;
   constexpr int kSide = Op::kSideWords > 0 ? Op::kSideWords : 1;
+  constexpr int kVec = IO<T>::kVec;
+  constexpr int kLanePackets = kE / kVec;
+  bool packed = false;
+  if constexpr (OpPacked<Op, kL>::value) {
+    packed = C == kL * kE &&
+        ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    op.set_packed(packed);
+  }
   op.template begin<kL>(l, C);
   for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rows_per_chunk; row0 < N;
        row0 += static_cast<int64_t>(gridDim.x) * rows_per_chunk) {
@@ -162,6 +186,33 @@ __global__ __launch_bounds__(kShortThreads) void short_rows(
       T* p0 = tile0 + static_cast<size_t>(r) * C;
       const T* p1 = tile1 + static_cast<size_t>(r) * C;
       A v0[kE], v1[kE];
+      if (OpPacked<Op, kL>::value && packed) {  // uniform over the grid; rows start on packets
+        u32x4* q0 = reinterpret_cast<u32x4*>(p0) + l * kLanePackets;
+        const u32x4* q1 = reinterpret_cast<const u32x4*>(p1) + l * kLanePackets;
+#pragma unroll
+        for (int k = 0; k < kLanePackets; ++k) {
+          A t[kVec];
+          IO<T>::unpack(q0[k], t);
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) v0[k * kVec + i] = t[i];
+          if constexpr (Op::kIn == 2) {
+            IO<T>::unpack(q1[k], t);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) v1[k * kVec + i] = t[i];
+          }
+        }
+        op.template row<kL>(row0 + r, side + r * kSide, l, C, v0, v1);
+        if constexpr (!OpReadOnly<Op>::value) {
+#pragma unroll
+          for (int k = 0; k < kLanePackets; ++k) {
+            A t[kVec];
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) t[i] = v0[k * kVec + i];
+            q0[k] = IO<T>::pack(t);
+          }
+        }
+        continue;
+      }
 #pragma unroll
       for (int j = 0; j < kE; ++j) {
         const int e = l + j * kL;

@@ -923,6 +923,9 @@ struct SoftmaxShortForwardOp {
   static constexpr int kIn = 1;
   static constexpr size_t kEndBytes = 0;
   static constexpr int kSideWords = 0;
+  __device__ __forceinline__ void set_packed(bool) {}  // no per-element state: any order
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
   __device__ __forceinline__ A fill0() const { return acc_neg_inf<A>(); }
   __device__ __forceinline__ A fill1() const { return A(0); }
   template <int kL>
@@ -966,6 +969,9 @@ struct SoftmaxShortBackwardOp {
   static constexpr int kIn = 2;
   static constexpr size_t kEndBytes = 0;
   static constexpr int kSideWords = 0;
+  __device__ __forceinline__ void set_packed(bool) {}  // no per-element state: any order
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
   __device__ __forceinline__ A fill0() const { return A(0); }
   __device__ __forceinline__ A fill1() const { return kKind == kSoftmax ? A(0) : acc_neg_inf<A>(); }
   template <int kL>
