@@ -172,6 +172,10 @@ struct ReduceRowOp {
   static constexpr bool kReadOnly = true;
   typename P::Out out;
   A inv_n;
+  // sums only: any element order (element 0 stays v[0] of lane 0 in both)
+  __device__ __forceinline__ void set_packed(bool) {}
+  template <int kL>
+  static constexpr bool packed_ok() { return true; }
   __device__ __forceinline__ A fill0() const { return A(0); }
   __device__ __forceinline__ A fill1() const { return A(0); }
   template <int kL>
