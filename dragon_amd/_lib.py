@@ -106,6 +106,7 @@ SIGNATURES = {
                                                        _vp]),
     "dragon_hip_exchange_timed_out": (_int, []),
     "dragon_hip_exchange_reset": (None, [ctypes.c_uint]),
+    "dragon_hip_exchange_plan": (_int, [_int, _i64, _i64, _i64, _int] + [ctypes.POINTER(_int)] * 4),
     "dragon_hip_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
 }
 

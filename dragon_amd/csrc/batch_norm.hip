@@ -541,6 +541,7 @@ template <typename T>
 struct CoopForward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 1;
+  static constexpr bool kBeginReadsInput = true;
   using Merge = PairSum;
   A inv_n, momentum, one_minus_momentum, eps;
   const A* gamma;
@@ -791,6 +792,18 @@ inline int check_scratch(const ChannelShape& sh, int dtype, const void* scratch,
   return (scratch && bytes >= scratch_bytes_for(dtype, sh)) ? DRAGON_HIP_OK : DRAGON_HIP_ESCRATCH;
 }
 
+template <typename T>
+int exchange_plan_of(const SliceUnits& u, int tensors, int* slices, int* slice_packets,
+                     int* packets_per_thread, int* grid) {
+  const CoopPlan p = plan_coop<T>(u, tensors);
+  if (!p.ok) return 0;
+  *slices = static_cast<int>(p.K);
+  *slice_packets = static_cast<int>(p.slice);
+  *packets_per_thread = p.r;
+  *grid = static_cast<int>(coop_grid(coop_rmax(tensors), tensors));
+  return 1;
+}
+
 } // namespace
 } // namespace dragon_hip
 
@@ -909,15 +922,29 @@ int dragon_hip_batch_norm_inference_grad(int dtype, int64_t N, int64_t C, int64_
   DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_inference_grad, sh, rsig, gamma, dy, dx, s);
 }
 
-int dragon_hip_exchange_timed_out(void) {
-  const dragon_hip::ExchangeState& ex = dragon_hip::exchange_state();
-  return ex.host_word && *static_cast<volatile uint32_t*>(ex.host_word) != 0u ? 1 : 0;
-}
-
-void dragon_hip_exchange_reset(unsigned patience) {
-  dragon_hip::ExchangeState& ex = dragon_hip::exchange_state();
-  if (ex.host_word) *static_cast<volatile uint32_t*>(ex.host_word) = 0u;
-  ex.patience = patience;
+int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seglen, int tensors,
+                             int* slices, int* slice_packets, int* packets_per_thread, int* grid) {
+  if (!slices || !slice_packets || !packets_per_thread || !grid) return 0;
+  if (tensors < 1 || tensors > 2 || units <= 0 || nseg <= 0 || seglen <= 0) return 0;
+  if (!dragon_hip::fits_int32(units * nseg * seglen)) return 0;
+  const dragon_hip::SliceUnits u{static_cast<uint32_t>(units), static_cast<uint32_t>(nseg),
+                                 static_cast<uint32_t>(seglen), static_cast<uint32_t>(seglen),
+                                 static_cast<uint32_t>(seglen)};
+  switch (dtype) {
+    case DRAGON_HIP_F16:
+      return dragon_hip::exchange_plan_of<dragon_hip::f16_t>(u, tensors, slices, slice_packets,
+                                                             packets_per_thread, grid);
+    case DRAGON_HIP_BF16:
+      return dragon_hip::exchange_plan_of<dragon_hip::bf16_t>(u, tensors, slices, slice_packets,
+                                                              packets_per_thread, grid);
+    case DRAGON_HIP_F32:
+      return dragon_hip::exchange_plan_of<float>(u, tensors, slices, slice_packets,
+                                                 packets_per_thread, grid);
+    case DRAGON_HIP_F64:
+      return dragon_hip::exchange_plan_of<double>(u, tensors, slices, slice_packets,
+                                                  packets_per_thread, grid);
+    default: return 0;
+  }
 }
 
 int dragon_hip_batch_norm_training_backward(int dtype, int64_t N, int64_t C, int64_t S,

@@ -149,7 +149,7 @@ inline int pick_col_tw(int64_t N, int64_t C, int64_t S, int vec, int max_r) {
 }
 
 inline unsigned col_launch_grid(int64_t tiles) {
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 64;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 64;
   return static_cast<unsigned>(tiles < cap ? (tiles > 0 ? tiles : 1) : cap);
 }
 

@@ -6,12 +6,36 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "dragon_hip.h"
 
 namespace dragon_hip {
 
 constexpr int kWaveSize = 64;  // CDNA wavefront width
-constexpr int kNumCUs = 256;   // MI355X compute units (8 XCDs x 32)
+constexpr int kMaxDevices = 64;  // per-device state is kept in arrays of this size
+
+// Compute units of the current device (256 on MI355X: 8 XCDs x 32), asked of the
+// runtime once per device. Where no device answers (size queries on a host
+// without one) the MI355X figure is assumed.
+inline int num_cus() {
+  constexpr int kAssumed = 256;
+  static std::atomic<int> cached[kMaxDevices];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    (void)hipGetLastError();
+    return kAssumed;
+  }
+  int n = cached[device].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+      n <= 0) {
+    (void)hipGetLastError();
+    n = kAssumed;
+  }
+  cached[device].store(n, std::memory_order_relaxed);
+  return n;
+}
 
 // 16-bit storage types: same bit layout as dragon::float16 / dragon::bfloat16
 // (dragon/core/types.h:36-42), a bare unsigned short.

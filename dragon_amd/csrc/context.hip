@@ -5,7 +5,37 @@
 
 namespace {
 inline int st(hipError_t e) { return e == hipSuccess ? DRAGON_HIP_OK : static_cast<int>(e); }
+
+// Items of the single-read kernels (slices.h) whose wait ran out, counted on
+// the device that ran them. Every device holds its own copy of the word.
+__device__ uint32_t g_exchange_gave_up;
+std::atomic<uint32_t> g_exchange_patience{0};
 } // namespace
+
+namespace dragon_hip {
+
+uint32_t exchange_patience() { return g_exchange_patience.load(std::memory_order_relaxed); }
+
+uint32_t* exchange_gave_up_counter() {
+  static std::atomic<uint32_t*> resolved[kMaxDevices];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  uint32_t* p = resolved[device].load(std::memory_order_acquire);
+  if (p) return p;
+  void* addr = nullptr;
+  if (hipGetSymbolAddress(&addr, HIP_SYMBOL(g_exchange_gave_up)) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  p = static_cast<uint32_t*>(addr);
+  resolved[device].store(p, std::memory_order_release);
+  return p;
+}
+
+} // namespace dragon_hip
 
 extern "C" {
 
@@ -16,8 +46,7 @@ const char* dragon_hip_status_string(int status) {
     case DRAGON_HIP_EDTYPE: return "unsupported dtype";
     case DRAGON_HIP_ESCRATCH: return "scratch buffer missing or too small";
     case DRAGON_HIP_ENODEVICE: return "no HIP device";
-    case DRAGON_HIP_ETIMEOUT:
-      return "an earlier single-read BatchNorm launch gave up waiting for partial sums";
+    case DRAGON_HIP_ETIMEOUT: return "timed out (not returned by any entry point)";
     default: break;
   }
   if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -109,6 +138,23 @@ int dragon_hip_event_sync(void* event) { return st(hipEventSynchronize(static_ca
 int dragon_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
   if (!ms) return DRAGON_HIP_EINVAL;
   return st(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+}
+
+
+int dragon_hip_exchange_timed_out(void) {
+  uint32_t* word = dragon_hip::exchange_gave_up_counter();
+  uint32_t n = 0;
+  if (!word || hipMemcpy(&n, word, sizeof(n), hipMemcpyDeviceToHost) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n > 0x7fffffffu ? 0x7fffffff : static_cast<int>(n);
+}
+
+void dragon_hip_exchange_reset(unsigned patience) {
+  g_exchange_patience.store(patience, std::memory_order_relaxed);
+  uint32_t* word = dragon_hip::exchange_gave_up_counter();
+  if (word && hipMemset(word, 0, sizeof(uint32_t)) != hipSuccess) (void)hipGetLastError();
 }
 
 } // extern "C"

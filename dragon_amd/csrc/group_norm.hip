@@ -453,7 +453,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
 // its workgroup visits; the workgroup's lane groups are combined through LDS
 // into one partial row per workgroup, summed by sum_partial_rows.
 // --------------------------------------------------------------------------
-constexpr int kShortGradMaxGrid = kNumCUs * 8;
+inline int short_grad_max_grid() { return num_cus() * 8; }
 
 template <typename T, int kE>
 struct LayerNormShortBackward {
@@ -561,7 +561,7 @@ inline bool layer_norm_grad_short_rows(int64_t G, int64_t D, int64_t S, size_t e
 }
 inline unsigned short_grad_grid(int64_t N, uint32_t rows_per_chunk) {
   const unsigned grid = short_grid(N, rows_per_chunk);
-  return grid < static_cast<unsigned>(kShortGradMaxGrid) ? grid : kShortGradMaxGrid;
+  return grid < static_cast<unsigned>(short_grad_max_grid()) ? grid : short_grad_max_grid();
 }
 
 // --------------------------------------------------------------------------
@@ -590,13 +590,13 @@ inline WideGradPlan plan_wide_grad(int64_t N, int64_t D, int kw) {
   const int64_t tile = static_cast<int64_t>(kReduceThreads) * kw;
   const int64_t col_blocks = ceil_div(D, tile);
   // first pass: enough workgroups for the chip, at least four tiles each
-  int64_t splits = ceil_div(static_cast<int64_t>(kNumCUs) * 4, N);
+  int64_t splits = ceil_div(static_cast<int64_t>(num_cus()) * 4, N);
   const int64_t max_splits = col_blocks / 4 > 1 ? col_blocks / 4 : 1;
   if (splits > max_splits) splits = max_splits;
   const int64_t tiles_per_split = ceil_div(col_blocks, splits);
   splits = ceil_div(col_blocks, tiles_per_split);
   // second pass: about eight workgroups per compute unit, eight rows or more per chunk
-  int64_t chunks = ceil_div(static_cast<int64_t>(kNumCUs) * 8, col_blocks);
+  int64_t chunks = ceil_div(static_cast<int64_t>(num_cus()) * 8, col_blocks);
   const int64_t max_chunks = N / 8 > 1 ? N / 8 : 1;
   if (chunks > max_chunks) chunks = max_chunks;
   const int64_t rows_per_chunk = ceil_div(N, chunks);
@@ -1713,7 +1713,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
 // device, at least ~64 rows each.
 inline uint32_t batched_split(int64_t N, int64_t S, int64_t C, int kw) {
   const int64_t tiles = ceil_div(C, kWaveSize * kw);
-  int64_t split = ceil_div(static_cast<int64_t>(kNumCUs) * 8, N * tiles);
+  int64_t split = ceil_div(static_cast<int64_t>(num_cus()) * 8, N * tiles);
   const int64_t by_work = ceil_div(S, 64);
   if (split > by_work) split = by_work;
   if (split < 1) split = 1;
@@ -1907,7 +1907,7 @@ RowGradPlan plan_row_grad(int64_t N, int64_t G, int64_t D, int64_t S) {
   const int per_cu = p.threads == 512 ? 2 : 1;
   const int64_t groups = p.threads / p.cfg.tpr;
   const int64_t want = ceil_div(N, groups);
-  const int64_t cap = kNumCUs * per_cu;
+  const int64_t cap = num_cus() * per_cu;
   p.grid = static_cast<unsigned>(want < cap ? want : cap);
   p.use_rows = true;
   return p;
@@ -1952,7 +1952,7 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   // kernels, or of the staged short-row kernel when the addresses select it
   size_t row_paths = rp.use_rows ? static_cast<size_t>(rp.grid) * D * 2 * sizeof(A) : 0;
   if (G == 1 && S == 1 && D <= 1024) {
-    const size_t staged = static_cast<size_t>(kShortGradMaxGrid) * D * 2 * sizeof(A);
+    const size_t staged = static_cast<size_t>(short_grad_max_grid()) * D * 2 * sizeof(A);
     if (staged > row_paths) row_paths = staged;
   }
   if (rp.use_rows) return row_paths;
@@ -1966,18 +1966,19 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   size_t pairs = static_cast<size_t>(N) * C;
   if (pairs * 2 * sizeof(A) < row_paths) pairs = row_paths / (2 * sizeof(A));
   if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
-  // the slice path: K pairs per group and one pair per wavefront block
+  size_t bytes = pairs * 2 * sizeof(A);
+  // the slice path: the exchange of K pairs per group, then one pair per wavefront block
   if (layout == DRAGON_HIP_NCHW && S % (IO<T>::kVec * kWaveSize) == 0) {
     const uint32_t L = static_cast<uint32_t>(D * S);
     const SliceUnits u{static_cast<uint32_t>(N * G), 1u, L, L, L};
     const CoopPlan p = plan_coop<T>(u, 2);
     if (p.ok) {
-      const size_t slices = static_cast<size_t>(u.units) * p.K +
-          static_cast<size_t>(N) * C * (S / IO<T>::kVec / kWaveSize);
-      if (slices > pairs) pairs = slices;
+      const size_t slices = coop_exchange_bytes(static_cast<size_t>(u.units) * p.K, sizeof(A)) +
+          static_cast<size_t>(N) * C * (S / IO<T>::kVec / kWaveSize) * 2 * sizeof(A);
+      if (slices > bytes) bytes = slices;
     }
   }
-  return pairs * 2 * sizeof(A);
+  return bytes;
 }
 
 // --------------------------------------------------------------------------
@@ -1994,6 +1995,7 @@ template <typename T>
 struct GroupSlicesForward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 1;
+  static constexpr bool kBeginReadsInput = true;
   using Merge = PairSum;
   A inv_l, eps;
   const A* gamma;
@@ -2133,7 +2135,9 @@ int try_group_norm_grad_slices(const GroupShape& sh, const void* x, const void* 
   const CoopPlan p = plan_coop<T>(u, 2);
   if (!p.ok) return kNotApplicable;
   A* pairs = static_cast<A*>(scratch);
-  A* chan_part = pairs + static_cast<size_t>(u.units) * p.K * 2;
+  A* chan_part = reinterpret_cast<A*>(
+      static_cast<char*>(scratch) +
+      coop_exchange_bytes(static_cast<size_t>(u.units) * p.K, sizeof(A)));
   const uint32_t blocks_per_chan = sh.S / kVec / kWaveSize;
   const GroupSlicesBackward<T> op{A(1) / A(static_cast<int64_t>(sh.D) * sh.S),
                                   static_cast<const A*>(mu),

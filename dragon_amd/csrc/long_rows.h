@@ -34,7 +34,7 @@ struct LongRowSplit {
 
 inline unsigned long_rows_grid(int64_t rows) {
   const int64_t want = ceil_div(rows, kLongThreads / kWaveSize);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 16;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 16;
   return static_cast<unsigned>(want < cap ? want : cap);
 }
 

@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kLossThreads) void softmax_ce_backward(
 
 inline unsigned loss_grid(int64_t work_items) {
   const int64_t want = ceil_div(work_items, kLossThreads);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 32;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 32;
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 

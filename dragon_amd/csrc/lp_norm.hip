@@ -322,7 +322,7 @@ __global__ __launch_bounds__(256) void lp_norm_columns(
 
 inline unsigned flat_grid(int64_t threads_needed) {
   const int64_t want = ceil_div(threads_needed, 256);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 64;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 64;
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 

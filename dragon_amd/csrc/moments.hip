@@ -336,7 +336,7 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
   } else if (plan.kind == kPlanStrided) {
     const SegmentedReduce& s = plan.seg;
     const unsigned grid = static_cast<unsigned>(
-        std::min<int64_t>(ceil_div(plan.n_out, kReduceThreads), static_cast<int64_t>(kNumCUs) * 32));
+        std::min<int64_t>(ceil_div(plan.n_out, kReduceThreads), static_cast<int64_t>(num_cus()) * 32));
     hipLaunchKernelGGL((reduce_strided_columns<T, P>), dim3(grid), dim3(kReduceThreads), 0, stream,
                        s.nseg, s.seglen, s.seg_stride, xp, out);
   } else if (plan.kind == kPlanSegments) {

@@ -45,7 +45,7 @@ struct ColumnReduce {
 // How many workgroups share one output: enough to put ~8 workgroups on every
 // compute unit, but never less than ~16K elements per workgroup.
 inline uint32_t pick_split(int64_t n_out, int64_t elems_per_out) {
-  const int64_t want_blocks = static_cast<int64_t>(kNumCUs) * 8;
+  const int64_t want_blocks = static_cast<int64_t>(num_cus()) * 8;
   int64_t split = ceil_div(want_blocks, n_out > 0 ? n_out : 1);
   const int64_t max_by_work = ceil_div(elems_per_out, 16384);
   if (split > max_by_work) split = max_by_work;
@@ -385,7 +385,7 @@ __global__ __launch_bounds__(256) void map_flat(const uint32_t total, const T* i
 
 inline unsigned map_grid(uint32_t npackets) {
   const int64_t want = ceil_div(npackets, 256);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 32;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 32;
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 

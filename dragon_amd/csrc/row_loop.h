@@ -76,7 +76,7 @@ struct RowLoop {
 
 // Workgroups of a looped row kernel: one per row, capped at a few per compute unit.
 inline unsigned loop_grid(int64_t rows) {
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 2;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 2;
   return static_cast<unsigned>(rows < cap ? (rows > 0 ? rows : 1) : cap);
 }
 

@@ -362,7 +362,7 @@ inline unsigned resident_grid(Kernel kernel, int threads, size_t dynamic_lds) {
     (void)hipGetLastError();
     per_cu = 1;
   }
-  const unsigned grid = static_cast<unsigned>(per_cu) * kNumCUs;
+  const unsigned grid = static_cast<unsigned>(per_cu) * num_cus();
   std::lock_guard<std::mutex> guard(lock);
   cache[key] = grid;
   return grid;
@@ -375,7 +375,7 @@ constexpr size_t kMaxStagedParamBytes = 144 * 1024;
 // grid-stride loop picks up the rest.
 inline unsigned row_grid(int64_t rows, int rows_per_block) {
   const int64_t want = ceil_div(rows, rows_per_block);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 2048;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 2048;
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 

@@ -271,7 +271,7 @@ inline bool plan_short_rows(int64_t C, size_t elem_bytes, int packets_per_thread
 }
 inline unsigned short_grid(int64_t N, uint32_t rows_per_chunk) {
   const int64_t chunks = ceil_div(N, rows_per_chunk);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 16;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 16;
   return static_cast<unsigned>(chunks < cap ? chunks : cap);
 }
 inline bool congruent16(const void* a, const void* b) {

@@ -12,14 +12,26 @@
 //
 // Work item w = u*K + k is taken by workgroup w % grid, and a workgroup walks
 // its items in ascending order. All `grid` workgroups are resident at once
-// (the grid is never larger than the occupancy query reports), so a workgroup
-// that waits for the peers of its item waits for workgroups that are running:
-// each of them holds a slice of the same unit or an item of an earlier unit,
-// which by induction completes. The wait is bounded all the same (a thread
-// that runs out of patience goes on with what it has read), so every wavefront
-// reaches the end of the kernel whatever happens.
+// (the grid is never larger than the occupancy query reports) and a unit never
+// has more slices than the grid has workgroups, so the K items of a unit are
+// held by K different workgroups, each of which is at that item or at an item
+// of an earlier unit, which by induction completes: a workgroup that waits for
+// the peers of its item waits for workgroups that are running.
 //
-// A small kernel fills the pairs with the "unset" pattern before every launch.
+// The wait is bounded all the same (other work on the device can keep part of
+// the grid from becoming resident, e.g. a second such kernel on another
+// stream). A workgroup whose wait runs out leaves its item alone: it writes no
+// output for it, the unit's leader writes no per-unit output, and the item is
+// flagged in the launch's own scratch. A second launch of the same code
+// (`channel_slices_repair`, enqueued right behind the first) ends at once when
+// nothing is flagged; otherwise it finishes every flagged item. By then every
+// slice of every unit has published its pair (a workgroup publishes before it
+// waits), so the repair needs no waiting and forms the same totals, bit for
+// bit, as the workgroups that did not give up. The outputs of a call are
+// therefore always complete in stream order, in place or not.
+//
+// A small kernel fills the pairs with the "unset" pattern and clears the flags
+// before every launch.
 //
 // The arithmetic is a policy Op:
 //   kIn                              tensors held (x; x and dy)
@@ -45,32 +57,14 @@ namespace dragon_hip {
 
 constexpr int kCoopThreads = 256;
 
-// A wait that gave up is reported through one word of pinned host memory that
-// the kernels write and the host reads without synchronising: the outputs of
-// that launch are invalid, and every later single-read launch is refused with
-// DRAGON_HIP_ETIMEOUT until the word is cleared. Allocated on first use (once
-// per process; before any stream capture, like the cached launch plans).
-struct ExchangeState {
-  uint32_t* host_word = nullptr;
-  uint32_t* device_word = nullptr;
-  uint32_t patience = 0;  // 0: the default
-};
-inline ExchangeState& exchange_state() {
-  static ExchangeState st = [] {
-    ExchangeState e;
-    void* p = nullptr;
-    if (hipHostMalloc(&p, sizeof(uint32_t), hipHostMallocMapped | hipHostMallocPortable) ==
-        hipSuccess) {
-      e.host_word = static_cast<uint32_t*>(p);
-      *e.host_word = 0u;
-      void* dp = nullptr;
-      if (hipHostGetDevicePointer(&dp, p, 0) == hipSuccess) e.device_word = static_cast<uint32_t*>(dp);
-    }
-    (void)hipGetLastError();
-    return e;
-  }();
-  return st;
-}
+// Process-wide settings and diagnostics of the exchange (defined in
+// context.hip). `exchange_patience` is how many polls of a slot a thread makes
+// before it gives up (0: the default). `exchange_gave_up_counter` is the address,
+// on the current device, of a word that counts the items whose wait ran out
+// (a diagnostic: such items are repaired, see above); null when it cannot be
+// resolved. Neither allocates.
+uint32_t exchange_patience();
+uint32_t* exchange_gave_up_counter();
 constexpr uint32_t kCoopPatience = 1u << 20;  // polls of about 1 us each (s_sleep 32 between them)
 
 struct CoopPlan {
@@ -87,7 +81,9 @@ struct CoopPlan {
 // smaller slices lose more to the per-item exchange than the extra residency
 // gains (8 packets: 81 us forward against 61; 4 + 4: 166 us backward against 125).
 inline int coop_rmax(int kIn) { return kIn == 1 ? 16 : 12; }
-inline uint32_t coop_grid(int r, int kIn) { return r * kIn > 16 ? kNumCUs * 3 : kNumCUs * 4; }
+inline uint32_t coop_grid(int r, int kIn) {
+  return static_cast<uint32_t>(r * kIn > 16 ? num_cus() * 3 : num_cus() * 4);
+}
 
 // What is reduced: `units` reduction units (BatchNorm channels, GroupNorm
 // groups), each `nseg` runs of `seglen` contiguous elements; run s of unit u
@@ -107,11 +103,14 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn) {
   const int rmax = coop_rmax(kIn);
   const int64_t grid = coop_grid(rmax, kIn);
   const int64_t kmin = ceil_div(P, static_cast<int64_t>(rmax) * kCoopThreads);
-  if (kmin > 1024) return p;
+  // The K slices of a unit must be held by K different workgroups (see the
+  // head of this file): never more slices than the grid has workgroups.
+  const int64_t klimit = grid < 1024 ? grid : 1024;
+  if (kmin > klimit) return p;
   // Slices of at least four packets per thread, unless the unit is smaller.
   int64_t kmax = P / (4 * kCoopThreads);
   if (kmax < kmin) kmax = kmin;
-  if (kmax > 1024) kmax = 1024;
+  if (kmax > klimit) kmax = klimit;
   if (kmax > kmin + 64) kmax = kmin + 64;
   // The K whose units*K items fill whole rounds of the resident grid best.
   int64_t best = kmin;
@@ -130,6 +129,14 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn) {
   return p;
 }
 
+// Scratch of one launch over `items` work items: the pairs, then one flag word
+// per item (set when the item's wait ran out) and one for the launch as a whole;
+// a multiple of 256 bytes, so that whatever a caller places behind it stays aligned.
+inline size_t coop_exchange_bytes(size_t items, size_t acc_size) {
+  const size_t bytes = items * 2 * acc_size + (items + 1) * sizeof(uint32_t);
+  return (bytes + 255) / 256 * 256;
+}
+
 // Scratch of the single-read path for `units`: the larger of the one- and the two-tensor plan.
 template <typename T>
 size_t coop_scratch_bytes(const SliceUnits& u) {
@@ -138,7 +145,7 @@ size_t coop_scratch_bytes(const SliceUnits& u) {
   for (int in = 1; in <= 2; ++in) {
     const CoopPlan p = plan_coop<T>(u, in);
     if (!p.ok) continue;
-    const size_t bytes = static_cast<size_t>(u.units) * p.K * 2 * sizeof(A);
+    const size_t bytes = coop_exchange_bytes(static_cast<size_t>(u.units) * p.K, sizeof(A));
     if (bytes > need) need = bytes;
   }
   return need;
@@ -152,11 +159,12 @@ struct CoopShape {
   uint32_t step_seg, step_p;  // kCoopThreads packets further on = step_seg segments and step_p packets
   uint32_t items;        // units * K
   uint32_t patience;     // polls of a slot before a thread gives up
-  uint32_t* timed_out;   // set to 1 by a thread that gave up (may be null)
+  uint32_t* flags;       // flags[w] = 1: item w gave up; flags[items] = 1: some item did
+  uint32_t* gave_up_count;  // device-wide count of such items (a diagnostic; may be null)
 };
 
 template <typename T>
-CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p) {
+CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p, typename IO<T>::Acc* scratch) {
   constexpr int kVec = IO<T>::kVec;
   CoopShape d;
   d.unit_stride = u.unit_stride, d.K = p.K, d.slice = p.slice;
@@ -165,9 +173,10 @@ CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p) {
   d.seg_stride = u.seg_stride;
   d.step_seg = kCoopThreads / d.pps, d.step_p = kCoopThreads % d.pps;
   d.items = u.units * p.K;
-  const ExchangeState& ex = exchange_state();
-  d.patience = ex.patience ? ex.patience : kCoopPatience;
-  d.timed_out = ex.device_word;
+  const uint32_t patience = exchange_patience();
+  d.patience = patience ? patience : kCoopPatience;
+  d.flags = reinterpret_cast<uint32_t*>(scratch + static_cast<size_t>(d.items) * 2);
+  d.gave_up_count = exchange_gave_up_counter();
   return d;
 }
 
@@ -191,25 +200,36 @@ struct CoopCursor {
   }
 };
 
-// Bit pattern of a partial sum that has not been published yet (a NaN that no
-// arithmetic here produces; the slots are filled with it before every launch).
+// Bit pattern of a partial sum that has not been published yet; the slots are
+// filled with it before every launch. It is a NaN, and the hardware carries the
+// payload of an input NaN into a sum, so a partial that is any NaN is published
+// as the canonical quiet NaN instead: no published value equals the pattern.
 template <typename A>
 struct Unset;
 template <>
 struct Unset<float> {
   using Bits = uint32_t;
   static constexpr Bits kValue = 0xffffffffu;
+  static constexpr Bits kQuietNaN = 0x7fc00000u;
 };
 template <>
 struct Unset<double> {
   using Bits = unsigned long long;
   static constexpr Bits kValue = ~0ull;
+  static constexpr Bits kQuietNaN = 0x7ff8000000000000ull;
 };
+template <typename A>
+__device__ __forceinline__ typename Unset<A>::Bits publishable_bits(const A v) {
+  return v != v ? Unset<A>::kQuietNaN : __builtin_bit_cast(typename Unset<A>::Bits, v);
+}
 
+// Before a launch: the n pair words take the unset pattern, the nflags flag words zero.
 template <typename Bits>
-__global__ __launch_bounds__(256) void fill_words(Bits* p, uint32_t n, Bits value) {
+__global__ __launch_bounds__(256) void fill_exchange(Bits* p, uint32_t n, Bits value,
+                                                     uint32_t* flags, uint32_t nflags) {
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
   if (i < n) p[i] = value;
+  if (i < nflags) flags[i] = 0u;
 }
 
 // Publishes this slice's pair, waits for the channel's K pairs and returns
@@ -257,40 +277,58 @@ __device__ __forceinline__ void block_merge_pair(A& a, A& b, A* lds /*2*kReduceW
   }
 }
 
-template <typename Merge, typename A>
-__device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t c, uint32_t w,
+// Returns false when a wait ran out (the same answer in every thread of the
+// workgroup): a and b are then meaningless and the item has been flagged.
+// kRepair: the second launch; every pair has been published, nothing is
+// published or waited for.
+template <typename Merge, bool kRepair, typename A>
+__device__ __forceinline__ bool coop_channel_totals(const CoopShape& d, uint32_t c, uint32_t w,
                                                     A& a, A& b, A* partial, A* lds_a, A* lds_b) {
   using Bits = typename Unset<A>::Bits;
-  block_merge_pair<Merge>(a, b, lds_a);
   Bits* slots = reinterpret_cast<Bits*>(partial);
-  if (threadIdx.x == 0) {
-    __hip_atomic_store(slots + 2 * static_cast<size_t>(w), __builtin_bit_cast(Bits, a),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(slots + 2 * static_cast<size_t>(w) + 1, __builtin_bit_cast(Bits, b),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if constexpr (!kRepair) {
+    block_merge_pair<Merge>(a, b, lds_a);
+    if (threadIdx.x == 0) {
+      __hip_atomic_store(slots + 2 * static_cast<size_t>(w), publishable_bits(a), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slots + 2 * static_cast<size_t>(w) + 1, publishable_bits(b),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
   A ta, tb;
   Merge::identity(ta, tb);
+  int gave_up = 0;
   const Bits* pairs = slots + 2 * static_cast<size_t>(c) * d.K;
   for (uint32_t q = threadIdx.x; q < d.K; q += kCoopThreads) {
     Bits ua, ub;
-    uint32_t patience = d.patience;
+    uint32_t patience = kRepair ? 1u : d.patience;
     for (;;) {
       ua = __hip_atomic_load(pairs + 2 * q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       ub = __hip_atomic_load(pairs + 2 * q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (ua != Unset<A>::kValue && ub != Unset<A>::kValue) break;
       if (--patience == 0) {
-        if (d.timed_out) {
-          __hip_atomic_store(d.timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        }
+        gave_up = 1;
         break;
       }
       __builtin_amdgcn_s_sleep(32);
     }
     Merge::merge(ta, tb, __builtin_bit_cast(A, ua), __builtin_bit_cast(A, ub));
   }
+  if constexpr (!kRepair) {
+    if (__syncthreads_or(gave_up)) {
+      if (threadIdx.x == 0) {
+        __hip_atomic_store(d.flags + w, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(d.flags + d.items, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d.gave_up_count) {
+          __hip_atomic_fetch_add(d.gave_up_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      return false;
+    }
+  }
   block_merge_pair<Merge>(ta, tb, lds_b);
   a = ta, b = tb;
+  return true;
 }
 
 // Optional parts of an Op, both off unless it declares them:
@@ -298,7 +336,7 @@ __device__ __forceinline__ void coop_channel_totals(const CoopShape& d, uint32_t
 //               accumulate (a thread-wide maximum, say);
 //   kRewrites   op.accumulate_rewrite(x, a, b) replaces the elements it is
 //               given, and the second pass reads those instead of the input
-//               (exact only where a packet holds accumulator-typed elements).
+//               (exact only where a packet holds accumulator-typed elements);
 template <typename Op, typename = void>
 struct OpScansFirst : std::false_type {};
 template <typename Op>
@@ -307,6 +345,15 @@ template <typename Op, typename = void>
 struct OpRewrites : std::false_type {};
 template <typename Op>
 struct OpRewrites<Op, std::void_t<decltype(Op::kRewrites)>> : std::bool_constant<Op::kRewrites> {};
+//   kBeginReadsInput  op.begin reads elements of the unit from memory (the sample
+//               a shifted sum is taken relative to). A repaired item must see
+//               the value the first launch saw, so such an Op is kept off
+//               calls whose output overwrites that input.
+template <typename Op, typename = void>
+struct OpBeginReadsInput : std::false_type {};
+template <typename Op>
+struct OpBeginReadsInput<Op, std::void_t<decltype(Op::kBeginReadsInput)>>
+    : std::bool_constant<Op::kBeginReadsInput> {};
 
 template <typename T, int kR, int kIn>
 struct CoopSlice {  // the raw packets of one item
@@ -345,7 +392,8 @@ __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const 
 // `next` is the item this workgroup takes after w (>= d.items: none): its
 // packets are requested one by one into the registers the second pass has just
 // written out, so they travel while the rest of this item is stored.
-template <typename T, int kR, typename Op>
+// kRepair: the second launch, which finishes the items whose wait ran out.
+template <typename T, int kR, typename Op, bool kRepair>
 __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uint32_t next,
                                              const T* in0, const T* in1, T* out, Op op,
                                              CoopSlice<T, kR, Op::kIn>& s,
@@ -386,20 +434,22 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
       }
     }
   }
-  coop_channel_totals<typename Op::Merge>(d, it.c, w, a, b, partial, lds_a, lds_b);
-  op.finish(it.c, it.k == 0 && threadIdx.x == 0, a, b);
+  // false (for the whole workgroup): the wait ran out, the item is left to the repair launch
+  const bool complete = coop_channel_totals<typename Op::Merge, kRepair>(d, it.c, w, a, b, partial,
+                                                                         lds_a, lds_b);
+  if (complete) op.finish(it.c, it.k == 0 && threadIdx.x == 0, a, b);
   // convert the packets again instead of keeping every converted element
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     asm volatile("" : "+v"(s.p0[i]));
     if constexpr (Op::kIn == 2) asm volatile("" : "+v"(s.p1[i]));
   }
-  const bool more = next < d.items;  // uniform over the workgroup
+  const bool more = !kRepair && next < d.items;  // uniform over the workgroup
   const CoopItem nit(d, more ? next : w);
   CoopCursor cur(d, it.j0), ncur(d, nit.j0);
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
-    if (it.has(i)) {
+    if (complete && it.has(i)) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
@@ -430,7 +480,29 @@ __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void chann
   CoopSlice<T, kR, Op::kIn> s;
   if (blockIdx.x < d.items) coop_load<T, kR, Op::kIn>(d, blockIdx.x, in0, in1, s);
   for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
-    coop_process<T, kR, Op>(d, w, w + gridDim.x, in0, in1, out, op, s, partial, lds_a, lds_b);
+    coop_process<T, kR, Op, false>(d, w, w + gridDim.x, in0, in1, out, op, s, partial, lds_a,
+                                   lds_b);
+  }
+}
+
+// The launch behind it: nothing to do unless a wait of the first launch ran
+// out; then every flagged item is finished from the pairs, which by now are all
+// published. Inputs of a flagged item are intact even when the call runs in
+// place: the workgroup that gave up wrote nothing for it.
+template <typename T, int kR, typename Op>
+__global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void channel_slices_repair(
+    const CoopShape d, const T* __restrict__ in0, const T* __restrict__ in1, T* __restrict__ out,
+    const Op op, typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds_a[2 * kReduceWaves];
+  __shared__ A lds_b[2 * kReduceWaves];
+  if (d.flags[d.items] == 0u) return;
+  for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
+    if (d.flags[w] == 0u) continue;  // the same word in every thread
+    CoopSlice<T, kR, Op::kIn> s;
+    coop_load<T, kR, Op::kIn>(d, w, in0, in1, s);
+    coop_process<T, kR, Op, true>(d, w, d.items, in0, in1, out, op, s, partial, lds_a, lds_b);
+    __syncthreads();  // the next item reuses the LDS words of the reductions
   }
 }
 
@@ -438,39 +510,50 @@ template <typename A>
 inline void fill_unset(A* pairs, const CoopShape& d, hipStream_t stream) {
   using Bits = typename Unset<A>::Bits;
   const uint32_t n = d.items * 2;
-  hipLaunchKernelGGL((fill_words<Bits>), dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0,
-                     stream, reinterpret_cast<Bits*>(pairs), n, Unset<A>::kValue);
+  hipLaunchKernelGGL((fill_exchange<Bits>), dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256),
+                     0, stream, reinterpret_cast<Bits*>(pairs), n, Unset<A>::kValue, d.flags,
+                     d.items + 1);
 }
 
 // DRAGON_HIP_OK when the single-read kernel was launched, kNotApplicable when
 // the shape or alignment leaves the call to the split path, or an error.
+// `scratch` holds coop_scratch_bytes<T>(sh) bytes.
 constexpr int kNotApplicable = 1;
+constexpr unsigned kCoopRepairGrid = 256;
 template <typename T, typename Op>
 int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T* in1, T* out,
                        typename IO<T>::Acc* scratch, hipStream_t stream) {
-  const CoopPlan p = plan_coop<T>(sh, Op::kIn);
-  if (!p.ok || !aligned16(in0) || !aligned16(in1) || !aligned16(out)) return kNotApplicable;
-  const ExchangeState& ex = exchange_state();
-  if (ex.host_word && *static_cast<volatile uint32_t*>(ex.host_word) != 0u) {
-    return DRAGON_HIP_ETIMEOUT;
-  }
-  const CoopShape d = make_coop_shape<T>(sh, p);
-  fill_unset(scratch, d, stream);
-#define LAUNCH(R)                                                                              \
-  {                                                                                            \
-    auto kernel = channel_slices<T, R, Op>;                                                    \
-    const unsigned resident = resident_grid(kernel, kCoopThreads, 0);                          \
-    const unsigned want = coop_grid(coop_rmax(Op::kIn), Op::kIn);                              \
-    const unsigned cap = resident < want ? resident : want;                                    \
-    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kCoopThreads), 0,     \
-                       stream, d, in0, in1, out, op, scratch);                                 \
-  }
   constexpr int kIn = Op::kIn;
-  if (p.r * kIn <= 4) LAUNCH(4 / kIn)
-  else if (p.r * kIn <= 8) LAUNCH(8 / kIn)
-  else if (p.r * kIn <= 16) LAUNCH(16 / kIn)
-  else if constexpr (kIn == 2) LAUNCH(12)  // one tensor: never more than 16 packets
-#undef LAUNCH
+  const CoopPlan p = plan_coop<T>(sh, kIn);
+  if (!p.ok || !aligned16(in0) || !aligned16(in1) || !aligned16(out)) return kNotApplicable;
+  if (OpBeginReadsInput<Op>::value && static_cast<const void*>(out) == in0) return kNotApplicable;
+  const CoopShape d = make_coop_shape<T>(sh, p, scratch);
+  // Workgroups launched: all of them resident at once, and at least as many as a unit has slices.
+#define DRAGON_HIP_COOP_GRID(R)                                                                \
+  [&] {                                                                                        \
+    const unsigned resident = resident_grid(channel_slices<T, R, Op>, kCoopThreads, 0);        \
+    const unsigned want = coop_grid(coop_rmax(kIn), kIn);                                      \
+    return resident < want ? resident : want;                                                  \
+  }()
+#define DRAGON_HIP_COOP_LAUNCH(R)                                                              \
+  {                                                                                            \
+    const unsigned cap = DRAGON_HIP_COOP_GRID(R);                                              \
+    if (p.K > cap) return kNotApplicable;                                                      \
+    fill_unset(scratch, d, stream);                                                            \
+    hipLaunchKernelGGL((channel_slices<T, R, Op>), dim3(d.items < cap ? d.items : cap),        \
+                       dim3(kCoopThreads), 0, stream, d, in0, in1, out, op, scratch);          \
+  }
+  if (p.r * kIn <= 4) DRAGON_HIP_COOP_LAUNCH(4 / kIn)
+  else if (p.r * kIn <= 8) DRAGON_HIP_COOP_LAUNCH(8 / kIn)
+  else if (p.r * kIn <= 16) DRAGON_HIP_COOP_LAUNCH(16 / kIn)
+  else if constexpr (kIn == 2) DRAGON_HIP_COOP_LAUNCH(12)  // one tensor: never more than 16 packets
+#undef DRAGON_HIP_COOP_LAUNCH
+#undef DRAGON_HIP_COOP_GRID
+  // the widest slice serves every plan: a repair is rare and its speed does not matter
+  constexpr int kRepairR = kIn == 2 ? 12 : 16;
+  hipLaunchKernelGGL((channel_slices_repair<T, kRepairR, Op>),
+                     dim3(d.items < kCoopRepairGrid ? d.items : kCoopRepairGrid), dim3(kCoopThreads),
+                     0, stream, d, in0, in1, out, op, scratch);
   return status_of_launch();
 }
 

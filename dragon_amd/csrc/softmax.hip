@@ -1013,7 +1013,7 @@ inline bool use_short_rows(int64_t C, size_t elem_bytes, bool forward, const voi
 
 inline unsigned flat_grid(int64_t threads_needed) {
   const int64_t want = ceil_div(threads_needed, 256);
-  const int64_t cap = static_cast<int64_t>(kNumCUs) * 64;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 64;
   return static_cast<unsigned>(want < cap ? (want > 0 ? want : 1) : cap);
 }
 

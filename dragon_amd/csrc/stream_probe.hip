@@ -49,8 +49,8 @@ extern "C" int dragon_hip_stream_probe(int mode, const void* src, void* dst, siz
   if (!aligned16(src) || !aligned16(dst)) return DRAGON_HIP_EINVAL;
   const size_t n = bytes / 16;
   const size_t want = (n + 255) / 256;
-  const unsigned grid = static_cast<unsigned>(want < static_cast<size_t>(kNumCUs) * 64
-                                                  ? want : static_cast<size_t>(kNumCUs) * 64);
+  const unsigned grid = static_cast<unsigned>(want < static_cast<size_t>(num_cus()) * 64
+                                                  ? want : static_cast<size_t>(num_cus()) * 64);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (mode == 0) {
     hipLaunchKernelGGL(probe_read, dim3(grid), dim3(256), 0, s, static_cast<const u32x4*>(src), n,

@@ -335,13 +335,26 @@ def batch_norm_training_backward(N, C, S, normalizer, data_format, x, mu, rsig, 
 
 
 def exchange_timed_out():
-    """True when a single-read BatchNorm launch gave up waiting for its peers' partial sums."""
-    return bool(_lib.lib().dragon_hip_exchange_timed_out())
+    """How many slices of the single-read kernels ran out of patience waiting for their
+    peers' partial results, and were finished by the repair launch, since the last reset."""
+    return int(_lib.lib().dragon_hip_exchange_timed_out())
 
 
 def exchange_reset(patience=0):
-    """Clears the time-out state; ``patience`` polls per wait (0 = the default)."""
+    """Clears that count; ``patience`` polls per wait from now on (0 = the default)."""
     _lib.lib().dragon_hip_exchange_reset(int(patience))
+
+
+def exchange_plan(dtype_name, units, nseg, seglen, tensors):
+    """(slices per unit, packets per slice, packets per thread, grid) of the single-read
+    path for ``units`` reduction units of ``nseg`` runs of ``seglen`` elements, or None
+    when the shape is left to the split path. Needs no device."""
+    import ctypes
+    out = [ctypes.c_int(0) for _ in range(4)]
+    tag = {"float16": 0, "bfloat16": 1, "float32": 2, "float64": 3}[dtype_name]
+    ok = _lib.lib().dragon_hip_exchange_plan(tag, units, nseg, seglen, tensors,
+                                             *[ctypes.byref(o) for o in out])
+    return tuple(o.value for o in out) if ok else None
 
 
 # ---------------------------------------------------------------- measurement

@@ -59,8 +59,7 @@ typedef enum {
   DRAGON_HIP_EDTYPE = -2,   /* dtype not in dragon_hip_dtype                  */
   DRAGON_HIP_ESCRATCH = -3, /* scratch missing or too small                   */
   DRAGON_HIP_ENODEVICE = -4, /* no gfx950 device visible                      */
-  DRAGON_HIP_ETIMEOUT = -5  /* an earlier single-read BatchNorm launch gave up
-                               waiting (dragon_hip_exchange_timed_out)         */
+  DRAGON_HIP_ETIMEOUT = -5  /* reserved: no entry point returns it             */
 } dragon_hip_status;
 
 /* Human-readable text for a status returned by any function below. */
@@ -378,18 +377,35 @@ int dragon_hip_batch_norm_training_backward(int dtype, int64_t N, int64_t C, int
                                             const void* dy, void* dgamma, void* dbeta, void* dx,
                                             void* scratch, size_t scratch_bytes, void* stream);
 
-/* The single-read path of the two training entry points above (NCHW, S a
- * whole number of 16-byte packets) keeps the slices of a channel in the
- * registers of several workgroups, which exchange partial sums inside one
- * kernel and wait for each other, bounded. No counterpart in the reference.
- * dragon_hip_exchange_timed_out: 1 when such a wait has given up since the
- * last reset: the outputs of that launch are invalid, and the two entry points
- * return DRAGON_HIP_ETIMEOUT until dragon_hip_exchange_reset is called.
- * dragon_hip_exchange_reset: clears that state and sets how many polls (of
- * about a microsecond) a wait lasts; 0 = the default (about a second). The first use
- * allocates four bytes of pinned host memory (do it before capturing a graph). */
+/* The single-read paths (BatchNorm training forward / backward on NCHW with S
+ * a whole number of 16-byte packets, GroupNorm groups beyond one workgroup,
+ * softmax rows of many thousands of packets when scratch is passed) keep the
+ * slices of a reduction unit in the registers of several workgroups, which
+ * exchange partial results inside one kernel and wait for each other. The wait
+ * is bounded; a workgroup whose wait runs out writes nothing for its slice and
+ * flags it in the call's scratch, and a second launch enqueued behind the first
+ * finishes every flagged slice, so the outputs of a call are always complete
+ * in stream order and no status is sticky. A wait can only run out when other
+ * work keeps part of the grid off the device (e.g. a second such kernel on
+ * another stream); the call is then correct but slow. No counterpart in the
+ * reference.
+ * dragon_hip_exchange_timed_out: how many slices of the current device had to
+ * be finished that way since the last reset (a diagnostic; copies one word from
+ * the device, so it waits for the null stream). Synchronise the streams of
+ * interest first.
+ * dragon_hip_exchange_reset: clears that count and sets how many polls (of
+ * about a microsecond) a wait lasts in later launches from any thread; 0 = the
+ * default (about a second).
+ * dragon_hip_exchange_plan: how the path would cut `units` reduction units,
+ * each `nseg` runs of `seglen` contiguous elements, with `tensors` (1 or 2)
+ * tensors held in registers: returns 1 and fills slices (per unit),
+ * slice_packets (16-byte packets per slice), packets_per_thread and grid (the
+ * workgroups it asks for; a unit never has more slices than that), or returns
+ * 0 when the shape is left to the split path. */
 int dragon_hip_exchange_timed_out(void);
 void dragon_hip_exchange_reset(unsigned patience);
+int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seglen, int tensors,
+                             int* slices, int* slice_packets, int* packets_per_thread, int* grid);
 
 /* ------------------------------------------------------------------------ */
 /* Measurement utility (no counterpart in the reference): a streaming read    */

@@ -75,3 +75,33 @@ def test_scratch_queries_need_no_device():
     assert lib.dragon_hip_batch_norm_reduce_scratch_bytes(2, 64, 256, 3136, 0) > 0
     assert lib.dragon_hip_group_norm_grad_scratch_bytes(1, 8192, 1, 12288, 1, 1) > 0
     assert lib.dragon_hip_batch_norm_reduce_scratch_bytes(2, 0, 256, 3136, 0) == 0
+
+
+def test_exchange_plan_never_has_more_slices_than_workgroups():
+    """The K slices of a reduction unit must sit in K different workgroups of a grid that is
+    resident at once, or a workgroup would wait for an item it holds itself. Sweeps channel /
+    group / row sizes up to the largest the planner accepts, for both tensor counts."""
+    from dragon_amd import kernels as K
+    rows = 0
+    for dtype, vec in (("float32", 4), ("bfloat16", 8), ("float64", 2)):
+        for tensors in (1, 2):
+            packets_per_unit = 64
+            while packets_per_unit * vec < (1 << 31):
+                for nseg in (1, 48, 768):
+                    seglen = max(16, packets_per_unit // nseg) * vec
+                    units = max(1, min(64, ((1 << 31) - 1) // (nseg * seglen)))
+                    plan = K.exchange_plan(dtype, units, nseg, seglen, tensors)
+                    if plan is None:
+                        continue
+                    slices, slice_packets, per_thread, grid = plan
+                    rows += 1
+                    assert 1 <= slices <= grid, (dtype, tensors, nseg, seglen, plan)
+                    assert slices * slice_packets >= nseg * (seglen // vec)
+                    assert per_thread <= (16 if tensors == 1 else 12)
+                    assert slice_packets % 64 == 0 and slice_packets <= per_thread * 256
+                packets_per_unit = packets_per_unit * 5 // 4 + 1
+    assert rows > 300
+    # the two shapes whose plans once exceeded the backward grid of 768 workgroups
+    for shape in ((4, 768, 112 * 112), (3, 48, 448 * 448)):
+        plan = K.exchange_plan("float32", shape[0], shape[1], shape[2], 2)
+        assert plan is None or plan[0] <= plan[3]

@@ -1,0 +1,255 @@
+"""The single-read kernels' exchange between workgroups (BatchNorm training on NCHW, GroupNorm
+groups and softmax rows beyond one workgroup): a wait that runs out is repaired in stream
+order, an input that holds the "unset" bit pattern does not stall it, and shapes whose
+units would need more slices than the grid has workgroups take the split path."""
+
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    import torch
+    assert torch.cuda.is_available()
+    from dragon_amd import kernels
+    return kernels
+
+
+def _bn_forward(K, t):
+    import torch
+    N, C, S = 8, 40, 56 * 56  # six slices per channel
+    x = t["x"] if "x" in t else t.setdefault("x", torch.randn((N, C, S), device="cuda") * 2 + 0.5)
+    g = t.setdefault("g", torch.rand(C, device="cuda") + 0.5)
+    b = t.setdefault("b", torch.randn(C, device="cuda") * 0.1)
+    rm, rv = torch.full((C,), 0.25, device="cuda"), torch.full((C,), 1.5, device="cuda")
+    mu, rsig, params = (torch.full((n,), -7.0, device="cuda") for n in (C, C, 2 * C))
+    y = torch.full_like(x, -7.0)
+    K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, x, g, b, rm, rv, mu, rsig, params, y)
+    return [y, mu, rsig, params, rm, rv]
+
+
+def _bn_backward(K, t):
+    import torch
+    N, C, S = 8, 40, 56 * 56
+    x = t.setdefault("x", torch.randn((N, C, S), device="cuda") * 2 + 0.5)
+    dy = t.setdefault("dy", torch.randn((N, C, S), device="cuda"))
+    g = t.setdefault("g", torch.rand(C, device="cuda") + 0.5)
+    mu = t.setdefault("mu", x.mean((0, 2)))
+    rsig = t.setdefault("rsig", torch.rsqrt(x.var((0, 2), unbiased=False) + 1e-5))
+    wg, dx = torch.full((2 * C,), -7.0, device="cuda"), torch.full_like(x, -7.0)
+    K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", x, mu, rsig, g, dy, wg, wg, dx)
+    return [dx, wg]
+
+
+def _gn_forward(K, t):
+    import torch
+    N, G, D, S = 2, 2, 4, 256 * 256  # groups of 1 MiB in bf16: 16 slices or more each
+    x = t.setdefault("x", (torch.randn((N, G * D, S), device="cuda") + 0.3).to(torch.bfloat16))
+    g = t.setdefault("g", torch.rand(G * D, device="cuda") + 0.5)
+    b = t.setdefault("b", torch.randn(G * D, device="cuda") * 0.1)
+    mu, rsig = torch.full((N * G,), -7.0, device="cuda"), torch.full((N * G,), -7.0, device="cuda")
+    y = torch.full_like(x, -7.0)
+    K.group_norm_forward(N, G, D, S, "NCHW", 1e-5, x, g, b, mu, rsig, y)
+    return [y, mu, rsig]
+
+
+def _gn_backward(K, t):
+    import torch
+    N, G, D, S = 2, 2, 4, 256 * 256
+    x = t.setdefault("x", (torch.randn((N, G * D, S), device="cuda") + 0.3).to(torch.bfloat16))
+    dy = t.setdefault("dy", torch.randn((N, G * D, S), device="cuda").to(torch.bfloat16))
+    g = t.setdefault("g", torch.rand(G * D, device="cuda") + 0.5)
+    xf = x.float().reshape(N * G, -1)
+    mu = t.setdefault("mu", xf.mean(1))
+    rsig = t.setdefault("rsig", torch.rsqrt(xf.var(1, unbiased=False) + 1e-5))
+    params = torch.full((2 * N * G,), -7.0, device="cuda")
+    dg, db = torch.full((G * D,), -7.0, device="cuda"), torch.full((G * D,), -7.0, device="cuda")
+    dx = torch.full_like(x, -7.0)
+    K.group_norm_grad(N, G, D, S, "NCHW", x, mu, rsig, g, dy, params, params, dg, db, dx)
+    return [dx, dg, db, params]
+
+
+def _softmax_in_place(K, t, log=False, dtype="float32"):
+    import torch
+    N, C = 6, 131072
+    x = t.setdefault("x", (torch.randn((N, C), device="cuda") * 3).to(U.torch_dtype(dtype)))
+    buf = x.clone()
+    (K.log_softmax if log else K.softmax)(N, 1, C, buf, buf)  # y aliases x
+    return [buf]
+
+
+def _softmax_grad_in_place(K, t):
+    import torch
+    N, C = 6, 131072
+    y = t.setdefault("y", torch.softmax(torch.randn((N, C), device="cuda") * 3, 1))
+    dy = t.setdefault("dy", torch.randn((N, C), device="cuda"))
+    buf = dy.clone()
+    K.softmax_grad(N, 1, C, buf, y, buf)  # dx aliases dy
+    return [buf]
+
+
+CALLS = {
+    "batch_norm_training_forward": _bn_forward,
+    "batch_norm_training_backward": _bn_backward,
+    "group_norm_forward": _gn_forward,
+    "group_norm_grad": _gn_backward,
+    "softmax_in_place": _softmax_in_place,
+    "log_softmax_in_place": lambda K, t: _softmax_in_place(K, t, log=True),
+    "softmax_bf16_in_place": lambda K, t: _softmax_in_place(K, t, dtype="bfloat16"),
+    "softmax_grad_in_place": _softmax_grad_in_place,
+}
+
+
+@pytest.mark.parametrize("name", sorted(CALLS))
+def test_waits_that_run_out_are_repaired_in_stream_order(K, name):
+    """With a patience of one poll most workgroups give up before their peers have published.
+    The call still returns complete outputs (the launch behind it finishes the flagged
+    slices), bit for bit those of an undisturbed call, per-unit outputs and running
+    statistics written exactly once, in place or not; nothing is sticky afterwards."""
+    import torch
+    call, tensors = CALLS[name], {}
+    K.exchange_reset(0)
+    want = [o.clone() for o in call(K, tensors)]
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    try:
+        K.exchange_reset(1)
+        repaired = 0
+        for _ in range(4):  # a peer that is late by one poll is all it takes
+            got = call(K, tensors)
+            torch.cuda.synchronize()
+            repaired = K.exchange_timed_out()
+            for g, w in zip(got, want):
+                assert torch.equal(g.view(torch.uint8), w.view(torch.uint8))
+            if repaired:
+                break
+        assert repaired > 0, "the forced give-up never happened: the repair path did not run"
+    finally:
+        K.exchange_reset(0)
+    assert K.exchange_timed_out() == 0
+    got = call(K, tensors)
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    for g, w in zip(got, want):
+        assert torch.equal(g.view(torch.uint8), w.view(torch.uint8))
+
+
+def test_repaired_batch_norm_matches_the_oracle(K):
+    import torch
+    N, C, S = 8, 40, 56 * 56
+    rng = U.rng_for(77)
+    x = (2 * rng.standard_normal((N, C, S)) + 0.5).astype(np.float32)
+    g, b = U.affine_params(rng, C, "float32")
+    rm_ref, rv_ref = np.zeros(C, np.float32), np.ones(C, np.float32)
+    y_ref, mu_ref, rsig_ref, params_ref = R.op_batch_norm_train("float32", x, g, b, rm_ref, rv_ref,
+                                                                1, 0.9, 1e-5)
+    t = {"x": torch.from_numpy(x).cuda(), "g": torch.from_numpy(g).cuda(),
+         "b": torch.from_numpy(b).cuda()}
+    try:
+        K.exchange_reset(1)
+        y, mu, rsig, params, rm, rv = _bn_forward(K, t)
+        torch.cuda.synchronize()
+    finally:
+        K.exchange_reset(0)
+    assert U.normwise(U.to_host(y), y_ref) <= 1e-5
+    assert U.normwise(U.to_host(mu), mu_ref) <= 1e-5
+    assert U.normwise(U.to_host(params), params_ref) <= 1e-5
+    # _bn_forward starts the running statistics at 0.25 / 1.5
+    assert U.normwise(U.to_host(rm), 0.9 * np.float32(0.25) + (1 - 0.9) * mu_ref) <= 1e-5
+    var_ref = 1.0 / np.asarray(rsig_ref, np.float64) ** 2 - 1e-5
+    assert U.normwise(U.to_host(rv), 0.9 * 1.5 + 0.1 * var_ref) <= 1e-4
+
+
+def test_an_input_holding_the_unset_pattern_does_not_stall_the_exchange(K):
+    """0xffffffff is a NaN; summed into a partial it would equal the pattern that marks a
+    slot as not yet published, and every peer would wait out its patience. Partials are
+    published as the canonical NaN instead: the poisoned unit is NaN as the CPU kernels
+    make it, the others are untouched, and nothing had to be repaired."""
+    import torch
+    K.exchange_reset(0)
+    N, C, S = 8, 40, 56 * 56
+    t = {}
+    want = _bn_forward(K, t)
+    xp = t["x"].clone()
+    xp.view(torch.int32)[3, 7, 1234] = -1  # 0xffffffff in channel 7
+    y, mu, rsig, params, rm, rv = _bn_forward(K, dict(t, x=xp))
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    assert bool(torch.isnan(y[:, 7]).all()) and bool(torch.isnan(mu[7])) and bool(torch.isnan(rm[7]))
+    clean = [c for c in range(C) if c != 7]
+    assert torch.equal(y[:, clean], want[0][:, clean]) and torch.equal(mu[clean], want[1][clean])
+    # backward, the pattern in dy
+    tb = {}
+    wantb = _bn_backward(K, tb)
+    dyp = tb["dy"].clone()
+    dyp.view(torch.int32)[0, 0, 0] = -1
+    dx, wg = _bn_backward(K, dict(tb, dy=dyp))
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    assert bool(torch.isnan(dx[:, 0]).all()) and torch.equal(dx[:, 1:], wantb[0][:, 1:])
+    # softmax rows held by several workgroups, fp32 (the exchanged pair is maximum and sum)
+    ts = {}
+    wants = _softmax_in_place(K, ts)
+    xs = ts["x"].clone()
+    xs.view(torch.int32)[2, 70000] = -1
+    (ys,) = _softmax_in_place(K, dict(ts, x=xs))
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    assert bool(torch.isnan(ys[2]).all())
+    rows = [0, 1, 3, 4, 5]
+    assert torch.equal(ys[rows], wants[0][rows])
+
+
+def test_batch_norm_backward_of_channels_beyond_the_grid(K):
+    """fp32 [768, 4, 112, 112]: 9.6 M elements per channel would be 784 slices of the
+    backward's twelve packets per thread, more than the 768 workgroups of its grid, and a
+    workgroup would hold two slices of one channel and wait for itself. Such shapes are
+    left to the split path."""
+    import torch
+    shape = (768, 4, 112, 112)
+    N, C, S = shape[0], shape[1], shape[2] * shape[3]
+    plan = K.exchange_plan("float32", C, N, S, 2)
+    assert plan is None or plan[0] <= plan[3]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(9)
+    x = torch.empty(shape, device="cuda").normal_(generator=gen).mul_(2).add_(0.5)
+    dy = torch.empty(shape, device="cuda").normal_(generator=gen)
+    g = torch.rand(C, device="cuda", generator=gen) + 0.5
+    x64, dy64 = x.double(), dy.double()
+    mu64 = x64.mean((0, 2, 3))
+    rsig64 = torch.rsqrt(x64.var((0, 2, 3), unbiased=False) + 1e-5)
+    mu, rsig = mu64.float(), rsig64.float()
+    wg, dx = torch.empty(2 * C, device="cuda"), torch.empty_like(x)
+    K.exchange_reset(0)
+    K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", x, mu, rsig, g, dy, wg, wg, dx)
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    # fp64 closed form (the reference's own tests spell it out, test_ops.py:4127-4181)
+    xh = (x64 - mu.double()[None, :, None, None]) * rsig.double()[None, :, None, None]
+    dg64 = (dy64 * xh).sum((0, 2, 3))
+    db64 = dy64.sum((0, 2, 3))
+    M = float(N * S)
+    dx64 = (g.double() * rsig.double())[None, :, None, None] * (
+        dy64 - (xh * dg64[None, :, None, None] + db64[None, :, None, None]) / M)
+    assert float((dx.double() - dx64).abs().max() / dx64.abs().max()) <= 1e-5
+    assert float((wg[:C].double() - dg64).abs().max() / dg64.abs().max()) <= 2e-5
+    assert float((wg[C:].double() - db64).abs().max() / db64.abs().max().clamp_min(1.0)) <= 2e-5
+    # and the oracle on a slice of the batch small enough for one CPU thread
+    n = 24
+    xs, dys = x[:n].cpu().numpy(), dy[:n].cpu().numpy()
+    mus, rss = xs.mean((0, 2, 3), dtype=np.float64), None
+    rss = 1.0 / np.sqrt(xs.var((0, 2, 3), dtype=np.float64) + 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_train_grad(
+        "float32", xs, g.cpu().numpy(), dys, mus.astype(np.float32), rss.astype(np.float32), 1)
+    wg2, dx2 = torch.empty(2 * C, device="cuda"), torch.empty((n,) + shape[1:], device="cuda")
+    K.batch_norm_training_backward(n, C, S, float(n * S), "NCHW", x[:n].contiguous(),
+                                   torch.from_numpy(mus.astype(np.float32)).cuda(),
+                                   torch.from_numpy(rss.astype(np.float32)).cuda(), g,
+                                   dy[:n].contiguous(), wg2, wg2, dx2)
+    assert U.normwise(U.to_host(dx2), dx_ref) <= 1e-5
+    assert U.normwise(U.to_host(wg2)[:C], dg_ref) <= 2e-5
