@@ -104,6 +104,9 @@ SIGNATURES = {
     "dragon_hip_batch_norm_training_backward": (_int, [_int, _i64, _i64, _i64, _f32, _int, _vp, _vp,
                                                        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz,
                                                        _vp]),
+    "dragon_hip_batch_norm_training_forward_noalloc": (_int, [_int, _i64, _i64, _i64, _int, _f32,
+                                                              _f32, _vp, _vp, _vp, _vp, _vp, _vp,
+                                                              _vp, _vp, _vp, _vp]),
     "dragon_hip_exchange_timed_out": (_int, []),
     "dragon_hip_exchange_reset": (None, [ctypes.c_uint]),
     "dragon_hip_exchange_plan": (_int, [_int, _i64, _i64, _i64, _int] + [ctypes.POINTER(_int)] * 4),

@@ -30,6 +30,13 @@
 #include "short_rows.h"
 #include "slices.h"
 
+// Scratch of dragon_hip_batch_norm_training_forward_noalloc: device memory that
+// exists from the moment the library is loaded, so the entry point never
+// allocates. Every device that runs the library holds its own copy at its own
+// address; in host code the name below is a stand-in for the symbol, not a
+// device address, and only static_scratch_on_current_device() may mention it.
+static __device__ __align__(256) unsigned char scratch[DRAGON_HIP_STATIC_SCRATCH_BYTES];
+
 namespace dragon_hip {
 namespace {
 
@@ -804,6 +811,24 @@ int exchange_plan_of(const SliceUnits& u, int tensors, int* slices, int* slice_p
   return 1;
 }
 
+// The device address of the static array on the current device, resolved on
+// the first call on that device and kept per device.
+int static_scratch_on_current_device(void** ptr) {
+  static std::atomic<void*> resolved[kMaxDevices];
+  int device = 0;
+  const hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (device < 0 || device >= kMaxDevices) return DRAGON_HIP_EINVAL;
+  void* p = resolved[device].load(std::memory_order_acquire);
+  if (!p) {
+    const hipError_t g = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (g != hipSuccess) return static_cast<int>(g);
+    resolved[device].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return DRAGON_HIP_OK;
+}
+
 } // namespace
 } // namespace dragon_hip
 
@@ -986,6 +1011,28 @@ int dragon_hip_batch_norm_training_forward(int dtype, int64_t N, int64_t C, int6
   hipStream_t s = static_cast<hipStream_t>(stream);
   DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_training_forward, sh, momentum, eps, x, gamma,
                             beta, running_mean, running_var, mu, rsig, params, y, scratch, s);
+}
+
+int dragon_hip_batch_norm_training_forward_noalloc(int dtype, int64_t N, int64_t C, int64_t S,
+                                                   int layout, float momentum, float eps,
+                                                   const void* x, const void* gamma,
+                                                   const void* beta, void* running_mean,
+                                                   void* running_var, void* mu, void* rsig,
+                                                   void* params, void* y, void* stream) {
+  ChannelShape sh;
+  const int st = dragon_hip::make_shape(N, C, S, layout, &sh);
+  if (st != DRAGON_HIP_OK) return st;
+  if (N * S == 0) return DRAGON_HIP_EINVAL;
+  if (dtype < DRAGON_HIP_F16 || dtype > DRAGON_HIP_F64) return DRAGON_HIP_EDTYPE;
+  if (dragon_hip::scratch_bytes_for(dtype, sh) > DRAGON_HIP_STATIC_SCRATCH_BYTES) {
+    return DRAGON_HIP_ELIMIT;
+  }
+  void* ptr = nullptr;  // the static array's address on this device; never the array's name
+  const int got = dragon_hip::static_scratch_on_current_device(&ptr);
+  if (got != DRAGON_HIP_OK) return got;
+  return dragon_hip_batch_norm_training_forward(dtype, N, C, S, layout, momentum, eps, x, gamma,
+                                                beta, running_mean, running_var, mu, rsig, params,
+                                                y, ptr, DRAGON_HIP_STATIC_SCRATCH_BYTES, stream);
 }
 
 } // extern "C"

@@ -47,6 +47,8 @@ const char* dragon_hip_status_string(int status) {
     case DRAGON_HIP_ESCRATCH: return "scratch buffer missing or too small";
     case DRAGON_HIP_ENODEVICE: return "no HIP device";
     case DRAGON_HIP_ETIMEOUT: return "timed out (not returned by any entry point)";
+    case DRAGON_HIP_ELIMIT:
+      return "shape needs more scratch than the static buffer of the no-allocation entry point";
     default: break;
   }
   if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

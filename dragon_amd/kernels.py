@@ -323,6 +323,18 @@ def batch_norm_training_forward(N, C, S, data_format, momentum, epsilon, x, gamm
           _ptr(params), _ptr(y), _ptr(ws), need, _stream())
 
 
+STATIC_SCRATCH_BYTES = 4 << 20  # DRAGON_HIP_STATIC_SCRATCH_BYTES
+
+
+def batch_norm_training_forward_noalloc(N, C, S, data_format, momentum, epsilon, x, gamma, beta,
+                                        running_mean, running_var, mu, rsig, params, y):
+    """batch_norm_training_forward on the library's static scratch: allocates nothing."""
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    _call("dragon_hip_batch_norm_training_forward_noalloc", tag, N, C, S, lay, momentum, epsilon,
+          _ptr(x), _ptr(gamma), _ptr(beta), _ptr(running_mean), _ptr(running_var), _ptr(mu),
+          _ptr(rsig), _ptr(params), _ptr(y), _stream())
+
+
 def batch_norm_training_backward(N, C, S, normalizer, data_format, x, mu, rsig, gamma, dy, dgamma,
                                  dbeta, dx):
     """BatchNormWGrad + BatchNormTrainingGrad in one call (x and dy read once where a

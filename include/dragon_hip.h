@@ -59,7 +59,9 @@ typedef enum {
   DRAGON_HIP_EDTYPE = -2,   /* dtype not in dragon_hip_dtype                  */
   DRAGON_HIP_ESCRATCH = -3, /* scratch missing or too small                   */
   DRAGON_HIP_ENODEVICE = -4, /* no gfx950 device visible                      */
-  DRAGON_HIP_ETIMEOUT = -5  /* reserved: no entry point returns it             */
+  DRAGON_HIP_ETIMEOUT = -5, /* reserved: no entry point returns it             */
+  DRAGON_HIP_ELIMIT = -6    /* the shape needs more scratch than the static
+                               buffer of a *_noalloc entry point holds         */
 } dragon_hip_status;
 
 /* Human-readable text for a status returned by any function below. */
@@ -376,6 +378,26 @@ int dragon_hip_batch_norm_training_backward(int dtype, int64_t N, int64_t C, int
                                             const void* mu, const void* rsig, const void* gamma,
                                             const void* dy, void* dgamma, void* dbeta, void* dx,
                                             void* scratch, size_t scratch_bytes, void* stream);
+
+/* dragon_hip_batch_norm_training_forward for callers that cannot allocate
+ * device memory and have no workspace to pass: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc. No counterpart in the
+ * reference, whose operators always take scratch from the context's workspace.
+ * Same arguments without the scratch pair, same kernels, same results; the
+ * scratch is a static device array of DRAGON_HIP_STATIC_SCRATCH_BYTES inside
+ * the library (each device that runs the library holds it until the process
+ * ends). Shapes for which dragon_hip_batch_norm_reduce_scratch_bytes() exceeds
+ * that return DRAGON_HIP_ELIMIT and enqueue nothing. The call allocates and
+ * frees nothing on the device. All calls on one device share the one array:
+ * two calls that overlap in time on one device (different streams or threads)
+ * race on it and must be ordered by the caller. */
+#define DRAGON_HIP_STATIC_SCRATCH_BYTES (4u << 20)
+int dragon_hip_batch_norm_training_forward_noalloc(int dtype, int64_t N, int64_t C, int64_t S,
+                                                   int layout, float momentum, float eps,
+                                                   const void* x, const void* gamma,
+                                                   const void* beta, void* running_mean,
+                                                   void* running_var, void* mu, void* rsig,
+                                                   void* params, void* y, void* stream);
 
 /* The single-read paths (BatchNorm training forward / backward on NCHW with S
  * a whole number of 16-byte packets, GroupNorm groups beyond one workgroup,
