@@ -7,20 +7,35 @@ A step is one pass of the workload's kernels (forward then backward) over one
 batch of synthetic input that is already resident in HBM. The headline
 workload is Softmax forward+backward, fp16 I/O, [16, 32, 512, 512] along the
 last axis; `value` is its algorithmic bytes per step divided by the time per
-step. One JSON line is printed. It also carries
+step. One JSON line is printed.
+
+Cold and warm. The device has a 256 MB last-level cache in front of HBM, and a
+kernel re-run on the same tensors finds part of them there. Every workload is
+therefore built several times over (distinct tensor sets, as many as it takes
+for more than 1 GiB to be touched between two uses of a set) and the calls
+rotate over the sets: that is the *cold* figure, the one `value`, `roofline`
+and `frac_hbm_peak` quote. The *warm* figure (the same set again and again) is
+reported beside it.
+
   roofline      the dominant kernel of the headline workload against the
-                MI355X HBM peak of 8 TB/s (average launch duration measured
-                with events on the launch stream),
+                MI355X HBM peak of 8 TB/s: cold average launch duration from
+                events on the launch stream over the timed region, HBM traffic
+                from the hardware counters recorded under profiles/,
   cpu_baseline  the CPU oracle (a loop-for-loop port of the reference's CPU
                 kernels, single thread as the reference runs them) timed on the
                 same workload on the host cores,
-  kernels       the same per-kernel measurement for every workload of the
-                sweep (LayerNorm, GroupNorm, BatchNorm and the >= 8192x4096
-                target shapes).
+  kernels       per kernel of every workload of the sweep (the BASELINE
+                configs, the >= 8192x4096 target shapes, shapes at the ends of
+                the row-length range): cold mean / median / p10 / p90, warm mean,
+                GB/s, elements/s, fraction of the HBM peak, fraction of the
+                streaming probe with the kernel's read : write mix, and for the
+                BASELINE configs the CPU oracle's rate and the speed-up.
 """
 
 import argparse
+import glob
 import json
+import math
 import os
 import sys
 import time
@@ -30,14 +45,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE hardware counters, each
-# scaled by what it reads for the 1 GiB streaming-copy probe (figures and
-# commands: profiles/hbm_traffic_softmax_f16_16x32x512x512.txt).
-MEASURED_TRAFFIC_BYTES = {
-    ("softmax_f16_16x32x512x512", "softmax"): 536.9e6,
-    ("softmax_f16_16x32x512x512", "softmax_grad"): 805.4e6,
-}
+LLC_BYTES = 256 << 20  # last-level cache in front of HBM
+COLD_BYTES = 4 * LLC_BYTES  # bytes touched between two uses of a tensor set
 
 
 def parse_args():
@@ -47,14 +56,28 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="softmax_f16_16x32x512x512")
     ap.add_argument("--no-sweep", action="store_true", help="measure the headline workload only")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return ap.parse_args()
+
+
+def measured_traffic():
+    """{(workload, kernel): HBM bytes per launch} from the counter summaries under
+    profiles/ (lines `traffic_bytes <workload> <kernel> <bytes>`)."""
+    out = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "hbm_traffic_*.txt"))):
+        for line in open(path):
+            parts = line.lstrip("# ").split()
+            if len(parts) == 4 and parts[0] == "traffic_bytes":
+                out[(parts[1], parts[2])] = float(parts[3])
+    return out
 
 
 # ----------------------------------------------------------------------------
 # Workloads: synthetic inputs with the distributions and seeds of the configs,
 # generated on the device (the timed region starts with everything in HBM).
-# Each returns (kernels, meta): kernels = [(name, fn, algorithmic_bytes)].
+# Each factory takes the index of the tensor set (which only moves the seed)
+# and returns (kernels, meta): kernels = [(name, fn, algorithmic_bytes, mix)],
+# mix = the read : write ratio of the kernel ("1:1" or "2:1").
 # ----------------------------------------------------------------------------
 
 def _randn(shape, dtype, gen, scale=1.0, shift=0.0):
@@ -80,11 +103,11 @@ def _gen(seed):
     return g
 
 
-def wl_softmax(shape, dtype_name, seed=1):
+def wl_softmax(shape, dtype_name, seed=1, k=0):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     C = shape[-1]
     N = 1
     for d in shape[:-1]:
@@ -98,34 +121,34 @@ def wl_softmax(shape, dtype_name, seed=1):
     y, dx = torch.empty_like(x), torch.empty_like(x)
     nbytes = x.numel() * x.element_size()
     kernels = [
-        ("softmax", lambda: K.softmax(N, 1, C, x, y), 2 * nbytes),
-        ("softmax_grad", lambda: K.softmax_grad(N, 1, C, dy, y, dx), 3 * nbytes),
+        ("softmax", lambda: K.softmax(N, 1, C, x, y), 2 * nbytes, "1:1"),
+        ("softmax_grad", lambda: K.softmax_grad(N, 1, C, dy, y, dx), 3 * nbytes, "2:1"),
     ]
-    return kernels, {"rows": N, "width": C, "tensors": (x, dy, y, dx)}
+    return kernels, {"rows": N, "width": C}
 
 
-def wl_lp_norm(N, C, dtype_name, p=2, seed=5):
+def wl_lp_norm(N, C, dtype_name, p=2, seed=5, k=0):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     x = _randn((N, C), dtype, gen)
     dy = _randn((N, C), dtype, gen)
     y, dx = torch.empty_like(x), torch.empty_like(x)
     nbytes = x.numel() * x.element_size()
     fwd, bwd = (K.l1_norm, K.l1_norm_grad) if p == 1 else (K.l2_norm, K.l2_norm_grad)
     kernels = [
-        ("l%d_norm" % p, lambda: fwd(N, 1, C, 1.0, 1e-12, x, y), 2 * nbytes),
-        ("l%d_norm_grad" % p, lambda: bwd(N, 1, C, 1.0, 1e-12, dy, x, dx), 3 * nbytes),
+        ("l%d_norm" % p, lambda: fwd(N, 1, C, 1.0, 1e-12, x, y), 2 * nbytes, "1:1"),
+        ("l%d_norm_grad" % p, lambda: bwd(N, 1, C, 1.0, 1e-12, dy, x, dx), 3 * nbytes, "2:1"),
     ]
     return kernels, {"rows": N, "width": C}
 
 
-def wl_softmax_cross_entropy(N, C, seed=6):
+def wl_softmax_cross_entropy(N, C, seed=6, k=0):
     """fp32 logits [N, C], int64 class indices, VALID reduction, 1 in 16 targets ignored."""
     import torch
     from dragon_amd import kernels as K
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     x = _randn((N, C), torch.float32, gen, scale=2.0)
     target = torch.randint(0, C, (N,), generator=gen, device="cuda", dtype=torch.int64)
     target[::16] = 255 if C > 255 else -1
@@ -136,19 +159,19 @@ def wl_softmax_cross_entropy(N, C, seed=6):
     kernels = [
         ("softmax_cross_entropy_loss_forward",
          lambda: K.softmax_cross_entropy_loss_forward(N, 1, C, ignore, "valid", x, target, prob, loss),
-         2 * nbytes + N * 8),
+         2 * nbytes + N * 8, "1:1"),
         ("softmax_cross_entropy_loss_backward",
          lambda: K.softmax_cross_entropy_loss_backward(N, 1, C, ignore, "valid", prob, target, dl, dx),
-         2 * nbytes + N * 8),
+         2 * nbytes + N * 8, "1:1"),
     ]
     return kernels, {"rows": N, "width": C}
 
 
-def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False):
+def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False, k=0):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     x = _randn((N, C), torch.float32, gen)
     if outliers:
         m = torch.empty((N, C), device="cuda").uniform_(generator=gen) < 0.01
@@ -160,7 +183,7 @@ def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False):
     mu, rsig = torch.empty(N, device="cuda"), torch.empty(N, device="cuda")
     nbytes = x.numel() * x.element_size()
     kernels = [("layer_norm", lambda: K.layer_norm(N, C, 1e-5, x, g, b, mu, rsig, y),
-                2 * nbytes + 2 * C * 4 + 2 * N * 4)]
+                2 * nbytes + 2 * C * 4 + 2 * N * 4, "1:1")]
     if backward:
         dy = _randn((N, C), dtype, gen)
         dx = torch.empty_like(x)
@@ -169,15 +192,15 @@ def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False):
         kernels.append(("layer_norm_grad",
                         lambda: K.group_norm_grad(N, 1, C, 1, "NHWC", x, mu, rsig, g, dy, params,
                                                   params, dg, db, dx),
-                        3 * nbytes + C * 4 + 2 * N * 4 + 2 * C * 4))
+                        3 * nbytes + C * 4 + 2 * N * 4 + 2 * C * 4, "2:1"))
     return kernels, {"rows": N, "width": C}
 
 
-def wl_group_norm(shape, G, dtype_name, seed=3):
+def wl_group_norm(shape, G, dtype_name, seed=3, k=0):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     N, C = shape[0], shape[1]
     S = 1
     for d in shape[2:]:
@@ -193,19 +216,20 @@ def wl_group_norm(shape, G, dtype_name, seed=3):
     nbytes = x.numel() * x.element_size()
     kernels = [
         ("group_norm_forward",
-         lambda: K.group_norm_forward(N, G, D, S, "NCHW", 1e-5, x, g, b, mu, rsig, y), 2 * nbytes),
+         lambda: K.group_norm_forward(N, G, D, S, "NCHW", 1e-5, x, g, b, mu, rsig, y), 2 * nbytes,
+         "1:1"),
         ("group_norm_grad",
          lambda: K.group_norm_grad(N, G, D, S, "NCHW", x, mu, rsig, g, dy, params, params, dg, db, dx),
-         3 * nbytes),
+         3 * nbytes, "2:1"),
     ]
     return kernels, {"shape": list(shape), "groups": G}
 
 
-def wl_batch_norm(shape, dtype_name, seed=2):
+def wl_batch_norm(shape, dtype_name, seed=2, k=0):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
-    gen = _gen(seed)
+    gen = _gen(seed + 1000 * k)
     N, C = shape[0], shape[1]
     S = 1
     for d in shape[2:]:
@@ -225,125 +249,248 @@ def wl_batch_norm(shape, dtype_name, seed=2):
     kernels = [
         ("batch_norm_training_forward",
          lambda: K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, x, g, b, rm, rv, mu, rsig,
-                                               params, y), 2 * nbytes),
-        ("batch_norm_training_backward", backward, 3 * nbytes),
+                                               params, y), 2 * nbytes, "1:1"),
+        ("batch_norm_training_backward", backward, 3 * nbytes, "2:1"),
     ]
     return kernels, {"shape": list(shape)}
 
 
 WORKLOADS = {
     # BASELINE configs
-    "softmax_f16_16x32x512x512": lambda: wl_softmax((16, 32, 512, 512), "float16", 1),
-    "layer_norm_f32_8192x1024_fwd": lambda: wl_layer_norm(8192, 1024, "float32", 0, backward=False),
-    "batch_norm_f32_64x256x56x56": lambda: wl_batch_norm((64, 256, 56, 56), "float32", 2),
-    "group_norm_bf16_32x512x64x64_g32": lambda: wl_group_norm((32, 512, 64, 64), 32, "bfloat16", 3),
-    "layer_norm_bf16_8192x12288": lambda: wl_layer_norm(8192, 12288, "bfloat16", 4, outliers=True),
-    "layer_norm_bf16_65536x1000": lambda: wl_layer_norm(65536, 1000, "bfloat16", 4, outliers=True),
+    "softmax_f16_16x32x512x512": lambda k: wl_softmax((16, 32, 512, 512), "float16", 1, k=k),
+    "layer_norm_f32_8192x1024_fwd": lambda k: wl_layer_norm(8192, 1024, "float32", 0, backward=False, k=k),
+    "batch_norm_f32_64x256x56x56": lambda k: wl_batch_norm((64, 256, 56, 56), "float32", 2, k=k),
+    "group_norm_bf16_32x512x64x64_g32": lambda k: wl_group_norm((32, 512, 64, 64), 32, "bfloat16", 3, k=k),
+    "layer_norm_bf16_8192x12288": lambda k: wl_layer_norm(8192, 12288, "bfloat16", 4, outliers=True, k=k),
+    "layer_norm_bf16_65536x1000": lambda k: wl_layer_norm(65536, 1000, "bfloat16", 4, outliers=True, k=k),
     # target shapes (>= 8192 x 4096)
-    "layer_norm_bf16_8192x4096": lambda: wl_layer_norm(8192, 4096, "bfloat16", 4),
-    "layer_norm_f32_8192x4096": lambda: wl_layer_norm(8192, 4096, "float32", 4),
-    "softmax_f16_8192x4096": lambda: wl_softmax((8192, 4096), "float16", 1),
-    "softmax_f32_8192x4096": lambda: wl_softmax((8192, 4096), "float32", 1),
+    "layer_norm_bf16_8192x4096": lambda k: wl_layer_norm(8192, 4096, "bfloat16", 4, k=k),
+    "layer_norm_f32_8192x4096": lambda k: wl_layer_norm(8192, 4096, "float32", 4, k=k),
+    "softmax_f16_8192x4096": lambda k: wl_softmax((8192, 4096), "float16", 1, k=k),
+    "softmax_f32_8192x4096": lambda k: wl_softmax((8192, 4096), "float32", 1, k=k),
     # sibling row reductions on the same skeleton
-    "softmax_cross_entropy_f32_8192x4096": lambda: wl_softmax_cross_entropy(8192, 4096),
-    "l2_norm_bf16_8192x4096": lambda: wl_lp_norm(8192, 4096, "bfloat16", 2),
-    "l2_norm_f32_8192x4096": lambda: wl_lp_norm(8192, 4096, "float32", 2),
+    "softmax_cross_entropy_f32_8192x4096": lambda k: wl_softmax_cross_entropy(8192, 4096, k=k),
+    "l2_norm_bf16_8192x4096": lambda k: wl_lp_norm(8192, 4096, "bfloat16", 2, k=k),
+    "l2_norm_f32_8192x4096": lambda k: wl_lp_norm(8192, 4096, "float32", 2, k=k),
     # shapes at the ends of the row-length range: attention rows of a vision transformer,
     # per-head normalisation, vocabulary-sized logits
-    "softmax_bf16_605184x197": lambda: wl_softmax((605184, 197), "bfloat16", 1),
-    "layer_norm_bf16_1048576x64": lambda: wl_layer_norm(1048576, 64, "bfloat16", 4),
-    "softmax_f32_2048x128256": lambda: wl_softmax((2048, 128256), "float32", 1),
+    "softmax_bf16_605184x197": lambda k: wl_softmax((605184, 197), "bfloat16", 1, k=k),
+    "layer_norm_bf16_1048576x64": lambda k: wl_layer_norm(1048576, 64, "bfloat16", 4, k=k),
+    "softmax_f32_2048x128256": lambda k: wl_softmax((2048, 128256), "float32", 1, k=k),
 }
 
 
-def time_calls(fn, steps, warmup):
-    """Average milliseconds per call of fn over `steps` calls, events on the launch stream."""
+def build_sets(name):
+    """The workload's tensor sets: enough of them that more than COLD_BYTES are touched
+    between two uses of a set even when only its smallest kernel is being timed."""
     import torch
-    for _ in range(warmup):
-        fn()
+    first = WORKLOADS[name](0)
+    smallest = min(k[2] for k in first[0])
+    count = max(2, min(24, int(math.ceil(COLD_BYTES / smallest)) + 1))
+    sets = [first] + [WORKLOADS[name](k) for k in range(1, count)]
+    for kernels, _ in sets:  # backward kernels read what the forward of their set wrote
+        for _, fn, _, _ in kernels:
+            fn()
+    torch.cuda.synchronize()
+    return sets
+
+
+def time_calls(fns, steps, warmup):
+    """fns[i % len(fns)] is call i. Returns (mean ms over `steps` calls from one pair of
+    events around the region, sorted per-call ms from an event between any two calls);
+    events are recorded on the stream the kernels are launched on."""
+    import torch
+    n = len(fns)
+    for i in range(max(warmup, n)):
+        fns[i % n]()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
-    for _ in range(steps):
-        fn()
+    for i in range(steps):
+        fns[i % n]()
     stop.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / steps
+    mean = start.elapsed_time(stop) / steps
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    marks[0].record()
+    for i in range(steps):
+        fns[i % n]()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    return mean, each
+
+
+def _pct(sorted_values, q):
+    return sorted_values[min(len(sorted_values) - 1, int(q * len(sorted_values)))]
 
 
 def measure_workload(name, steps, warmup):
     import torch
-    kernels, meta = WORKLOADS[name]()
+    sets = build_sets(name)
+    meta = sets[0][1]
+    elems = 1
+    for d in meta.get("shape", (meta.get("rows", 1), meta.get("width", 1))):
+        elems *= d
     per_kernel = []
-    for kname, fn, nbytes in kernels:
-        ms = time_calls(fn, steps, warmup)
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        elems = 1
-        for d in meta.get("shape", (meta.get("rows", 1), meta.get("width", 1))):
-            elems *= d
-        per_kernel.append({"workload": name, "kernel": kname, "us": round(ms * 1e3, 2),
-                           "algorithmic_bytes": nbytes, "GB/s": round(gbs, 1),
-                           "Gelem/s": round(elems / (ms * 1e-3) / 1e9, 1),
-                           "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
+    for j, (kname, _, nbytes, mix) in enumerate(sets[0][0]):
+        cold_mean, cold_each = time_calls([s[0][j][1] for s in sets], steps, warmup)
+        warm_mean, _ = time_calls([sets[0][0][j][1]], steps, warmup)
+        gbs = nbytes / (cold_mean * 1e-3) / 1e9
+        warm_gbs = nbytes / (warm_mean * 1e-3) / 1e9
+        per_kernel.append({
+            "workload": name, "kernel": kname, "mix": mix, "tensor_sets": len(sets),
+            "us": round(cold_mean * 1e3, 2),
+            "us_median": round(_pct(cold_each, 0.5) * 1e3, 2),
+            "us_p10": round(_pct(cold_each, 0.1) * 1e3, 2),
+            "us_p90": round(_pct(cold_each, 0.9) * 1e3, 2),
+            "algorithmic_bytes": nbytes, "GB/s": round(gbs, 1),
+            "Gelem/s": round(elems / (cold_mean * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "warm_us": round(warm_mean * 1e3, 2),
+            "frac_hbm_peak_warm": round(warm_gbs / HBM_PEAK_GBS, 4)})
 
-    def step():
-        for _, fn, _ in kernels:
+    def step(i):
+        for _, fn, _, _ in sets[i % len(sets)][0]:
             fn()
 
-    # the contract's timed region: W warm-up steps, then exactly K steps between syncs
-    for _ in range(warmup):
-        step()
+    # the contract's timed region: W warm-up steps, then exactly K steps between syncs,
+    # rotating over the tensor sets
+    for i in range(warmup):
+        step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
+    for i in range(steps):
+        step(i)
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / steps
-    total_bytes = sum(k[2] for k in kernels)
-    del kernels, meta
+    total_bytes = sum(k[2] for k in sets[0][0])
+    del sets
     torch.cuda.empty_cache()
     return per_kernel, ms_step, total_bytes
 
 
 def streaming_ceiling(steps, warmup):
-    """Achieved GB/s of plain streaming kernels over 1 GiB buffers (far beyond the
-    256 MB last-level cache): read only, copy (read + write bytes) and fill."""
+    """Achieved GB/s of plain streaming kernels over 1 GiB buffers of non-zero data (far
+    beyond the last-level cache): read only, copy, fill, and two reads with one write."""
     import torch
     from dragon_amd import kernels as K
     n = 1 << 30
-    a = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    a = torch.randint(1, 255, (2 * n,), dtype=torch.uint8, device="cuda")
     b = torch.empty(n, dtype=torch.uint8, device="cuda")
     out = {}
-    for name, mode, moved in (("read", 0, n), ("copy", 1, 2 * n), ("fill", 2, n)):
-        ms = time_calls(lambda: K.stream_probe(mode, a, b, n), steps, warmup)
+    for name, mode, moved in (("read", 0, n), ("copy", 1, 2 * n), ("fill", 2, n),
+                              ("two_reads_one_write", 3, 3 * n)):
+        ms, _ = time_calls([lambda: K.stream_probe(mode, a, b, n)], steps, warmup)
         out[name] = round(moved / (ms * 1e-3) / 1e9, 1)
     return out
 
 
-def cpu_baseline_softmax(shape, reps=3):
-    """Oracle Softmax + SoftmaxGrad (fp32 kernels on the fp16-rounded inputs) on the
-    full headline workload, single thread, median of `reps`."""
-    import numpy as np
-    from oracle import ref_cpu as R
-    C = shape[-1]
-    N = int(np.prod(shape[:-1]))
-    rng = np.random.default_rng(1)
-    x = (rng.standard_normal((N, C), dtype=np.float32) * 3)
-    x[rng.random((N, C), dtype=np.float32) < 0.05] = -1e4
-    x = R.from_bits(R.to_bits(x, "float16"), "float16")
-    dy = R.from_bits(R.to_bits(rng.standard_normal((N, C), dtype=np.float32), "float16"), "float16")
+# ----------------------------------------------------------------------------
+# CPU baseline: the oracle (a port of the reference's CPU kernels, one thread,
+# as the reference runs them) on the same seeded distributions, full size where
+# a pass takes about a second, otherwise on a stated share of the rows.
+# Returns {(workload, kernel): {"GB/s": ..., "sample": ...}} with the same
+# algorithmic bytes per element the GPU figure is quoted on.
+# ----------------------------------------------------------------------------
+
+def _timed(fn, reps):
     times = []
+    out = None
     for _ in range(reps):
         t0 = time.perf_counter()
-        y = R.softmax("float32", N, 1, C, x)
-        R.softmax_grad("float32", N, 1, C, dy, y)
+        out = fn()
         times.append(time.perf_counter() - t0)
-    t = sorted(times)[len(times) // 2]
-    nbytes_fp16 = 5 * N * C * 2  # the same algorithmic bytes the GPU number is quoted on
-    return {"value": round(nbytes_fp16 / t / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "host_cores": os.cpu_count(),
-            "sample": "full workload [%d, %d], Softmax+SoftmaxGrad fp32 oracle on fp16-rounded "
-                      "inputs, median of %d, %.2f s per pass" % (N, C, reps, t)}
+    return sorted(times)[len(times) // 2], out
+
+
+def cpu_baselines(reps=3):
+    import numpy as np
+    from oracle import ref_cpu as R
+    out = {}
+
+    def put(workload, kernel, nbytes, seconds, sample, passes=reps):
+        out[(workload, kernel)] = {"GB/s": round(nbytes / seconds / 1e9, 3),
+                                   "sample": "%s, median of %d, %.2f s per pass" % (sample, passes, seconds)}
+
+    def rounded(a, dtype):
+        return R.from_bits(R.to_bits(a, dtype), dtype)
+
+    # cfg 2: Softmax + SoftmaxGrad, fp32 kernels on the fp16-rounded inputs, a quarter of the rows
+    N, C = 16 * 32 * 512 // 4, 512
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((N, C), dtype=np.float32) * 3
+    x[rng.random((N, C), dtype=np.float32) < 0.05] = -1e4
+    x = rounded(x, "float16")
+    dy = rounded(rng.standard_normal((N, C), dtype=np.float32), "float16")
+    t_f, y = _timed(lambda: R.softmax("float32", N, 1, C, x), reps)
+    t_b, _ = _timed(lambda: R.softmax_grad("float32", N, 1, C, dy, y), reps)
+    name = "softmax_f16_16x32x512x512"
+    what = "%d of %d rows of %d, fp32 oracle on fp16-rounded inputs" % (N, 4 * N, C)
+    put(name, "softmax", 2 * N * C * 2, t_f, what)
+    put(name, "softmax_grad", 3 * N * C * 2, t_b, what)
+    del x, dy, y
+
+    # cfg 1: LayerNorm forward fp32, full size
+    N, C = 8192, 1024
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((N, C), dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    t, _ = _timed(lambda: R.layer_norm("float32", x, g, b, 1e-5), reps)
+    put("layer_norm_f32_8192x1024_fwd", "layer_norm", 2 * N * C * 4, t, "full [%d, %d] fp32" % (N, C))
+
+    # cfg 3: BatchNorm training forward + backward fp32 NCHW, full size
+    shape = (64, 256, 56, 56)
+    rng = np.random.default_rng(2)
+    x = (2 * rng.standard_normal(shape, dtype=np.float32) + 0.5).astype(np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, shape[1]).astype(np.float32)
+    b = (rng.standard_normal(shape[1]) * 0.1).astype(np.float32)
+    rm, rv = np.zeros(shape[1], np.float32), np.ones(shape[1], np.float32)
+    t_f, (y, mu, rsig, _) = _timed(
+        lambda: R.op_batch_norm_train("float32", x, g, b, rm.copy(), rv.copy(), 1, 0.9, 1e-5), 1)
+    t_b, _ = _timed(lambda: R.op_batch_norm_train_grad("float32", x, g, dy, mu, rsig, 1), 1)
+    name = "batch_norm_f32_64x256x56x56"
+    put(name, "batch_norm_training_forward", 2 * x.size * 4, t_f, "full %s fp32" % (list(shape),), 1)
+    put(name, "batch_norm_training_backward", 3 * x.size * 4, t_b, "full %s fp32" % (list(shape),), 1)
+    del x, dy, y
+
+    # cfg 4: GroupNorm bf16 NCHW, 32 groups: 4 of the 32 samples (the forward in the
+    # reference's software bf16, the backward as its fp32 kernel on the rounded inputs)
+    shape = (4, 512, 64, 64)
+    rng = np.random.default_rng(3)
+    xb = R.to_bits(rng.standard_normal(shape, dtype=np.float32), "bfloat16")
+    dyf = rounded(rng.standard_normal(shape, dtype=np.float32), "bfloat16")
+    g = rng.uniform(0.5, 1.5, shape[1]).astype(np.float32)
+    b = (rng.standard_normal(shape[1]) * 0.1).astype(np.float32)
+    t_f, (_, mu, rsig) = _timed(lambda: R.op_group_norm("bfloat16", xb, g, b, 1, 32, 1e-5), reps)
+    xf = R.from_bits(xb, "bfloat16")
+    t_b, _ = _timed(lambda: R.op_group_norm_grad("float32", xf, g, dyf, mu, rsig, 1, 32), reps)
+    name = "group_norm_bf16_32x512x64x64_g32"
+    put(name, "group_norm_forward", 2 * xb.size * 2, t_f, "4 of 32 samples, %s bf16" % (list(shape),))
+    put(name, "group_norm_grad", 3 * xb.size * 2, t_b,
+        "4 of 32 samples, %s, fp32 oracle on bf16-rounded inputs" % (list(shape),))
+    del xb, xf, dyf
+
+    # cfg 5: LayerNorm bf16 forward + backward on a share of the rows
+    for (rows, C, sample) in ((8192, 12288, 512), (65536, 1000, 4096)):
+        rng = np.random.default_rng(4)
+        x = rng.standard_normal((sample, C), dtype=np.float32)
+        x[rng.random((sample, C), dtype=np.float32) < 0.01] *= 50
+        xb = R.to_bits(x, "bfloat16")
+        dyf = rounded(rng.standard_normal((sample, C), dtype=np.float32), "bfloat16")
+        g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+        b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+        t_f, (_, mu, rsig) = _timed(lambda: R.layer_norm("bfloat16", xb, g, b, 1e-5), reps)
+        xf = R.from_bits(xb, "bfloat16")
+        t_b, _ = _timed(lambda: R.group_norm_grad("float32", sample, 1, C, 1, "NHWC", xf, mu, rsig, g,
+                                                  dyf), reps)
+        name = "layer_norm_bf16_%dx%d" % (rows, C)
+        put(name, "layer_norm", 2 * sample * C * 2, t_f, "%d of %d rows of %d, bf16" % (sample, rows, C))
+        put(name, "layer_norm_grad", 3 * sample * C * 2, t_b,
+            "%d of %d rows of %d, fp32 oracle on bf16-rounded inputs" % (sample, rows, C))
+    return out
 
 
 def main():
@@ -367,14 +514,29 @@ def main():
     if not args.no_sweep:
         for name in WORKLOADS:
             if name != head:
-                all_kernels += measure_workload(name, max(10, args.steps // 2), args.warmup)[0]
+                all_kernels += measure_workload(name, args.steps, args.warmup)[0]
     ceiling = streaming_ceiling(20, 5)
-    for k in all_kernels:  # the second denominator: an achieved 1:1 streaming copy on this device
-        k["frac_copy_probe"] = round(k["GB/s"] / ceiling["copy"], 3)
+    for k in all_kernels:  # the second denominator: an achieved streaming kernel of the same mix
+        probe = ceiling["copy"] if k["mix"] == "1:1" else ceiling["two_reads_one_write"]
+        k["frac_stream_probe"] = round(k["GB/s"] / probe, 3)
 
     cpu = None
-    if not args.no_cpu and head == "softmax_f16_16x32x512x512":
-        cpu = cpu_baseline_softmax((16, 32, 512, 512))
+    if not args.no_cpu:
+        cpus = cpu_baselines()
+        for k in all_kernels:
+            c = cpus.get((k["workload"], k["kernel"]))
+            if c:
+                k["cpu_GB/s"] = c["GB/s"]
+                k["cpu_sample"] = c["sample"]
+                k["speedup_vs_cpu"] = round(k["GB/s"] / c["GB/s"], 1)
+        mine = [cpus[(head, k["kernel"])] for k in per_kernel if (head, k["kernel"]) in cpus]
+        if len(mine) == len(per_kernel):
+            # the whole step on the CPU: total bytes over the summed pass times
+            secs = sum(k["algorithmic_bytes"] / (c["GB/s"] * 1e9) for k, c in zip(per_kernel, mine))
+            cpu = {"value": round(total_bytes / secs / 1e9, 3), "unit": "GB/s", "cores": 1,
+                   "kind": "port", "host_cores": os.cpu_count(),
+                   "sample": "; ".join("%s: %s" % (k["kernel"], c["sample"])
+                                       for k, c in zip(per_kernel, mine))}
 
     out = {
         "metric": "GB/s and % of HBM roofline per norm/softmax kernel; speedup vs host-CPU ref",
@@ -390,13 +552,15 @@ def main():
         "dtype": "f32",  # every reduction and the element-wise math run in fp32; I/O type is in config
         "data": "synthetic",
         "config": {"workload": head, "io_dtype": "f16" if "f16" in head else ("bf16" if "bf16" in head else "f32"),
-                   "step": "forward + backward, inputs resident in HBM",
+                   "step": "forward + backward, inputs resident in HBM, rotating over tensor sets "
+                           "so that no call finds its tensors in the last-level cache",
                    "algorithmic_bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "kernel": dominant["kernel"],
                      "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dominant["GB/s"] / HBM_PEAK_GBS, 4),
                      "avg_launch_us": dominant["us"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((head, dominant["kernel"])),
+                     "frac_warm": dominant["frac_hbm_peak_warm"],
+                     "traffic": measured_traffic().get((head, dominant["kernel"])),
                      "streaming_kernels_GB/s": ceiling},
         "cpu_baseline": cpu,
         "kernels": all_kernels,

@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     }
   } else {
     for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
-      staged[i] = load_packet(gamma + i * kPerPacket);
+      staged[i] = load_packet_keep(gamma + i * kPerPacket);
     }
   }
   __syncthreads();
@@ -623,7 +623,7 @@ __device__ __forceinline__ void load_run(const T* p, typename IO<T>::Acc (&v)[kW
   if constexpr (kW == 1) {
     v[0] = IO<T>::load1(p);
   } else {
-    IO<T>::unpack(load_packet(p), v);
+    IO<T>::unpack(load_packet_keep(p), v);
   }
 }
 template <int kW, typename A>
@@ -1674,8 +1674,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_batched_columns(
         x0[0] = IO<T>::load1(in0 + off);
         x1[0] = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
       } else {
-        load_unpack<T>(in0 + off, x0);
-        if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
+        load_unpack_keep<T>(in0 + off, x0);
+        if constexpr (kIn == 2) load_unpack_keep<T>(in1 + off, x1);
       }
 #pragma unroll
       for (int e = 0; e < kW; ++e) fs[e].add(x0[e], kIn == 2 ? x1[e] : A(0), a[e], b[e]);

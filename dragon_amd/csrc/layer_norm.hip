@@ -108,8 +108,8 @@ __global__ __launch_bounds__(kThreads) void layer_norm_wide_rows(
   A* lds_gamma = reinterpret_cast<A*>(staged);
   A* lds_beta = lds_gamma + C;
   for (int i = threadIdx.x; i < C / kPerPacket; i += kThreads) {
-    staged[i] = load_packet(gamma + i * kPerPacket);
-    staged[C / kPerPacket + i] = load_packet(beta + i * kPerPacket);
+    staged[i] = load_packet_keep(gamma + i * kPerPacket);
+    staged[C / kPerPacket + i] = load_packet_keep(beta + i * kPerPacket);
   }
   __syncthreads();
 

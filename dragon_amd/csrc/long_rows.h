@@ -61,8 +61,8 @@ __global__ __launch_bounds__(kLongThreads) void long_rows_sums(
 #pragma unroll 4
     for (int p = lane; p < sp.body; p += kWaveSize) {
       A x0[kVec], x1[kVec];
-      load_unpack<T>(r0 + sp.head + p * kVec, x0);
-      if constexpr (kIn == 2) load_unpack<T>(r1 + sp.head + p * kVec, x1);
+      load_unpack_keep<T>(r0 + sp.head + p * kVec, x0);
+      if constexpr (kIn == 2) load_unpack_keep<T>(r1 + sp.head + p * kVec, x1);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) op.add(w, x0[e], kIn == 2 ? x1[e] : A(0), a, b);
     }

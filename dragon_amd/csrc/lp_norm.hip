@@ -281,8 +281,8 @@ __global__ __launch_bounds__(256) void lp_norm_columns(
         v[0] = IO<T>::load1(x + base + k * S);
         if (kGrad) g[0] = IO<T>::load1(dy + base + k * S);
       } else {
-        load_unpack<T>(x + base + k * S, v);
-        if (kGrad) load_unpack<T>(dy + base + k * S, g);
+        load_unpack_keep<T>(x + base + k * S, v);
+        if (kGrad) load_unpack_keep<T>(dy + base + k * S, g);
       }
 #pragma unroll
       for (int e = 0; e < kW; ++e) {

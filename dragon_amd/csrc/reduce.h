@@ -105,8 +105,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_segments(
       x0[0] = IO<T>::load1(in0 + off);
       x1[0] = kIn == 2 ? IO<T>::load1(in1 + off) : A(0);
     } else {
-      load_unpack<T>(in0 + off, x0);
-      if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
+      load_unpack_keep<T>(in0 + off, x0);
+      if constexpr (kIn == 2) load_unpack_keep<T>(in1 + off, x1);
     }
     f.add(o, seg, p, off, x0, x1, a, b);
   }
@@ -207,8 +207,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_columns_packets(
          r += d.split * kReduceWaves * rows_per_wave) {
       const uint32_t off = r * d.cols + c0;
       A x0[kVec], x1[kVec];
-      load_unpack<T>(in0 + off, x0);
-      if constexpr (kIn == 2) load_unpack<T>(in1 + off, x1);
+      load_unpack_keep<T>(in0 + off, x0);
+      if constexpr (kIn == 2) load_unpack_keep<T>(in1 + off, x1);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
         fs[e].add(r, c0 + e, off + e, x0[e], kIn == 2 ? x1[e] : A(0), a[e], b[e]);

@@ -70,12 +70,14 @@ struct StagedRange {
 // Copies the packets of `r` into stage[0 .. r.packets). A packet that reaches
 // outside the tensor (only the tensor's first or last can) is read element by
 // element; what lies outside reads as zero.
-template <typename T>
+// kStream: the tensor is read once and not again soon (non-temporal loads).
+template <typename T, bool kStream>
 __device__ __forceinline__ void stage_in(const StagedRange& r, u32x4* stage) {
   for (uint32_t p = threadIdx.x; p < r.packets; p += kShortThreads) {
     const uintptr_t addr = r.first + 16u * p;
     if (addr >= r.base && addr + 16 <= r.base + r.total) {
-      stage[p] = *reinterpret_cast<const u32x4*>(addr);
+      stage[p] = kStream ? load_packet(reinterpret_cast<const T*>(addr))
+                         : load_packet_keep(reinterpret_cast<const T*>(addr));
     } else {
       T* out = reinterpret_cast<T*>(stage + p);
 #pragma unroll
@@ -174,10 +176,10 @@ __global__ __launch_bounds__(kShortThreads) void short_rows(
         for (int q = 0; q < kSide; ++q) side[i * kSide + q] = w[q];
       }
     }
-    stage_in<T>(r0, stage);
+    stage_in<T, !OpReadOnly<Op>::value>(r0, stage);
     if constexpr (Op::kIn == 2) {
       const StagedRange r1(in1, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-      stage_in<T>(r1, stage1);
+      stage_in<T, !OpReadOnly<Op>::value>(r1, stage1);
     }
     __syncthreads();
     T* tile0 = reinterpret_cast<T*>(reinterpret_cast<char*>(stage) + r0.lead());

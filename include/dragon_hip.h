@@ -431,10 +431,13 @@ int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seg
 
 /* ------------------------------------------------------------------------ */
 /* Measurement utility (no counterpart in the reference): a streaming read    */
-/* (mode 0: dst receives at most one word), copy (mode 1) or fill (mode 2) of */
-/* `bytes` bytes (a multiple of 16, 16-byte aligned buffers) with 128-bit      */
-/* accesses. Gives the achieved streaming ceiling of the device and a         */
-/* known-size kernel for calibrating profiler byte counters.                  */
+/* (mode 0: dst receives at most one word), copy (mode 1), fill (mode 2) or    */
+/* two reads and one write (mode 3: src holds two tensors of `bytes` bytes     */
+/* back to back, dst their xor) of `bytes` bytes (a multiple of 16, 16-byte    */
+/* aligned buffers) with 128-bit accesses, several in flight per thread.       */
+/* Gives the achieved streaming ceiling of the device at the read : write      */
+/* mixes of the kernels here, and a known-size kernel for calibrating          */
+/* profiler byte counters.                                                     */
 /* ------------------------------------------------------------------------ */
 int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes, void* stream);
 
