@@ -56,6 +56,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="softmax_f16_16x32x512x512")
     ap.add_argument("--no-sweep", action="store_true", help="measure the headline workload only")
+    ap.add_argument("--sweep", default="", help="comma-separated workloads to sweep instead of all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return ap.parse_args()
 
@@ -512,7 +513,7 @@ def main():
     dominant = max(per_kernel, key=lambda k: k["us"])
     all_kernels = list(per_kernel)
     if not args.no_sweep:
-        for name in WORKLOADS:
+        for name in (args.sweep.split(",") if args.sweep else WORKLOADS):
             if name != head:
                 all_kernels += measure_workload(name, args.steps, args.warmup)[0]
     ceiling = streaming_ceiling(20, 5)

@@ -248,22 +248,24 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   // packets and the accumulators fit the register budget (128 per thread; 168
   // for the 768-thread workgroup, which runs three wavefronts per SIMD).
   constexpr int kDepth = (kVPT * kVec <= 8 || kGradThreads == 768) ? 2 : 1;
+  constexpr bool kSplit = !kRagged && kVec == 2 * kPerPacket;
   extern __shared__ u32x4 staged[];  // gamma[C]
   __shared__ A slots[2 * Tile::kSlots];
   __shared__ A red[kRedWords];
   const A* lds_gamma = reinterpret_cast<const A*>(staged);
+  const int npackets_of_row = (C + kVec - 1) / kVec;
+  // gamma of the kVec columns of packet `packet` of the row
+  auto gamma_of = [&](const int packet, A(&g)[kVec]) {
+    if constexpr (kSplit) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(lds_gamma + packet * 4);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(lds_gamma + (npackets_of_row + packet) * 4);
+      g[0] = lo.x, g[1] = lo.y, g[2] = lo.z, g[3] = lo.w;
+      g[4] = hi.x, g[5] = hi.y, g[6] = hi.z, g[7] = hi.w;
+    } else {
+      load_params<kVec>(lds_gamma + packet * kVec, g);
+    }
+  };
   const int npackets = (C + kVec - 1) / kVec;
-  if constexpr (kRagged) {
-    A* stage_gamma = reinterpret_cast<A*>(staged);
-    for (int i = threadIdx.x; i < npackets * kVec; i += kGradThreads) {
-      stage_gamma[i] = i < C ? gamma[i] : A(0);
-    }
-  } else {
-    for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
-      staged[i] = load_packet_keep(gamma + i * kPerPacket);
-    }
-  }
-  __syncthreads();
 
   const int lane = Tile::lane();
   const int sub = Tile::sub_row();
@@ -306,6 +308,24 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
 #pragma unroll
   for (int k = 0; k < kDepth; ++k) request(rx[k], rdy[k], rm[k], rr[k], row + k * stride);
 
+  // gamma is staged while the first rows travel
+  if constexpr (kRagged) {
+    A* stage_gamma = reinterpret_cast<A*>(staged);
+    for (int i = threadIdx.x; i < npackets * kVec; i += kGradThreads) {
+      stage_gamma[i] = i < C ? gamma[i] : A(0);
+    }
+  } else {
+    // Rows of 8-element packets against 4-float LDS words: the first halves of
+    // all packets, then the second halves, so that the lanes of a wavefront read
+    // adjacent 16-byte words (eight consecutive floats per lane put lanes l and
+    // l + 8 on the same banks: a two-way conflict on every access).
+    for (int i = threadIdx.x; i < C / kPerPacket; i += kGradThreads) {
+      const int at = kSplit ? (i & 1) * npackets + (i >> 1) : i;
+      staged[at] = load_packet_keep(gamma + i * kPerPacket);
+    }
+  }
+  __syncthreads();
+
   // One row: tx / tdy hold it, nx / ndy the row after it.
   auto step = [&](Raw& tx, Raw& tdy, const A m, const A r, Raw& nx, Raw& ndy) {
     const bool valid = row < N;
@@ -316,7 +336,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
         A xv[kVec], dv[kVec], g[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
-        load_params<kVec>(lds_gamma + (i * kTPR + lane) * kVec, g);
+        gamma_of(i * kTPR + lane, g);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
           const A t = g[e] * dv[e];
@@ -343,8 +363,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
         // A slot beyond the row reads gamma of column 0 .. kVec - 1: its dx is not stored.
-        const int col = Tile::active(i, npackets) ? (i * kTPR + lane) * kVec : 0;
-        load_params<kVec>(lds_gamma + col, g);
+        gamma_of(Tile::active(i, npackets) ? i * kTPR + lane : 0, g);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
           const A xc = xv[e] - m;
@@ -1857,6 +1876,88 @@ __global__ __launch_bounds__(1024) void sum_partial_rows(const uint32_t P, const
   }
 }
 
+// The same for rows of whole 16-byte packets (C even for fp32: a packet holds
+// the (dgamma, dbeta) pairs of two adjacent columns, or one pair of doubles).
+// A workgroup owns kLanes adjacent packets of every partial row; its
+// 1024 / kLanes lane groups take rows g, g + groups, ..., several loads in
+// flight per lane, and are added up through LDS in a fixed order. kLanes is 32
+// (512 contiguous bytes per row) for wide rows and 8 (one cache line) for
+// narrow ones, which would otherwise leave all but a few compute units idle.
+template <typename A, int kLanes>
+__global__ __launch_bounds__(1024) void sum_partial_rows_packets(const uint32_t P, const uint32_t C,
+                                                                 const A* __restrict__ partial,
+                                                                 A* __restrict__ dgamma,
+                                                                 A* __restrict__ dbeta) {
+  constexpr int kPer = 16 / sizeof(A);  // words per packet
+  constexpr int kGroups = 1024 / kLanes;
+  constexpr int kWords = kLanes * kPer;  // words of the result a workgroup owns
+  constexpr int kParts = 1024 / kWords < 8 ? 1024 / kWords : 8;
+  __shared__ A lds[kGroups][kWords];
+  __shared__ A parts[kParts][kWords];
+  const uint32_t lane = threadIdx.x % kLanes;
+  const uint32_t group = threadIdx.x / kLanes;
+  const uint32_t packets = 2 * C / kPer;
+  const uint32_t packet = blockIdx.x * kLanes + lane;
+  A acc[kPer];
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) acc[e] = A(0);
+  if (packet < packets) {
+    const A* col = partial + static_cast<size_t>(packet) * kPer;
+#pragma unroll 4
+    for (uint32_t p = group; p < P; p += kGroups) {
+      A v[kPer];
+      IO<A>::unpack(load_packet(col + static_cast<size_t>(p) * 2 * C), v);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) acc[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) lds[group][lane * kPer + e] = acc[e];
+  __syncthreads();
+  // kParts threads per word each add a run of the lane groups, then one thread adds the runs
+  if (threadIdx.x < kParts * kWords) {
+    const uint32_t w = threadIdx.x % kWords, part = threadIdx.x / kWords;
+    constexpr int kRun = kGroups / kParts;
+    A t = lds[part * kRun][w];
+#pragma unroll 8
+    for (int g = 1; g < kRun; ++g) t += lds[part * kRun + g][w];
+    parts[part][w] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < kWords) {
+    const uint32_t word = blockIdx.x * kWords + threadIdx.x;
+    A total = parts[0][threadIdx.x];
+#pragma unroll
+    for (int q = 1; q < kParts; ++q) total += parts[q][threadIdx.x];
+    if (word < 2 * C) {
+      if (word & 1) {
+        dbeta[word >> 1] = total;
+      } else {
+        dgamma[word >> 1] = total;
+      }
+    }
+  }
+}
+
+template <typename A>
+void launch_sum_partial_rows(uint32_t P, uint32_t C, const A* partial, A* dgamma, A* dbeta,
+                             hipStream_t stream) {
+  constexpr uint32_t kPer = 16 / sizeof(A);
+  const uint32_t packets = 2 * C / kPer;
+  if ((2 * C) % kPer != 0 || !aligned16(partial)) {
+    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * C, kWaveSize))),
+                       dim3(1024), 0, stream, P, C, partial, dgamma, dbeta);
+  } else if (packets >= 32 * 64) {
+    hipLaunchKernelGGL((sum_partial_rows_packets<A, 32>),
+                       dim3(static_cast<unsigned>(ceil_div(packets, 32))), dim3(1024), 0, stream, P,
+                       C, partial, dgamma, dbeta);
+  } else {
+    hipLaunchKernelGGL((sum_partial_rows_packets<A, 8>),
+                       dim3(static_cast<unsigned>(ceil_div(packets, 8))), dim3(1024), 0, stream, P, C,
+                       partial, dgamma, dbeta);
+  }
+}
+
 struct RowGradPlan {
   bool use_rows;
   RowConfig cfg;
@@ -2314,8 +2415,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     DRAGON_HIP_SHORT_LAUNCH(T, LayerNormShortBackward, sp, lds, grid, stream, rows,
                             static_cast<int>(sh.D), xp, dyp, dxp, A(1) / A(sh.D), mup, rsp, gp, dsp,
                             dbp, part, {}, {}, {});
-    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
-                       dim3(1024), 0, stream, grid, sh.D, part, dgp, dbtp);
+    launch_sum_partial_rows<A>(grid, sh.D, part, dgp, dbtp, stream);
     return status_of_launch();
   }
 
@@ -2362,8 +2462,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     else LAUNCH(1024, 4)
 #undef LAUNCH_T
 #undef LAUNCH
-    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
-                       dim3(1024), 0, stream, rp.grid, sh.D, part, dgp, dbtp);
+    launch_sum_partial_rows<A>(rp.grid, sh.D, part, dgp, dbtp, stream);
     return status_of_launch();
   }
 
@@ -2389,8 +2488,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          static_cast<int64_t>(sh.N), D, wp, xp, dyp, gp, mup, rsp, pairs, dsp, dbp,
                          dxp, rows);
     }
-    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.D, kWaveSize))),
-                       dim3(1024), 0, stream, wp.row_chunks, sh.D, rows, dgp, dbtp);
+    launch_sum_partial_rows<A>(wp.row_chunks, sh.D, rows, dgp, dbtp, stream);
     return status_of_launch();
   }
 
@@ -2425,8 +2523,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     else if (gcfg.tpr == 1024 && gcfg.vpt == 4) LAUNCH(1024, 4)
     else LAUNCH(1024, 8)
 #undef LAUNCH
-    hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * sh.C, kWaveSize))),
-                       dim3(1024), 0, stream, sh.N, sh.C, part, dgp, dbtp);
+    launch_sum_partial_rows<A>(sh.N, sh.C, part, dgp, dbtp, stream);
     return status_of_launch();
   }
 
