@@ -29,8 +29,11 @@
 //                                  form of test_ops.py:4480-4512
 //   f16 / bf16 conversions         exhaustive comparison against numpy float16 and
 //                                  a bit-level bf16 RNE over all 2^16 encodings
-//   running-stat update (axpby)    PARITY UNPINNED by any reference test; pinned
-//                                  only by the closed form rm*m + (1-m)*mu
+//   running-stat update (axpby)    the formula the reference states for its operator,
+//                                  running = momentum * running + (1 - momentum) * batch
+//                                  (dragon/python/core/ops/normalization_ops.py:36-39),
+//                                  with the biased batch variance of batch_norm_op.cc:60-63;
+//                                  no reference test asserts the running tensors
 //   batch_norm_expectation         PARITY UNPINNED by any reference test (SyncBN is
 //                                  never run multi-rank); checked against E[x], E[x^2]
 //
