@@ -1,120 +1,85 @@
 """HIP device utilities with the names and arguments of ``dragon.cuda``
 (dragon/python/core/device/cuda.py:23-277): stream objects, device queries,
-the default device and synchronisation, all over the C ABI of
-``libdragon_hip.so`` (include/dragon_hip.h). cuBLAS / cuDNN flag setters have
+the default device and synchronisation, over the compiled module of the host
+layer (``backend``: pybind11 bindings of HIPContext / HIPStream, the
+counterpart of dragon/modules/python/cuda.h). cuBLAS / cuDNN flag setters have
 no counterpart: this library has no vendor-library switches.
 """
 
-import ctypes
-
-from . import _lib
+from . import backend
 
 # The process-wide default device of ``dragon.device`` scopes
 # (dragon/python/core/framework/config.py): type "hip" with an index, or "cpu".
 _default = {"device_type": "cpu", "device_index": 0}
-_seeds = {}
-
-
-def _call(name, *args):
-    _lib.check(name, getattr(_lib.lib(), name)(*args))
 
 
 class Stream:
-    """A non-blocking HIP stream at the default priority (cuda.py:23-67)."""
+    """A non-blocking HIP stream at the default priority (cuda.py:23-67): the next
+    unused stream index of the calling thread's device objects."""
 
     def __init__(self, device_index=None):
         self.device_index = current_device() if device_index is None else int(device_index)
-        prev = current_device()
-        set_device(self.device_index)
-        handle = ctypes.c_void_p()
-        try:
-            _call("dragon_hip_stream_create", ctypes.byref(handle))
-        finally:
-            set_device(prev)
-        self._ptr = handle
+        self._impl = backend.HIPStream(self.device_index)
+
+    @property
+    def index(self):
+        """The stream index operators are run on (``Workspace.run_operator(..., stream=index)``)."""
+        return self._impl.index
 
     @property
     def ptr(self):
         """The ``hipStream_t`` as an integer."""
-        return self._ptr.value
+        return self._impl.ptr
 
     def query(self):
         """True when everything enqueued on the stream has finished."""
-        done = ctypes.c_int()
-        _call("dragon_hip_stream_query", self._ptr, ctypes.byref(done))
-        return bool(done.value)
+        return self._impl.Query()
 
     def synchronize(self):
-        _call("dragon_hip_stream_sync", self._ptr)
+        self._impl.Synchronize()
 
     def close(self):
-        if self._ptr is not None and self._ptr.value:
-            _call("dragon_hip_stream_destroy", self._ptr)
-        self._ptr = None
-
-    def __del__(self):
-        try:
-            self.close()
-        except Exception:
-            pass
+        """Streams belong to the thread's device objects and are destroyed with them."""
+        self._impl = None
 
 
 def is_available():
-    """True when the kernel library loads and sees at least one device (cuda.py:134-143)."""
+    """True when the compiled module loads and sees at least one device (cuda.py:134-143)."""
     try:
-        return get_device_count() > 0
-    except (OSError, _lib.DragonHipError):
+        return backend.hipIsDriverSufficient() and get_device_count() > 0
+    except (OSError, RuntimeError):
         return False
 
 
 def get_device_count():
-    n = ctypes.c_int()
-    _call("dragon_hip_device_count", ctypes.byref(n))
-    return n.value
+    return backend.hipGetDeviceCount()
 
 
 def current_device():
-    d = ctypes.c_int()
-    _call("dragon_hip_get_device", ctypes.byref(d))
-    return d.value
+    return backend.hipGetDevice()
 
 
 def set_device(device_index=0):
-    _call("dragon_hip_set_device", int(device_index))
+    backend.hipSetDevice(int(device_index))
 
 
 def get_device_name(device_index=None):
-    buf = ctypes.create_string_buffer(256)
-    idx = current_device() if device_index is None else int(device_index)
-    _call("dragon_hip_device_name", idx, buf, 256)
-    return buf.value.decode()
+    return backend.hipGetDeviceName(-1 if device_index is None else int(device_index))
 
 
 def get_device_capability(device_index=None):
     """(major, minor) of the device's ISA version, (9, 5) for gfx950 (cuda.py:82-99)."""
-    major, minor = ctypes.c_int(), ctypes.c_int()
-    idx = current_device() if device_index is None else int(device_index)
-    _call("dragon_hip_device_capability", idx, ctypes.byref(major), ctypes.byref(minor))
-    return major.value, minor.value
+    return backend.hipGetDeviceCapability(-1 if device_index is None else int(device_index))
 
 
-def memory_allocated(device_index=None):
-    """Bytes of device memory in use on the device (total minus free).
-
-    ``dragon.cuda.memory_allocated`` reports the workspace pool's own bytes
-    (cuda.py:146-169); this library keeps no pool, so the device-wide figure is
-    the closest observable.
-    """
-    prev = current_device()
-    if device_index is not None:
-        set_device(device_index)
-    free, total = ctypes.c_size_t(), ctypes.c_size_t()
-    try:
-        _call("dragon_hip_mem_info", ctypes.byref(free), ctypes.byref(total))
-    finally:
-        if device_index is not None:
-            set_device(prev)
-    return total.value - free.value
+def memory_allocated(device_index=None, workspace=None):
+    """Bytes of device memory held by the tensors of a workspace (cuda.py:146-169).
+    ``workspace`` is a ``runtime.Workspace``; without one the answer is 0 (this package
+    keeps no process-wide default workspace)."""
+    if workspace is None:
+        return 0
+    index = current_device() if device_index is None else int(device_index)
+    return workspace.memory_allocated("hip", index)
 
 
 def set_default_device(device_index=0):
@@ -130,19 +95,20 @@ def default_device():
 
 
 def set_random_seed(device_index=None, seed=3):
-    """Record the seed of a device's generator (cuda.py:248-262). No kernel on
-    this path draws random numbers; the value is kept for callers that query it."""
-    _seeds[current_device() if device_index is None else int(device_index)] = int(seed)
+    """The seed of a device's generator (cuda.py:248-262). No kernel on this path draws
+    random numbers; the device objects keep the value for operators that would."""
+    backend.hipSetRandomSeed(-1 if device_index is None else int(device_index), int(seed))
 
 
-def synchronize(device_index=None, stream_index=0):
-    """Wait for all work on a device (cuda.py:265-277). ``stream_index`` selects a
-    workspace stream in the reference; here every stream of the device is waited for."""
-    prev = current_device()
-    if device_index is not None:
-        set_device(device_index)
-    try:
-        _call("dragon_hip_device_sync")
-    finally:
-        if device_index is not None:
-            set_device(prev)
+def get_random_seed(device_index=None):
+    return backend.hipGetRandomSeed(-1 if device_index is None else int(device_index))
+
+
+def synchronize(device_index=None, stream_index=None):
+    """Wait for a workspace stream of a device (cuda.py:265-277), or for every stream of
+    the device when ``stream_index`` is None."""
+    index = -1 if device_index is None else int(device_index)
+    if stream_index is None:
+        backend.hipDeviceSynchronize(index)
+    else:
+        backend.hipStreamSynchronize(index, int(stream_index))

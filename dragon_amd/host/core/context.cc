@@ -34,7 +34,27 @@ void HipCheck(int status, const char* what) {
 
 // ---------------------------------------------------------------- HIPObjects
 
-HIPObjects::HIPObjects() {}
+HIPObjects::HIPObjects() {
+  for (int& seed : seeds_) seed = 3;  // DEFAULT_RNG_SEED of the reference's device objects
+}
+
+int HIPObjects::num_streams(int device_id) const {
+  CHECK(device_id >= 0 && device_id < kMaxDevices) << "\nBad device id: " << device_id;
+  const size_t n = streams_[device_id].size();
+  return n == 0 ? 1 : static_cast<int>(n);  // id 0, the default stream, always exists
+}
+
+void HIPObjects::SetRandomSeed(int device_id, int seed) {
+  CHECK(device_id >= 0 && device_id < kMaxDevices) << "\nBad device id: " << device_id;
+  seeds_[device_id] = seed;
+}
+
+int HIPObjects::GetRandomSeed(int device_id) const {
+  CHECK(device_id >= 0 && device_id < kMaxDevices) << "\nBad device id: " << device_id;
+  return seeds_[device_id];
+}
+
+void HIPObjects::SetDevice(int device_id) { HIP_CHECK(dragon_hip_set_device(device_id)); }
 
 HIPObjects::~HIPObjects() {
   for (int d = 0; d < kMaxDevices; ++d) {
@@ -161,6 +181,20 @@ HIPObjects& HIPContext::objects() {
   static thread_local HIPObjects objects;
   return objects;
 }
+
+HIPStream::HIPStream(int device_id) : device_id_(device_id) {
+  HIPObjects& objects = HIPContext::objects();
+  stream_id_ = objects.num_streams(device_id);
+  impl_ = objects.stream(device_id, stream_id_);
+}
+
+bool HIPStream::Query() {
+  int done = 0;
+  HIP_CHECK(dragon_hip_stream_query(impl_, &done));
+  return done != 0;
+}
+
+void HIPStream::Synchronize() { HIPContext::SynchronizeStream(impl_); }
 
 HIPDeviceGuard::HIPDeviceGuard(int new_id) : prev_id_(HIPContext::current_device()) {
   if (prev_id_ != new_id) HIP_CHECK(dragon_hip_set_device(new_id));

@@ -49,12 +49,19 @@ class HIPObjects {
   // non-blocking at the default priority on first use.
   void* stream(int device_id, int stream_id);
   Workspace* workspace(int device_id, int stream_id);
+  // How many stream ids of the device have been handed out (id 0 included).
+  int num_streams(int device_id) const;
+  // The seed operators created for the device start from (CUDAObjects::SetRandomSeed's role).
+  void SetRandomSeed(int device_id, int seed);
+  int GetRandomSeed(int device_id) const;
+  void SetDevice(int device_id);
 
   static constexpr int kMaxDevices = 16;
 
  private:
   vector<void*> streams_[kMaxDevices];
   vector<std::unique_ptr<Workspace>> workspaces_[kMaxDevices];
+  int seeds_[kMaxDevices];
 };
 
 class HIPContext {
@@ -100,6 +107,23 @@ class HIPContext {
  private:
   int device_id_, stream_id_ = 0;
   uint32_t random_seed_;
+};
+
+// A stream of the calling thread's device objects behind a handle that a front
+// end can hold (CUDAStream's role, dragon/core/context_cuda.h:339-395): the next
+// unused stream id of the device, created non-blocking at the default priority.
+class HIPStream {
+ public:
+  explicit HIPStream(int device_id);
+  bool Query();
+  void Synchronize();
+  void* impl() const { return impl_; }
+  int device_id() const { return device_id_; }
+  int stream_id() const { return stream_id_; }
+
+ private:
+  int device_id_, stream_id_;
+  void* impl_;
 };
 
 // Switches the current device for a scope (CUDADeviceGuard's role).

@@ -26,6 +26,14 @@ class UnifiedMemory {
   void* mutable_hip_data(int device);
 
   size_t size() const { return size_; }
+  // Bytes held on the given device ("cpu" or "hip"), 0 when nothing is allocated there.
+  size_t size(const string& device_type, int device_id) const {
+    if (device_type == "cpu") return cpu_ptr_ ? size_ : 0;
+    if (device_type == "hip") return hip_ptr_ && device_id_ == device_id ? size_ : 0;
+    return 0;
+  }
+  // Where the up-to-date copy lives (UnifiedMemory::info's "device_type" / "device_id").
+  string device_type() const { return state_ == STATE_AT_HIP ? "hip" : "cpu"; }
   State state() const { return state_; }
   int device() const { return device_id_; }
 

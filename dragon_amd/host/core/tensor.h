@@ -54,6 +54,7 @@ class Tensor {
   int64_t count(int start) const { return count(start, ndim()); }
   size_t size() const { return size_; }
   size_t nbytes() const { return size_ * SizeOf(meta_); }
+  size_t capacity() const { return capacity_; }
   DType meta() const { return meta_; }
   void set_meta(DType meta) { meta_ = meta; }
   bool has_memory() const { return memory_ != nullptr; }

@@ -1,4 +1,5 @@
-"""Python front end of the C++ host layer (``libdragon_hip_ops.so``).
+"""Python front end of the C++ host layer (``libdragon_hip_ops.so`` through its
+compiled Python module, ``backend``).
 
 A thin stand-in for what ``dragon.Workspace`` / ``OpLib.execute`` /
 ``GradientTape`` do in the reference (dragon/python/core/autograph/op_lib.py:56-235,
@@ -9,51 +10,40 @@ operator on the HIP device, and results are fetched back to numpy. Nothing is
 computed in Python.
 """
 
-import ctypes
 import itertools
-import os
 
 import numpy as np
 
-from . import _lib
+from . import backend
 
-_HERE = os.path.dirname(os.path.abspath(__file__))
-OPS_LIB_PATH = os.path.join(_HERE, "lib", "libdragon_hip_ops.so")
 PROTO_HIP = 4
-
-_handle = None
+# DeviceTypeProto values by device name: the reference's table
+# (dragon/python/core/framework/proto_util.py:132) with the HIP device added.
+_DEVICE_TO_IDENTIFIER = {"cpu": 0, "cuda": 1, "mps": 2, "mlu": 3, "hip": PROTO_HIP}
 
 
 class DragonError(RuntimeError):
     """What the reference reports through LOG(FATAL) before aborting."""
 
 
-def ops_lib():
-    global _handle
-    if _handle is None:
-        if not os.path.exists(OPS_LIB_PATH):
-            raise RuntimeError("%s is missing: run __graft_entry__.build()" % OPS_LIB_PATH)
-        _lib.lib()  # binds the kernel library (and the HIP runtime torch ships) first
-        h = ctypes.CDLL(OPS_LIB_PATH)
-        h.dragon_c_last_error.restype = ctypes.c_char_p
-        _handle = h
-    return _handle
-
-
-def _check(status):
-    if status != 0:
-        raise DragonError(ops_lib().dragon_c_last_error().decode())
+def _guard(fn, *args, **kwargs):
+    """Calls into the compiled module; its fatal errors surface as DragonError."""
+    try:
+        return fn(*args, **kwargs)
+    except RuntimeError as e:
+        raise DragonError(str(e)) from None
 
 
 def registered_operators():
-    buf = ctypes.create_string_buffer(1 << 14)
-    _check(ops_lib().dragon_c_registered_operators(buf, len(buf)))
-    return [s for s in buf.value.decode().split("\n") if s]
+    return list(backend.RegisteredOperators())
 
 
-def _np_storage(dtype):
-    return {"float16": np.uint16, "bfloat16": np.uint16, "float32": np.float32,
-            "float64": np.float64, "int64": np.int64, "int32": np.int32}[dtype]
+def get_device_option(device_type, device_index=0, random_seed=None):
+    """DeviceOption in protobuf text format (proto_util.py:135-147)."""
+    text = "device_type: %d device_id: %d" % (_DEVICE_TO_IDENTIFIER[device_type.lower()], device_index)
+    if random_seed is not None:
+        text += " random_seed: %d" % random_seed
+    return "device_option { %s }" % text
 
 
 def _quote(s):
@@ -84,84 +74,69 @@ def make_def(op_type, inputs, outputs, name="", device_id=0, **args):
         else:
             raise TypeError("unsupported argument %s=%r" % (key, value))
         parts.append("arg { name: %s %s }" % (_quote(key), field))
-    parts.append("device_option { device_type: %d device_id: %d }" % (PROTO_HIP, device_id))
+    parts.append(get_device_option("hip", device_id))
     return " ".join(parts)
 
 
 class Workspace:
-    """Named tensors plus operator execution on the HIP device."""
+    """Named tensors plus operator execution on the HIP device: the compiled module's
+    Workspace (C++ ``dragon::Workspace``) behind the method names the tests use."""
 
     _uid = itertools.count()
 
     def __init__(self, name="default"):
-        self._ws = ctypes.c_void_p()
-        _check(ops_lib().dragon_c_workspace_create(name.encode(), ctypes.byref(self._ws)))
+        self._impl = backend.Workspace(name)
 
     def close(self):
-        if self._ws:
-            ops_lib().dragon_c_workspace_destroy(self._ws)
-            self._ws = ctypes.c_void_p()
-
-    def __del__(self):
-        try:
-            self.close()
-        except Exception:
-            pass
+        self._impl = None
 
     def unique_name(self, prefix):
         return "%s_%d" % (prefix, next(Workspace._uid))
 
-    def feed(self, name, array, dtype=None):
-        """Feed a numpy array; 16-bit floats travel as uint16 bit patterns with ``dtype`` given."""
-        if dtype is None:
-            dtype = {np.dtype(np.float16): "float16", np.dtype(np.float32): "float32",
-                     np.dtype(np.float64): "float64", np.dtype(np.int64): "int64",
-                     np.dtype(np.int32): "int32"}[array.dtype]
-            if dtype == "float16":
-                array = array.view(np.uint16)
-        a = np.ascontiguousarray(array, dtype=_np_storage(dtype))
-        dims = (ctypes.c_int64 * a.ndim)(*a.shape)
-        _check(ops_lib().dragon_c_feed_tensor(self._ws, name.encode(), dtype.encode(), a.ndim, dims,
-                                              ctypes.c_void_p(a.ctypes.data)))
+    def feed(self, name, array, dtype=None, device=None):
+        """Feed a numpy array (``Tensor.FromNumpy``). bfloat16 travels as uint16 bit patterns
+        with ``dtype`` given, and so may float16. ``device`` = ("hip", index) writes straight
+        into device memory; by default the tensor moves there when an operator first reads it."""
+        array = np.asarray(array)
+        if dtype == "float16" and array.dtype == np.uint16:
+            array, dtype = array.view(np.float16), None
+        device_type, device_id = device if device is not None else ("cpu", 0)
+        tensor = self._impl.CreateTensor(name)
+        _guard(tensor.FromNumpy, array, dtype or "", device_type, device_id)
         return name
 
     def has(self, name):
-        flag = ctypes.c_int()
-        _check(ops_lib().dragon_c_has_tensor(self._ws, name.encode(), ctypes.byref(flag)))
-        return bool(flag.value)
+        return self._impl.HasTensor(name)
+
+    def tensor(self, name):
+        """The compiled module's Tensor (name, dims, dtype, device, data pointers)."""
+        t = self._impl.GetTensor(name)
+        if t is None:
+            raise DragonError("Tensor(%s) is not in workspace." % name)
+        return t
 
     def info(self, name):
-        buf = ctypes.create_string_buffer(32)
-        ndim = ctypes.c_int()
-        dims = (ctypes.c_int64 * 8)()
-        _check(ops_lib().dragon_c_tensor_info(self._ws, name.encode(), buf, len(buf),
-                                              ctypes.byref(ndim), dims))
-        return buf.value.decode(), tuple(dims[i] for i in range(ndim.value))
+        t = self.tensor(name)
+        return t.dtype, tuple(t.dims)
 
     def fetch(self, name, raw=False):
-        """numpy copy of a tensor. float16 comes back as float16, bfloat16 as uint16 bit
-        patterns (``raw=True`` keeps float16 as uint16 too)."""
-        dtype, shape = self.info(name)
-        out = np.empty(shape, _np_storage(dtype))
-        _check(ops_lib().dragon_c_fetch_tensor(self._ws, name.encode(), ctypes.c_void_p(out.ctypes.data),
-                                               out.nbytes))
-        if dtype == "float16" and not raw:
-            return out.view(np.float16)
+        """numpy copy of a tensor (``Tensor.ToNumpy``). float16 comes back as float16, bfloat16
+        as uint16 bit patterns (``raw=True`` gives float16 as uint16 too)."""
+        out = _guard(self.tensor(name).ToNumpy)
+        if raw and out.dtype == np.float16:
+            return out.view(np.uint16)
         return out
 
+    def memory_allocated(self, device_type="cpu", device_index=0):
+        return self._impl.MemoryAllocated(device_type, device_index)
+
     def run_operator(self, def_text, stream=0, sync=True):
-        _check(ops_lib().dragon_c_run_operator(self._ws, def_text.encode(), stream, int(sync)))
+        _guard(self._impl.RunOperator, def_text, stream, sync)
 
     def gradient_defs(self, def_text, output_grads):
         """Gradient OperatorDefs of a forward definition and the names of the input gradients."""
-        arr = (ctypes.c_char_p * len(output_grads))(*[g.encode() for g in output_grads])
-        defs = ctypes.create_string_buffer(1 << 16)
-        gis = ctypes.create_string_buffer(1 << 14)
-        _check(ops_lib().dragon_c_make_gradient_defs(def_text.encode(), arr, len(output_grads), defs,
-                                                     len(defs), gis, len(gis)))
-        grad_defs = [d for d in defs.value.decode().split("\n") if d.strip()]
-        grad_inputs = gis.value.decode().split("\n")[:-1]
-        return grad_defs, grad_inputs
+        defs, grad_inputs = _guard(backend.MakeGradientDefs, def_text, list(output_grads))
+        return list(defs), list(grad_inputs)
 
 
 class Tape:

@@ -111,5 +111,55 @@ def test_hip_module_without_a_device():
     if not torch.cuda.is_available():
         assert hip.is_available() is False
         assert hip.get_device_count() == 0
-        with pytest.raises(_lib.DragonHipError):
+        with pytest.raises(RuntimeError, match="no ROCm-capable device"):
             hip.get_device_name(0)
+
+
+def test_compiled_module_binds_the_host_classes():
+    """The pybind11 module exposes what the reference's compiled module does for this path:
+    Workspace, Tensor, the device functions of dragon/modules/python/cuda.h under hip names,
+    and the stream class."""
+    from dragon_amd import backend
+    for name in ("Workspace", "Tensor", "HIPStream", "hipIsDriverSufficient", "hipGetDevice",
+                 "hipGetDeviceCount", "hipGetDeviceName", "hipGetDeviceCapability", "hipSetDevice",
+                 "hipSetRandomSeed", "hipStreamSynchronize", "RegisteredOperators",
+                 "MakeGradientDefs"):
+        assert hasattr(backend, name), name
+    assert rt._DEVICE_TO_IDENTIFIER == {"cpu": 0, "cuda": 1, "mps": 2, "mlu": 3, "hip": 4}
+    assert rt.get_device_option("hip", 2) == "device_option { device_type: 4 device_id: 2 }"
+
+
+def test_tensor_numpy_conversions_on_the_host_side():
+    """Tensor.FromNumpy / ToNumpy (dragon/modules/python/numpy.h:31-150) for every dtype of
+    this path, without a device: shape, dtype, bytes, and where the memory lives."""
+    from dragon_amd import backend
+    ws = backend.Workspace("numpy_test")
+    rng = np.random.default_rng(3)
+    for dtype in (np.float16, np.float32, np.float64, np.int64, np.int32, np.uint8):
+        a = (rng.standard_normal((2, 3, 4)) * 9).astype(dtype)
+        t = ws.CreateTensor("t_" + np.dtype(dtype).name)
+        t.FromNumpy(a)
+        assert (t.name, t.dtype, tuple(t.dims), t.size) == ("t_" + np.dtype(dtype).name,
+                                                             np.dtype(dtype).name, (2, 3, 4), 24)
+        assert t.itemsize == a.itemsize and t.nbytes == a.nbytes and t.capacity >= t.nbytes
+        assert t.device == ("cpu", 0)
+        out = t.ToNumpy()
+        assert out.dtype == a.dtype and np.array_equal(out, a)
+        assert t.data("cpu") != 0
+    bits = rng.integers(0, 65535, (5, 3)).astype(np.uint16)
+    b = ws.CreateTensor("b")
+    b.FromNumpy(bits, "bfloat16")
+    assert b.dtype == "bfloat16" and np.array_equal(b.ToNumpy(), bits)
+    # a non-contiguous array is made contiguous, as PyArray_GETCONTIGUOUS does
+    a = rng.standard_normal((6, 4)).astype(np.float32)
+    t = ws.CreateTensor("strided")
+    t.FromNumpy(a.T)
+    assert np.array_equal(t.ToNumpy(), a.T)
+    assert ws.MemoryAllocated("cpu", 0) >= a.nbytes and ws.MemoryAllocated("hip", 0) == 0
+    assert ws.GetTensor("missing") is None and not ws.HasTensor("missing")
+    with pytest.raises(RuntimeError, match="cannot hold"):
+        b.FromNumpy(bits.astype(np.uint8), "bfloat16")
+    with pytest.raises(RuntimeError, match="Unsupported numpy type"):
+        b.FromNumpy(np.zeros(3, np.complex64))
+    with pytest.raises(RuntimeError, match="empty tensor"):
+        ws.CreateTensor("never_written").ToNumpy()
