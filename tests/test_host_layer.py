@@ -163,3 +163,30 @@ def test_tensor_numpy_conversions_on_the_host_side():
         b.FromNumpy(np.zeros(3, np.complex64))
     with pytest.raises(RuntimeError, match="empty tensor"):
         ws.CreateTensor("never_written").ToNumpy()
+
+
+def test_c_runtime_api_still_answers():
+    """The C API of the host layer (host/capi/dragon_c_api.h, the counterpart of the
+    reference's C++ runtime API) beside the compiled Python module: registry, feed, fetch,
+    and a fatal error reported as a message."""
+    import ctypes
+    import os
+    from dragon_amd import _lib
+    _lib.lib()
+    here = os.path.dirname(os.path.abspath(rt.__file__))
+    api = ctypes.CDLL(os.path.join(here, "lib", "libdragon_hip_ops.so"))
+    api.dragon_c_last_error.restype = ctypes.c_char_p
+    buf = ctypes.create_string_buffer(1 << 14)
+    assert api.dragon_c_registered_operators(buf, len(buf)) == 0
+    assert "LayerNorm" in buf.value.decode().split("\n")
+    ws = ctypes.c_void_p()
+    assert api.dragon_c_workspace_create(b"capi", ctypes.byref(ws)) == 0
+    a = np.arange(12, dtype=np.float32).reshape(3, 4)
+    dims = (ctypes.c_int64 * 2)(3, 4)
+    assert api.dragon_c_feed_tensor(ws, b"a", b"float32", 2, dims, ctypes.c_void_p(a.ctypes.data)) == 0
+    out = np.empty_like(a)
+    assert api.dragon_c_fetch_tensor(ws, b"a", ctypes.c_void_p(out.ctypes.data), out.nbytes) == 0
+    assert np.array_equal(out, a)
+    assert api.dragon_c_run_operator(ws, b'type: "Nope" device_option { device_type: 4 }', 0, 1) == -1
+    assert b"not registered" in api.dragon_c_last_error()
+    assert api.dragon_c_workspace_destroy(ws) == 0
