@@ -665,6 +665,163 @@ __global__ __launch_bounds__(kColThreads) void softmax_grad_col_tiles(const ColG
   }
 }
 
+// S > 1 with a reduced axis too long for a register tile (more than 1024
+// classes): a workgroup owns a panel of all C rows by kTW * kVec adjacent
+// columns of one n and walks it in chunks of ColTile::kMaxC rows, twice. Pass
+// one keeps, per thread and column, a running maximum and a sum rescaled to it;
+// the row threads of a column are then combined once. Pass two reads the
+// chunks again (from the caches where the panel fits them), normalises and
+// writes. Each chunk is read before it is written, so y may alias x.
+constexpr int kPanelPackets = 8;  // packets per thread and chunk
+
+template <typename T, int kKind, int kTW>
+__global__ __launch_bounds__(kColThreads) void softmax_col_panels(const ColGrid g, const T* x,
+                                                                  T* y) {
+  using Tile = ColTile<T, kTW, kPanelPackets>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  constexpr int kR = kPanelPackets;
+  __shared__ A lds[Tile::kLdsWords];
+  for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
+    const int64_t n = tile / g.strips;
+    const int64_t s0 = (tile - n * g.strips) * Tile::kCols + Tile::tw() * kVec;
+    const int64_t left = g.S - s0;
+    const int nvalid = left >= kVec ? kVec : (left > 0 ? static_cast<int>(left) : 0);
+    const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
+    A m[kVec], sum[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) m[e] = acc_neg_inf<A>(), sum[e] = A(0);
+    for (int c0 = 0; c0 < g.C; c0 += Tile::kMaxC) {
+      Tile t;
+      t.load(x + base + static_cast<int64_t>(c0) * g.S, g.S, g.C - c0, nvalid, acc_neg_inf<A>());
+      A pm[kVec];
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) pm[e] = acc_neg_inf<A>();
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) pm[e] = MaxOp()(pm[e], v[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (pm[e] > m[e]) {
+          sum[e] *= M::exp_of(m[e] - pm[e]);  // m == -inf so far: the sum is 0 and stays 0
+          m[e] = pm[e];
+        }
+      }
+      t.refresh();
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (m[e] > acc_neg_inf<A>()) sum[e] += M::exp_of(v[e] - m[e]);  // padding: exp(-inf) = 0
+        }
+      }
+    }
+    A top[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) top[e] = m[e];
+    Tile::reduce_rows(top, MaxOp(), lds);
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      sum[e] = m[e] > acc_neg_inf<A>() ? sum[e] * M::exp_of(m[e] - top[e]) : A(0);
+    }
+    Tile::reduce_rows(sum, SumOp(), lds);
+    A inv[kVec], l[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) inv[e] = A(1) / sum[e], l[e] = acc_log(sum[e]);
+    for (int c0 = 0; c0 < g.C; c0 += Tile::kMaxC) {
+      const int64_t at = base + static_cast<int64_t>(c0) * g.S;
+      Tile t;
+      t.load(x + at, g.S, g.C - c0, nvalid, acc_neg_inf<A>());
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        A v[kVec];
+        t.unpack(r, v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A d = v[e] - top[e];
+          v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), sum[e], inv[e]) : d - l[e];
+        }
+        Tile::store(y + at, g.S, g.C - c0, nvalid, r, v);
+      }
+    }
+  }
+}
+
+// The backward of the same panels: pass one sums dy * y (softmax) or dy
+// (log-softmax) over C, pass two reads both tensors again. dx may alias dy.
+template <typename T, int kKind, int kTW>
+__global__ __launch_bounds__(kColThreads) void softmax_grad_col_panels(const ColGrid g, const T* dy,
+                                                                       const T* y, T* dx) {
+  using Tile = ColTile<T, kTW, kPanelPackets>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  constexpr int kR = kPanelPackets;
+  __shared__ A lds[Tile::kLdsWords];
+  const A y_fill = kKind == kSoftmax ? A(0) : acc_neg_inf<A>();
+  for (int64_t tile = blockIdx.x; tile < g.tiles; tile += gridDim.x) {
+    const int64_t n = tile / g.strips;
+    const int64_t s0 = (tile - n * g.strips) * Tile::kCols + Tile::tw() * kVec;
+    const int64_t left = g.S - s0;
+    const int nvalid = left >= kVec ? kVec : (left > 0 ? static_cast<int>(left) : 0);
+    const int64_t base = n * g.C * g.S + (nvalid > 0 ? s0 : 0);
+    A sum[kVec];
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) sum[e] = A(0);
+    for (int c0 = 0; c0 < g.C; c0 += Tile::kMaxC) {
+      const int64_t at = base + static_cast<int64_t>(c0) * g.S;
+      Tile tg, to;
+      tg.load(dy + at, g.S, g.C - c0, nvalid, A(0));
+      if (kKind == kSoftmax) to.load(y + at, g.S, g.C - c0, nvalid, y_fill);
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        A gv[kVec], ov[kVec];
+        tg.unpack(r, gv);
+        if (kKind == kSoftmax) to.unpack(r, ov);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) sum[e] += kKind == kSoftmax ? gv[e] * ov[e] : gv[e];
+      }
+    }
+    Tile::reduce_rows(sum, SumOp(), lds);
+    for (int c0 = 0; c0 < g.C; c0 += Tile::kMaxC) {
+      const int64_t at = base + static_cast<int64_t>(c0) * g.S;
+      Tile tg, to;
+      tg.load(dy + at, g.S, g.C - c0, nvalid, A(0));
+      to.load(y + at, g.S, g.C - c0, nvalid, y_fill);
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        A gv[kVec], ov[kVec];
+        tg.unpack(r, gv);
+        to.unpack(r, ov);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          gv[e] = kKind == kSoftmax ? (gv[e] - sum[e]) * ov[e] : gv[e] - M::exp_of(ov[e]) * sum[e];
+        }
+        Tile::store(dx + at, g.S, g.C - c0, nvalid, r, gv);
+      }
+    }
+  }
+}
+
+// Threads along the columns of a panel: the widest of 64 / 16 / 4 that the
+// columns fill and that still gives every compute unit a couple of panels.
+inline int pick_panel_tw(int64_t N, int64_t S, int vec) {
+  const int64_t packets = ceil_div(S, vec);
+  const int tw_cap = packets > 16 ? 64 : (packets > 4 ? 16 : 4);
+  for (int tw : {64, 16}) {
+    if (tw > tw_cap) continue;
+    if (N * ceil_div(S, static_cast<int64_t>(tw) * vec) >= 2 * num_cus()) return tw;
+  }
+  return 4;
+}
+
 // One thread per (n, s) column, elements S apart.
 template <typename T, int kKind>
 __global__ __launch_bounds__(256) void softmax_columns(
@@ -1119,6 +1276,17 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
   }
     if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
 #undef LAUNCH
+  } else if (C > 1024) {
+    // no register tile holds the reduced axis: panels walked in chunks, twice
+    const int tw = pick_panel_tw(N, S, kVec);
+#define LAUNCH(TW)                                                                        \
+  {                                                                                       \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                  \
+    hipLaunchKernelGGL((softmax_col_panels<T, kKind, TW>), dim3(col_launch_grid(g.tiles)), \
+                       dim3(kColThreads), 0, stream, g, xp, yp);                          \
+  }
+    if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
   } else {
     hipLaunchKernelGGL((softmax_columns<T, kKind>), dim3(flat_grid(N * S)), dim3(256), 0, stream, N,
                        S, C, xp, yp);
@@ -1209,6 +1377,16 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
       hipLaunchKernelGGL((softmax_grad_col_tiles<T, kKind, TW, 16>), grid, block, 0, stream, g, \
                          gp, yp, dp);                                                     \
     }                                                                                     \
+  }
+    if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
+#undef LAUNCH
+  } else if (C > 1024) {
+    const int tw = pick_panel_tw(N, S, kVec);
+#define LAUNCH(TW)                                                                          \
+  {                                                                                         \
+    const ColGrid g = make_col_grid(N, S, C, TW * kVec);                                    \
+    hipLaunchKernelGGL((softmax_grad_col_panels<T, kKind, TW>), dim3(col_launch_grid(g.tiles)), \
+                       dim3(kColThreads), 0, stream, g, gp, yp, dp);                        \
   }
     if (tw == 64) LAUNCH(64) else if (tw == 16) LAUNCH(16) else LAUNCH(4)
 #undef LAUNCH

@@ -132,7 +132,12 @@ SM_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 100000), 
              # scratch the wrapper passes); (3, 100000) above takes the same path
              ((5, 131072), -1),
              # short rows staged through LDS, several rows per wavefront
-             ((64, 64), -1), ((33, 197), -1), ((9, 577), -1), ((100, 128), -1), ((300, 8), -1)]
+             ((64, 64), -1), ((33, 197), -1), ((9, 577), -1), ((100, 128), -1), ((300, 8), -1),
+             # a strided axis beyond the register tiles (more than 1024 classes): panels of
+             # columns walked in chunks of rows, twice; wide, medium and narrow panels, a
+             # partial last chunk, columns that are not whole packets
+             ((2, 1500, 40), 1), ((3, 4096, 24), 1), ((1, 1100, 530), 1), ((300, 1030, 70), 1),
+             ((2, 2051, 3), 1)]
 
 
 def _softmax_inputs(shape, dtype, seed):
@@ -195,7 +200,8 @@ def test_softmax_forward_backward(K, shape, axis, dtype, log):
     assert U.normwise(dxw[ok], np.asarray(dx_ref)[ok]) <= U.TIGHT[dtype]
 
 
-@pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (2, 66000), (3, 10, 33)])
+@pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (2, 66000), (3, 10, 33),
+                                   (2, 1300, 20)])
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_softmax_in_place(K, dtype, shape):
     x, dy = _softmax_inputs(shape, dtype, 5)
