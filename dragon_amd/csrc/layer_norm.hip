@@ -107,13 +107,30 @@ __global__ __launch_bounds__(kThreads) void layer_norm_wide_rows(
   __shared__ A slots[2][Tile::kSlots];
   A* lds_gamma = reinterpret_cast<A*>(staged);
   A* lds_beta = lds_gamma + C;
+  const int npackets = C / kVec;
+  // Rows of 8-element packets against 4-float LDS words: the first halves of
+  // all packets, then the second halves, so that the lanes of a wavefront read
+  // adjacent 16-byte words (eight consecutive floats per lane put lanes l and
+  // l + 8 on the same banks: a two-way conflict on every access).
+  constexpr bool kSplit = kVec == 2 * kPerPacket;
   for (int i = threadIdx.x; i < C / kPerPacket; i += kThreads) {
-    staged[i] = load_packet_keep(gamma + i * kPerPacket);
-    staged[C / kPerPacket + i] = load_packet_keep(beta + i * kPerPacket);
+    const int at = kSplit ? (i & 1) * npackets + (i >> 1) : i;
+    staged[at] = load_packet_keep(gamma + i * kPerPacket);
+    staged[C / kPerPacket + at] = load_packet_keep(beta + i * kPerPacket);
   }
   __syncthreads();
+  // the kVec parameters of packet `packet` of the row
+  auto params_of = [&](const A* lds, const int packet, A(&v)[kVec]) {
+    if constexpr (kSplit) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(lds + packet * 4);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(lds + (npackets + packet) * 4);
+      v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
+      v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    } else {
+      load_params<kVec>(lds + packet * kVec, v);
+    }
+  };
 
-  const int npackets = C / kVec;
   const A inv_c = A(1) / A(C);
   const int lane = Tile::lane();
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
@@ -159,10 +176,9 @@ __global__ __launch_bounds__(kThreads) void layer_norm_wide_rows(
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (Tile::active(i, npackets)) {
-        const int col = (i * kTPR + lane) * kVec;
         A g[kVec], b[kVec];
-        load_params<kVec>(lds_gamma + col, g);
-        load_params<kVec>(lds_beta + col, b);
+        params_of(lds_gamma, i * kTPR + lane, g);
+        params_of(lds_beta, i * kTPR + lane, b);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * rs * g[e] + b[e];
       }
