@@ -181,11 +181,14 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
   constexpr int kVec = IO<T>::kVec;
   const unsigned fin_grid = static_cast<unsigned>(ceil_div(sh.C, kReduceThreads));
   ShortPlan sp;
+  auto lds_of = [](const ShortPlan& q) {
+    return static_cast<size_t>(q.stage_packets) * 16 * kIn + q.rows_per_chunk * sizeof(A);
+  };
   if (short_channel_rows(sh, sizeof(T), in0, in1, in0) &&
-      plan_short_rows(sh.S, sizeof(T), kIn == 1 ? 4 : 2, false, &sp)) {
+      plan_short_rows_within(sh.S, sizeof(T), kIn == 1 ? 4 : 3, false, lds_of, &sp)) {
     using Holder = RowSumsOf<F, kIn>;
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
-    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 * kIn + sp.rows_per_chunk * sizeof(A);
+    const size_t lds = lds_of(sp);
     T* none = nullptr;
     DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
                             short_grid(rows, sp.rows_per_chunk), stream, rows,
@@ -503,14 +506,17 @@ void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hi
   const bool vec_ok = aligned16(in0) && aligned16(in1) && aligned16(out) &&
       (sh.nchw ? sh.S % kVec == 0 : sh.C % kVec == 0);
   ShortPlan sp;
+  auto lds_of = [](const ShortPlan& q) {
+    return static_cast<size_t>(q.stage_packets) * 16 * kIn +
+        static_cast<size_t>(q.rows_per_chunk) * F<T, 1>::kParams * sizeof(A);
+  };
   if (short_channel_rows(sh, sizeof(T), in0, in1, out) &&
-      plan_short_rows(sh.S, sizeof(T), kIn == 1 ? 4 : 2, false, &sp)) {
+      plan_short_rows_within(sh.S, sizeof(T), kIn == 1 ? 4 : 3, false, lds_of, &sp)) {
     using Fn = F<T, 1>;
     using Holder = RowMapOf<Fn, kIn>;
     const Fn fn{ChannelIndex{sh}, args...};
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
-    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16 * kIn +
-        static_cast<size_t>(sp.rows_per_chunk) * Fn::kParams * sizeof(A);
+    const size_t lds = lds_of(sp);
     DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
                             short_grid(rows, sp.rows_per_chunk), stream, rows,
                             static_cast<int>(sh.S), in0, in1, out, fn, sh.C);

@@ -18,6 +18,9 @@
 namespace dragon_hip {
 namespace {
 
+// A wavefront that holds a whole row in one or two packets per lane takes two
+// neighbouring rows at a time: their dependent cross-lane reduction steps
+// interleave, and one fetch of gamma and beta serves both.
 template <typename T, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
     const int64_t N, const int C, const typename IO<T>::Acc eps, const T* __restrict__ x,
@@ -27,39 +30,58 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
   using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
+  constexpr int kR = wave_rows_at_a_time<kTPR, kVPT>();
+  constexpr int kRowsPerStep = Tile::kRowsPerBlock * kR;
   __shared__ A slots[2][Tile::kSlots];
   const int npackets = Tile::extent_of(C);
   const A inv_c = A(1) / A(C);
   const int lane = Tile::lane();
 
-  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
-       row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
-    Tile t;
-    t.load(x + row * C, npackets, A(0));
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerStep + Tile::sub_row() * kR;
+       row < N; row += static_cast<int64_t>(gridDim.x) * kRowsPerStep) {
+    Tile t[kR];
+    bool on[kR];  // uniform over the row's threads
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      on[r] = row + r < N;
+      t[r].load(x + (on[r] ? row + r : row) * C, npackets, A(0));
+    }
 
-    A s = A(0);
+    A mean[kR];
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i)
+    for (int r = 0; r < kR; ++r) {
+      mean[r] = A(0);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) s += t.v[i][e];
-    const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_c;
+      for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) mean[r] += t[r].v[i][e];
+    }
+#pragma unroll
+    for (int r = 0; r < kR; ++r) mean[r] = Tile::reduce(mean[r], SumOp(), slots[0]) * inv_c;
 
-    A q = A(0);
+    A rs[kR];
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i) {
-      if (Tile::active(i, npackets)) {
+    for (int r = 0; r < kR; ++r) {
+      rs[r] = A(0);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) {
-          const A d = t.v[i][e] - mean;
-          if (Tile::elem_active(i, e, npackets)) q += d * d;
+      for (int i = 0; i < kVPT; ++i) {
+        if (Tile::active(i, npackets)) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            const A d = t[r].v[i][e] - mean[r];
+            if (Tile::elem_active(i, e, npackets)) rs[r] += d * d;
+          }
         }
       }
     }
-    const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_c;
-    const A rs = acc_rsqrt_exact(var + eps);
-    if (lane == 0) {
-      mu[row] = mean;
-      rsig[row] = rs;
+#pragma unroll
+    for (int r = 0; r < kR; ++r) {
+      const A var = Tile::reduce(rs[r], SumOp(), slots[1]) * inv_c;
+      rs[r] = acc_rsqrt_exact(var + eps);
+      if (lane == 0 && on[r]) {
+        mu[row + r] = mean[r];
+        rsig[row + r] = rs[r];
+      }
     }
 
 #pragma unroll
@@ -75,10 +97,15 @@ __global__ __launch_bounds__(row_threads(kTPR)) void layer_norm_rows(
           load_params<kVec>(beta + col, b);
         }
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * rs * g[e] + b[e];
+        for (int r = 0; r < kR; ++r)
+#pragma unroll
+          for (int e = 0; e < kVec; ++e)
+            t[r].v[i][e] = (t[r].v[i][e] - mean[r]) * rs[r] * g[e] + b[e];
       }
     }
-    t.store(y + row * C, npackets);
+#pragma unroll
+    for (int r = 0; r < kR; ++r)
+      if (on[r]) t[r].store(y + (row + r) * C, npackets);
     if (kTPR != kWaveSize) __syncthreads();  // slots are reused by the next row
   }
 }
@@ -372,7 +399,8 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
   {                                                                                        \
     using Tile = RowTile<T, TPR, VPT>;                                                     \
     hipLaunchKernelGGL((layer_norm_rows<T, TPR, VPT, false>),                              \
-                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       dim3(row_grid(N, Tile::kRowsPerBlock * wave_rows_at_a_time<TPR, VPT>())), \
+                       dim3(Tile::kThreads), 0, stream,                                    \
                        N, static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);            \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
@@ -383,7 +411,8 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
   {                                                                                        \
     using Tile = RowTile<T, TPR, VPT>;                                                     \
     hipLaunchKernelGGL((layer_norm_rows<T, TPR, VPT, true>),                               \
-                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0, stream, \
+                       dim3(row_grid(N, Tile::kRowsPerBlock * wave_rows_at_a_time<TPR, VPT>())), \
+                       dim3(Tile::kThreads), 0, stream,                                    \
                        N, static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);            \
   }
     DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);

@@ -423,7 +423,7 @@ int launch_lp_norm(int64_t N, int64_t S, int64_t C, float normalizer, float epsi
   const bool packets_ok = aligned16(x) && aligned16(out) && (!kGrad || aligned16(dy));
   ShortPlan sp;
   if (S == 1 && lp_norm_short_rows(C, sizeof(T), kGrad, x, dy, out) &&
-      plan_short_rows(C, sizeof(T), kGrad ? 1 : 4, aligned16(x), &sp)) {
+      plan_short_rows(C, sizeof(T), 4, aligned16(x), &sp)) {
     const size_t lds = static_cast<size_t>(sp.stage_packets) * (kGrad ? 32 : 16);
     const unsigned grid = short_grid(N, sp.rows_per_chunk);
     if constexpr (kGrad && kP == 1) {

@@ -287,6 +287,16 @@ struct RawRowTile {
   }
 };
 
+// How many neighbouring rows a forward row kernel holds per thread group at a
+// time. A wavefront that holds a whole row in one or two packets per lane takes
+// two: the dependent cross-lane reduction steps of the two rows interleave
+// instead of each waiting out the latency of the one before, and twice the
+// loads are in flight per wavefront.
+template <int kTPR, int kVPT>
+constexpr int wave_rows_at_a_time() {
+  return kTPR == kWaveSize && kVPT <= 2 ? 2 : 1;
+}
+
 // Picks the tile for a row of `npackets` packets: the fewest threads per row
 // whose tile still holds it, because short rows on few threads leave many rows
 // in flight per compute unit (wave-per-row up to 4 packets per lane, then a

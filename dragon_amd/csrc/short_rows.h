@@ -67,27 +67,70 @@ struct StagedRange {
   __device__ __forceinline__ uint32_t lead() const { return static_cast<uint32_t>(a0 - first); }
 };
 
-// Copies the packets of `r` into stage[0 .. r.packets). A packet that reaches
-// outside the tensor (only the tensor's first or last can) is read element by
-// element; what lies outside reads as zero.
-// kStream: the tensor is read once and not again soon (non-temporal loads).
-template <typename T, bool kStream>
-__device__ __forceinline__ void stage_in(const StagedRange& r, u32x4* stage) {
-  for (uint32_t p = threadIdx.x; p < r.packets; p += kShortThreads) {
-    const uintptr_t addr = r.first + 16u * p;
-    if (addr >= r.base && addr + 16 <= r.base + r.total) {
-      stage[p] = kStream ? load_packet(reinterpret_cast<const T*>(addr))
-                         : load_packet_keep(reinterpret_cast<const T*>(addr));
-    } else {
-      T* out = reinterpret_cast<T*>(stage + p);
+// Packets a thread requests before it waits for the first of them.
+constexpr int kStageBatch = 4;
+
+// One packet of `r` that may reach outside the tensor (only the tensor's first
+// or last can): read element by element; what lies outside reads as zero.
+template <typename T>
+__device__ __forceinline__ void stage_in_edge(const StagedRange& r, u32x4* stage, uint32_t p) {
+  const uintptr_t addr = r.first + 16u * p;
+  T* out = reinterpret_cast<T*>(stage + p);
 #pragma unroll
-      for (uint32_t i = 0; i < 16 / sizeof(T); ++i) {
-        const uintptr_t ea = addr + i * sizeof(T);
-        T zero{};
-        out[i] = (ea >= r.base && ea + sizeof(T) <= r.base + r.total)
-                     ? *reinterpret_cast<const T*>(ea) : zero;
+  for (uint32_t i = 0; i < 16 / sizeof(T); ++i) {
+    const uintptr_t ea = addr + i * sizeof(T);
+    T zero{};
+    out[i] = (ea >= r.base && ea + sizeof(T) <= r.base + r.total)
+                 ? *reinterpret_cast<const T*>(ea) : zero;
+  }
+}
+
+// Copies the packets of the ranges into stage0 / stage1 [0 .. r.packets); the
+// two ranges (kIn == 2) cover the same bytes of two congruent tensors. A thread
+// requests a batch of packets of every tensor before it waits for the first and
+// moves them to LDS: the loads of a workgroup travel together instead of one per
+// thread at a time. The conditions around the loads are uniform over the
+// workgroup. kStream: the tensors are read once and not again soon
+// (non-temporal loads).
+template <typename T, bool kStream, int kIn>
+__device__ __forceinline__ void stage_in(const StagedRange& r0, u32x4* stage0,
+                                         const StagedRange& r1, u32x4* stage1) {
+  // packets [lo, hi) lie inside the tensor
+  const bool head_out = r0.first < r0.base;
+  const bool tail_out = r0.first + 16u * static_cast<uintptr_t>(r0.packets) > r0.base + r0.total;
+  const uint32_t lo = head_out ? 1u : 0u;
+  const uint32_t hi = r0.packets - (tail_out ? 1u : 0u);
+  for (uint32_t p0 = lo; p0 < hi; p0 += kShortThreads * kStageBatch) {
+    u32x4 v0[kStageBatch], v1[kStageBatch];
+#pragma unroll
+    for (int k = 0; k < kStageBatch; ++k) {
+      if (p0 + k * kShortThreads < hi) {  // uniform
+        const uint32_t want = p0 + k * kShortThreads + threadIdx.x;
+        const uint32_t p = want < hi ? want : hi - 1;
+        const T* a0 = reinterpret_cast<const T*>(r0.first + 16u * static_cast<uintptr_t>(p));
+        v0[k] = kStream ? load_packet(a0) : load_packet_keep(a0);
+        if constexpr (kIn == 2) {
+          const T* a1 = reinterpret_cast<const T*>(r1.first + 16u * static_cast<uintptr_t>(p));
+          v1[k] = kStream ? load_packet(a1) : load_packet_keep(a1);
+        }
       }
     }
+#pragma unroll
+    for (int k = 0; k < kStageBatch; ++k) {
+      const uint32_t p = p0 + k * kShortThreads + threadIdx.x;
+      if (p < hi) {
+        stage0[p] = v0[k];
+        if constexpr (kIn == 2) stage1[p] = v1[k];
+      }
+    }
+  }
+  if (head_out && threadIdx.x == 0) {
+    stage_in_edge<T>(r0, stage0, 0);
+    if constexpr (kIn == 2) stage_in_edge<T>(r1, stage1, 0);
+  }
+  if (tail_out && threadIdx.x == kWaveSize && !(head_out && r0.packets == 1)) {
+    stage_in_edge<T>(r0, stage0, r0.packets - 1);
+    if constexpr (kIn == 2) stage_in_edge<T>(r1, stage1, r0.packets - 1);
   }
 }
 
@@ -176,11 +219,9 @@ __global__ __launch_bounds__(kShortThreads) void short_rows(
         for (int q = 0; q < kSide; ++q) side[i * kSide + q] = w[q];
       }
     }
-    stage_in<T, !OpReadOnly<Op>::value>(r0, stage);
-    if constexpr (Op::kIn == 2) {
-      const StagedRange r1(in1, total, row0 * row_bytes, (row0 + rows) * row_bytes);
-      stage_in<T, !OpReadOnly<Op>::value>(r1, stage1);
-    }
+    const StagedRange r1(Op::kIn == 2 ? in1 : in0, total, row0 * row_bytes,
+                         (row0 + rows) * row_bytes);
+    stage_in<T, !OpReadOnly<Op>::value, Op::kIn>(r0, stage, r1, stage1);
     __syncthreads();
     T* tile0 = reinterpret_cast<T*>(reinterpret_cast<char*>(stage) + r0.lead());
     const T* tile1 = reinterpret_cast<const T*>(reinterpret_cast<const char*>(stage1) + r0.lead());
@@ -269,6 +310,18 @@ inline bool plan_short_rows(int64_t C, size_t elem_bytes, int packets_per_thread
   if (rows == 0) rows = per_pass;  // at least one row per lane group (at most 16 KB)
   p->rows_per_chunk = rows;
   p->stage_packets = static_cast<uint32_t>((rows * row_bytes + 15) / 16 + 2);
+  return true;
+}
+// The plan with the most packets per thread, up to `packets_per_thread`, whose
+// LDS need `lds_of(plan)` (stage plus per-row scalars) stays within the 48 KB a
+// kernel may use without its limit being raised.
+template <typename LdsOf>
+inline bool plan_short_rows_within(int64_t C, size_t elem_bytes, int packets_per_thread,
+                                   bool base_aligned, LdsOf lds_of, ShortPlan* p) {
+  for (int ppt = packets_per_thread; ppt >= 1; --ppt) {
+    if (!plan_short_rows(C, elem_bytes, ppt, base_aligned, p)) return false;
+    if (lds_of(*p) <= 48 * 1024) break;
+  }
   return true;
 }
 inline unsigned short_grid(int64_t N, uint32_t rows_per_chunk) {
