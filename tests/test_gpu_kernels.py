@@ -310,6 +310,48 @@ def test_softmax_short_rows_at_shifted_bases(K, dtype, shift_x, shift_y):
     assert np.all(flat[:shift_x] == 0) and np.all(flat[shift_x + N * C:] == 0)
 
 
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
+@pytest.mark.parametrize("C", [16411, 20001, 30522, 50257])
+@pytest.mark.parametrize("shift_x,shift_y", [(0, 0), (3, 3), (1, 0)])
+def test_softmax_wide_rows_that_are_not_whole_packets(K, C, dtype, shift_x, shift_y, log):
+    """Vocabulary-sized rows whose width or base address is not a multiple of 16 bytes (the
+    ragged register tiles, 1024 threads per row and up to sixteen packets per thread), with
+    equal and unequal shifts of input and output. What surrounds the input is poisoned with a
+    huge logit that must not leak into a row; forward against fp64, and nothing outside the
+    output may be written."""
+    N = 5
+    shape = (N, C)
+    x, _ = _softmax_inputs(shape, dtype, 31)
+    x64 = np.asarray(U.widen(x, dtype), np.float64).reshape(shape)
+    e64 = np.exp(x64 - x64.max(1, keepdims=True))
+    y_ref = e64 / e64.sum(1, keepdims=True)
+    if log:
+        y_ref = (x64 - x64.max(1, keepdims=True)) - np.log(e64.sum(1, keepdims=True))
+    guard = 24
+
+    def shifted(shift, bits=None, fill=0.0):
+        buf = empty((N * C + shift + guard,), dtype)
+        buf.fill_(fill)
+        view = buf[shift:shift + N * C].view(N, C)
+        if bits is not None:
+            view.copy_(U.to_device(bits, dtype))
+        return buf, view
+
+    # what lies around the input must not leak into the rows: poison it with a huge logit
+    _, xd = shifted(shift_x, x, fill=6e4)
+    ybuf, y = shifted(shift_y, fill=-7.0)
+    (K.log_softmax if log else K.softmax)(N, 1, C, xd, y)
+    yw = U.widen(U.to_host(y.contiguous()), dtype).reshape(shape)
+    if log:
+        keep = y_ref > -1e3
+        assert np.max(np.abs(yw[keep] - y_ref[keep]) / (1 + np.abs(y_ref[keep]))) <= U.TIGHT[dtype]
+    else:
+        assert U.rowwise_normwise(yw, y_ref) <= U.TIGHT[dtype]
+    flat = U.widen(U.to_host(ybuf), dtype).ravel()
+    assert np.all(flat[:shift_y] == -7.0) and np.all(flat[shift_y + N * C:] == -7.0)
+
+
 def test_softmax_masked_logits_are_exact_zero(K):
     x = np.zeros((4, 512), np.float32)
     x[:, ::2] = -1e4
