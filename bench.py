@@ -267,6 +267,10 @@ WORKLOADS = {
     # target shapes (>= 8192 x 4096)
     "layer_norm_bf16_8192x4096": lambda k: wl_layer_norm(8192, 4096, "bfloat16", 4, k=k),
     "layer_norm_f32_8192x4096": lambda k: wl_layer_norm(8192, 4096, "float32", 4, k=k),
+    # the same row widths with four times the rows: what the kernels sustain once the fixed
+    # cost of a call (first loads, last stores, the second stage of dgamma / dbeta) is spread
+    "layer_norm_bf16_32768x4096": lambda k: wl_layer_norm(32768, 4096, "bfloat16", 4, k=k),
+    "layer_norm_bf16_32768x12288": lambda k: wl_layer_norm(32768, 12288, "bfloat16", 4, k=k),
     "softmax_f16_8192x4096": lambda k: wl_softmax((8192, 4096), "float16", 1, k=k),
     "softmax_f32_8192x4096": lambda k: wl_softmax((8192, 4096), "float32", 1, k=k),
     # sibling row reductions on the same skeleton

@@ -107,11 +107,14 @@ def test_layer_norm_8192x4096_whole_tensor_against_the_oracle(K, dtype):
 
 @pytest.mark.parametrize("shape,dtype,outliers", [((8192, 12288), "bfloat16", True),
                                                   ((1048576, 64), "bfloat16", False),
-                                                  ((65536, 1000), "bfloat16", True)])
+                                                  ((65536, 1000), "bfloat16", True),
+                                                  ((32768, 4096), "bfloat16", False),
+                                                  ((32768, 12288), "bfloat16", False)])
 def test_layer_norm_bench_shapes_sampled_rows_and_column_sums(K, shape, dtype, outliers):
     """bench workloads layer_norm_bf16_8192x12288 (32 rows per workgroup of the 768-thread
     backward tile), layer_norm_bf16_1048576x64 (more chunks of staged short rows than the grid
-    holds) and layer_norm_bf16_65536x1000 (ragged rows)."""
+    holds), layer_norm_bf16_65536x1000 (ragged rows), and layer_norm_bf16_32768x4096 /
+    32768x12288 (32 and 128 iterations per persistent workgroup)."""
     N, C = shape
     x, dy, g, b = _layer_norm_inputs(N, C, dtype, 42, outliers)
     y, mu, rsig, dx, dg, db, params = _layer_norm_run(K, N, C, x, dy, g, b)
