@@ -128,6 +128,8 @@ def test_layer_norm_large_mean_stays_accurate(K):
 SM_SHAPES = [((256, 512), -1), ((10, 1000), -1), ((4, 4096), -1), ((3, 100000), -1), ((5, 37), -1),
              ((6, 300), -1), ((3, 7, 5), 1), ((2, 3, 4, 6), 2), ((4, 1), -1), ((2, 16, 8, 8), -1),
              ((3, 8200), -1),
+             # a wavefront takes two rows at a time: odd row counts, a single row
+             ((7, 512), -1), ((1, 512), -1), ((33, 1000), -1), ((9, 1024), -1),
              # rows beyond the one-workgroup tiles: several workgroups per row (with the
              # scratch the wrapper passes); (3, 100000) above takes the same path
              ((5, 131072), -1),
