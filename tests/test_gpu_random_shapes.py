@@ -1,0 +1,281 @@
+"""Seeded random shapes around the widths at which the launchers switch kernels (rows of one
+packet per lane, the LDS-staged short rows, 256- and 1024-thread tiles, raw-packet tiles,
+the looped and the sliced kernels; channel rows that are or are not whole packets), with
+odd row counts, every I/O type and tensors that start a few elements past a 16-byte
+boundary. The checker is the defining formula in fp64 (numpy), which the oracle itself is
+pinned against; tolerances as in tests/util.py. Every output lies in a poisoned buffer whose
+surroundings must come back untouched."""
+
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ("float32", "bfloat16", "float16")
+EDGES = (8, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, 65536, 131072)
+GUARD = 16
+POISON = -7.0
+
+
+@pytest.fixture(scope="module")
+def K():
+    import torch
+    assert torch.cuda.is_available()
+    from dragon_amd import kernels
+    return kernels
+
+
+def _row_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        edge = int(rng.choice(EDGES))
+        C = max(1, edge + int(rng.integers(-9, 10)) * int(rng.choice((1, 1, 8))))
+        N = int(rng.integers(1, max(2, min(48, 1_500_000 // C))))
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        sx = int(rng.choice((0, 0, 0, 1, 3, 4)))
+        sy = sx if rng.random() < 0.7 else int(rng.choice((0, 2, 5)))
+        cases.append((N, C, dtype, sx, sy, 1000 + i))
+    return cases
+
+
+def _held(n, dtype, shift, bits=None):
+    """A poisoned buffer and the view of n elements that starts `shift` elements into it."""
+    import torch
+    buf = torch.full((n + shift + GUARD,), POISON, dtype=U.torch_dtype(dtype), device="cuda")
+    view = buf[shift:shift + n]
+    if bits is not None:
+        view.copy_(U.to_device(np.ascontiguousarray(bits).ravel(), dtype))
+    return buf, view
+
+
+def _untouched(buf, dtype, shift, n):
+    flat = U.widen(U.to_host(buf), dtype).ravel()
+    return bool(np.all(flat[:shift] == POISON) and np.all(flat[shift + n:] == POISON))
+
+
+def _mean_ok(got, want, x):
+    """A mean of values that nearly cancel is held to the scale of the values, not of the mean."""
+    err = np.max(np.abs(np.asarray(got, np.float64).ravel() - np.asarray(want).ravel()))
+    return err <= 2e-5 * (np.max(np.abs(want)) + np.sqrt(np.mean(np.asarray(x) ** 2)))
+
+
+def _values(rng, shape, dtype, scale=1.0):
+    bits = R.to_bits((rng.standard_normal(shape) * scale).astype(np.float32), dtype)
+    return bits, U.widen(bits, dtype).reshape(shape)
+
+
+@pytest.mark.parametrize("N,C,dtype,sx,sy,seed", _row_cases(60, 1))
+def test_softmax_rows(K, N, C, dtype, sx, sy, seed):
+    rng = np.random.default_rng(seed)
+    log = bool(seed & 1)
+    xb, x = _values(rng, (N, C), dtype, 3.0)
+    dyb, dy = _values(rng, (N, C), dtype)
+    e = np.exp(x - x.max(1, keepdims=True))
+    p = e / e.sum(1, keepdims=True)
+    y_ref = np.log(p) if log else p
+    _, xd = _held(N * C, dtype, sx, xb)
+    ybuf, yd = _held(N * C, dtype, sy)
+    (K.log_softmax if log else K.softmax)(N, 1, C, xd, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, C)
+    if log:
+        assert np.max(np.abs(y - y_ref) / (1 + np.abs(y_ref))) <= U.TIGHT[dtype]
+    else:
+        assert U.rowwise_normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, sy, N * C)
+    # backward from the forward's own (rounded) output, as the operator graph does
+    _, dyd = _held(N * C, dtype, sx, dyb)
+    _, yin = _held(N * C, dtype, sx, U.to_host(yd.contiguous()))
+    dxbuf, dxd = _held(N * C, dtype, sy)
+    (K.log_softmax_grad if log else K.softmax_grad)(N, 1, C, dyd, yin, dxd)
+    dx = U.widen(U.to_host(dxd.contiguous()), dtype).reshape(N, C)
+    dx_ref = (dy - np.exp(y) * dy.sum(1, keepdims=True)) if log else \
+        (dy - (dy * y).sum(1, keepdims=True)) * y
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert _untouched(dxbuf, dtype, sy, N * C)
+
+
+@pytest.mark.parametrize("N,C,dtype,sx,sy,seed", _row_cases(60, 2))
+def test_layer_norm_rows(K, N, C, dtype, sx, sy, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    xb, x = _values(rng, (N, C), dtype, 2.0)
+    dyb, dy = _values(rng, (N, C), dtype)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    eps = 1e-5
+    mean = x.mean(1, keepdims=True)
+    var = ((x - mean) ** 2).mean(1, keepdims=True)
+    rs = 1 / np.sqrt(var + np.float64(np.float32(eps)))
+    xh = (x - mean) * rs
+    y_ref = xh * g + b
+    _, xd = _held(N * C, dtype, sx, xb)
+    ybuf, yd = _held(N * C, dtype, sy)
+    gd, bd = torch.from_numpy(g).cuda(), torch.from_numpy(b).cuda()
+    mu, rsig = torch.empty(N, device="cuda"), torch.empty(N, device="cuda")
+    K.layer_norm(N, C, eps, xd, gd, bd, mu, rsig, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, C)
+    assert _mean_ok(mu.cpu().numpy(), mean, x)
+    assert np.max(np.abs(rsig.cpu().numpy().astype(np.float64) / rs.ravel() - 1)) <= 2e-5
+    assert U.normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, sy, N * C)
+    # backward = GroupNormGrad with one group and S = 1, from the kernel's own statistics
+    m32 = mu.cpu().numpy().astype(np.float64)[:, None]
+    r32 = rsig.cpu().numpy().astype(np.float64)[:, None]
+    _, dyd = _held(N * C, dtype, sx, dyb)
+    dxbuf, dxd = _held(N * C, dtype, sy)
+    params = torch.empty(2 * N, device="cuda")
+    dg, db = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    K.group_norm_grad(N, 1, C, 1, "NHWC", xd, mu, rsig, gd, dyd, params, params, dg, db, dxd)
+    ds_ref = (g * dy * x).sum(1)
+    db_ref = (g * dy).sum(1)
+    u = (db_ref[:, None] * m32 - ds_ref[:, None]) * (x - m32) * r32 ** 3
+    dx_ref = g * dy * r32 + (u - db_ref[:, None] * r32) / C
+    dx = U.widen(U.to_host(dxd.contiguous()), dtype).reshape(N, C)
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(dg.cpu().numpy(), (dy * (x - m32) * r32).sum(0)) <= 2e-5
+    assert U.normwise(db.cpu().numpy(), dy.sum(0)) <= 2e-5
+    assert U.normwise(params[:N].cpu().numpy(), ds_ref) <= 2e-5
+    assert U.normwise(params[N:].cpu().numpy(), db_ref) <= 2e-5
+    assert _untouched(dxbuf, dtype, sy, N * C)
+
+
+@pytest.mark.parametrize("N,C,dtype,sx,sy,seed", _row_cases(40, 3))
+def test_l2_norm_rows(K, N, C, dtype, sx, sy, seed):
+    rng = np.random.default_rng(seed)
+    xb, x = _values(rng, (N, C), dtype)
+    dyb, dy = _values(rng, (N, C), dtype)
+    eps = 1e-12
+    nrm = np.sqrt((x * x).sum(1, keepdims=True))
+    nrm = np.maximum(nrm, eps)
+    _, xd = _held(N * C, dtype, sx, xb)
+    ybuf, yd = _held(N * C, dtype, sy)
+    K.l2_norm(N, 1, C, 1.0, eps, xd, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, C)
+    assert U.normwise(y, x / nrm) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, sy, N * C)
+    _, dyd = _held(N * C, dtype, sx, dyb)
+    dxbuf, dxd = _held(N * C, dtype, sy)
+    K.l2_norm_grad(N, 1, C, 1.0, eps, dyd, xd, dxd)
+    dx = U.widen(U.to_host(dxd.contiguous()), dtype).reshape(N, C)
+    dx_ref = dy / nrm - x * (dy * x).sum(1, keepdims=True) / nrm ** 3
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert _untouched(dxbuf, dtype, sy, N * C)
+
+
+def _channel_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        N = int(rng.integers(1, 7))
+        G = int(rng.choice((1, 2, 4, 8)))
+        D = int(rng.choice((1, 2, 3, 4, 16)))
+        S = int(rng.choice((1, 7, 49, 64, 196, 200, 1024, 1030, 3136, 4099)))
+        fmt = "NCHW" if rng.random() < 0.6 else "NHWC"
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        cases.append((N, G, D, S, fmt, dtype, 2000 + i))
+    return cases
+
+
+def _as_ncs(a, N, C, S, fmt):
+    """fp64 view [N, C, S] of a tensor stored in `fmt`."""
+    return a.reshape(N, C, S) if fmt == "NCHW" else a.reshape(N, S, C).transpose(0, 2, 1)
+
+
+@pytest.mark.parametrize("N,G,D,S,fmt,dtype,seed", _channel_cases(40, 4))
+def test_group_norm_shapes(K, N, G, D, S, fmt, dtype, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    C = G * D
+    n = N * C * S
+    xb, xs = _values(rng, (n,), dtype, 2.0)
+    dyb, dys = _values(rng, (n,), dtype)
+    x, dy = _as_ncs(xs, N, C, S, fmt), _as_ncs(dys, N, C, S, fmt)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    eps = 1e-5
+    xg = x.reshape(N, G, D * S)
+    mean = xg.mean(2)
+    rs = 1 / np.sqrt(((xg - mean[..., None]) ** 2).mean(2) + np.float64(np.float32(eps)))
+    mc, rc = np.repeat(mean, D, 1)[..., None], np.repeat(rs, D, 1)[..., None]
+    y_ref = (x - mc) * rc * g[None, :, None] + b[None, :, None]
+    _, xd = _held(n, dtype, 0, xb)
+    ybuf, yd = _held(n, dtype, 0)
+    gd, bd = torch.from_numpy(g).cuda(), torch.from_numpy(b).cuda()
+    mu, rsig = torch.empty(N * G, device="cuda"), torch.empty(N * G, device="cuda")
+    K.group_norm_forward(N, G, D, S, fmt, eps, xd, gd, bd, mu, rsig, yd)
+    y = _as_ncs(U.widen(U.to_host(yd.contiguous()), dtype), N, C, S, fmt)
+    assert _mean_ok(mu.cpu().numpy(), mean, x)
+    assert np.max(np.abs(rsig.cpu().numpy().astype(np.float64) / rs.ravel() - 1)) <= 5e-5
+    assert U.normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, 0, n)
+    m32 = np.repeat(mu.cpu().numpy().astype(np.float64).reshape(N, G), D, 1)[..., None]
+    r32 = np.repeat(rsig.cpu().numpy().astype(np.float64).reshape(N, G), D, 1)[..., None]
+    _, dyd = _held(n, dtype, 0, dyb)
+    dxbuf, dxd = _held(n, dtype, 0)
+    params = torch.empty(2 * N * G, device="cuda")
+    dg, db = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    K.group_norm_grad(N, G, D, S, fmt, xd, mu, rsig, gd, dyd, params, params, dg, db, dxd)
+    gc = g[None, :, None]
+    ds_ref = (gc * dy * x).reshape(N, G, D * S).sum(2)
+    db_ref = (gc * dy).reshape(N, G, D * S).sum(2)
+    dsc, dbc = np.repeat(ds_ref, D, 1)[..., None], np.repeat(db_ref, D, 1)[..., None]
+    dx_ref = gc * dy * r32 + ((dbc * m32 - dsc) * (x - m32) * r32 ** 3 - dbc * r32) / (D * S)
+    dx = _as_ncs(U.widen(U.to_host(dxd.contiguous()), dtype), N, C, S, fmt)
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(dg.cpu().numpy(), (dy * (x - m32) * r32).sum((0, 2))) <= 5e-5
+    assert U.normwise(db.cpu().numpy(), dy.sum((0, 2))) <= 5e-5
+    assert _untouched(dxbuf, dtype, 0, n)
+
+
+@pytest.mark.parametrize("N,G,D,S,fmt,dtype,seed", _channel_cases(40, 5))
+def test_batch_norm_training_shapes(K, N, G, D, S, fmt, dtype, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    C = G * D * int(rng.choice((1, 5, 16)))
+    if N * S < 2:
+        S = 2
+    n = N * C * S
+    xb, xs = _values(rng, (n,), dtype, 2.0)
+    dyb, dys = _values(rng, (n,), dtype)
+    x, dy = _as_ncs(xs, N, C, S, fmt), _as_ncs(dys, N, C, S, fmt)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    eps, momentum = 1e-5, 0.9
+    mean = x.mean((0, 2))
+    var = ((x - mean[None, :, None]) ** 2).mean((0, 2))
+    rs = 1 / np.sqrt(var + np.float64(np.float32(eps)))
+    y_ref = (x - mean[None, :, None]) * (rs * g)[None, :, None] + b[None, :, None]
+    _, xd = _held(n, dtype, 0, xb)
+    ybuf, yd = _held(n, dtype, 0)
+    gd, bd = torch.from_numpy(g).cuda(), torch.from_numpy(b).cuda()
+    rm0 = rng.standard_normal(C).astype(np.float32)
+    rv0 = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    rm, rv = torch.from_numpy(rm0.copy()).cuda(), torch.from_numpy(rv0.copy()).cuda()
+    mu, rsig = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    params = torch.empty(2 * C, device="cuda")
+    K.batch_norm_training_forward(N, C, S, fmt, momentum, eps, xd, gd, bd, rm, rv, mu, rsig, params, yd)
+    y = _as_ncs(U.widen(U.to_host(yd.contiguous()), dtype), N, C, S, fmt)
+    assert _mean_ok(mu.cpu().numpy(), mean, x)
+    assert np.max(np.abs(rsig.cpu().numpy().astype(np.float64) / rs - 1)) <= 5e-5
+    assert U.normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert U.normwise(rm.cpu().numpy(), momentum * rm0 + (1 - momentum) * mean) <= 2e-5
+    assert U.normwise(rv.cpu().numpy(), momentum * rv0 + (1 - momentum) * var) <= 5e-5
+    assert _untouched(ybuf, dtype, 0, n)
+    m32 = mu.cpu().numpy().astype(np.float64)[None, :, None]
+    r32 = rsig.cpu().numpy().astype(np.float64)[None, :, None]
+    _, dyd = _held(n, dtype, 0, dyb)
+    dxbuf, dxd = _held(n, dtype, 0)
+    wg = torch.empty(2 * C, device="cuda")
+    K.batch_norm_training_backward(N, C, S, float(N * S), fmt, xd, mu, rsig, gd, dyd, wg, wg, dxd)
+    xh = (x - m32) * r32
+    dg_ref, db_ref = (dy * xh).sum((0, 2)), dy.sum((0, 2))
+    dx_ref = (g[None, :, None] * r32) * (dy - (xh * dg_ref[None, :, None] + db_ref[None, :, None]) / (N * S))
+    dx = _as_ncs(U.widen(U.to_host(dxd.contiguous()), dtype), N, C, S, fmt)
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert U.normwise(wg[:C].cpu().numpy(), dg_ref) <= 5e-5
+    assert U.normwise(wg[C:].cpu().numpy(), db_ref) <= 5e-5
+    assert _untouched(dxbuf, dtype, 0, n)
