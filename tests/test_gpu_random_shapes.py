@@ -279,3 +279,123 @@ def test_batch_norm_training_shapes(K, N, G, D, S, fmt, dtype, seed):
     assert U.normwise(wg[:C].cpu().numpy(), dg_ref) <= 5e-5
     assert U.normwise(wg[C:].cpu().numpy(), db_ref) <= 5e-5
     assert _untouched(dxbuf, dtype, 0, n)
+
+
+def _strided_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        C = max(1, int(rng.choice((1, 2, 7, 21, 64, 150, 1024, 1030, 2051))) + int(rng.integers(-1, 2)))
+        S = max(2, int(rng.choice((2, 3, 8, 24, 70, 530, 4096))) + int(rng.integers(-1, 2)))
+        N = int(rng.integers(1, max(2, min(9, 1_200_000 // (C * S)))))
+        cases.append((N, C, S, DTYPES[int(rng.integers(0, 3))], 3000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,S,dtype,seed", _strided_cases(40, 6))
+def test_softmax_along_a_strided_axis(K, N, C, S, dtype, seed):
+    rng = np.random.default_rng(seed)
+    log = bool(seed & 1)
+    xb, x = _values(rng, (N, C, S), dtype, 3.0)
+    dyb, dy = _values(rng, (N, C, S), dtype)
+    e = np.exp(x - x.max(1, keepdims=True))
+    p = e / e.sum(1, keepdims=True)
+    n = N * C * S
+    _, xd = _held(n, dtype, 0, xb)
+    ybuf, yd = _held(n, dtype, 0)
+    (K.log_softmax if log else K.softmax)(N, S, C, xd, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, C, S)
+    if log:
+        assert np.max(np.abs(y - np.log(p)) / (1 + np.abs(np.log(p)))) <= U.TIGHT[dtype]
+    else:
+        assert U.rowwise_normwise(y, p, axis=1) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, 0, n)
+    _, dyd = _held(n, dtype, 0, dyb)
+    dxbuf, dxd = _held(n, dtype, 0)
+    (K.log_softmax_grad if log else K.softmax_grad)(N, S, C, dyd, yd, dxd)
+    dx = U.widen(U.to_host(dxd.contiguous()), dtype).reshape(N, C, S)
+    dx_ref = (dy - np.exp(y) * dy.sum(1, keepdims=True)) if log else \
+        (dy - (dy * y).sum(1, keepdims=True)) * y
+    assert U.normwise(dx, dx_ref) <= U.TIGHT[dtype]
+    assert _untouched(dxbuf, dtype, 0, n)
+
+
+def _moment_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        nd = int(rng.integers(1, 5))
+        dims = [int(rng.choice((1, 2, 3, 7, 16, 33, 64, 200, 1031))) for _ in range(nd)]
+        while int(np.prod(dims)) > 1_500_000:
+            dims[int(np.argmax(dims))] = max(1, max(dims) // 4)
+        k = int(rng.integers(1, nd + 1))
+        axes = sorted(int(a) for a in rng.choice(nd, size=k, replace=False))
+        cases.append((tuple(dims), tuple(axes), DTYPES[int(rng.integers(0, 3))], 4000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("dims,axes,dtype,seed", _moment_cases(50, 7))
+def test_moments_over_random_axes(K, dims, axes, dtype, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    xb = R.to_bits((rng.standard_normal(dims) * 2 + 0.5).astype(np.float32), dtype)
+    x = U.widen(xb, dtype).reshape(dims)
+    want_m, want_v = x.mean(axes), x.var(axes)
+    out = int(np.prod(want_m.shape)) if want_m.shape else 1
+    mean, var = torch.empty(out, device="cuda"), torch.empty(out, device="cuda")
+    K.moments(list(dims), list(axes), U.to_device(xb, dtype), mean, var)
+    scale = np.sqrt(np.mean(x ** 2)) + 1e-30
+    assert np.max(np.abs(mean.cpu().numpy() - want_m.ravel())) <= 2e-5 * scale
+    assert np.max(np.abs(var.cpu().numpy() - want_v.ravel())) <= 4e-5 * scale ** 2
+
+
+def _loss_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        C = max(2, int(rng.choice((2, 10, 21, 100, 1000, 4096, 32000))) + int(rng.integers(-1, 2)))
+        S = int(rng.choice((1, 1, 1, 5, 64)))
+        N = int(rng.integers(1, max(2, min(300, 600_000 // (C * S)))))
+        cases.append((N, C, S, ("none", "sum", "mean", "valid")[int(rng.integers(0, 4))],
+                      ("int64", "int32")[int(rng.integers(0, 2))], 5000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,S,reduction,tdtype,seed", _loss_cases(40, 8))
+def test_fused_softmax_cross_entropy_loss_shapes(K, N, C, S, reduction, tdtype, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    dtype = "float32"
+    x = (rng.standard_normal((N, C, S)) * 3).astype(np.float32)
+    target = rng.integers(0, C, (N, S)).astype(tdtype)
+    target[rng.random((N, S)) < 0.1] = 255 if C <= 255 else -1
+    ignore = 255 if C <= 255 else -1
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    p = e / e.sum(1, keepdims=True)
+    valid = target != ignore
+    safe = np.where(valid, target, 0).astype(np.int64)
+    picked = np.take_along_axis(p, safe[:, None, :], 1)[:, 0, :]
+    losses = np.where(valid, -np.log(np.maximum(picked, np.finfo(np.float32).tiny)), 0.0)
+    nvalid = max(int(valid.sum()), 1)
+    want = {"none": losses, "sum": losses.sum(), "mean": losses.sum() / (N * S),
+            "valid": losses.sum() / nvalid}[reduction]
+    xd, td = torch.from_numpy(x).cuda(), torch.from_numpy(target).cuda()
+    prob = torch.empty((N, C, S), device="cuda")
+    loss = torch.empty((N, S) if reduction == "none" else (1,), device="cuda")
+    K.softmax_cross_entropy_loss_forward(N, S, C, ignore, reduction, xd, td, prob, loss)
+    assert U.rowwise_normwise(prob.cpu().numpy(), p, axis=1) <= 1e-5
+    got = loss.cpu().numpy().reshape(np.shape(want))
+    assert np.max(np.abs(got - want)) <= 4e-5 * max(1.0, float(np.max(np.abs(want))))
+    dl = rng.standard_normal((N, S)).astype(np.float32) if reduction == "none" else np.float32(1.7)
+    dx = torch.empty((N, C, S), device="cuda")
+    K.softmax_cross_entropy_loss_backward(N, S, C, ignore, reduction, prob, td,
+                                          torch.from_numpy(np.atleast_1d(dl)).cuda(), dx)
+    ph = prob.cpu().numpy().astype(np.float64)
+    onehot = np.zeros((N, C, S))
+    np.put_along_axis(onehot, safe[:, None, :], 1.0, 1)
+    g = (ph - onehot) * valid[:, None, :]
+    w = {"none": np.asarray(dl, np.float64)[:, None, :] if reduction == "none" else 0,
+         "sum": 1.7, "mean": 1.7 / (N * S), "valid": 1.7 / nvalid}[reduction]
+    assert U.normwise(dx.cpu().numpy(), g * w) <= 1e-5
+    assert np.all(dx.cpu().numpy()[np.broadcast_to(~valid[:, None, :], (N, C, S))] == 0)
