@@ -1044,15 +1044,18 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
         }
       }
       if (Tile::active(i, npackets)) {
+        // gamma is one value per thread and slot: it multiplies the slot's sums once
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
+        A p1 = A(0), p2 = A(0);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const A t = gam[i] * dv[e];
-          s1 += t * xv[e];
-          s2 += t;
+          p1 += dv[e] * xv[e];
+          p2 += dv[e];
         }
+        s1 += gam[i] * p1;
+        s2 += gam[i] * p2;
       }
     }
     Tile::reduce_sum_pair(s1, s2, slots);
@@ -1060,8 +1063,9 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
       ds[row] = s1;
       db[row] = s2;
     }
-    const A u0 = (s2 * m - s1) * (r * r * r);
-    const A v0 = s2 * r;
+    // dx = gamma*rsig * dy + (u*(x - mu) - v) with the row's u, v divided by D*S once
+    const A u0 = (s2 * m - s1) * (r * r * r) * denom;
+    const A v0 = s2 * r * denom;
     tx.refresh();
     tdy.refresh();
 #pragma unroll
@@ -1071,13 +1075,15 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
+        const A gr = gam[i] * r;
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
           const A xc = xv[e] - m;
-          t1 += dv[e] * xc * r;
+          t1 += dv[e] * xc;
           t2 += dv[e];
-          xv[e] = gam[i] * dv[e] * r + (u0 * xc - v0) * denom;
+          xv[e] = gr * dv[e] + (u0 * xc - v0);
         }
+        t1 *= r;
         tx.store_slot(dx + row * L, i, xv);
       }
       if (next_valid) {
