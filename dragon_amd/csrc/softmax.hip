@@ -245,6 +245,260 @@ __global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const
   }
 }
 
+// A row of any width at any element-aligned address, as the aligned 16-byte
+// packets that cover it (its window): the window starts `lead` elements before
+// the row and its last packet holds `tail_valid` elements of the row. The
+// softmax gradient does not care which column an element is, so a row can be
+// read, reduced and written window packet by window packet: every access to HBM
+// is an aligned packet except the element-wise stores of a row's first and last
+// packet, whose other elements belong to the neighbouring rows. An aligned
+// packet that holds one byte of a tensor lies in the same page as that byte, so
+// reading all of it is safe at the tensor's ends too.
+template <typename T>
+struct RowWindow {
+  static constexpr int kVec = IO<T>::kVec;
+  int lead, packets, tail_valid;
+  __device__ __forceinline__ RowWindow(const T* row, int C) {
+    lead = static_cast<int>((reinterpret_cast<uintptr_t>(row) & 15u) / sizeof(T));
+    packets = (lead + C + kVec - 1) / kVec;
+    tail_valid = lead + C - (packets - 1) * kVec;  // 1 .. kVec
+  }
+};
+
+// softmax_wide_rows for rows that are not whole aligned packets, through their
+// windows; x and y must be congruent modulo 16 bytes. A window may be one packet
+// longer than the row has whole packets: the caller picks kVPT for C / kVec + 2
+// packets. What the window's first and last packet hold of the neighbouring rows
+// is set to -inf in the two lanes concerned before the row is reduced, so the
+// passes are those of rows of whole packets; those two packets go through LDS
+// and are stored element by element by the first threads of the workgroup.
+template <typename T, int kKind, int kVPT>
+__global__ __launch_bounds__(1024) void softmax_wide_windows(const int64_t N, const int C,
+                                                             const T* x, T* y) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT, kTPR, false>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  __shared__ u32x4 edge[2];
+  const int lane = threadIdx.x;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  auto request = [&](Raw& t, const int64_t at, const bool valid) {
+    const int64_t from = valid ? at : 0;
+    const RowWindow<T> w(x + from * C, C);
+    t.load(x + from * C - w.lead, w.packets, valid);
+  };
+  Raw cur;
+  request(cur, row, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    request(nxt, row + stride, row + stride < N);
+    const RowWindow<T> w(x + row * C, C);
+    const int tail_slot = (w.packets - 1) / kTPR, tail_lane = (w.packets - 1) % kTPR;
+    const bool head_partial = w.lead > 0 || (w.packets == 1 && w.tail_valid < kVec);
+    const bool tail_partial = w.packets > 1 && w.tail_valid < kVec;
+    auto keep = [&](u32x4& packet, const int first, const int last) {
+      A v[kVec];
+      IO<T>::unpack(packet, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (e < first || e >= last) v[e] = acc_neg_inf<A>();
+      }
+      packet = IO<T>::pack(v);
+    };
+    if (head_partial && lane == 0) keep(cur.p[0], w.lead, w.packets == 1 ? w.tail_valid : kVec);
+    if (tail_partial && lane == tail_lane) {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        if (i == tail_slot) keep(cur.p[i], 0, w.tail_valid);
+      }
+    }
+    Tile t;
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      cur.unpack(i, t.v[i]);
+      const bool on = Tile::active(i, w.packets);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = on ? t.v[i][e] : acc_neg_inf<A>();  // raw padding is zero bits
+        m = MaxOp()(m, t.v[i][e]);
+      }
+    }
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (kKind == kSoftmax) {
+          t.v[i][e] = M::exp_of(t.v[i][e] - m);
+          s += t.v[i][e];
+        } else {
+          t.v[i][e] = t.v[i][e] - m;
+          s += M::exp_of(t.v[i][e]);
+        }
+      }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    const A inv = A(1) / s;
+    const A l = acc_log(s);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = kKind == kSoftmax ? M::normalise(t.v[i][e], s, inv) : t.v[i][e] - l;
+      }
+    nxt.wait_ready();
+    cur = nxt;
+    T* base = y + row * C - w.lead;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int idx = i * kTPR + lane;
+      if (idx < w.packets) {
+        const u32x4 packet = IO<T>::pack(t.v[i]);
+        if (idx == 0 && head_partial) {
+          edge[0] = packet;
+        } else if (idx == w.packets - 1 && tail_partial) {
+          edge[1] = packet;
+        } else {
+          store_packet(base + static_cast<int64_t>(idx) * kVec, packet);
+        }
+      }
+    }
+    __syncthreads();  // slots are reused by the next row; the edge packets are in LDS
+    if (lane < 2 * kVec) {
+      const int which = lane / kVec, e = lane % kVec;
+      const T* from = reinterpret_cast<const T*>(&edge[which]);
+      if (which == 0 && head_partial) {
+        const int last = w.packets == 1 ? w.tail_valid : kVec;
+        if (e >= w.lead && e < last) base[e] = from[e];
+      } else if (which == 1 && tail_partial) {
+        if (e < w.tail_valid) base[static_cast<int64_t>(w.packets - 1) * kVec + e] = from[e];
+      }
+    }
+  }
+}
+
+// 16-bit rows of 4097 to 8192 packets that are not whole aligned packets (a
+// 50257-entry vocabulary), through their windows like softmax_wide_windows:
+// eight packets per thread of a 1024-thread workgroup do not leave room for
+// their 64 converted elements beside the next row's packets, so the row stays
+// in raw packets, which are converted in each of the three passes (the
+// exponential is taken twice), and the next row is requested ahead.
+template <typename T, int kKind>
+__global__ __launch_bounds__(1024) void softmax_wide_raw_windows(const int64_t N, const int C,
+                                                                 const T* x, T* y) {
+  constexpr int kTPR = 1024, kVPT = 8;
+  using Tile = RowTile<T, kTPR, kVPT, kTPR, false>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  __shared__ u32x4 edge[2];
+  const int lane = threadIdx.x;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  auto request = [&](Raw& t, const int64_t at, const bool valid) {
+    const int64_t from = valid ? at : 0;
+    const RowWindow<T> w(x + from * C, C);
+    t.load(x + from * C - w.lead, w.packets, valid);
+  };
+  Raw cur;
+  request(cur, row, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    request(nxt, row + stride, row + stride < N);
+    const RowWindow<T> w(x + row * C, C);
+    const int tail_slot = (w.packets - 1) / kTPR, tail_lane = (w.packets - 1) % kTPR;
+    const bool head_partial = w.lead > 0 || (w.packets == 1 && w.tail_valid < kVec);
+    const bool tail_partial = w.packets > 1 && w.tail_valid < kVec;
+    auto keep = [&](u32x4& packet, const int first, const int last) {
+      A v[kVec];
+      IO<T>::unpack(packet, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (e < first || e >= last) v[e] = acc_neg_inf<A>();
+      }
+      packet = IO<T>::pack(v);
+    };
+    if (head_partial && lane == 0) keep(cur.p[0], w.lead, w.packets == 1 ? w.tail_valid : kVec);
+    if (tail_partial && lane == tail_lane) {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        if (i == tail_slot) keep(cur.p[i], 0, w.tail_valid);
+      }
+    }
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      cur.unpack(i, v);
+      if (Tile::active(i, w.packets)) {  // slots beyond the window hold zero bits
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) m = MaxOp()(m, v[e]);
+      }
+    }
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    cur.refresh();
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      cur.unpack(i, v);
+      if (Tile::active(i, w.packets)) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) s += M::exp_of(v[e] - m);  // exp(-inf) = 0 beside the row
+      }
+    }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    cur.refresh();
+    const A inv = A(1) / s;
+    const A l = acc_log(s);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A v[kVec];
+      cur.unpack(i, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A d = v[e] - m;
+        v[e] = kKind == kSoftmax ? M::normalise(M::exp_of(d), s, inv) : d - l;
+      }
+      cur.p[i] = IO<T>::pack(v);
+    }
+    nxt.wait_ready();
+    T* base = y + row * C - w.lead;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int idx = i * kTPR + lane;
+      if (idx < w.packets) {
+        if (idx == 0 && head_partial) {
+          edge[0] = cur.p[i];
+        } else if (idx == w.packets - 1 && tail_partial) {
+          edge[1] = cur.p[i];
+        } else {
+          store_packet(base + static_cast<int64_t>(idx) * kVec, cur.p[i]);
+        }
+      }
+    }
+    cur = nxt;
+    __syncthreads();  // slots are reused by the next row; the edge packets are in LDS
+    if (lane < 2 * kVec) {
+      const int which = lane / kVec, e = lane % kVec;
+      const T* from = reinterpret_cast<const T*>(&edge[which]);
+      if (which == 0 && head_partial) {
+        const int last = w.packets == 1 ? w.tail_valid : kVec;
+        if (e >= w.lead && e < last) base[e] = from[e];
+      } else if (which == 1 && tail_partial) {
+        if (e < w.tail_valid) base[static_cast<int64_t>(w.packets - 1) * kVec + e] = from[e];
+      }
+    }
+  }
+}
+
 template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
     const int64_t N, const int C, const T* dy, const T* y, T* dx) {
@@ -441,6 +695,129 @@ __global__ __launch_bounds__(1024) void softmax_grad_wide_rows(const int64_t N, 
     }
     if (kPrefetch) tg = ng, to = no;
     __syncthreads();  // slots are reused by the next row
+  }
+}
+
+// softmax_grad_wide_rows for rows that are not whole aligned packets, through
+// their windows: dy, y and dx must be congruent modulo 16 bytes. A window may be
+// one packet longer than the row has whole packets: the caller picks kVPT for
+// C / kVec + 2 packets. Without it such rows take two passes over dy and y.
+template <typename T, int kKind, int kVPT, bool kPrefetch>
+__global__ __launch_bounds__(1024) void softmax_grad_wide_windows(const int64_t N, const int C,
+                                                                  const T* dy, const T* y, T* dx) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  using M = SoftmaxMath<T>;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[Tile::kSlots];
+  __shared__ u32x4 edge[2];
+  const int lane = threadIdx.x;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  auto request = [&](Raw& g, Raw& o, const int64_t at, const bool valid) {
+    const int64_t from = valid ? at : 0;
+    const RowWindow<T> w(dy + from * C, C);
+    g.load(dy + from * C - w.lead, w.packets, valid);
+    o.load(y + from * C - w.lead, w.packets, valid);
+  };
+  Raw tg, to;
+  if (kPrefetch) request(tg, to, row, row < N);
+  for (; row < N; row += stride) {
+    Raw ng, no;
+    if (kPrefetch) {
+      request(ng, no, row + stride, row + stride < N);
+    } else {
+      request(tg, to, row, true);
+    }
+    const RowWindow<T> w(dy + row * C, C);
+    const int tail_slot = (w.packets - 1) / kTPR, tail_lane = (w.packets - 1) % kTPR;
+    const bool head_partial = w.lead > 0 || (w.packets == 1 && w.tail_valid < kVec);
+    const bool tail_partial = w.packets > 1 && w.tail_valid < kVec;
+    // What the window's first and last packet hold of the neighbouring rows is zeroed in
+    // the two lanes concerned before the row is summed (slots beyond the window hold zero
+    // bits already), so the passes below are those of rows of whole packets.
+    auto keep = [&](u32x4& packet, const int first, const int last) {
+      A v[kVec];
+      IO<T>::unpack(packet, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (e < first || e >= last) v[e] = A(0);
+      }
+      packet = IO<T>::pack(v);
+    };
+    if (head_partial && lane == 0) {
+      const int last = w.packets == 1 ? w.tail_valid : kVec;
+      keep(tg.p[0], w.lead, last);
+      keep(to.p[0], w.lead, last);
+    }
+    if (tail_partial && lane == tail_lane) {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        if (i == tail_slot) {
+          keep(tg.p[i], 0, w.tail_valid);
+          keep(to.p[i], 0, w.tail_valid);
+        }
+      }
+    }
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A g[kVec], o[kVec];
+      tg.unpack(i, g);
+      to.unpack(i, o);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s += kKind == kSoftmax ? g[e] * o[e] : g[e];
+    }
+    s = Tile::reduce(s, SumOp(), slots);
+    tg.refresh();
+    to.refresh();
+    // the results replace the packets of dy: no third set of registers
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      A g[kVec], o[kVec];
+      tg.unpack(i, g);
+      to.unpack(i, o);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        g[e] = kKind == kSoftmax ? (g[e] - s) * o[e] : g[e] - M::exp_of(o[e]) * s;
+      }
+      tg.p[i] = IO<T>::pack(g);
+    }
+    if (kPrefetch) {
+      ng.wait_ready();
+      no.wait_ready();
+    }
+    // Whole packets of the row are stored as they are; the window's first and last
+    // packet, when they also hold elements of the neighbouring rows, go through LDS
+    // and are stored element by element by the first threads of the workgroup.
+    T* base = dx + row * C - w.lead;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int idx = i * kTPR + lane;
+      if (idx < w.packets) {
+        if (idx == 0 && head_partial) {
+          edge[0] = tg.p[i];
+        } else if (idx == w.packets - 1 && tail_partial) {
+          edge[1] = tg.p[i];
+        } else {
+          store_packet(base + static_cast<int64_t>(idx) * kVec, tg.p[i]);
+        }
+      }
+    }
+    if (kPrefetch) tg = ng, to = no;
+    __syncthreads();  // slots are reused by the next row; the edge packets are in LDS
+    if (lane < 2 * kVec) {
+      const int which = lane / kVec, e = lane % kVec;
+      const T* from = reinterpret_cast<const T*>(&edge[which]);
+      if (which == 0 && head_partial) {
+        const int last = w.packets == 1 ? w.tail_valid : kVec;
+        if (e >= w.lead && e < last) base[e] = from[e];
+      } else if (which == 1 && tail_partial) {
+        if (e < w.tail_valid) base[static_cast<int64_t>(w.packets - 1) * kVec + e] = from[e];
+      }
+    }
   }
 }
 
@@ -1230,6 +1607,35 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
     // 1024-thread tiles: persistent workgroups that prefetch the next row
     // (not the ragged flavour of eight 16-bit packets per thread: 64 converted
     // elements beside the next row's packets do not fit 128 registers)
+    // 16-bit rows beyond four packets per thread that are not whole aligned packets: raw
+    // packets through windows, the next row ahead (rows of whole packets measured 4% faster
+    // with their converted elements held, softmax_wide_rows below)
+    if (sizeof(T) == 2 && !regular && congruent16(x, y) && C / kVec + 2 > 4 * 1024 &&
+        C / kVec + 2 <= 8 * 1024) {
+      if constexpr (sizeof(T) == 2) {
+        auto kernel = softmax_wide_raw_windows<T, kKind>;
+        const unsigned resident = resident_grid(kernel, 1024, 0);
+        const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), xp, yp);
+        return status_of_launch();
+      }
+    }
+    // rows of 1024-thread size that are not whole aligned packets: the same through windows
+    RowConfig wcfg;
+    if (!regular && sizeof(T) <= 4 && congruent16(x, y) &&
+        pick_row_config(C / kVec + 2, 8, &wcfg) && wcfg.tpr == 1024 &&
+        !(wcfg.vpt == 8 && sizeof(T) == 2)) {
+#define LAUNCH_WINDOWS(VPT)                                                                  \
+  {                                                                                          \
+    auto kernel = softmax_wide_windows<T, kKind, VPT>;                                       \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), xp, yp); \
+  }
+      if (wcfg.vpt == 2) LAUNCH_WINDOWS(2) else if (wcfg.vpt == 4) LAUNCH_WINDOWS(4) else LAUNCH_WINDOWS(8)
+#undef LAUNCH_WINDOWS
+      return status_of_launch();
+    }
     if (cfg.tpr == 1024 && (regular || (N > 1 && !(cfg.vpt == 8 && sizeof(T) == 2)))) {
       // ragged rows: all but the last here (whole packets may read past a row's
       // end), the last one through the element-exact tile below
@@ -1363,6 +1769,22 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
     if (cfg.vpt == 2) LAUNCH_WIDE(2, true) else if (cfg.vpt == 4) LAUNCH_WIDE(4, true)
     else LAUNCH_WIDE(8, false)
 #undef LAUNCH_WIDE
+    return status_of_launch();
+  }
+  // rows of 1024-thread size that are not whole aligned packets: the same through windows
+  if (S == 1 && !regular && sizeof(T) <= 4 && congruent16(dy, y) && congruent16(dy, dx) &&
+      pick_row_config(C / kVec + 2, 8, &cfg) && cfg.tpr == 1024) {
+#define LAUNCH_WINDOWS(VPT, PREFETCH)                                                        \
+  {                                                                                          \
+    auto kernel = softmax_grad_wide_windows<T, kKind, VPT, PREFETCH>;                        \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C), gp, yp, \
+                       dp);                                                                  \
+  }
+    if (cfg.vpt == 2) LAUNCH_WINDOWS(2, true) else if (cfg.vpt == 4) LAUNCH_WINDOWS(4, true)
+    else LAUNCH_WINDOWS(8, false)
+#undef LAUNCH_WINDOWS
     return status_of_launch();
   }
   // Two tiles live at once: halve the packets a thread may hold.

@@ -203,7 +203,7 @@ def test_softmax_forward_backward(K, shape, axis, dtype, log):
 
 
 @pytest.mark.parametrize("shape", [(64, 512), (7, 197), (2, 66001), (2, 66000), (3, 10, 33),
-                                   (2, 1300, 20)])
+                                   (2, 1300, 20), (3, 30522), (2, 50257)])
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_softmax_in_place(K, dtype, shape):
     x, dy = _softmax_inputs(shape, dtype, 5)
@@ -318,10 +318,11 @@ def test_softmax_short_rows_at_shifted_bases(K, dtype, shift_x, shift_y):
 @pytest.mark.parametrize("shift_x,shift_y", [(0, 0), (3, 3), (1, 0)])
 def test_softmax_wide_rows_that_are_not_whole_packets(K, C, dtype, shift_x, shift_y, log):
     """Vocabulary-sized rows whose width or base address is not a multiple of 16 bytes (the
-    ragged register tiles, 1024 threads per row and up to sixteen packets per thread), with
-    equal and unequal shifts of input and output. What surrounds the input is poisoned with a
-    huge logit that must not leak into a row; forward against fp64, and nothing outside the
-    output may be written."""
+    ragged register tiles, 1024 threads per row and up to sixteen packets per thread; in the
+    backward pass, with congruent tensors, the aligned packets that cover a row), with equal
+    and unequal shifts of input and output. What surrounds the inputs is poisoned (a huge
+    logit, NaN for the backward) and must not leak into a row; against fp64, and nothing
+    outside the outputs may be written."""
     N = 5
     shape = (N, C)
     x, _ = _softmax_inputs(shape, dtype, 31)
@@ -351,6 +352,21 @@ def test_softmax_wide_rows_that_are_not_whole_packets(K, C, dtype, shift_x, shif
     else:
         assert U.rowwise_normwise(yw, y_ref) <= U.TIGHT[dtype]
     flat = U.widen(U.to_host(ybuf), dtype).ravel()
+    assert np.all(flat[:shift_y] == -7.0) and np.all(flat[shift_y + N * C:] == -7.0)
+    # backward from the forward's own output; what surrounds dy and y is NaN and must not
+    # reach a row's sum
+    _, dyb = _softmax_inputs(shape, dtype, 32)
+    dy64 = np.asarray(U.widen(dyb, dtype), np.float64).reshape(shape)
+    _, dyd = shifted(shift_x, dyb, fill=float("nan"))
+    _, yin = shifted(shift_x, U.to_host(y.contiguous()).reshape(shape), fill=float("nan"))
+    dxbuf, dx = shifted(shift_y, fill=-7.0)
+    (K.log_softmax_grad if log else K.softmax_grad)(N, 1, C, dyd, yin, dx)
+    dxw = U.widen(U.to_host(dx.contiguous()), dtype).reshape(shape)
+    dx_ref = (dy64 - np.exp(yw) * dy64.sum(1, keepdims=True)) if log else \
+        (dy64 - (dy64 * yw).sum(1, keepdims=True)) * yw
+    assert np.all(np.isfinite(dxw))
+    assert U.normwise(dxw, dx_ref) <= U.TIGHT[dtype]
+    flat = U.widen(U.to_host(dxbuf), dtype).ravel()
     assert np.all(flat[:shift_y] == -7.0) and np.all(flat[shift_y + N * C:] == -7.0)
 
 
