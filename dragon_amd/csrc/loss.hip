@@ -487,6 +487,73 @@ __global__ __launch_bounds__(kLossThreads) void softmax_ce_backward(
   }
 }
 
+// The same for S == 1 in whole packets: a workgroup takes chunks of kLossThreads * 4
+// consecutive packets (16 KB) and requests a thread's four packets, and their rows'
+// targets, before it uses the first; the row of a packet comes from one division per chunk
+// and a 32-bit one per packet.
+template <typename T, typename TargetT, bool kPerPosition>
+__global__ __launch_bounds__(kLossThreads) void softmax_ce_backward_chunks(
+    const int64_t npackets, const int64_t C, const int64_t ignore_index,
+    const T* __restrict__ prob, const TargetT* __restrict__ target, const T* __restrict__ dl,
+    const T* __restrict__ scale, T* __restrict__ dx) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  constexpr int kBatch = 4;
+  constexpr int64_t kChunk = static_cast<int64_t>(kLossThreads) * kBatch;
+  const A alpha = kPerPosition ? A(0) : static_cast<A>(scale[0]);
+  for (int64_t c0 = static_cast<int64_t>(blockIdx.x) * kChunk; c0 < npackets;
+       c0 += static_cast<int64_t>(gridDim.x) * kChunk) {
+    const int64_t n0 = c0 * kVec / C;                       // uniform over the workgroup
+    const uint32_t k_start = static_cast<uint32_t>(c0 * kVec - n0 * C);
+    u32x4 raw[kBatch];
+    int64_t rn[kBatch];
+    uint32_t rk[kBatch];
+    TargetT tg[kBatch];
+    A wl[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int64_t p = c0 + j * kLossThreads + threadIdx.x;
+      const bool on = p < npackets;
+      raw[j] = load_packet(prob + (on ? p : c0) * kVec);
+      const uint32_t k = k_start + static_cast<uint32_t>(on ? j * kLossThreads + threadIdx.x : 0) * kVec;
+      const uint32_t dn = k / static_cast<uint32_t>(C);
+      rn[j] = n0 + dn;
+      rk[j] = k - dn * static_cast<uint32_t>(C);
+      tg[j] = target[rn[j]];
+      wl[j] = kPerPosition ? static_cast<A>(dl[rn[j]]) : alpha;
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int64_t p = c0 + j * kLossThreads + threadIdx.x;
+      if (p >= npackets) continue;
+      A v[kVec];
+      IO<T>::unpack(raw[j], v);
+      if (rk[j] + kVec <= C) {  // the packet lies within one row
+        const bool valid = target_valid(tg[j], ignore_index, C);
+        const A w = valid ? wl[j] : A(0);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A hot = (valid && static_cast<int64_t>(rk[j]) + e == static_cast<int64_t>(tg[j])) ? A(1) : A(0);
+          v[e] = (v[e] - hot) * w;
+        }
+      } else {  // C is not a multiple of the packet: this one straddles two rows
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const bool next = rk[j] + e >= C;
+          const int64_t ne = rn[j] + (next ? 1 : 0);
+          const int64_t ke = static_cast<int64_t>(rk[j]) + e - (next ? C : 0);
+          const TargetT tgt = target[ne];
+          const bool valid = target_valid(tgt, ignore_index, C);
+          const A w = valid ? (kPerPosition ? static_cast<A>(dl[ne]) : alpha) : A(0);
+          const A hot = (valid && ke == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+          v[e] = (v[e] - hot) * w;
+        }
+      }
+      pack_store<T>(dx + p * kVec, v);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ launchers
 
 inline unsigned loss_grid(int64_t work_items) {
@@ -748,7 +815,20 @@ int launch_fused_backward(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
   hipLaunchKernelGGL((softmax_ce_backward<T, TargetT, VEC, ALONG_C, PER_POS>),                 \
                      dim3(loss_grid(total / VEC)), dim3(kLossThreads), 0, stream, total / VEC, \
                      S, C, ignore_index, pp, tp, dlp, scalar, dp)
-  if (S == 1 && total % kVec == 0 && aligned) {
+  if (S == 1 && total % kVec == 0 && aligned && C >= kVec && C < (int64_t(1) << 30)) {
+    // a packet touches two rows at most, and a chunk's offsets fit 32 bits
+    const int64_t npackets = total / kVec;
+    const int64_t chunks = ceil_div(npackets, static_cast<int64_t>(kLossThreads) * 4);
+    const int64_t cap = static_cast<int64_t>(num_cus()) * 64;
+    const dim3 grid(static_cast<unsigned>(chunks < cap ? chunks : cap));
+    if (reduction == kNone) {
+      hipLaunchKernelGGL((softmax_ce_backward_chunks<T, TargetT, true>), grid, dim3(kLossThreads), 0,
+                         stream, npackets, C, ignore_index, pp, tp, dlp, scalar, dp);
+    } else {
+      hipLaunchKernelGGL((softmax_ce_backward_chunks<T, TargetT, false>), grid, dim3(kLossThreads),
+                         0, stream, npackets, C, ignore_index, pp, tp, dlp, scalar, dp);
+    }
+  } else if (S == 1 && total % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, true, true); else LAUNCH(kVec, true, false);
   } else if (S > 1 && S % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, false, true); else LAUNCH(kVec, false, false);
