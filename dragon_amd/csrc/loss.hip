@@ -422,6 +422,126 @@ __global__ __launch_bounds__(1024) void softmax_ce_wide_rows(
   }
 }
 
+// softmax_ce_wide_rows for rows that are not whole aligned packets, through the
+// aligned packets that cover a row (RowWindow; x and prob congruent modulo 16
+// bytes; the caller picks kVPT for C / kVec + 2 packets). What the window's
+// first and last packet hold of the neighbouring rows is set to -inf in the two
+// lanes concerned before the row is reduced; those two packets of the output go
+// through LDS and are stored element by element. The target's column moves by
+// the window's lead.
+template <typename T, typename TargetT, int kVPT>
+__global__ __launch_bounds__(1024) void softmax_ce_wide_windows(
+    const int64_t N, const int C, const int64_t ignore_index, const T* __restrict__ x,
+    const TargetT* __restrict__ target, T* __restrict__ prob, T* __restrict__ loss,
+    T* __restrict__ mask) {
+  constexpr int kTPR = 1024;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  __shared__ u32x4 edge[2];
+  const int lane = threadIdx.x;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  auto request = [&](Raw& t, const int64_t at, const bool valid) {
+    const int64_t from = valid ? at : 0;
+    const RowWindow<T> w(x + from * C, C);
+    t.load(x + from * C - w.lead, w.packets, valid);
+  };
+  Raw cur;
+  request(cur, row, row < N);
+  for (; row < N; row += stride) {
+    Raw nxt;
+    request(nxt, row + stride, row + stride < N);
+    const RowWindow<T> w(x + row * C, C);
+    const int tail_slot = (w.packets - 1) / kTPR, tail_lane = (w.packets - 1) % kTPR;
+    const bool head_partial = w.lead > 0 || (w.packets == 1 && w.tail_valid < kVec);
+    const bool tail_partial = w.packets > 1 && w.tail_valid < kVec;
+    auto keep = [&](u32x4& packet, const int first, const int last) {
+      A v[kVec];
+      IO<T>::unpack(packet, v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (e < first || e >= last) v[e] = acc_neg_inf<A>();
+      }
+      packet = IO<T>::pack(v);
+    };
+    if (head_partial && lane == 0) keep(cur.p[0], w.lead, w.packets == 1 ? w.tail_valid : kVec);
+    if (tail_partial && lane == tail_lane) {
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        if (i == tail_slot) keep(cur.p[i], 0, w.tail_valid);
+      }
+    }
+    const TargetT tgt = target[row];
+    Tile t;
+    A m = acc_neg_inf<A>();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      cur.unpack(i, t.v[i]);
+      const bool on = Tile::active(i, w.packets);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = on ? t.v[i][e] : acc_neg_inf<A>();  // raw padding is zero bits
+        m = MaxOp()(m, t.v[i][e]);
+      }
+    }
+    m = Tile::reduce(m, MaxOp(), slots[0]);
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = acc_exp(t.v[i][e] - m);
+        s += t.v[i][e];
+      }
+    s = Tile::reduce(s, SumOp(), slots[1]);
+    const bool valid = target_valid(tgt, ignore_index, C);
+    const int col = valid ? static_cast<int>(tgt) + w.lead : -1;  // from the window's start
+    const A inv = A(1) / s;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        t.v[i][e] = sizeof(A) == 4 ? t.v[i][e] * inv : t.v[i][e] / s;
+        if ((i * kTPR + lane) * kVec + e == col) {
+          loss[row] = neg_log_clamped(t.v[i][e]);
+          mask[row] = T(1);
+        }
+      }
+    if (!valid && lane == 0) loss[row] = mask[row] = T(0);
+    nxt.wait_ready();
+    cur = nxt;
+    T* base = prob + row * C - w.lead;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int idx = i * kTPR + lane;
+      if (idx < w.packets) {
+        const u32x4 packet = IO<T>::pack(t.v[i]);
+        if (idx == 0 && head_partial) {
+          edge[0] = packet;
+        } else if (idx == w.packets - 1 && tail_partial) {
+          edge[1] = packet;
+        } else {
+          store_packet(base + static_cast<int64_t>(idx) * kVec, packet);
+        }
+      }
+    }
+    __syncthreads();  // slots are reused by the next row; the edge packets are in LDS
+    if (lane < 2 * kVec) {
+      const int which = lane / kVec, e = lane % kVec;
+      const T* from = reinterpret_cast<const T*>(&edge[which]);
+      if (which == 0 && head_partial) {
+        const int last = w.packets == 1 ? w.tail_valid : kVec;
+        if (e >= w.lead && e < last) base[e] = from[e];
+      } else if (which == 1 && tail_partial) {
+        if (e < w.tail_valid) base[static_cast<int64_t>(w.packets - 1) * kVec + e] = from[e];
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ fused backward
 
 // dx = (p - [k == target]) * w over [N, C, S], with w = 0 where the target is
@@ -727,6 +847,20 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
   }
       if (cfg.vpt == 2) LAUNCH_WIDE(2) else if (cfg.vpt == 4) LAUNCH_WIDE(4) else LAUNCH_WIDE(8)
 #undef LAUNCH_WIDE
+    } else if (RowConfig wcfg; !regular && congruent16(x, prob) &&
+               pick_row_config(C / kVec + 2, 8, &wcfg) && wcfg.tpr == 1024) {
+      // rows of 1024-thread size that are not whole aligned packets: through their windows
+#define LAUNCH_WINDOWS(VPT)                                                                     \
+  {                                                                                             \
+    auto kernel = softmax_ce_wide_windows<T, TargetT, VPT>;                                     \
+    const unsigned resident = resident_grid(kernel, 1024, 0);                                   \
+    const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(1024), 0, stream, N, static_cast<int>(C),       \
+                       ignore_index, xp, tp, pp, loss, mask);                                   \
+  }
+      if (wcfg.vpt == 2) LAUNCH_WINDOWS(2) else if (wcfg.vpt == 4) LAUNCH_WINDOWS(4)
+      else LAUNCH_WINDOWS(8)
+#undef LAUNCH_WINDOWS
     } else {
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \

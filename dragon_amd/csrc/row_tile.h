@@ -287,6 +287,27 @@ struct RawRowTile {
   }
 };
 
+// A row of any width at any element-aligned address, as the aligned 16-byte
+// packets that cover it (its window): the window starts `lead` elements before
+// the row and its last packet holds `tail_valid` elements of the row. Where a
+// kernel does not care which column an element is (softmax and its gradient;
+// the fused loss adds `lead` to the target's column), a row can be read,
+// reduced and written window packet by window packet: every access to HBM
+// is an aligned packet except the element-wise stores of a row's first and last
+// packet, whose other elements belong to the neighbouring rows. An aligned
+// packet that holds one byte of a tensor lies in the same page as that byte, so
+// reading all of it is safe at the tensor's ends too.
+template <typename T>
+struct RowWindow {
+  static constexpr int kVec = IO<T>::kVec;
+  int lead, packets, tail_valid;
+  __device__ __forceinline__ RowWindow(const T* row, int C) {
+    lead = static_cast<int>((reinterpret_cast<uintptr_t>(row) & 15u) / sizeof(T));
+    packets = (lead + C + kVec - 1) / kVec;
+    tail_valid = lead + C - (packets - 1) * kVec;  // 1 .. kVec
+  }
+};
+
 // How many neighbouring rows a forward row kernel holds per thread group at a
 // time. A wavefront that holds a whole row in one or two packets per lane takes
 // two: the dependent cross-lane reduction steps of the two rows interleave

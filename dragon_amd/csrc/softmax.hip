@@ -245,26 +245,6 @@ __global__ __launch_bounds__(1024) void softmax_wide_rows(const int64_t N, const
   }
 }
 
-// A row of any width at any element-aligned address, as the aligned 16-byte
-// packets that cover it (its window): the window starts `lead` elements before
-// the row and its last packet holds `tail_valid` elements of the row. The
-// softmax gradient does not care which column an element is, so a row can be
-// read, reduced and written window packet by window packet: every access to HBM
-// is an aligned packet except the element-wise stores of a row's first and last
-// packet, whose other elements belong to the neighbouring rows. An aligned
-// packet that holds one byte of a tensor lies in the same page as that byte, so
-// reading all of it is safe at the tensor's ends too.
-template <typename T>
-struct RowWindow {
-  static constexpr int kVec = IO<T>::kVec;
-  int lead, packets, tail_valid;
-  __device__ __forceinline__ RowWindow(const T* row, int C) {
-    lead = static_cast<int>((reinterpret_cast<uintptr_t>(row) & 15u) / sizeof(T));
-    packets = (lead + C + kVec - 1) / kVec;
-    tail_valid = lead + C - (packets - 1) * kVec;  // 1 .. kVec
-  }
-};
-
 // softmax_wide_rows for rows that are not whole aligned packets, through their
 // windows; x and y must be congruent modulo 16 bytes. A window may be one packet
 // longer than the row has whole packets: the caller picks kVPT for C / kVec + 2

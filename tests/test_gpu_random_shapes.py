@@ -353,7 +353,7 @@ def _loss_cases(count, seed):
     rng = np.random.default_rng(seed)
     cases = []
     for i in range(count):
-        C = max(2, int(rng.choice((2, 10, 21, 100, 1000, 4096, 32000))) + int(rng.integers(-1, 2)))
+        C = max(2, int(rng.choice((2, 10, 21, 100, 1000, 4096, 20001, 30522, 32000))) + int(rng.integers(-1, 2)))
         S = int(rng.choice((1, 1, 1, 5, 64)))
         N = int(rng.integers(1, max(2, min(300, 600_000 // (C * S)))))
         cases.append((N, C, S, ("none", "sum", "mean", "valid")[int(rng.integers(0, 4))],
@@ -399,3 +399,36 @@ def test_fused_softmax_cross_entropy_loss_shapes(K, N, C, S, reduction, tdtype, 
          "sum": 1.7, "mean": 1.7 / (N * S), "valid": 1.7 / nvalid}[reduction]
     assert U.normwise(dx.cpu().numpy(), g * w) <= 1e-5
     assert np.all(dx.cpu().numpy()[np.broadcast_to(~valid[:, None, :], (N, C, S))] == 0)
+
+
+@pytest.mark.parametrize("C", [20001, 30522, 32002])
+@pytest.mark.parametrize("shift", [0, 1, 3])
+def test_fused_loss_on_wide_rows_at_shifted_bases(K, C, shift):
+    """Vocabulary-sized fp32 rows that are not whole packets, logits and probabilities starting
+    `shift` elements past a 16-byte boundary: the rows go through the aligned packets that cover
+    them, the target's column moves with the window, and what surrounds the logits (a huge
+    value) must not reach a row."""
+    import torch
+    N = 6
+    rng = np.random.default_rng(C + shift)
+    x = (rng.standard_normal((N, C)) * 3).astype(np.float32)
+    target = rng.integers(0, C, N).astype(np.int64)
+    target[1] = -1
+    target[2], target[3] = 0, C - 1  # the row's first and last class: the window's edge packets
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    p = e / e.sum(1, keepdims=True)
+    valid = target != -1
+    picked = p[np.arange(N), np.where(valid, target, 0)]
+    want = np.where(valid, -np.log(picked), 0.0)
+    xbuf = torch.full((N * C + shift + GUARD,), 3e4, device="cuda")
+    xd = xbuf[shift:shift + N * C]
+    xd.copy_(torch.from_numpy(x.ravel()).cuda())
+    pbuf, pd = _held(N * C, "float32", shift)
+    loss = torch.empty(N, device="cuda")
+    K.softmax_cross_entropy_loss_forward(N, 1, C, -1, "none", xd, torch.from_numpy(target).cuda(),
+                                         pd, loss)
+    got = pd.contiguous().cpu().numpy().reshape(N, C)
+    assert U.rowwise_normwise(got, p) <= 1e-5
+    assert np.max(np.abs(loss.cpu().numpy() - want)) <= 4e-5 * max(1.0, float(want.max()))
+    assert _untouched(pbuf, "float32", shift, N * C)
