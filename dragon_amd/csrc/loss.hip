@@ -674,6 +674,56 @@ __global__ __launch_bounds__(kLossThreads) void softmax_ce_backward_chunks(
   }
 }
 
+// The same for a class axis in the middle (S > 1, a multiple of the packet): the packet runs
+// along S, so its elements share a class and belong to kVec consecutive positions.
+template <typename T, typename TargetT, bool kPerPosition>
+__global__ __launch_bounds__(kLossThreads) void softmax_ce_backward_chunks_strided(
+    const int64_t npackets, const uint32_t S, const uint32_t C, const int64_t ignore_index,
+    const T* __restrict__ prob, const TargetT* __restrict__ target, const T* __restrict__ dl,
+    const T* __restrict__ scale, T* __restrict__ dx) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  constexpr int kBatch = 4;
+  constexpr int64_t kChunk = static_cast<int64_t>(kLossThreads) * kBatch;
+  const A alpha = kPerPosition ? A(0) : static_cast<A>(scale[0]);
+  const uint32_t CS = C * S;  // the caller keeps it below 2^30
+  for (int64_t c0 = static_cast<int64_t>(blockIdx.x) * kChunk; c0 < npackets;
+       c0 += static_cast<int64_t>(gridDim.x) * kChunk) {
+    const int64_t n0 = c0 * kVec / CS;  // uniform over the workgroup
+    const uint32_t rem0 = static_cast<uint32_t>(c0 * kVec - n0 * CS);
+    u32x4 raw[kBatch];
+    uint32_t rk[kBatch];
+    int64_t pos[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int64_t p = c0 + j * kLossThreads + threadIdx.x;
+      const bool on = p < npackets;
+      raw[j] = load_packet(prob + (on ? p : c0) * kVec);
+      uint32_t r = rem0 + static_cast<uint32_t>(on ? j * kLossThreads + threadIdx.x : 0) * kVec;
+      const uint32_t dn = r / CS;
+      r -= dn * CS;
+      rk[j] = r / S;
+      pos[j] = (n0 + dn) * S + (r - rk[j] * S);
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int64_t p = c0 + j * kLossThreads + threadIdx.x;
+      if (p >= npackets) continue;
+      A v[kVec];
+      IO<T>::unpack(raw[j], v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const TargetT tgt = target[pos[j] + e];
+        const bool valid = target_valid(tgt, ignore_index, C);
+        const A w = valid ? (kPerPosition ? static_cast<A>(dl[pos[j] + e]) : alpha) : A(0);
+        const A hot = (valid && static_cast<int64_t>(rk[j]) == static_cast<int64_t>(tgt)) ? A(1) : A(0);
+        v[e] = (v[e] - hot) * w;
+      }
+      pack_store<T>(dx + p * kVec, v);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ launchers
 
 inline unsigned loss_grid(int64_t work_items) {
@@ -964,6 +1014,20 @@ int launch_fused_backward(int64_t N, int64_t S, int64_t C, int64_t ignore_index,
     }
   } else if (S == 1 && total % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, true, true); else LAUNCH(kVec, true, false);
+  } else if (S > 1 && S % kVec == 0 && aligned && C * S < (int64_t(1) << 30)) {
+    const int64_t npackets = total / kVec;
+    const int64_t chunks = ceil_div(npackets, static_cast<int64_t>(kLossThreads) * 4);
+    const int64_t cap = static_cast<int64_t>(num_cus()) * 64;
+    const dim3 grid(static_cast<unsigned>(chunks < cap ? chunks : cap));
+    if (reduction == kNone) {
+      hipLaunchKernelGGL((softmax_ce_backward_chunks_strided<T, TargetT, true>), grid,
+                         dim3(kLossThreads), 0, stream, npackets, static_cast<uint32_t>(S),
+                         static_cast<uint32_t>(C), ignore_index, pp, tp, dlp, scalar, dp);
+    } else {
+      hipLaunchKernelGGL((softmax_ce_backward_chunks_strided<T, TargetT, false>), grid,
+                         dim3(kLossThreads), 0, stream, npackets, static_cast<uint32_t>(S),
+                         static_cast<uint32_t>(C), ignore_index, pp, tp, dlp, scalar, dp);
+    }
   } else if (S > 1 && S % kVec == 0 && aligned) {
     if (reduction == kNone) LAUNCH(kVec, false, true); else LAUNCH(kVec, false, false);
   } else {
