@@ -183,14 +183,17 @@ def test_softmax_8192x4096_whole_tensor_against_the_oracle(K, dtype):
 
 
 @pytest.mark.parametrize("shape,dtype", [((2048, 128256), "float32"), ((2048, 128256), "bfloat16"),
-                                         ((605184, 197), "bfloat16")])
+                                         ((605184, 197), "bfloat16"), ((4096, 50257), "bfloat16"),
+                                         ((4096, 30522), "float16")])
 @pytest.mark.parametrize("log", [False, True])
 def test_softmax_bench_shapes_sampled_rows_and_every_row(K, shape, dtype, log):
     """bench workloads softmax_f32_2048x128256 (vocabulary-sized rows cut into slices that
     several workgroups hold: tens of thousands of work items over many rounds of the resident
     grid, each round's packets requested into the registers the round before has just
-    rewritten) and softmax_bf16_605184x197 (rows that are not whole packets, far more chunks
-    of staged rows than the grid holds)."""
+    rewritten), softmax_bf16_605184x197 (rows that are not whole packets, far more chunks
+    of staged rows than the grid holds) and softmax_bf16_4096x50257 (rows that are not whole
+    packets through the aligned packets that cover them, many rows per persistent workgroup;
+    [4096, 30522] for the flavour that holds the converted row)."""
     import torch
     N, C = shape
     x, dy = _softmax_inputs(N, C, dtype, 44)
