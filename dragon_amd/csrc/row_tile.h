@@ -31,6 +31,27 @@ namespace dragon_hip {
 // Workgroup size of a row kernel: wave-per-row tiles share a 256-thread group.
 constexpr int row_threads(int tpr) { return tpr == kWaveSize ? 256 : tpr; }
 
+// A row of any width at any element-aligned address, as the aligned 16-byte
+// packets that cover it (its window): the window starts `lead` elements before
+// the row and its last packet holds `tail_valid` elements of the row. Where a
+// kernel does not care which column an element is (softmax and its gradient;
+// the fused loss adds `lead` to the target's column), a row can be read,
+// reduced and written window packet by window packet: every access to HBM
+// is an aligned packet except the element-wise stores of a row's first and last
+// packet, whose other elements belong to the neighbouring rows. An aligned
+// packet that holds one byte of a tensor lies in the same page as that byte, so
+// reading all of it is safe at the tensor's ends too.
+template <typename T>
+struct RowWindow {
+  static constexpr int kVec = IO<T>::kVec;
+  int lead, packets, tail_valid;
+  __device__ __forceinline__ RowWindow(const T* row, int C) {
+    lead = static_cast<int>((reinterpret_cast<uintptr_t>(row) & 15u) / sizeof(T));
+    packets = (lead + C + kVec - 1) / kVec;
+    tail_valid = lead + C - (packets - 1) * kVec;  // 1 .. kVec
+  }
+};
+
 // kThreads is the workgroup size; a workgroup runs kThreads / kTPR rows at a
 // time. Kernels whose rows span several wavefronts and that run more than one
 // row per workgroup must keep their row loop uniform across the workgroup
@@ -112,6 +133,55 @@ struct RowTile {
     for (int s = 0; s < kVPT; ++s) {
       if (valid && active(s, npackets)) {
         pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v[s]);
+      }
+    }
+  }
+
+  // The row through its window (regular tiles only): aligned packets, and what the
+  // window's first and last packet hold of the neighbouring rows replaced by `fill`.
+  // `row` is the row's own (element-aligned) address.
+  __device__ __forceinline__ void load_window(const T* row, const RowWindow<T>& w, A fill,
+                                              bool valid = true) {
+    static_assert(!kRagged, "windows use the regular tile");
+    load(row - w.lead, w.packets, fill, valid);
+    const int tail_slot = (w.packets - 1) / kTPR, tail_lane = (w.packets - 1) % kTPR;
+    if (w.lead > 0 && lane() == 0) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (e < w.lead) v[0][e] = fill;
+      }
+    }
+    if (w.tail_valid < kVec && lane() == tail_lane) {
+#pragma unroll
+      for (int s = 0; s < kVPT; ++s) {
+        if (s == tail_slot) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (e >= w.tail_valid) v[s][e] = fill;
+          }
+        }
+      }
+    }
+  }
+  // Whole packets of the row as aligned packets; the elements of the row in the
+  // window's first and last packet one by one (the others belong to its neighbours).
+  __device__ __forceinline__ void store_window(T* row, const RowWindow<T>& w,
+                                               bool valid = true) const {
+    static_assert(!kRagged, "windows use the regular tile");
+    T* base = row - w.lead;
+#pragma unroll
+    for (int s = 0; s < kVPT; ++s) {
+      const int idx = s * kTPR + lane();
+      if (!valid || idx >= w.packets) continue;
+      const int first = idx == 0 ? w.lead : 0;
+      const int last = idx == w.packets - 1 ? w.tail_valid : kVec;
+      if (first == 0 && last == kVec) {
+        pack_store<T>(base + static_cast<int64_t>(idx) * kVec, v[s]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (e >= first && e < last) IO<T>::store1(base + static_cast<int64_t>(idx) * kVec + e, v[s][e]);
+        }
       }
     }
   }
@@ -284,27 +354,6 @@ struct RawRowTile {
   }
   __device__ __forceinline__ void store_slot(T* row, int s, const A (&v)[kVec]) const {
     pack_store<T>(row + static_cast<int64_t>(s * kTPR + lane()) * kVec, v);
-  }
-};
-
-// A row of any width at any element-aligned address, as the aligned 16-byte
-// packets that cover it (its window): the window starts `lead` elements before
-// the row and its last packet holds `tail_valid` elements of the row. Where a
-// kernel does not care which column an element is (softmax and its gradient;
-// the fused loss adds `lead` to the target's column), a row can be read,
-// reduced and written window packet by window packet: every access to HBM
-// is an aligned packet except the element-wise stores of a row's first and last
-// packet, whose other elements belong to the neighbouring rows. An aligned
-// packet that holds one byte of a tensor lies in the same page as that byte, so
-// reading all of it is safe at the tensor's ends too.
-template <typename T>
-struct RowWindow {
-  static constexpr int kVec = IO<T>::kVec;
-  int lead, packets, tail_valid;
-  __device__ __forceinline__ RowWindow(const T* row, int C) {
-    lead = static_cast<int>((reinterpret_cast<uintptr_t>(row) & 15u) / sizeof(T));
-    packets = (lead + C + kVec - 1) / kVec;
-    tail_valid = lead + C - (packets - 1) * kVec;  // 1 .. kVec
   }
 };
 

@@ -59,9 +59,11 @@ enum SoftmaxKind { kSoftmax = 0, kLogSoftmax = 1 };
 // Rows held in registers by kTPR threads; a wavefront that holds a whole row in
 // one or two packets per lane takes two neighbouring rows at a time
 // (wave_rows_at_a_time).
-template <typename T, int kKind, int kTPR, int kVPT, bool kRagged, bool kFull = false>
+template <typename T, int kKind, int kTPR, int kVPT, bool kRagged, bool kFull = false,
+          bool kWindow = false>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
     const int64_t N, const int C, const T* x, T* y) {
+  static_assert(!(kWindow && (kRagged || kFull)), "windows use the regular tile");
   using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
@@ -79,7 +81,9 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
     for (int r = 0; r < kR; ++r) {
       on[r] = row + r < N;
       const T* src = x + (on[r] ? row + r : row) * C;
-      if constexpr (kFull) {
+      if constexpr (kWindow) {
+        t[r].load_window(src, RowWindow<T>(src, C), acc_neg_inf<A>());
+      } else if constexpr (kFull) {
         t[r].load_full(src);  // the row fills the tile: nothing to mask
       } else {
         t[r].load(src, npackets, acc_neg_inf<A>());
@@ -133,7 +137,11 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_rows(
 #pragma unroll
           for (int e = 0; e < kVec; ++e) t[r].v[i][e] = t[r].v[i][e] - l;
       }
-      if (on[r]) t[r].store(y + (row + r) * C, npackets);
+      if constexpr (kWindow) {
+        if (on[r]) t[r].store_window(y + (row + r) * C, RowWindow<T>(x + (row + r) * C, C));
+      } else {
+        if (on[r]) t[r].store(y + (row + r) * C, npackets);
+      }
     }
     if (kTPR != kWaveSize) __syncthreads();
   }
@@ -479,9 +487,10 @@ __global__ __launch_bounds__(1024) void softmax_wide_raw_windows(const int64_t N
   }
 }
 
-template <typename T, int kKind, int kTPR, int kVPT, bool kRagged>
+template <typename T, int kKind, int kTPR, int kVPT, bool kRagged, bool kWindow = false>
 __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
     const int64_t N, const int C, const T* dy, const T* y, T* dx) {
+  static_assert(!(kWindow && kRagged), "windows use the regular tile");
   using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), kRagged>;
   using A = typename Tile::A;
   using M = SoftmaxMath<T>;
@@ -492,8 +501,14 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < N; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
     Tile g, o;
-    g.load(dy + row * C, npackets, A(0));
-    o.load(y + row * C, npackets, kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
+    const RowWindow<T> w(dy + row * C, C);  // the same for y and dx: congruent tensors
+    if constexpr (kWindow) {
+      g.load_window(dy + row * C, w, A(0));
+      o.load_window(y + row * C, w, kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
+    } else {
+      g.load(dy + row * C, npackets, A(0));
+      o.load(y + row * C, npackets, kKind == kSoftmax ? A(0) : acc_neg_inf<A>());
+    }
 
     A s = A(0);
 #pragma unroll
@@ -518,7 +533,11 @@ __global__ __launch_bounds__(row_threads(kTPR)) void softmax_grad_rows(
           g.v[i][e] = g.v[i][e] - M::exp_of(o.v[i][e]) * s;
         }
       }
-    g.store(dx + row * C, npackets);
+    if constexpr (kWindow) {
+      g.store_window(dx + row * C, w);
+    } else {
+      g.store(dx + row * C, npackets);
+    }
     if (kTPR != kWaveSize) __syncthreads();
   }
 }
@@ -1637,6 +1656,20 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
 #undef LAUNCH_WIDE
       return status_of_launch();
     }
+    // rows of the smaller tiles that are not whole aligned packets: through their windows
+    if (RowConfig wc; !regular && congruent16(x, y) && pick_row_config(C / kVec + 2, 8, &wc) &&
+                      wc.tpr < 1024) {
+#define LAUNCH(TPR, VPT)                                                                     \
+  {                                                                                          \
+    using Tile = RowTile<T, TPR, VPT>;                                                       \
+    const dim3 grid(row_grid(N, Tile::kRowsPerBlock * wave_rows_at_a_time<TPR, VPT>()));     \
+    hipLaunchKernelGGL((softmax_rows<T, kKind, TPR, VPT, false, false, true>), grid,         \
+                       dim3(Tile::kThreads), 0, stream, N, static_cast<int>(C), xp, yp);     \
+  }
+      DRAGON_HIP_ROW_SWITCH(wc, LAUNCH);
+#undef LAUNCH
+      return status_of_launch();
+    }
 #define LAUNCH(TPR, VPT)                                                                     \
   {                                                                                          \
     using Tile = RowTile<T, TPR, VPT>;                                                       \
@@ -1765,6 +1798,20 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
     if (cfg.vpt == 2) LAUNCH_WINDOWS(2, true) else if (cfg.vpt == 4) LAUNCH_WINDOWS(4, true)
     else LAUNCH_WINDOWS(8, false)
 #undef LAUNCH_WINDOWS
+    return status_of_launch();
+  }
+  // rows of the register tiles that are not whole aligned packets: through their windows
+  if (S == 1 && !regular && congruent16(dy, y) && congruent16(dy, dx) &&
+      pick_row_config(C / kVec + 2, 4, &cfg)) {
+#define LAUNCH(TPR, VPT)                                                                     \
+  {                                                                                          \
+    using Tile = RowTile<T, TPR, VPT>;                                                       \
+    hipLaunchKernelGGL((softmax_grad_rows<T, kKind, TPR, VPT, false, true>),                 \
+                       dim3(row_grid(N, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,      \
+                       stream, N, static_cast<int>(C), gp, yp, dp);                          \
+  }
+    DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
+#undef LAUNCH
     return status_of_launch();
   }
   // Two tiles live at once: halve the packets a thread may hold.
