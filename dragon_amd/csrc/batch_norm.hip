@@ -555,6 +555,7 @@ struct CoopForward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 1;
   static constexpr bool kBeginReadsInput = true;
+  static constexpr bool kWindows = true;
   using Merge = PairSum;
   A inv_n, momentum, one_minus_momentum, eps;
   const A* gamma;
@@ -605,6 +606,7 @@ template <typename T>
 struct CoopBackward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 2;
+  static constexpr bool kWindows = true;
   using Merge = PairSum;
   A normalizer;
   const A* mu;
@@ -784,7 +786,7 @@ inline size_t acc_bytes(int dtype) { return dtype == DRAGON_HIP_F64 ? 8 : 4; }
 template <typename T>
 size_t scratch_bytes_of(const ChannelShape& sh, size_t* out) {
   const size_t split = channel_scratch_bytes(sh, sizeof(typename IO<T>::Acc));
-  const size_t coop = sh.nchw ? coop_scratch_bytes<T>(channel_units(sh)) : 0;
+  const size_t coop = sh.nchw ? coop_scratch_bytes<T>(channel_units(sh), true) : 0;
   *out = split > coop ? split : coop;
   return *out;
 }

@@ -352,6 +352,10 @@ __device__ __forceinline__ double acc_neg_inf<double>() { return -__builtin_inf(
 // Host-side helpers
 // ---------------------------------------------------------------------------
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// The same offset from a 16-byte boundary: the aligned packets of one tensor line up with the other's.
+inline bool congruent16(const void* a, const void* b) {
+  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+}
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int status_of_launch() {
   const hipError_t e = hipGetLastError();

@@ -348,6 +348,10 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
     if (vec_ok) {
       hipLaunchKernelGGL((reduce2_segments<T, 1, kVec, Accum>), grid, dim3(kReduceThreads), 0,
                          stream, s, xp, xp, f, part);
+    } else if (s.seglen >= 4 * kVec && sizeof(T) <= 4) {
+      // segments that are not whole aligned packets, through the packets that cover them
+      hipLaunchKernelGGL((reduce2_segments_windows<T, 1, Accum>), grid, dim3(kReduceThreads), 0,
+                         stream, s, xp, xp, f, part);
     } else {
       hipLaunchKernelGGL((reduce2_segments<T, 1, 1, Accum>), grid, dim3(kReduceThreads), 0, stream,
                          s, xp, xp, f, part);

@@ -117,6 +117,64 @@ __global__ __launch_bounds__(kReduceThreads) void reduce2_segments(
   }
 }
 
+// Stage one over segments of any length at any element-aligned address, read as
+// the aligned 16-byte packets that cover each segment (two tensors must be
+// congruent modulo 16 bytes): a segment of seglen elements takes
+// seglen / kVec + 2 packet slots, of which the last may lie wholly behind it
+// and is skipped. A packet wholly inside its segment goes to F's packet
+// interface; the elements of a segment in its first and last packet go to the
+// scalar one, one call per element, so F sees exactly the elements and indices
+// it would see element by element. An aligned packet that holds a byte of a
+// tensor lies in that byte's page, so packets that reach beyond a tensor's ends
+// may be read whole.
+template <typename T, int kIn, typename F>
+__global__ __launch_bounds__(kReduceThreads) void reduce2_segments_windows(
+    const SegmentedReduce d, const T* __restrict__ in0, const T* __restrict__ in1, F f,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  __shared__ A lds[2 * kReduceWaves];
+  const uint32_t o = blockIdx.x / d.split;
+  const uint32_t k = blockIdx.x - o * d.split;
+  const uint32_t o1 = o / d.outer2;
+  const uint32_t o2 = o - o1 * d.outer2;
+  const uint32_t base = o1 * d.stride1 + o2 * d.stride2;
+  const uint32_t slots_per_seg = d.seglen / kVec + 2;
+  const uint32_t nslots = d.nseg * slots_per_seg;
+  f.begin(o, base);
+  A a = A(0), b = A(0);
+#pragma unroll 4
+  for (uint32_t js = k * kReduceThreads + threadIdx.x; js < nslots;
+       js += d.split * kReduceThreads) {
+    const uint32_t seg = js / slots_per_seg;
+    const uint32_t q = js - seg * slots_per_seg;
+    const uint32_t s0 = base + seg * d.seg_stride;  // the segment's first element
+    const int lead = static_cast<int>((reinterpret_cast<uintptr_t>(in0 + s0) & 15u) / sizeof(T));
+    const int pe = static_cast<int>(q * kVec) - lead;  // the packet's first element, in the segment
+    if (pe >= static_cast<int>(d.seglen)) continue;
+    A x0[kVec], x1[kVec];
+    load_unpack_keep<T>(in0 + (static_cast<int64_t>(s0) + pe), x0);
+    if constexpr (kIn == 2) load_unpack_keep<T>(in1 + (static_cast<int64_t>(s0) + pe), x1);
+    if (pe >= 0 && pe + kVec <= static_cast<int>(d.seglen)) {
+      f.add(o, seg, static_cast<uint32_t>(pe), s0 + pe, x0, x1, a, b);
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (pe + e >= 0 && pe + e < static_cast<int>(d.seglen)) {
+          const A y0[1] = {x0[e]};
+          const A y1[1] = {kIn == 2 ? x1[e] : A(0)};
+          f.add(o, seg, static_cast<uint32_t>(pe + e), s0 + pe + e, y0, y1, a, b);
+        }
+      }
+    }
+  }
+  block_reduce_pair(a, b, lds);
+  if (threadIdx.x == 0) {
+    partial[(static_cast<size_t>(o) * d.split + k) * 2] = a;
+    partial[(static_cast<size_t>(o) * d.split + k) * 2 + 1] = b;
+  }
+}
+
 // Stage one over columns: a workgroup owns a tile of 64 adjacent columns
 // (one per lane, so a wavefront reads 64 adjacent elements) and its four
 // wavefronts stride over the rows of slice k. F provides

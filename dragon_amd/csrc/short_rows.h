@@ -329,9 +329,6 @@ inline unsigned short_grid(int64_t N, uint32_t rows_per_chunk) {
   const int64_t cap = static_cast<int64_t>(num_cus()) * 16;
   return static_cast<unsigned>(chunks < cap ? chunks : cap);
 }
-inline bool congruent16(const void* a, const void* b) {
-  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
-}
 
 // Launches short_rows<T, L, E, OP<T, E>> for the plan; OP is the policy
 // template, the trailing arguments its constructor arguments.

@@ -46,6 +46,19 @@
 // A slice is a whole number of wavefronts of packets, and so is a unit whenever
 // its packet count is a multiple of 64: accumulate / transform are then entered
 // by whole wavefronts and may reduce across the wavefront.
+//
+// Runs that are not whole aligned packets (a 57x57 or 15x15 feature map, a
+// tensor at an element-aligned address) go through the same kernel in its
+// window flavour, for an Op that declares kWindows: a run of seglen elements is
+// read as the aligned 16-byte packets that cover it, seglen / kVec + 2 packet
+// slots of which the last may lie behind the run and is skipped. A packet
+// wholly inside the run is accumulated, transformed and stored as a packet; of
+// a packet at either end only the run's own elements are accumulated (one call
+// of accumulate<1> each) and stored (one element store each), the neighbouring
+// run's elements in it belonging to another unit and another workgroup. All
+// tensors of a call must then be congruent modulo 16 bytes. An aligned packet
+// that holds a byte of a tensor lies in that byte's page, so a packet that
+// reaches beyond either end of a tensor may be read whole.
 #pragma once
 
 #include <type_traits>
@@ -93,12 +106,15 @@ struct SliceUnits {
 };
 
 template <typename T>
-CoopPlan plan_coop(const SliceUnits& u, int kIn) {
+CoopPlan plan_coop(const SliceUnits& u, int kIn, bool windows = false) {
   constexpr int kVec = IO<T>::kVec;
   CoopPlan p = {false, 0, 0, 0};
-  if (u.seglen % kVec != 0) return p;
-  const uint32_t pps = u.seglen / kVec;
-  if (pps < 16) return p;  // runs shorter than 256 bytes: left to the split reduction
+  if (!windows && u.seglen % kVec != 0) return p;
+  // Runs shorter than 256 bytes are left to the split reduction, and so are window
+  // runs under 384 bytes, two of whose packets are taken element by element
+  // (measured on 9x9 fp32 maps: 25.9 us against the split path's 21.3).
+  if (u.seglen / kVec < (windows ? 24u : 16u)) return p;
+  const uint32_t pps = u.seglen / kVec + (windows ? 2 : 0);
   const int64_t P = static_cast<int64_t>(u.nseg) * pps;  // packets per unit
   const int rmax = coop_rmax(kIn);
   const int64_t grid = coop_grid(rmax, kIn);
@@ -137,23 +153,28 @@ inline size_t coop_exchange_bytes(size_t items, size_t acc_size) {
   return (bytes + 255) / 256 * 256;
 }
 
-// Scratch of the single-read path for `units`: the larger of the one- and the two-tensor plan.
+// Scratch of the single-read path for `units`: the larger of the one- and the
+// two-tensor plan (`windows_too`: and of their window flavours, which the
+// addresses of a call may select).
 template <typename T>
-size_t coop_scratch_bytes(const SliceUnits& u) {
+size_t coop_scratch_bytes(const SliceUnits& u, bool windows_too = false) {
   using A = typename IO<T>::Acc;
   size_t need = 0;
   for (int in = 1; in <= 2; ++in) {
-    const CoopPlan p = plan_coop<T>(u, in);
-    if (!p.ok) continue;
-    const size_t bytes = coop_exchange_bytes(static_cast<size_t>(u.units) * p.K, sizeof(A));
-    if (bytes > need) need = bytes;
+    for (int win = 0; win <= (windows_too ? 1 : 0); ++win) {
+      const CoopPlan p = plan_coop<T>(u, in, win != 0);
+      if (!p.ok) continue;
+      const size_t bytes = coop_exchange_bytes(static_cast<size_t>(u.units) * p.K, sizeof(A));
+      if (bytes > need) need = bytes;
+    }
   }
   return need;
 }
 
 struct CoopShape {
   uint32_t unit_stride, K, slice;
-  uint32_t pps;          // packets per run
+  uint32_t pps;          // packets (window flavour: packet slots) per run
+  uint32_t seglen;       // elements per run
   uint32_t P;            // packets per unit
   uint32_t seg_stride;   // elements between two runs of a unit
   uint32_t step_seg, step_p;  // kCoopThreads packets further on = step_seg segments and step_p packets
@@ -164,11 +185,13 @@ struct CoopShape {
 };
 
 template <typename T>
-CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p, typename IO<T>::Acc* scratch) {
+CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p, typename IO<T>::Acc* scratch,
+                          bool windows = false) {
   constexpr int kVec = IO<T>::kVec;
   CoopShape d;
   d.unit_stride = u.unit_stride, d.K = p.K, d.slice = p.slice;
-  d.pps = u.seglen / kVec;
+  d.pps = u.seglen / kVec + (windows ? 2 : 0);
+  d.seglen = u.seglen;
   d.P = u.nseg * d.pps;
   d.seg_stride = u.seg_stride;
   d.step_seg = kCoopThreads / d.pps, d.step_p = kCoopThreads % d.pps;
@@ -199,6 +222,47 @@ struct CoopCursor {
     if (p >= d.pps) p -= d.pps, ++seg;
   }
 };
+
+// Where the cursor's packet lies, as an element offset from the tensors' bases
+// (window flavour: below zero for the packet that holds the tensor's first
+// elements at an unaligned base), and which of its elements [lo, hi) belong to
+// the run; hi <= lo for the slot behind a run, whose packet is not touched.
+struct CoopSlot {
+  int32_t off;
+  int lo, hi;
+  template <int kVec>
+  __device__ __forceinline__ bool whole() const { return lo == 0 && hi == kVec; }
+};
+template <typename T, bool kWin>
+__device__ __forceinline__ CoopSlot coop_slot(const CoopShape& d, const CoopCursor& cur,
+                                              uint32_t base, const T* in0) {
+  constexpr int kVec = IO<T>::kVec;
+  const uint32_t run = base + cur.seg * d.seg_stride;
+  CoopSlot s;
+  if constexpr (!kWin) {
+    s.off = static_cast<int32_t>(run + cur.p * kVec), s.lo = 0, s.hi = kVec;
+  } else {
+    const int lead = static_cast<int>((reinterpret_cast<uintptr_t>(in0 + run) & 15u) / sizeof(T));
+    const int pe = static_cast<int>(cur.p * kVec) - lead;  // the packet's first element, in the run
+    const int rest = static_cast<int>(d.seglen) - pe;
+    s.off = static_cast<int32_t>(run) + pe;
+    s.lo = pe < 0 ? -pe : 0;
+    s.hi = rest < kVec ? rest : kVec;
+  }
+  return s;
+}
+// An aligned packet that may always be read: the one that holds the unit's first element.
+template <typename T, bool kWin>
+__device__ __forceinline__ int32_t coop_safe_offset(uint32_t base, const T* in0) {
+  if constexpr (!kWin) return static_cast<int32_t>(base);
+  return static_cast<int32_t>(base) -
+      static_cast<int32_t>((reinterpret_cast<uintptr_t>(in0 + base) & 15u) / sizeof(T));
+}
+// Keeps the compiler from carrying every slot of one pass over an item to the
+// next pass in registers: the slots are recomputed from the cursor instead.
+__device__ __forceinline__ void coop_forget(CoopCursor& cur) {
+  asm volatile("" : "+v"(cur.seg), "+v"(cur.p));
+}
 
 // Bit pattern of a partial sum that has not been published yet; the slots are
 // filled with it before every launch. It is a NaN, and the hardware carries the
@@ -355,6 +419,13 @@ template <typename Op>
 struct OpBeginReadsInput<Op, std::void_t<decltype(Op::kBeginReadsInput)>>
     : std::bool_constant<Op::kBeginReadsInput> {};
 
+//   kWindows    the Op's accumulate and transform do not depend on the packet
+//               index j and accept V == 1: the window flavour may serve it.
+template <typename Op, typename = void>
+struct OpTakesWindows : std::false_type {};
+template <typename Op>
+struct OpTakesWindows<Op, std::void_t<decltype(Op::kWindows)>> : std::bool_constant<Op::kWindows> {};
+
 template <typename T, int kR, int kIn>
 struct CoopSlice {  // the raw packets of one item
   u32x4 p0[kR];
@@ -374,15 +445,16 @@ struct CoopItem {
   __device__ __forceinline__ bool has(int i) const { return i * kCoopThreads + threadIdx.x < len; }
 };
 
-template <typename T, int kR, int kIn>
+template <typename T, int kR, int kIn, bool kWin>
 __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const T* in0, const T* in1,
                                           CoopSlice<T, kR, kIn>& s) {
-  constexpr int kVec = IO<T>::kVec;
   const CoopItem it(d, w);
   CoopCursor cur(d, it.j0);
+  const int32_t safe = coop_safe_offset<T, kWin>(it.base, in0);
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
-    const uint32_t off = it.has(i) ? cur.template offset<kVec>(d, it.base) : it.base;
+    const CoopSlot at = coop_slot<T, kWin>(d, cur, it.base, in0);
+    const int32_t off = it.has(i) && at.hi > at.lo ? at.off : safe;
     s.p0[i] = load_packet(in0 + off);
     if constexpr (kIn == 2) s.p1[i] = load_packet(in1 + off);
     cur.advance(d);
@@ -393,7 +465,7 @@ __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const 
 // packets are requested one by one into the registers the second pass has just
 // written out, so they travel while the rest of this item is stored.
 // kRepair: the second launch, which finishes the items whose wait ran out.
-template <typename T, int kR, typename Op, bool kRepair>
+template <typename T, int kR, typename Op, bool kRepair, bool kWin>
 __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uint32_t next,
                                              const T* in0, const T* in1, T* out, Op op,
                                              CoopSlice<T, kR, Op::kIn>& s,
@@ -406,6 +478,8 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
   op.begin(it.c, it.base, in0);
   A a, b;
   Op::Merge::identity(a, b);
+  static_assert(!kWin || (!OpScansFirst<Op>::value && !OpRewrites<Op>::value),
+                "the window flavour serves plain accumulate / transform Ops");
   if constexpr (OpScansFirst<Op>::value) {
 #pragma unroll
     for (int i = 0; i < kR; ++i) {
@@ -419,9 +493,12 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
 #pragma unroll
     for (int i = 0; i < kR; ++i) asm volatile("" : "+v"(s.p0[i]));
   }
+  CoopCursor acur(d, it.j0);
+  if constexpr (kWin) coop_forget(acur);
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
-    if (it.has(i)) {
+    const CoopSlot at = coop_slot<T, kWin>(d, acur, it.base, in0);
+    if (it.has(i) && at.hi > at.lo) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
@@ -429,10 +506,20 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
         static_assert(sizeof(T) == sizeof(A), "rewritten elements must survive the packet");
         op.accumulate_rewrite(xv, a, b);
         s.p0[i] = IO<T>::pack(xv);
-      } else {
+      } else if (!kWin || at.template whole<kVec>()) {
         op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (e >= at.lo && e < at.hi) {
+            const A x1[1] = {xv[e]};
+            const A d1[1] = {Op::kIn == 2 ? dv[e] : A(0)};
+            op.accumulate(it.c, 0u, x1, d1, a, b);
+          }
+        }
       }
     }
+    if constexpr (kWin) acur.advance(d);
   }
   // false (for the whole workgroup): the wait ran out, the item is left to the repair launch
   const bool complete = coop_channel_totals<typename Op::Merge, kRepair>(d, it.c, w, a, b, partial,
@@ -447,18 +534,29 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
   const bool more = !kRepair && next < d.items;  // uniform over the workgroup
   const CoopItem nit(d, more ? next : w);
   CoopCursor cur(d, it.j0), ncur(d, nit.j0);
+  if constexpr (kWin) coop_forget(cur), coop_forget(ncur);
+  const int32_t nsafe = coop_safe_offset<T, kWin>(nit.base, in0);
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
-    if (complete && it.has(i)) {
+    const CoopSlot at = coop_slot<T, kWin>(d, cur, it.base, in0);
+    if (complete && it.has(i) && at.hi > at.lo) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
       op.transform(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv);
-      store_packet(out + cur.template offset<kVec>(d, it.base), IO<T>::pack(xv));
+      if (!kWin || at.template whole<kVec>()) {
+        store_packet(out + at.off, IO<T>::pack(xv));
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (e >= at.lo && e < at.hi) IO<T>::store1(out + at.off + e, xv[e]);
+        }
+      }
     }
     cur.advance(d);
     if (more) {
-      const uint32_t off = nit.has(i) ? ncur.template offset<kVec>(d, nit.base) : nit.base;
+      const CoopSlot nat = coop_slot<T, kWin>(d, ncur, nit.base, in0);
+      const int32_t off = nit.has(i) && nat.hi > nat.lo ? nat.off : nsafe;
       s.p0[i] = load_packet(in0 + off);
       if constexpr (Op::kIn == 2) s.p1[i] = load_packet(in1 + off);
       ncur.advance(d);
@@ -470,7 +568,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
 // exchange costs a few microseconds per item whatever its size. Four
 // workgroups per compute unit, or three with up to 168 registers for the
 // widest slices.
-template <typename T, int kR, typename Op>
+template <typename T, int kR, typename Op, bool kWin>
 __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void channel_slices(
     const CoopShape d, const T* __restrict__ in0, const T* __restrict__ in1, T* __restrict__ out,
     const Op op, typename IO<T>::Acc* __restrict__ partial) {
@@ -478,10 +576,10 @@ __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void chann
   __shared__ A lds_a[2 * kReduceWaves];
   __shared__ A lds_b[2 * kReduceWaves];
   CoopSlice<T, kR, Op::kIn> s;
-  if (blockIdx.x < d.items) coop_load<T, kR, Op::kIn>(d, blockIdx.x, in0, in1, s);
+  if (blockIdx.x < d.items) coop_load<T, kR, Op::kIn, kWin>(d, blockIdx.x, in0, in1, s);
   for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
-    coop_process<T, kR, Op, false>(d, w, w + gridDim.x, in0, in1, out, op, s, partial, lds_a,
-                                   lds_b);
+    coop_process<T, kR, Op, false, kWin>(d, w, w + gridDim.x, in0, in1, out, op, s, partial, lds_a,
+                                         lds_b);
   }
 }
 
@@ -489,7 +587,7 @@ __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void chann
 // out; then every flagged item is finished from the pairs, which by now are all
 // published. Inputs of a flagged item are intact even when the call runs in
 // place: the workgroup that gave up wrote nothing for it.
-template <typename T, int kR, typename Op>
+template <typename T, int kR, typename Op, bool kWin>
 __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void channel_slices_repair(
     const CoopShape d, const T* __restrict__ in0, const T* __restrict__ in1, T* __restrict__ out,
     const Op op, typename IO<T>::Acc* __restrict__ partial) {
@@ -500,8 +598,9 @@ __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void chann
   for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
     if (d.flags[w] == 0u) continue;  // the same word in every thread
     CoopSlice<T, kR, Op::kIn> s;
-    coop_load<T, kR, Op::kIn>(d, w, in0, in1, s);
-    coop_process<T, kR, Op, true>(d, w, d.items, in0, in1, out, op, s, partial, lds_a, lds_b);
+    coop_load<T, kR, Op::kIn, kWin>(d, w, in0, in1, s);
+    coop_process<T, kR, Op, true, kWin>(d, w, d.items, in0, in1, out, op, s, partial, lds_a,
+                                        lds_b);
     __syncthreads();  // the next item reuses the LDS words of the reductions
   }
 }
@@ -520,18 +619,15 @@ inline void fill_unset(A* pairs, const CoopShape& d, hipStream_t stream) {
 // `scratch` holds coop_scratch_bytes<T>(sh) bytes.
 constexpr int kNotApplicable = 1;
 constexpr unsigned kCoopRepairGrid = 256;
-template <typename T, typename Op>
-int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T* in1, T* out,
-                       typename IO<T>::Acc* scratch, hipStream_t stream) {
+template <typename T, typename Op, bool kWin>
+int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op, const T* in0,
+                          const T* in1, T* out, typename IO<T>::Acc* scratch, hipStream_t stream) {
   constexpr int kIn = Op::kIn;
-  const CoopPlan p = plan_coop<T>(sh, kIn);
-  if (!p.ok || !aligned16(in0) || !aligned16(in1) || !aligned16(out)) return kNotApplicable;
-  if (OpBeginReadsInput<Op>::value && static_cast<const void*>(out) == in0) return kNotApplicable;
-  const CoopShape d = make_coop_shape<T>(sh, p, scratch);
+  const CoopShape d = make_coop_shape<T>(sh, p, scratch, kWin);
   // Workgroups launched: all of them resident at once, and at least as many as a unit has slices.
 #define DRAGON_HIP_COOP_GRID(R)                                                                \
   [&] {                                                                                        \
-    const unsigned resident = resident_grid(channel_slices<T, R, Op>, kCoopThreads, 0);        \
+    const unsigned resident = resident_grid(channel_slices<T, R, Op, kWin>, kCoopThreads, 0);  \
     const unsigned want = coop_grid(coop_rmax(kIn), kIn);                                      \
     return resident < want ? resident : want;                                                  \
   }()
@@ -540,7 +636,7 @@ int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T
     const unsigned cap = DRAGON_HIP_COOP_GRID(R);                                              \
     if (p.K > cap) return kNotApplicable;                                                      \
     fill_unset(scratch, d, stream);                                                            \
-    hipLaunchKernelGGL((channel_slices<T, R, Op>), dim3(d.items < cap ? d.items : cap),        \
+    hipLaunchKernelGGL((channel_slices<T, R, Op, kWin>), dim3(d.items < cap ? d.items : cap),  \
                        dim3(kCoopThreads), 0, stream, d, in0, in1, out, op, scratch);          \
   }
   if (p.r * kIn <= 4) DRAGON_HIP_COOP_LAUNCH(4 / kIn)
@@ -551,10 +647,31 @@ int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T
 #undef DRAGON_HIP_COOP_GRID
   // the widest slice serves every plan: a repair is rare and its speed does not matter
   constexpr int kRepairR = kIn == 2 ? 12 : 16;
-  hipLaunchKernelGGL((channel_slices_repair<T, kRepairR, Op>),
+  hipLaunchKernelGGL((channel_slices_repair<T, kRepairR, Op, kWin>),
                      dim3(d.items < kCoopRepairGrid ? d.items : kCoopRepairGrid), dim3(kCoopThreads),
                      0, stream, d, in0, in1, out, op, scratch);
   return status_of_launch();
+}
+
+template <typename T, typename Op>
+int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T* in1, T* out,
+                       typename IO<T>::Acc* scratch, hipStream_t stream) {
+  constexpr int kIn = Op::kIn;
+  if (OpBeginReadsInput<Op>::value && static_cast<const void*>(out) == in0) return kNotApplicable;
+  const bool packets = sh.seglen % IO<T>::kVec == 0 && sh.unit_stride % IO<T>::kVec == 0 &&
+      sh.seg_stride % IO<T>::kVec == 0 && aligned16(in0) && aligned16(in1) && aligned16(out);
+  if (packets) {
+    const CoopPlan p = plan_coop<T>(sh, kIn);
+    if (!p.ok) return kNotApplicable;
+    return launch_channel_slices<T, Op, false>(sh, p, op, in0, in1, out, scratch, stream);
+  }
+  if constexpr (OpTakesWindows<Op>::value) {
+    if (sizeof(T) > 4 || !congruent16(in0, in1) || !congruent16(in0, out)) return kNotApplicable;
+    const CoopPlan p = plan_coop<T>(sh, kIn, true);
+    if (!p.ok) return kNotApplicable;
+    return launch_channel_slices<T, Op, true>(sh, p, op, in0, in1, out, scratch, stream);
+  }
+  return kNotApplicable;
 }
 
 

@@ -681,6 +681,85 @@ def test_batch_norm_training(K, shape, axis, dtype):
     assert U.normwise(U.widen(U.to_host(dx2), dtype), dx_ref) <= U.TIGHT[dtype]
 
 
+# (N, C, H, W): slices per channel and rounds of work items as in BN_CASES above, on maps
+# that are not whole packets
+BN_WINDOW_CASES = [(8, 40, 57, 57), (2, 1100, 15, 15), (32, 350, 27, 27), (4, 24, 35, 35),
+                   (3, 10, 71, 71), (16, 96, 14, 14)]
+
+
+@pytest.mark.parametrize("shift,shift_out", [(0, 0), (1, 1), (3, 3), (5, 5), (2, 0)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
+@pytest.mark.parametrize("N,C,H,W", BN_WINDOW_CASES)
+def test_batch_norm_training_on_maps_that_are_not_whole_packets(K, N, C, H, W, dtype, shift,
+                                                                shift_out):
+    """NCHW feature maps whose (n, c) runs are not whole 16-byte packets, at bases shifted by
+    whole elements: the single-read kernels take the aligned packets that cover each run
+    (inputs and outputs shifted alike), or the call goes the split way (shifted differently).
+    What surrounds the inputs is NaN and must not reach a channel's sums; nothing outside the
+    outputs may be written; the backward may overwrite dy."""
+    shape, S = (N, C, H, W), H * W
+    rng = U.rng_for(540 + N + H)
+    an = acc_name(dtype)
+    x = R.to_bits((2 * rng.standard_normal(shape) + 0.5).astype(np.float32), dtype)
+    dy = R.to_bits(rng.standard_normal(shape).astype(np.float32), dtype)
+    g, b = U.affine_params(rng, C, dtype)
+    rm0 = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    rv0 = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    xo, od = oracle_dtype_inputs(x, dtype)
+    dyo, _ = oracle_dtype_inputs(dy, dtype)
+    rm_ref, rv_ref = rm0.copy(), rv0.copy()
+    y_ref, mu_ref, rsig_ref, params_ref = R.op_batch_norm_train(
+        od, np.asarray(xo).reshape(shape), g, b, rm_ref, rv_ref, 1, 0.9, 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_train_grad(
+        od, np.asarray(xo).reshape(shape), g, np.asarray(dyo).reshape(shape), mu_ref, rsig_ref, 1)
+    n, guard = N * C * S, 24
+
+    def shifted(shift, bits=None, fill=0.0):
+        buf = empty((n + shift + guard,), dtype)
+        buf.fill_(fill)
+        view = buf[shift:shift + n].view(shape)
+        if bits is not None:
+            view.copy_(U.to_device(bits, dtype).view(shape))
+        return buf, view
+
+    def untouched(buf, shift):
+        flat = U.widen(U.to_host(buf), dtype).ravel()
+        return np.all(flat[:shift] == -7.0) and np.all(flat[shift + n:] == -7.0)
+
+    _, xd = shifted(shift, x, fill=float("nan"))
+    _, dyd = shifted(shift, dy, fill=float("nan"))
+    gd, bd = U.to_device(g, an), U.to_device(b, an)
+    mu, rsig, params = empty((C,), an), empty((C,), an), empty((2 * C,), an)
+    rm, rv = U.to_device(rm0, an), U.to_device(rv0, an)
+    ybuf, y = shifted(shift_out, fill=-7.0)
+    K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, xd, gd, bd, rm, rv, mu, rsig, params, y)
+    assert U.normwise(U.to_host(mu), mu_ref) <= 1e-5
+    assert np.max(np.abs(U.to_host(rsig) / rsig_ref - 1)) <= 1e-5
+    assert U.normwise(U.to_host(params), params_ref) <= 1e-5
+    assert U.normwise(U.to_host(rm), rm_ref) <= 1e-5 and U.normwise(U.to_host(rv), rv_ref) <= 1e-5
+    assert U.normwise(U.widen(U.to_host(y.contiguous()), dtype), y_ref) <= U.TIGHT[dtype]
+    assert untouched(ybuf, shift_out)
+
+    mud, rsd = U.to_device(mu_ref, an), U.to_device(rsig_ref, an)
+    wg = empty((2 * C,), an)
+    dxbuf, dx = shifted(shift_out, fill=-7.0)
+    K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", xd, mud, rsd, gd, dyd, wg, wg, dx)
+    w = U.to_host(wg)
+    assert U.normwise(w[:C], dg_ref) <= 2e-5 and U.normwise(w[C:], db_ref) <= 2e-5
+    got = U.to_host(dx.contiguous())
+    assert U.normwise(U.widen(got, dtype), dx_ref) <= U.TIGHT[dtype]
+    assert untouched(dxbuf, shift_out)
+    if shift == shift_out:
+        # dx over dy: the same bits, and the guards around dy still as they were
+        inbuf, dyin = shifted(shift, dy, fill=-7.0)
+        wg2 = empty((2 * C,), an)
+        K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", xd, mud, rsd, gd, dyin, wg2, wg2,
+                                       dyin)
+        assert np.array_equal(U.to_host(dyin.contiguous()), got)
+        assert np.array_equal(U.to_host(wg2), w)
+        assert untouched(inbuf, shift)
+
+
 def _same_specials(got, want):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     assert np.array_equal(np.isnan(got), np.isnan(want))
