@@ -967,7 +967,18 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
 // a channel is a group of adjacent lanes of one (slot, wavefront) pair, reduced
 // with shuffles and written by its first lane; gamma is read per lane.
 // partial[(n*C + c)*2 + {0,1}] receives this group's share of dgamma / dbeta.
-enum ChannelMode { kChannelWaves = 0, kChannelStraddles = 1, kChannelLanes = 2, kChannelPackets = 3 };
+// kChannelStraddlesAny is kChannelStraddles for channels that are not whole
+// packets (S any number of elements from 64 packets' worth on, the group still
+// whole aligned packets): the 64 packets of a (slot, wavefront) pair lie in at
+// most two channels, and the boundary may fall inside one packet, whose lane
+// then picks gamma and the channel share per element.
+enum ChannelMode {
+  kChannelWaves = 0,
+  kChannelStraddles = 1,
+  kChannelLanes = 2,
+  kChannelPackets = 3,
+  kChannelStraddlesAny = 4
+};
 // kChannelPackets (group_norm_grad_rows_any): at most this many packets per
 // group, 4 accumulator words of LDS each.
 constexpr int kMaxEntryPackets = 4096;
@@ -985,7 +996,8 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   constexpr int kWaves = kTPR / kWaveSize;
-  constexpr bool kStraddle = kMode == kChannelStraddles;
+  constexpr bool kAnyS = kMode == kChannelStraddlesAny;
+  constexpr bool kStraddle = kMode == kChannelStraddles || kAnyS;
   constexpr bool kLanes = kMode == kChannelLanes;
   constexpr int kParts = kStraddle ? 4 : 2;  // per entry: (dgamma, dbeta) of one or two channels
   __shared__ A slots[2 * Tile::kSlots];
@@ -1007,6 +1019,15 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     chan = p0 / packets_per_chan;
     in_first = (chan + 1) * packets_per_chan - p0;
     if (chan >= D) chan = D - 1, in_first = kWaveSize;
+  };
+  // kAnyS, the same in elements: the channel of the first element of the 64
+  // packets, and how many of their 64 * kVec elements lie in it.
+  constexpr uint32_t kSpan = kWaveSize * kVec;
+  auto first_channel_elems = [&](int i, uint32_t& chan, uint32_t& in_first) {
+    const uint32_t e0 = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) * kVec;
+    chan = e0 / S;
+    in_first = (chan + 1) * S - e0;
+    if (chan >= D) chan = D - 1, in_first = kSpan;
   };
 
   // A workgroup fills the compute unit's registers, so the next group cannot be
@@ -1031,7 +1052,37 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     A s1 = A(0), s2 = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      if constexpr (kLanes) {
+      if constexpr (kAnyS) {
+        uint32_t chan, in_first;
+        first_channel_elems(i, chan, in_first);
+        const A ga = gamma[c0 + chan], gb = gamma[c0 + (chan + 1 < D ? chan + 1 : chan)];
+        // The boundary falls into the packet of lane `edge`, `km` elements into
+        // it (0: between two packets); both are uniform over the wavefront.
+        const int edge = static_cast<int>(in_first / kVec), km = static_cast<int>(in_first % kVec);
+        if (Tile::active(i, npackets)) {
+          A xv[kVec], dv[kVec];
+          tx.unpack(i, xv);
+          tdy.unpack(i, dv);
+          if (km == 0 || wave_lane != edge) {
+            A p1 = A(0), p2 = A(0);
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              p1 += dv[e] * xv[e];
+              p2 += dv[e];
+            }
+            const A g = wave_lane < edge ? ga : gb;
+            s1 += g * p1;
+            s2 += g * p2;
+          } else {
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              const A t = (e < km ? ga : gb) * dv[e];
+              s1 += t * xv[e];
+              s2 += t;
+            }
+          }
+        }
+      } else if constexpr (kLanes) {
         const uint32_t chan = static_cast<uint32_t>(i * kTPR + lane) / packets_per_chan;
         gam[i] = gamma[c0 + (chan < D ? chan : D - 1)];
       } else {
@@ -1043,7 +1094,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           gam[i] = static_cast<uint32_t>(wave_lane) < in_first ? gam[i] : second;
         }
       }
-      if (Tile::active(i, npackets)) {
+      if (!kAnyS && Tile::active(i, npackets)) {
         // gamma is one value per thread and slot: it multiplies the slot's sums once
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
@@ -1071,7 +1122,44 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       A t1 = A(0), t2 = A(0);
-      if (Tile::active(i, npackets)) {
+      A u1 = A(0), u2 = A(0);  // kAnyS: the second channel's share of a packet on the boundary
+      if constexpr (kAnyS) {
+        uint32_t chan, in_first;
+        first_channel_elems(i, chan, in_first);
+        const int edge = static_cast<int>(in_first / kVec), km = static_cast<int>(in_first % kVec);
+        if (Tile::active(i, npackets)) {
+          const A ga = gamma[c0 + chan] * r, gb = gamma[c0 + (chan + 1 < D ? chan + 1 : chan)] * r;
+          A xv[kVec], dv[kVec];
+          tx.unpack(i, xv);
+          tdy.unpack(i, dv);
+          if (km == 0 || wave_lane != edge) {
+            const A gr = wave_lane < edge ? ga : gb;
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              const A xc = xv[e] - m;
+              t1 += dv[e] * xc;
+              t2 += dv[e];
+              xv[e] = gr * dv[e] + (u0 * xc - v0);
+            }
+            if (wave_lane >= edge) u1 = t1, u2 = t2, t1 = A(0), t2 = A(0);
+          } else {
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              const bool head = e < km;
+              const A xc = xv[e] - m;
+              const A w = dv[e] * xc;
+              t1 += head ? w : A(0);
+              t2 += head ? dv[e] : A(0);
+              u1 += head ? A(0) : w;
+              u2 += head ? A(0) : dv[e];
+              xv[e] = (head ? ga : gb) * dv[e] + (u0 * xc - v0);
+            }
+          }
+          t1 *= r;
+          u1 *= r;
+          tx.store_slot(dx + row * L, i, xv);
+        }
+      } else if (Tile::active(i, npackets)) {
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
@@ -1090,7 +1178,23 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
         tx.load_slot_unmasked(nx, i, npackets);
         tdy.load_slot_unmasked(ndy, i, npackets);
       }
-      if constexpr (kLanes) {
+      if constexpr (kAnyS) {
+        uint32_t chan, in_first;
+        first_channel_elems(i, chan, in_first);
+        const A a1 = wave_allreduce(t1, SumOp());
+        const A a2 = wave_allreduce(t2, SumOp());
+        A b1 = A(0), b2 = A(0);
+        if (in_first < kSpan) {  // uniform over the wavefront
+          b1 = wave_allreduce(u1, SumOp());
+          b2 = wave_allreduce(u2, SumOp());
+        }
+        if (wave_lane == 0) {
+          chan_part[i][wave][0] = a1;
+          chan_part[i][wave][1] = a2;
+          chan_part[i][wave][2] = b1;
+          chan_part[i][wave][3] = b2;
+        }
+      } else if constexpr (kLanes) {
         // packets_per_chan is a power of two below 64: xor-shuffles within the channel's lanes
         for (uint32_t o = 1; o < packets_per_chan; o <<= 1) {
           t1 += __shfl_xor(t1, static_cast<int>(o), kWaveSize);
@@ -1135,7 +1239,17 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
       // `lane` owns the packets [lane * packets_per_chan, (lane + 1) * packets_per_chan).
       A a = A(0), b = A(0);
       const A* entries = &chan_part[0][0][0];
-      if constexpr (kStraddle) {
+      if constexpr (kAnyS) {
+        // the same in elements: entry q covers elements [q kSpan, (q + 1) kSpan)
+        const uint32_t lo = static_cast<uint32_t>(lane) * S;
+        const uint32_t q0 = lo / kSpan, q1 = (lo + S - 1) / kSpan;
+#pragma nounroll
+        for (uint32_t q = q0; q <= q1; ++q) {
+          const uint32_t part = q * kSpan >= lo ? 0u : 2u;
+          a += entries[4 * q + part];
+          b += entries[4 * q + part + 1];
+        }
+      } else if constexpr (kStraddle) {
         const uint32_t lo = static_cast<uint32_t>(lane) * packets_per_chan;
         const uint32_t q0 = lo / kWaveSize, q1 = (lo + packets_per_chan - 1) / kWaveSize;
 #pragma nounroll
@@ -2033,6 +2147,13 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
     *mode = per_chan % kWaveSize == 0 ? kChannelWaves : kChannelStraddles;
   } else if (S % kVec == 0 && (per_chan & (per_chan - 1)) == 0) {
     *mode = kChannelLanes;
+  } else if (S >= kWaveSize * kVec && (D * S) % kVec == 0 &&
+             !(kVec == 8 && D * S / kVec > 4096)) {
+    // Channels of 64 packets' worth or more that are not whole packets. Not for
+    // 16-bit groups of more than 4096 packets: eight packets per thread and tensor
+    // plus the per-element boundary code spill 156 bytes at 128 registers, and
+    // the kernel then runs no faster than the general path.
+    *mode = kChannelStraddlesAny;
   } else if (S >= kVec && (D * S) % kVec == 0 && D * S / kVec <= kMaxEntryPackets) {
     // channels that are not whole packets (or a number of packets the lane
     // flavour does not take): one LDS entry per packet
@@ -2522,6 +2643,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     }                                                                                           \
   } else {                                                                                      \
     auto kernel = mode == kChannelStraddles ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddles> \
+        : mode == kChannelStraddlesAny ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddlesAny>   \
         : mode == kChannelLanes             ? group_norm_grad_rows<T, TPR, VPT, kChannelLanes>     \
                                             : group_norm_grad_rows<T, TPR, VPT, kChannelWaves>;    \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), 0, stream, rows, L, sh.G, sh.D, sh.S, xp, \

@@ -519,7 +519,12 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             ((2, 6, 33, 35), 1, 2), ((1, 2, 301, 303), 1, 2),
             # 14x14 and 7x7 maps in groups of whole packets: the fused backward with one LDS
             # entry per packet (up to 100 KB of dynamic LDS in fp64)
-            ((2, 64, 14, 14), 1, 2), ((3, 128, 7, 7), 1, 4)]
+            ((2, 64, 14, 14), 1, 2), ((3, 128, 7, 7), 1, 4),
+            # channels of 64 packets' worth or more that are not whole packets, in groups that
+            # are: a wavefront's packets split between two channels inside one packet (or, for
+            # (2, 8, 4, 257) in 16-bit types, inside one and between two by turns)
+            ((2, 32, 35, 35), 1, 4), ((2, 16, 23, 23), 1, 2), ((1, 32, 63, 63), 1, 4),
+            ((2, 8, 4, 257), 1, 2)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
