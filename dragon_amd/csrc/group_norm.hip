@@ -773,8 +773,9 @@ __global__ __launch_bounds__(kReduceThreads) void layer_norm_wide_grad(
 // Moments -> InvStd -> GroupNorm in one pass over x: the group stays in
 // registers between the statistics and the normalisation.
 // kAnyS: a channel is not whole packets (the group still is), so the elements
-// of a packet may belong to different channels.
-template <typename T, int kTPR, int kVPT, bool kAnyS = false>
+// of a packet may belong to different channels; 2 where a channel is 64 packets'
+// worth or more, 1 for shorter ones.
+template <typename T, int kTPR, int kVPT, int kAnyS = 0>
 __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const typename IO<T>::Acc eps, const T* __restrict__ x,
@@ -849,7 +850,31 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
       const uint32_t first = Tile::active(i, npackets) ? col / S : 0u;
       A v[kVec];
       t.unpack(i, v);
-      if constexpr (kAnyS) {
+      if constexpr (kAnyS == 2) {
+        {
+          // The wavefront's 64 packets lie in at most two channels, and the
+          // boundary in the packet of one lane: its place and both channels'
+          // parameters are uniform over the wavefront (scalar registers); only
+          // that lane picks per element.
+          const uint32_t e0 = static_cast<uint32_t>(
+              i * kTPR + __builtin_amdgcn_readfirstlane(lane / kWaveSize) * kWaveSize) * kVec;
+          uint32_t chan = e0 / S;
+          uint32_t in_first = (chan + 1) * S - e0;
+          if (chan >= D) chan = D - 1, in_first = kWaveSize * kVec;
+          const uint32_t ca = c0 + chan, cb = c0 + (chan + 1 < D ? chan + 1 : chan);
+          const A ga = gamma[ca] * rs, gb = gamma[cb] * rs, ba = beta[ca], bb = beta[cb];
+          const int edge = static_cast<int>(in_first / kVec), km = static_cast<int>(in_first % kVec);
+          const int wave_lane = lane & (kWaveSize - 1);
+          if (km == 0 || wave_lane != edge) {
+            const A gam = wave_lane < edge ? ga : gb, bet = wave_lane < edge ? ba : bb;
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+          } else {
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * (e < km ? ga : gb) + (e < km ? ba : bb);
+          }
+        }
+      } else if constexpr (kAnyS == 1) {
         const uint32_t rem = Tile::active(i, npackets) ? col - first * S : 0u;
         if (S >= static_cast<uint32_t>(kVec)) {
           // at most two channels per packet: their parameters once, picked per element
@@ -2453,8 +2478,10 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
     const unsigned one_shot = row_grid(rows, Tile::kRowsPerBlock);                              \
-    auto kernel = sh.S % kVec != 0 ? group_norm_forward_rows<T, TPR, VPT, true>                 \
-                                   : group_norm_forward_rows<T, TPR, VPT, false>;               \
+    auto kernel = sh.S % kVec == 0 ? group_norm_forward_rows<T, TPR, VPT, 0>                    \
+        : sh.S >= kWaveSize * kVec && !(kVec == 8 && VPT == 8 && TPR == 1024) /* spills: 82 us against 66 */ \
+            ? group_norm_forward_rows<T, TPR, VPT, 2>                                           \
+            : group_norm_forward_rows<T, TPR, VPT, 1>;                                          \
     const unsigned resident = TPR == 1024 ? resident_grid(kernel, TPR, 0) : one_shot;           \
     hipLaunchKernelGGL(kernel,                                                                  \
                        dim3(one_shot < resident ? one_shot : resident), dim3(Tile::kThreads), 0, stream, \
