@@ -282,6 +282,8 @@ WORKLOADS = {
     "softmax_bf16_605184x197": lambda k: wl_softmax((605184, 197), "bfloat16", 1, k=k),
     "layer_norm_bf16_1048576x64": lambda k: wl_layer_norm(1048576, 64, "bfloat16", 4, k=k),
     "softmax_f32_2048x128256": lambda k: wl_softmax((2048, 128256), "float32", 1, k=k),
+    # feature maps that are not whole 16-byte packets (the BASELINE BatchNorm shape at 57x57)
+    "batch_norm_f32_64x256x57x57": lambda k: wl_batch_norm((64, 256, 57, 57), "float32", 2, k=k),
     # a vocabulary whose rows are not whole 16-byte packets
     "softmax_bf16_4096x50257": lambda k: wl_softmax((4096, 50257), "bfloat16", 1, k=k),
 }

@@ -251,3 +251,72 @@ def test_softmax_bench_shapes_sampled_rows_and_every_row(K, shape, dtype, log):
     e_go, e_ge, e_oe = (U.rowwise_normwise(dxw, dx_ref), U.rowwise_normwise(dxw, dx64),
                         U.rowwise_normwise(dx_ref, dx64))
     assert e_ge <= tol and e_go <= tol + e_oe, (e_go, e_ge, e_oe)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_batch_norm_64x256x57x57_sampled_channels_and_every_channel(K, dtype):
+    """bench workload batch_norm_f32_64x256x57x57: feature maps that are not whole packets
+    through the single-read kernels, four rounds of work items over the resident grid. The
+    oracle's operator checks sampled channels (channels are independent); every channel goes
+    through the closed forms in fp64 on the device and through the property that a
+    batch-normalised channel's input gradient sums to zero."""
+    import torch
+    N, C, H, W = 64, 256, 57, 57
+    S = H * W
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    td = U.torch_dtype(dtype)
+    x = torch.empty((N, C, S), device="cuda").normal_(generator=gen).mul_(2).add_(0.5).to(td)
+    dy = torch.empty((N, C, S), device="cuda").normal_(generator=gen).to(td)
+    g = torch.empty(C, device="cuda").uniform_(0.5, 1.5, generator=gen)
+    b = torch.empty(C, device="cuda").normal_(generator=gen).mul_(0.1)
+    rm, rv = torch.zeros(C, device="cuda"), torch.ones(C, device="cuda")
+    mu, rsig, params = (torch.empty(n, device="cuda") for n in (C, C, 2 * C))
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    wg = torch.empty(2 * C, device="cuda")
+    K.batch_norm_training_forward(N, C, S, "NCHW", 0.9, 1e-5, x, g, b, rm, rv, mu, rsig, params, y)
+    K.batch_norm_training_backward(N, C, S, float(N * S), "NCHW", x, mu, rsig, g, dy, wg, wg, dx)
+    torch.cuda.synchronize()
+    tol = U.TIGHT[dtype]
+    # every channel: fp64 closed forms on the device
+    x64, dy64 = x.double(), dy.double()
+    mu64 = x64.mean((0, 2))
+    var64 = x64.var((0, 2), unbiased=False)
+    rsig64 = torch.rsqrt(var64 + 1e-5)
+    assert float((mu.double() - mu64).abs().max()) <= 1e-5 * float(mu64.abs().max())
+    assert float((rsig.double() / rsig64 - 1).abs().max()) <= 1e-5
+    assert float((rm.double() - 0.1 * mu64).abs().max()) <= 1e-5
+    assert float((rv.double() - (0.9 + 0.1 * var64)).abs().max()) <= 1e-4
+    xh = (x64 - mu.double()[None, :, None]) * rsig.double()[None, :, None]
+    y64 = xh * g.double()[None, :, None] + b.double()[None, :, None]
+    assert float((y.double() - y64).norm() / y64.norm()) <= tol
+    dg64, db64 = (dy64 * xh).sum((0, 2)), dy64.sum((0, 2))
+    assert float((wg[:C].double() - dg64).norm() / dg64.norm()) <= 2e-5
+    assert float((wg[C:].double() - db64).norm() / db64.norm()) <= 2e-5
+    dx64 = (g.double() * rsig.double())[None, :, None] * (
+        dy64 - (xh * dg64[None, :, None] + db64[None, :, None]) / (N * S))
+    assert float((dx.double() - dx64).norm() / dx64.norm()) <= tol
+    # (16-bit outputs: 207936 roundings per channel, bounded relative to the sum of magnitudes)
+    sums, mags = dx.double().sum((0, 2)).abs(), dx.double().abs().sum((0, 2))
+    assert float(sums.max()) < 5e-2 if dtype == "float32" else bool((sums <= 1e-3 * mags).all())
+    del x64, dy64, xh, y64, dx64
+    # sampled channels against the oracle's operator (first, last, and ones that later
+    # rounds of the grid reach)
+    chans = [0, 1, 100, 191, 254, 255]
+    idx = torch.as_tensor(chans, device="cuda")
+    xs = U.to_host(x[:, idx].contiguous()).reshape(N, len(chans), H, W)
+    dys = U.to_host(dy[:, idx].contiguous()).reshape(N, len(chans), H, W)
+    gs, bs = U.to_host(g[idx]), U.to_host(b[idx])
+    xo, od = (R.from_bits(xs, dtype), "float32") if dtype != "float32" else (xs, "float32")
+    dyo = R.from_bits(dys, dtype) if dtype != "float32" else dys
+    rm_ref, rv_ref = np.zeros(len(chans), np.float32), np.ones(len(chans), np.float32)
+    y_ref, mu_ref, rsig_ref, _ = R.op_batch_norm_train(od, xo, gs, bs, rm_ref, rv_ref, 1, 0.9, 1e-5)
+    dx_ref, dg_ref, db_ref = R.op_batch_norm_train_grad(od, xo, gs, dyo, mu_ref, rsig_ref, 1)
+    # the oracle's sequential fp32 sums over 207936 terms are themselves ~5e-5 off fp64
+    assert U.normwise(U.to_host(mu[idx]), mu_ref) <= 1e-4
+    assert np.max(np.abs(U.to_host(rsig[idx]) / rsig_ref - 1)) <= 1e-4
+    yg = U.to_host(y[:, idx].contiguous()).reshape(xs.shape)
+    dxg = U.to_host(dx[:, idx].contiguous()).reshape(xs.shape)
+    assert U.normwise(U.widen(yg, dtype), y_ref) <= max(tol, 1e-4)
+    assert U.normwise(U.widen(dxg, dtype), dx_ref) <= max(tol, 1e-4)
+    assert U.normwise(U.to_host(wg[:C][idx]), dg_ref) <= 1e-4
+    assert U.normwise(U.to_host(wg[C:][idx]), db_ref) <= 1e-4
