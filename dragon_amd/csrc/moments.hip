@@ -223,7 +223,47 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_strided_columns(
   }
 }
 
-enum PlanKind { kPlanSegments, kPlanColumns, kPlanGather, kPlanShortRows, kPlanStrided };
+// Rows of a few thousand contiguous elements, thousands of them: one wavefront
+// per row (four rows per workgroup), no LDS and no second stage. A row is read
+// as the aligned 16-byte packets that cover it, whatever its width and address;
+// of its first and last packet only the row's own elements are folded in.
+template <typename T, typename P>
+__global__ __launch_bounds__(kReduceThreads) void reduce_wave_rows(
+    const uint32_t rows, const uint32_t len, const T* __restrict__ x, const typename P::Out out,
+    const typename IO<T>::Acc inv_n) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const uint32_t wave = threadIdx.x / kWaveSize;
+  const int n = static_cast<int>(len);
+  for (uint32_t row = blockIdx.x * kReduceWaves + wave; row < rows; row += gridDim.x * kReduceWaves) {
+    const T* r = x + static_cast<size_t>(row) * len;
+    const A shift = P::kShift ? load_shift(r) : A(0);
+    const int lead = static_cast<int>((reinterpret_cast<uintptr_t>(r) & 15u) / sizeof(T));
+    const int packets = (lead + n + kVec - 1) / kVec;
+    A a = A(0), b = A(0);
+#pragma unroll 4
+    for (int p = lane; p < packets; p += kWaveSize) {
+      const int pe = p * kVec - lead;  // the packet's first element, in the row
+      A v[kVec];
+      load_unpack_keep<T>(r + pe, v);
+      if (pe >= 0 && pe + kVec <= n) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) P::term(P::kShift ? v[e] - shift : v[e], a, b);
+      } else {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (pe + e >= 0 && pe + e < n) P::term(P::kShift ? v[e] - shift : v[e], a, b);
+        }
+      }
+    }
+    a = wave_allreduce(a, SumOp());
+    b = wave_allreduce(b, SumOp());
+    if (lane == 0) P::finish(out, row, shift, a, b, inv_n);
+  }
+}
+
+enum PlanKind { kPlanSegments, kPlanColumns, kPlanGather, kPlanShortRows, kPlanStrided, kPlanWaveRows };
 struct MomentsPlan {
   PlanKind kind;
   SegmentedReduce seg;
@@ -277,6 +317,14 @@ int make_plan(int dtype, int num_dims, const int64_t* dims, int num_axes, const 
     // enough outputs to fill the device with a thread each
     plan->kind = kPlanStrided;
     s.nseg = u32(ext[0]), s.seglen = u32(ext[1]), s.seg_stride = u32(ext[2]);  // N, C, S
+  } else if (pat == "KR" && plan->n_out >= 2048 && dtype != DRAGON_HIP_F64 &&
+             plan->n_red * (dtype == DRAGON_HIP_F32 ? 4 : 2) <= 20 * 1024) {
+    // Rows of up to 20 KB, 2048 of them or more: a wavefront each. Measured against
+    // a workgroup per row: fp32 [65536,1025] 49 us against 83, [16384,4097] 46
+    // against 53, [8192,8192] 51 against 47 (left to the workgroups); bf16
+    // [32768,2048] 27 against 37, [8192,8192] 26 against 28; with 2048 rows of
+    // 128 KB the wavefronts are too few (78 us against 50).
+    plan->kind = kPlanWaveRows;
   } else if (pat == "R" || pat == "KR") {
     plan->kind = kPlanSegments;
     s.stride1 = u32(plan->n_red), s.seglen = u32(plan->n_red);
@@ -333,6 +381,13 @@ int launch_reduce(const MomentsPlan& plan, const void* x, const typename P::Out&
     DRAGON_HIP_SHORT_LAUNCH(T, typename Holder::template Op, sp, lds,
                             short_grid(plan.n_out, sp.rows_per_chunk), stream, plan.n_out,
                             static_cast<int>(plan.n_red), xp, xp, none, out, inv_n);
+  } else if (plan.kind == kPlanWaveRows) {
+    if (sizeof(T) > 4) return DRAGON_HIP_EINVAL;  // the planner keeps fp64 on the segment kernels
+    const int64_t want = ceil_div(plan.n_out, kReduceWaves);
+    const int64_t cap = static_cast<int64_t>(num_cus()) * 32;
+    hipLaunchKernelGGL((reduce_wave_rows<T, P>), dim3(static_cast<unsigned>(want < cap ? want : cap)),
+                       dim3(kReduceThreads), 0, stream, static_cast<uint32_t>(plan.n_out),
+                       static_cast<uint32_t>(plan.n_red), xp, out, inv_n);
   } else if (plan.kind == kPlanStrided) {
     const SegmentedReduce& s = plan.seg;
     const unsigned grid = static_cast<unsigned>(

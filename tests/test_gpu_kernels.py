@@ -907,7 +907,12 @@ MOMENT_CASES = [((4, 5, 6), (0, 2)), ((20, 5), (0,)), ((6, 35), (1,)), ((3, 4, 2
                 # a reduced axis between kept ones, a thread per output
                 ((70, 9, 300), (1,)), ((4200, 33, 4), (1,)),
                 # fewer than 64 columns: the lanes a row leaves idle take adjacent rows
-                ((20000, 2), (0,)), ((3000, 24), (0,))]
+                ((20000, 2), (0,)), ((3000, 24), (0,)),
+                # thousands of rows of a few KB: a wavefront per row through the aligned packets
+                # that cover it
+                ((2100, 1025), (1,)), ((2048, 4099), (1,)), ((2500, 2048), (1,)),
+                # segments that are not whole packets, a workgroup or several per output
+                ((40, 4097), (1,)), ((6, 10, 3137), (0, 2)), ((3, 20001), (1,))]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "float64"])
@@ -933,7 +938,8 @@ def test_moments(K, shape, axes, dtype):
 @pytest.mark.parametrize("shape,axes", [((6, 35), (1,)), ((16, 8192), (1,)), ((6, 70000), (1,)),
                                         ((1000, 72), (0,)), ((64, 40, 49), (0, 2)),
                                         ((5000, 7), (1,)), ((70, 9, 300), (1,)),
-                                        ((20000, 2), (0,)), ((2, 3, 4), (0, 1, 2))])
+                                        ((20000, 2), (0,)), ((2, 3, 4), (0, 1, 2)),
+                                        ((2100, 1025), (1,)), ((40, 4097), (1,))])
 def test_moments_special_values_follow_the_reference(K, shape, axes, dtype):
     """inf and nan among the reduced elements, the first one included (the sample the
     shifted sums are taken from): the mean is the infinity or nan that the CPU kernel's
