@@ -43,10 +43,13 @@ struct ColumnReduce {
 };
 
 // How many workgroups share one output: enough to put ~8 workgroups on every
-// compute unit, but never less than ~16K elements per workgroup.
+// compute unit, but never less than ~16K elements per workgroup. Rounded down:
+// a few workgroups more than the device holds at once would run as a second,
+// nearly empty round (48 column tiles x 43 = 2064 workgroups on 256 compute
+// units: 88 us; x 42: one round).
 inline uint32_t pick_split(int64_t n_out, int64_t elems_per_out) {
   const int64_t want_blocks = static_cast<int64_t>(num_cus()) * 8;
-  int64_t split = ceil_div(want_blocks, n_out > 0 ? n_out : 1);
+  int64_t split = want_blocks / (n_out > 0 ? n_out : 1);
   const int64_t max_by_work = ceil_div(elems_per_out, 16384);
   if (split > max_by_work) split = max_by_work;
   if (split < 1) split = 1;
@@ -319,6 +322,12 @@ inline uint32_t launch_reduce2_columns(uint32_t rows, uint32_t cols, const T* in
     while (lanes_per_row < kWaveSize && lanes_per_row * kVec < cols) lanes_per_row <<= 1;
     const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, lanes_per_row * kVec));
     d.split = pick_split(tiles, static_cast<int64_t>(rows) * kWaveSize * kVec);
+    // The pairs are written once and read once, 16 bytes per column and split
+    // against rows * sizeof(T) bytes of input per column: where that is more
+    // than a twelfth, half as many workgroups with twice the rows each.
+    if (static_cast<int64_t>(d.split) * 16 * 12 > static_cast<int64_t>(rows) * sizeof(T)) {
+      d.split = (d.split + 1) / 2;
+    }
     hipLaunchKernelGGL((reduce2_columns_packets<T, kIn, F>), dim3(tiles * d.split),
                        dim3(kReduceThreads), 0, stream, d, lanes_per_row, in0, in1, f, partial);
   } else {
