@@ -196,7 +196,11 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
     launch_reduce2_finalize<A, E>(sh.C, sh.N, false, part, e, stream);
     return;
   }
-  if (long_channel_rows(sh, sizeof(T), in0, in1, in0)) {
+  // (Fewer than 2048 such rows are too few wavefronts: they go to the split
+  // segment reduction below, through their packet windows. [16,32,225,225] bf16,
+  // 512 rows: 104 us a wavefront per row, 30 us split.)
+  if (long_channel_rows(sh, sizeof(T), in0, in1, in0) &&
+      !(sizeof(T) <= 4 && static_cast<int64_t>(sh.N) * sh.C < 2048)) {
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
     const ChannelRowSumsOp<T, 8, F, kIn> op{f, sh.C, sh.S, part};
     hipLaunchKernelGGL((long_rows_sums<T, kIn, ChannelRowSumsOp<T, 8, F, kIn>>),
@@ -212,6 +216,9 @@ void reduce_channels(const ChannelShape& sh, const T* in0, const T* in1, F f, E 
     if (vec_ok) {
       hipLaunchKernelGGL((reduce2_segments<T, kIn, kVec, F>), grid, dim3(kReduceThreads), 0, stream,
                          s, in0, in1, f, part);
+    } else if (sizeof(T) <= 4 && sh.S >= 4u * kVec && congruent16(in0, in1)) {
+      hipLaunchKernelGGL((reduce2_segments_windows<T, kIn, F>), grid, dim3(kReduceThreads), 0,
+                         stream, s, in0, in1, f, part);
     } else {
       hipLaunchKernelGGL((reduce2_segments<T, kIn, 1, F>), grid, dim3(kReduceThreads), 0, stream, s,
                          in0, in1, f, part);
@@ -510,6 +517,19 @@ void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hi
     return static_cast<size_t>(q.stage_packets) * 16 * kIn +
         static_cast<size_t>(q.rows_per_chunk) * F<T, 1>::kParams * sizeof(A);
   };
+  // Maps of 48 packets or more that are not whole aligned packets: the aligned
+  // packets that cover the tensor, the channel found once per packet. Shorter
+  // ones have a packet across two maps in every wavefront and do better staged
+  // through LDS (bf16 7x7 with two inputs: 43 us against 32; fp32 15x15: 62
+  // against 67 the other way).
+  if (sizeof(T) <= 4 && sh.S / kVec >= 48 && ragged_channel_rows(sh, sizeof(T), in0, in1, out)) {
+    using Fn = F<T, 1>;
+    const ChannelRowMapOp<T, 8, Fn, kIn> op{Fn{ChannelIndex{sh}, args...}, sh.C};
+    hipLaunchKernelGGL((map_flat_windows<T, kIn, ChannelRowMapOp<T, 8, Fn, kIn>>),
+                       dim3(map_grid(total / kVec + 2)), dim3(256), 0, stream, total, sh.S, in0, in1,
+                       out, op);
+    return;
+  }
   if (short_channel_rows(sh, sizeof(T), in0, in1, out) &&
       plan_short_rows_within(sh.S, sizeof(T), kIn == 1 ? 4 : 3, false, lds_of, &sp)) {
     using Fn = F<T, 1>;
@@ -522,7 +542,7 @@ void map_channels(const ChannelShape& sh, const T* in0, const T* in1, T* out, hi
                             static_cast<int>(sh.S), in0, in1, out, fn, sh.C);
     return;
   }
-  if (long_channel_rows(sh, sizeof(T), in0, in1, out)) {
+  if (long_channel_rows(sh, sizeof(T), in0, in1, out)) {  // (fp64 only: see above)
     using Fn = F<T, 1>;
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
     const ChannelRowMapOp<T, 8, Fn, kIn> op{Fn{ChannelIndex{sh}, args...}, sh.C};

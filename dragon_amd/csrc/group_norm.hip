@@ -1552,6 +1552,39 @@ __global__ __launch_bounds__(256) void channel_pair_sums_short(
 // maps): policies of the LDS-staged short-row kernel (short_rows.h), which
 // moves aligned packets whatever S is. The row's scalars are fetched once per
 // row with the range's packets.
+// The same pairs by the split segment reduction (reduce.h), for long (n, c) rows
+// that are too few to give every compute unit a wavefront each: several
+// workgroups per row, then `StorePairs` as the second stage's epilogue.
+template <typename T>
+struct RowPairAccum {
+  using A = typename IO<T>::Acc;
+  const A* mu;
+  uint32_t D;
+  A m;
+  __device__ __forceinline__ void begin(uint32_t row, uint32_t) { m = mu[row / D]; }
+  template <int V>
+  __device__ __forceinline__ void add(uint32_t, uint32_t, uint32_t, uint32_t, const A (&x)[V],
+                                      const A (&dy)[V], A& a, A& b) const {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      a += dy[e] * (x[e] - m);
+      b += dy[e];
+    }
+  }
+};
+template <typename A>
+struct StorePairs {
+  A* out;
+  __device__ __forceinline__ void operator()(uint32_t o, A a, A b) const {
+    out[2 * o] = a;
+    out[2 * o + 1] = b;
+  }
+};
+// Rows of more than 1024 elements, fewer than 2048 of them: how many workgroups share one.
+inline uint32_t few_long_rows_split(int64_t rows, int64_t S) {
+  return rows < 2048 && S > 1024 ? pick_split(rows, S) : 0u;
+}
+
 template <typename T, int kE>
 struct GroupRowPairSums {  // in0 = x, in1 = dy; reads only
   using A = typename IO<T>::Acc;
@@ -2219,6 +2252,8 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   size_t pairs = static_cast<size_t>(N) * C;
   if (pairs * 2 * sizeof(A) < row_paths) pairs = row_paths / (2 * sizeof(A));
   if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
+  // few long rows: the split reduction's partial pairs behind the N*C pairs
+  if (layout == DRAGON_HIP_NCHW) pairs += static_cast<size_t>(N) * C * few_long_rows_split(N * C, S);
   size_t bytes = pairs * 2 * sizeof(A);
   // the slice path: the exchange of K pairs per group, then one pair per wavefront block
   if (layout == DRAGON_HIP_NCHW && S % (IO<T>::kVec * kWaveSize) == 0) {
@@ -2519,8 +2554,15 @@ int launch_group_norm(const GroupShape& sh, const void* x, const void* mu, const
         sh, static_cast<const A*>(mu), static_cast<const A*>(rsig), static_cast<const A*>(gamma),
         static_cast<const A*>(beta)}};
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
-    hipLaunchKernelGGL((long_rows_map<T, 1, GroupRowApply<T, 8>>), dim3(long_rows_grid(rows)),
-                       dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, xp, yp, op);
+    if constexpr (sizeof(T) <= 4) {
+      // the aligned packets that cover the tensor, the row's scalars found once per packet
+      hipLaunchKernelGGL((map_flat_windows<T, 1, GroupRowApply<T, 8>>),
+                         dim3(map_grid(total / kVec + 2)), dim3(256), 0, stream, total, sh.S, xp, xp,
+                         yp, op);
+    } else {
+      hipLaunchKernelGGL((long_rows_map<T, 1, GroupRowApply<T, 8>>), dim3(long_rows_grid(rows)),
+                         dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, xp, yp, op);
+    }
   } else if (vec_ok) {
     GroupNormApply<T, kVec> f{sh, static_cast<const A*>(mu), static_cast<const A*>(rsig),
                               static_cast<const A*>(gamma), static_cast<const A*>(beta)};
@@ -2709,6 +2751,17 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       T* none = nullptr;
       DRAGON_HIP_SHORT_LAUNCH(T, GroupRowPairSums, sp, lds, short_grid(rows, sp.rows_per_chunk),
                               stream, rows, static_cast<int>(sh.S), xp, dyp, none, mup, sh.D, part);
+    } else if (const uint32_t split = few_long_rows_split(rows, sh.S);
+               split > 0 && sizeof(T) <= 4 && long_group_rows(sh, sizeof(T), x, dy, dx)) {
+      const SegmentedReduce s{static_cast<uint32_t>(rows), 1u, sh.S, 0u, 1u, sh.S, 0u, split};
+      A* partial = part + static_cast<size_t>(rows) * 2;
+      hipLaunchKernelGGL((reduce2_segments_windows<T, 2, RowPairAccum<T>>), dim3(s.n_out * s.split),
+                         dim3(kReduceThreads), 0, stream, s, xp, dyp, RowPairAccum<T>{mup, sh.D, A(0)},
+                         partial);
+      hipLaunchKernelGGL((reduce2_finalize<A, StorePairs<A>>),
+                         dim3(static_cast<unsigned>(ceil_div(rows, kReduceThreads))),
+                         dim3(kReduceThreads), 0, stream, s.n_out, s.split, true, partial,
+                         StorePairs<A>{part});
     } else if (long_group_rows(sh, sizeof(T), x, dy, dx)) {
       const GroupRowPairSums<T, 8> op{mup, sh.D, part};
       hipLaunchKernelGGL((long_rows_sums<T, 2, GroupRowPairSums<T, 8>>), dim3(long_rows_grid(rows)),
@@ -2775,9 +2828,15 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     } else if (long_group_rows(sh, sizeof(T), x, dy, dx)) {
       const GroupRowGradMap<T, 8> op{GroupNormGradApply<T, 1>{sh, mup, rsp, gp, dsp, dbp, denom}};
       const int64_t rows = static_cast<int64_t>(sh.N) * sh.C;
-      hipLaunchKernelGGL((long_rows_map<T, 2, GroupRowGradMap<T, 8>>), dim3(long_rows_grid(rows)),
-                         dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, dyp, dxp,
-                         op);
+      if constexpr (sizeof(T) <= 4) {
+        hipLaunchKernelGGL((map_flat_windows<T, 2, GroupRowGradMap<T, 8>>),
+                           dim3(map_grid(total / kVec + 2)), dim3(256), 0, stream, total, sh.S, xp,
+                           dyp, dxp, op);
+      } else {
+        hipLaunchKernelGGL((long_rows_map<T, 2, GroupRowGradMap<T, 8>>), dim3(long_rows_grid(rows)),
+                           dim3(kLongThreads), 0, stream, rows, static_cast<int>(sh.S), xp, dyp, dxp,
+                           op);
+      }
     } else if (vec_ok) {
       GroupNormGradApply<T, kVec> f{sh, mup, rsp, gp, dsp, dbp, denom};
       hipLaunchKernelGGL((map_flat<T, 2, kVec, GroupNormGradApply<T, kVec>>),
@@ -2805,6 +2864,8 @@ int try_group_norm_stats_rows(const GroupShape& sh, float eps, const void* x, vo
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
   const bool packets = L % kVec == 0 && aligned16(x);
   if (!sh.nchw || packets || L <= 1024 || !fits_int32(L)) return kNotApplicable;
+  // fewer rows than that are too few wavefronts: Moments splits each row over several workgroups
+  if (rows < 2048 && sizeof(T) <= 4) return kNotApplicable;
   if (!scratch || scratch_bytes < static_cast<size_t>(rows) * 2 * sizeof(A)) return kNotApplicable;
   const T* xp = static_cast<const T*>(x);
   A* pairs = static_cast<A*>(scratch);

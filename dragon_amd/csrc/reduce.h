@@ -450,6 +450,57 @@ __global__ __launch_bounds__(256) void map_flat(const uint32_t total, const T* i
   }
 }
 
+// An element-wise map with per-run parameters over a tensor whose runs of
+// `run` elements (the feature maps of an NCHW tensor) are not whole packets, or
+// that starts at an element-aligned address (all tensors congruent modulo 16
+// bytes): the aligned 16-byte packets that cover the tensor. Op provides
+//   static constexpr int kParams;  void row_params(int64_t r, A (&w)[kParams]) const
+//   A apply(const A* w, A x0, A x1) const
+// (the interface of long_rows_map). The run is found once per packet; a packet
+// that straddles two runs takes the next run's parameters from the boundary on. Of the packets that reach beyond the tensor's ends only the
+// tensor's own elements are computed and stored. An aligned packet that holds
+// a byte of the tensor lies in that byte's page, so those may be read whole.
+template <typename T, int kIn, typename Op>
+__global__ __launch_bounds__(256) void map_flat_windows(const uint32_t total, const uint32_t run,
+                                                        const T* in0, const T* in1, T* out,
+                                                        const Op f) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const int lead = static_cast<int>((reinterpret_cast<uintptr_t>(in0) & 15u) / sizeof(T));
+  const uint32_t npackets = (static_cast<uint32_t>(lead) + total + kVec - 1) / kVec;
+  for (uint32_t ip = blockIdx.x * 256 + threadIdx.x; ip < npackets; ip += gridDim.x * 256) {
+    const int64_t i = static_cast<int64_t>(ip) * kVec - lead;  // the packet's first element
+    A v0[kVec], v1[kVec];
+    load_unpack<T>(in0 + i, v0);
+    if constexpr (kIn == 2) load_unpack<T>(in1 + i, v1);
+    const bool inside = i >= 0 && i + kVec <= static_cast<int64_t>(total);
+    const uint32_t first = static_cast<uint32_t>(i < 0 ? 0 : i);  // first element inside the tensor
+    const uint32_t r = first / run;
+    // elements of the packet, counted from `first`, that still lie in run r
+    const uint32_t left = (r + 1) * run - first;
+    A w[Op::kParams];
+    f.row_params(r, w);
+    if (inside && left >= static_cast<uint32_t>(kVec)) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) v0[e] = f.apply(w, v0[e], kIn == 2 ? v1[e] : A(0));
+      pack_store<T>(out + i, v0);
+    } else {
+      A w2[Op::kParams];
+      f.row_params((r + 2) * run <= total ? r + 1 : r, w2);  // (no run behind the last one)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const int64_t j = i + e;
+        if (j >= 0 && j < static_cast<int64_t>(total)) {
+          const bool next = static_cast<uint32_t>(j) - first >= left;
+          v0[e] = f.apply(next ? w2 : w, v0[e], kIn == 2 ? v1[e] : A(0));
+          if (!inside) IO<T>::store1(out + j, v0[e]);
+        }
+      }
+      if (inside) pack_store<T>(out + i, v0);
+    }
+  }
+}
+
 inline unsigned map_grid(uint32_t npackets) {
   const int64_t want = ceil_div(npackets, 256);
   const int64_t cap = static_cast<int64_t>(num_cus()) * 32;

@@ -754,6 +754,23 @@ def test_batch_norm_training_on_maps_that_are_not_whole_packets(K, N, C, H, W, d
     got = U.to_host(dx.contiguous())
     assert U.normwise(U.widen(got, dtype), dx_ref) <= U.TIGHT[dtype]
     assert untouched(dxbuf, shift_out)
+    # the separate entry points (the operator's own sequence): element-wise maps over the
+    # aligned packets that cover the tensor
+    y2buf, y2 = shifted(shift_out, fill=-7.0)
+    K.batch_norm(N, C, S, "NCHW", xd, mud, rsd, gd, bd, params, params, y2)
+    assert U.normwise(U.widen(U.to_host(y2.contiguous()), dtype), y_ref) <= U.TIGHT[dtype]
+    assert untouched(y2buf, shift_out)
+    wref = U.to_device(np.concatenate([dg_ref, db_ref]).astype(np.float32), an)
+    dx2buf, dx2 = shifted(shift_out, fill=-7.0)
+    K.batch_norm_training_grad(N, C, S, float(N * S), "NCHW", xd, mud, rsd, gd, wref, wref, dyd, dx2)
+    assert U.normwise(U.widen(U.to_host(dx2.contiguous()), dtype), dx_ref) <= U.TIGHT[dtype]
+    assert untouched(dx2buf, shift_out)
+    dx3buf, dx3 = shifted(shift_out, fill=-7.0)
+    K.batch_norm_inference_grad(N, C, S, "NCHW", xd, mud, rsd, gd, dyd, None, None, dx3)
+    want = np.asarray(dyo, np.float64).reshape(shape) * (
+        np.asarray(g, np.float64) * np.asarray(rsig_ref, np.float64))[None, :, None, None]
+    assert U.normwise(U.widen(U.to_host(dx3.contiguous()), dtype), want) <= U.TIGHT[dtype]
+    assert untouched(dx3buf, shift_out)
     if shift == shift_out:
         # dx over dy: the same bits, and the guards around dy still as they were
         inbuf, dyin = shifted(shift, dy, fill=-7.0)
