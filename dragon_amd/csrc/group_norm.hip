@@ -917,14 +917,17 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
 // The same for any S and any alignment (S not a multiple of a packet, so
 // that a packet may straddle channels and groups start at element-aligned
 // addresses): ragged tiles, the channel of an element found from its column.
-template <typename T, int kTPR, int kVPT>
+// kWindow: x and y congruent modulo 16 bytes; a group is read and written as the
+// aligned packets that cover it (RowWindow), with regular tiles sized for
+// L / kVec + 2 packets.
+template <typename T, int kTPR, int kVPT, bool kWindow = false>
 __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
     T* __restrict__ y) {
-  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), true>;
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), !kWindow>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
@@ -932,8 +935,15 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
   const int lane = Tile::lane();
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    const RowWindow<T> w(x + row * L, L);
+    const int lead = kWindow ? w.lead : 0;          // elements of slot 0, lane 0 before the group
+    const int extent = kWindow ? w.packets : L;     // what Tile::active counts in
     Tile t;
-    t.load(x + row * L, L, A(0));
+    if constexpr (kWindow) {
+      t.load_window(x + row * L, w, A(0));
+    } else {
+      t.load(x + row * L, L, A(0));
+    }
     A s = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i)
@@ -946,7 +956,8 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
         const A d = t.v[i][e] - mean;
-        if (Tile::elem_active(i, e, L)) q += d * d;
+        const int col = (i * kTPR + lane) * kVec + e - lead;
+        if (col >= 0 && col < L) q += d * d;
       }
     const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_l;
     const A rs = acc_rsqrt_exact(var + eps);
@@ -957,26 +968,33 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
     const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      if (Tile::active(i, L)) {
-        const uint32_t col = static_cast<uint32_t>(i * kTPR + lane) * kVec;
-        const uint32_t first = col / S;
-        const uint32_t rem = col - first * S;
-        if (rem + kVec <= S) {  // the packet lies within one channel
+      if (Tile::active(i, extent)) {
+        const int col = (i * kTPR + lane) * kVec - lead;  // below zero: the group's first packet
+        const uint32_t colp = static_cast<uint32_t>(col < 0 ? 0 : col);
+        const uint32_t first = colp / S;
+        const uint32_t rem = colp - first * S;
+        if (col >= 0 && rem + kVec <= S) {  // the packet lies within one channel
           const A gam = gamma[c0 + first] * rs, bet = beta[c0 + first];
 #pragma unroll
           for (int e = 0; e < kVec; ++e) t.v[i][e] = (t.v[i][e] - mean) * gam + bet;
         } else {
 #pragma unroll
           for (int e = 0; e < kVec; ++e) {
-            uint32_t k = rem + e, c = first;
-            while (k >= S) k -= S, ++c;
+            int k = static_cast<int>(rem) + e + (col < 0 ? col : 0);
+            if (k < 0) k = 0;  // before the group: not stored
+            uint32_t c = first;
+            while (static_cast<uint32_t>(k) >= S) k -= static_cast<int>(S), ++c;
             if (c >= D) c = D - 1;  // padding beyond the group: not stored
             t.v[i][e] = (t.v[i][e] - mean) * (gamma[c0 + c] * rs) + beta[c0 + c];
           }
         }
       }
     }
-    t.store(y + row * L, L);
+    if constexpr (kWindow) {
+      t.store_window(y + row * L, w);
+    } else {
+      t.store(y + row * L, L);
+    }
     if (kTPR != kWaveSize) __syncthreads();
   }
 }
@@ -2495,6 +2513,22 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   if (!sh.nchw || !pick_row_config(ceil_div(L, kVec), 8, &cfg)) return false;
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
   if (L % kVec != 0 || !aligned16(x) || !aligned16(y)) {
+    if (RowConfig wc; sizeof(T) <= 4 && congruent16(x, y) && pick_row_config(L / kVec + 2, 8, &wc)) {
+      // the aligned packets that cover each group
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    using Tile = RowTile<T, TPR, VPT>;                                                          \
+    hipLaunchKernelGGL((group_norm_forward_rows_any<T, TPR, VPT, true>),                        \
+                       dim3(row_grid(rows, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,      \
+                       stream, rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),             \
+                       static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig), \
+                       static_cast<T*>(y));                                                     \
+  }
+      DRAGON_HIP_ROW_SWITCH(wc, LAUNCH);
+#undef LAUNCH
+      return true;
+    }
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
