@@ -112,7 +112,8 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn, bool windows = false) {
   if (!windows && u.seglen % kVec != 0) return p;
   // Runs shorter than 256 bytes are left to the split reduction, and so are window
   // runs under 384 bytes, two of whose packets are taken element by element
-  // (measured on 9x9 fp32 maps: 25.9 us against the split path's 21.3).
+  // (measured on 9x9 fp32 maps: 25.9 us against the split path's 21.3; single-slice
+  // channels of 7x7 maps, which need no exchange: 49.9 us against 32.7).
   if (u.seglen / kVec < (windows ? 24u : 16u)) return p;
   const uint32_t pps = u.seglen / kVec + (windows ? 2 : 0);
   const int64_t P = static_cast<int64_t>(u.nseg) * pps;  // packets per unit
@@ -522,8 +523,17 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
     if constexpr (kWin) acur.advance(d);
   }
   // false (for the whole workgroup): the wait ran out, the item is left to the repair launch
-  const bool complete = coop_channel_totals<typename Op::Merge, kRepair>(d, it.c, w, a, b, partial,
-                                                                         lds_a, lds_b);
+  bool complete = true;
+  if (d.K == 1) {
+    // a unit in one slice: its totals are this workgroup's own, nothing is
+    // exchanged (the host launches neither the fill nor the repair). Items take
+    // the two LDS buffers by turns: the barrier of one item's reduction lies
+    // between another's reads and writes of the same buffer.
+    block_merge_pair<typename Op::Merge>(a, b, ((w / gridDim.x) & 1u) ? lds_b : lds_a);
+  } else {
+    complete = coop_channel_totals<typename Op::Merge, kRepair>(d, it.c, w, a, b, partial, lds_a,
+                                                                lds_b);
+  }
   if (complete) op.finish(it.c, it.k == 0 && threadIdx.x == 0, a, b);
   // convert the packets again instead of keeping every converted element
 #pragma unroll
@@ -635,7 +645,7 @@ int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op,
   {                                                                                            \
     const unsigned cap = DRAGON_HIP_COOP_GRID(R);                                              \
     if (p.K > cap) return kNotApplicable;                                                      \
-    fill_unset(scratch, d, stream);                                                            \
+    if (p.K > 1) fill_unset(scratch, d, stream);                                               \
     hipLaunchKernelGGL((channel_slices<T, R, Op, kWin>), dim3(d.items < cap ? d.items : cap),  \
                        dim3(kCoopThreads), 0, stream, d, in0, in1, out, op, scratch);          \
   }
@@ -645,6 +655,7 @@ int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op,
   else if constexpr (kIn == 2) DRAGON_HIP_COOP_LAUNCH(12)  // one tensor: never more than 16 packets
 #undef DRAGON_HIP_COOP_LAUNCH
 #undef DRAGON_HIP_COOP_GRID
+  if (p.K == 1) return status_of_launch();  // nothing was exchanged: nothing to repair
   // the widest slice serves every plan: a repair is rare and its speed does not matter
   constexpr int kRepairR = kIn == 2 ? 12 : 16;
   hipLaunchKernelGGL((channel_slices_repair<T, kRepairR, Op, kWin>),
