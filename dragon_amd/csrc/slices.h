@@ -31,7 +31,9 @@
 // therefore always complete in stream order, in place or not.
 //
 // A small kernel fills the pairs with the "unset" pattern and clears the flags
-// before every launch.
+// before every launch. Units of a single slice (K = 1) exchange nothing: the
+// workgroup's own pair is the unit's, and neither the fill nor the repair is
+// launched.
 //
 // The arithmetic is a policy Op:
 //   kIn                              tensors held (x; x and dy)
