@@ -2564,6 +2564,197 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   return true;
 }
 
+// --------------------------------------------------------------------------
+// NHWC, fused forward: one 1024-thread workgroup per sample. A sample is S rows
+// of C channels; thread (r, cp) holds packet cp of rows r, r + R, r + 2R, ...
+// (R = 1024 / (C / kVec) rows at a time), so its channels, their group and
+// their gamma / beta are fixed, and a sample of up to 256 KB stays in registers
+// between the statistics and the normalisation: x is read once. A group's sums
+// are formed in a fixed order: every thread leaves its partial in LDS, one
+// thread per group adds the R * (D / kVec) partials of its group.
+// Requires D % kVec == 0 (a packet lies in one group) and C / kVec <= 1024.
+// --------------------------------------------------------------------------
+constexpr int kSampleThreads = 1024;
+
+// kTwo: D is not a multiple of kVec (but at least kVec): a packet may lie in two
+// groups; the thread then carries a share for each, and the elements pick their
+// group's statistics one by one.
+template <typename T, int kVPT, bool kTwo>
+__global__ __launch_bounds__(kSampleThreads) void group_norm_nhwc_samples(
+    const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
+    const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  __shared__ A part[kTwo ? 2 : 1][kSampleThreads];
+  __shared__ A total[kSampleThreads];  // one word per group (G <= C / kVec <= 1024)
+  const uint32_t cps = C / kVec;                     // packets per row
+  const uint32_t rows_at_a_time = kSampleThreads / cps;
+  const uint32_t t = threadIdx.x;
+  const uint32_t r = t / cps, cp = t - r * cps;
+  const bool on = r < rows_at_a_time;
+  // the group of the packet's first channel, and how many of its channels lie in it
+  const uint32_t g = on ? cp * kVec / D : 0u;
+  const int k0 = kTwo ? static_cast<int>(min(static_cast<uint32_t>(kVec), (g + 1) * D - cp * kVec)) : kVec;
+  const uint32_t g1 = g + 1 < G ? g + 1 : g;
+  const A inv_l = A(1) / A(static_cast<int64_t>(D) * S);
+  // The groups' totals of one value per thread and share, the same bits in every
+  // thread: the thread that owns group t adds the shares of the packets that
+  // touch it, row by row.
+  auto group_sums = [&](A v0, A v1, A& t0, A& t1) {
+    part[0][t] = on ? v0 : A(0);
+    if constexpr (kTwo) part[1][t] = on ? v1 : A(0);
+    __syncthreads();
+    if (t < G) {
+      const uint32_t lo = t * D / kVec, hi = ((t + 1) * D - 1) / kVec;
+      A acc = A(0);
+      for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+        for (uint32_t c = lo; c <= hi; ++c) {
+          // packet c starts in this group, or (only c == lo) in the one before it
+          const int share = kTwo && c * kVec < t * D ? 1 : 0;
+          acc += part[share][rr * cps + c];
+        }
+      }
+      total[t] = acc;
+    }
+    __syncthreads();
+    t0 = total[g];
+    t1 = kTwo ? total[g1] : A(0);
+    __syncthreads();  // (total is rewritten by the next call)
+  };
+
+  for (uint32_t n = blockIdx.x; n < N; n += gridDim.x) {
+    const T* xs = x + static_cast<size_t>(n) * S * C;
+    T* ys = y + static_cast<size_t>(n) * S * C;
+    // element offsets inside a sample fit 32 bits (a sample is at most 256 KB)
+    const uint32_t first = r * C + cp * kVec, step = rows_at_a_time * C;
+    u32x4 raw[kVPT];
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const bool has = on && r + i * rows_at_a_time < S;
+      raw[i] = load_packet(xs + (has ? first + i * step : 0u));
+    }
+    A s0 = A(0), s1 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (on && r + i * rows_at_a_time < S) {
+        A v[kVec];
+        IO<T>::unpack(raw[i], v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (!kTwo || e < k0) s0 += v[e]; else s1 += v[e];
+        }
+      }
+    }
+    A mean0, mean1;
+    group_sums(s0, s1, mean0, mean1);
+    mean0 *= inv_l, mean1 *= inv_l;
+    // convert the packets again in each pass instead of keeping every converted element
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
+    A q0 = A(0), q1 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (on && r + i * rows_at_a_time < S) {
+        A v[kVec];
+        IO<T>::unpack(raw[i], v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          if (!kTwo || e < k0) {
+            const A d = v[e] - mean0;
+            q0 += d * d;
+          } else {
+            const A d = v[e] - mean1;
+            q1 += d * d;
+          }
+        }
+      }
+    }
+    A rs0, rs1;
+    group_sums(q0, q1, rs0, rs1);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
+    rs0 = acc_rsqrt_exact(rs0 * inv_l + eps);
+    rs1 = kTwo ? acc_rsqrt_exact(rs1 * inv_l + eps) : A(0);
+    if (on && r == 0) {
+      if (cp * kVec == g * D) {  // the packet opens its first group
+        mu[static_cast<size_t>(n) * G + g] = mean0;
+        rsig[static_cast<size_t>(n) * G + g] = rs0;
+      }
+      if (kTwo && k0 < kVec) {  // and its second group starts inside it
+        mu[static_cast<size_t>(n) * G + g1] = mean1;
+        rsig[static_cast<size_t>(n) * G + g1] = rs1;
+      }
+    }
+    // The thread's channels are the same for every sample, but their parameters
+    // are fetched here, per sample, so that they do not occupy registers while
+    // the sample is loaded and reduced.
+    const A* gp = gamma + (on ? cp * kVec : 0u);
+    const A* bp = beta + (on ? cp * kVec : 0u);
+    asm volatile("" : "+v"(gp), "+v"(bp));
+    A gam[kVec], bet[kVec], mean[kVec];
+    load_params_ragged<kVec>(gp, kVec, gam);
+    load_params_ragged<kVec>(bp, kVec, bet);
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) {
+      const bool head = !kTwo || e < k0;
+      gam[e] *= head ? rs0 : rs1;
+      mean[e] = head ? mean0 : mean1;
+    }
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const uint32_t row = r + i * rows_at_a_time;
+      if (on && row < S) {
+        A v[kVec];
+        IO<T>::unpack(raw[i], v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - (kTwo ? mean[e] : mean0)) * gam[e] + bet[e];
+        store_packet(ys + (first + i * step), IO<T>::pack(v));
+      }
+    }
+  }
+}
+
+// true when the kernel above was launched
+template <typename T>
+bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const void* x,
+                                         const void* gamma, const void* beta, void* mu, void* rsig,
+                                         void* y, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  if constexpr (sizeof(T) > 4) {
+    return false;
+  } else {
+    if (sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D < static_cast<uint32_t>(kVec) ||
+        !aligned16(x) || !aligned16(y)) {
+      return false;
+    }
+    const bool two = sh.D % kVec != 0;  // a packet may lie in two groups
+    const uint32_t cps = sh.C / kVec;
+    if (cps > kSampleThreads) return false;
+    const uint32_t rows_at_a_time = kSampleThreads / cps;
+    const int64_t slots = ceil_div(sh.S, rows_at_a_time);
+    if (slots > (two ? 8 : 16)) return false;
+    // most of the workgroup's threads must have a row to hold
+    if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < kSampleThreads * 3) return false;
+#define LAUNCH(VPT)                                                                              \
+  {                                                                                              \
+    auto kernel = two ? group_norm_nhwc_samples<T, VPT < 16 ? VPT : 8, true>                     \
+                      : group_norm_nhwc_samples<T, VPT, false>;                                  \
+    const unsigned resident = resident_grid(kernel, kSampleThreads, 0);                          \
+    hipLaunchKernelGGL(kernel, dim3(sh.N < resident ? sh.N : resident), dim3(kSampleThreads), 0, \
+                       stream, sh.N, sh.S, sh.C, sh.G, sh.D, A(eps), static_cast<const T*>(x),   \
+                       static_cast<const A*>(gamma), static_cast<const A*>(beta),                \
+                       static_cast<A*>(mu), static_cast<A*>(rsig), static_cast<T*>(y));          \
+  }
+    if (slots <= 4) LAUNCH(4) else if (slots <= 8) LAUNCH(8) else LAUNCH(16)
+#undef LAUNCH
+    return true;
+  }
+}
+
 template <typename T>
 int launch_group_norm(const GroupShape& sh, const void* x, const void* mu, const void* rsig,
                       const void* gamma, const void* beta, void* y, hipStream_t stream) {
@@ -3087,6 +3278,21 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
       break;
     default:
       return DRAGON_HIP_EDTYPE;
+  }
+  if (!fused) {
+    switch (dtype) {
+      case DRAGON_HIP_F16:
+        fused = dragon_hip::try_group_norm_forward_nhwc_samples<dragon_hip::f16_t>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+        break;
+      case DRAGON_HIP_BF16:
+        fused = dragon_hip::try_group_norm_forward_nhwc_samples<dragon_hip::bf16_t>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+        break;
+      case DRAGON_HIP_F32:
+        fused = dragon_hip::try_group_norm_forward_nhwc_samples<float>(sh, eps, x, gamma, beta, mu, rsig, y, hs);
+        break;
+      default:
+        break;
+    }
   }
   if (fused) return dragon_hip::status_of_launch();
   switch (dtype) {
