@@ -2248,6 +2248,13 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
   return false;
 }
 
+// The most workgroups the NHWC sample backward (group_norm_grad_nhwc_samples) is
+// launched with: sizes its partial rows.
+inline uint32_t nhwc_sample_rows(int64_t N) {
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 2;
+  return static_cast<uint32_t>(N < cap ? N : cap);
+}
+
 template <typename T>
 size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
   using A = typename IO<T>::Acc;
@@ -2269,7 +2276,12 @@ size_t group_norm_grad_scratch(int64_t N, int64_t G, int64_t D, int64_t S, int l
   // per-(n, c) pairs of the fused and the general path; NHWC adds the stage-one partial pairs
   size_t pairs = static_cast<size_t>(N) * C;
   if (pairs * 2 * sizeof(A) < row_paths) pairs = row_paths / (2 * sizeof(A));
-  if (layout != DRAGON_HIP_NCHW) pairs += batched_partial_pairs(N, S, C);
+  if (layout != DRAGON_HIP_NCHW) {
+    pairs += batched_partial_pairs(N, S, C);
+    // or one partial (dgamma, dbeta) row per workgroup of the sample kernel
+    const size_t sample_pairs = static_cast<size_t>(nhwc_sample_rows(N)) * C;
+    if (pairs < sample_pairs) pairs = sample_pairs;
+  }
   // few long rows: the split reduction's partial pairs behind the N*C pairs
   if (layout == DRAGON_HIP_NCHW) pairs += static_cast<size_t>(N) * C * few_long_rows_split(N * C, S);
   size_t bytes = pairs * 2 * sizeof(A);
@@ -2755,6 +2767,135 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
   }
 }
 
+// The backward the same way: x and dy of a sample in registers (up to eight
+// packets per thread each, samples of up to 128 KB per tensor), groups of whole
+// packets. ds / db per group go through the group reduction above; a thread's
+// channels are the same for every sample it sees, so their dgamma / dbeta
+// shares stay in registers across samples and leave the workgroup once, as one
+// partial row of 2*C interleaved words per workgroup (summed by
+// sum_partial_rows).
+template <typename T, int kVPT>
+__global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
+    const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
+    const T* __restrict__ x, const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
+    const typename IO<T>::Acc* __restrict__ mu, const typename IO<T>::Acc* __restrict__ rsig,
+    typename IO<T>::Acc* __restrict__ ds, typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  __shared__ A part[2][kSampleThreads];
+  __shared__ A total[2][kSampleThreads];
+  const uint32_t cps = C / kVec;
+  const uint32_t rows_at_a_time = kSampleThreads / cps;
+  const uint32_t t = threadIdx.x;
+  const uint32_t r = t / cps, cp = t - r * cps;
+  const bool on = r < rows_at_a_time;
+  const uint32_t lanes_per_group = D / kVec;
+  const uint32_t g = on ? cp / lanes_per_group : 0u;
+  const A denom = A(1) / A(static_cast<int64_t>(D) * S);
+  A gam[kVec];
+  load_params_ragged<kVec>(gamma + (on ? cp * kVec : 0u), kVec, gam);
+  A t1[kVec], t2[kVec];
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) t1[e] = t2[e] = A(0);
+
+  for (uint32_t n = blockIdx.x; n < N; n += gridDim.x) {
+    const size_t base = static_cast<size_t>(n) * S * C;
+    const uint32_t first = r * C + cp * kVec, step = rows_at_a_time * C;
+    u32x4 rx[kVPT], rd[kVPT];
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const bool has = on && r + i * rows_at_a_time < S;
+      rx[i] = load_packet(x + base + (has ? first + i * step : 0u));
+      rd[i] = load_packet(dy + base + (has ? first + i * step : 0u));
+    }
+    const A m = mu[static_cast<size_t>(n) * G + g], rs = rsig[static_cast<size_t>(n) * G + g];
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (on && r + i * rows_at_a_time < S) {
+        A xv[kVec], dv[kVec];
+        IO<T>::unpack(rx[i], xv);
+        IO<T>::unpack(rd[i], dv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A gd = gam[e] * dv[e];
+          s1 += gd * xv[e];
+          s2 += gd;
+          t1[e] += dv[e] * (xv[e] - m) * rs;
+          t2[e] += dv[e];
+        }
+      }
+    }
+    // the group's ds and db: one LDS word per thread and sum, added by the group's owner thread
+    part[0][t] = on ? s1 : A(0);
+    part[1][t] = on ? s2 : A(0);
+    __syncthreads();
+    if (t < G) {
+      A a = A(0), b = A(0);
+      for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+        for (uint32_t k = 0; k < lanes_per_group; ++k) {
+          a += part[0][rr * cps + t * lanes_per_group + k];
+          b += part[1][rr * cps + t * lanes_per_group + k];
+        }
+      }
+      total[0][t] = a, total[1][t] = b;
+      ds[static_cast<size_t>(n) * G + t] = a;
+      db[static_cast<size_t>(n) * G + t] = b;
+    }
+    __syncthreads();
+    s1 = total[0][g], s2 = total[1][g];
+    const A u0 = (s2 * m - s1) * (rs * rs * rs) * denom;
+    const A v0 = s2 * rs * denom;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(rx[i]), "+v"(rd[i]));
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (on && r + i * rows_at_a_time < S) {
+        A xv[kVec], dv[kVec];
+        IO<T>::unpack(rx[i], xv);
+        IO<T>::unpack(rd[i], dv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
+        store_packet(dx + base + (first + i * step), IO<T>::pack(xv));
+      }
+    }
+    __syncthreads();  // total is rewritten for the next sample
+  }
+  // this workgroup's partial row: per channel, the shares of its row threads in row order
+  A* row = partial + static_cast<size_t>(blockIdx.x) * 2 * C;
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) {
+    part[0][t] = on ? t1[e] : A(0);
+    part[1][t] = on ? t2[e] : A(0);
+    __syncthreads();
+    if (t < cps) {
+      A a = A(0), b = A(0);
+      for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+        a += part[0][rr * cps + t];
+        b += part[1][rr * cps + t];
+      }
+      row[2 * (t * kVec + e)] = a;
+      row[2 * (t * kVec + e) + 1] = b;
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+bool group_norm_grad_nhwc_samples_ok(const GroupShape& sh, int* slots_out) {
+  constexpr int kVec = IO<T>::kVec;
+  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D % kVec != 0) return false;
+  const uint32_t cps = sh.C / kVec;
+  if (cps > kSampleThreads) return false;
+  const uint32_t rows_at_a_time = kSampleThreads / cps;
+  const int64_t slots = ceil_div(sh.S, rows_at_a_time);
+  if (slots > 8) return false;
+  if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < kSampleThreads * 3) return false;
+  *slots_out = static_cast<int>(slots);
+  return true;
+}
+
 template <typename T>
 int launch_group_norm(const GroupShape& sh, const void* x, const void* mu, const void* rsig,
                       const void* gamma, const void* beta, void* y, hipStream_t stream) {
@@ -2958,6 +3099,28 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     const int st = try_group_norm_grad_slices<T>(sh, x, mu, rsig, gamma, dy, ds, db, dgamma, dbeta,
                                                  dx, scratch, stream);
     if (st != kNotApplicable) return st;
+  }
+
+  if constexpr (sizeof(T) <= 4) {
+    int slots = 0;
+    if (group_norm_grad_nhwc_samples_ok<T>(sh, &slots) && aligned16(x) && aligned16(dy) &&
+        aligned16(dx)) {
+      // NHWC samples that fit one workgroup's registers: x and dy read once
+      unsigned grid = 0;
+#define LAUNCH(VPT)                                                                              \
+  {                                                                                              \
+    auto kernel = group_norm_grad_nhwc_samples<T, VPT>;                                          \
+    const unsigned resident = resident_grid(kernel, kSampleThreads, 0);                          \
+    grid = nhwc_sample_rows(sh.N);                                                               \
+    if (grid > resident) grid = resident;                                                        \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kSampleThreads), 0, stream, sh.N, sh.S, sh.C,    \
+                       sh.G, sh.D, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                  \
+  }
+      if (slots <= 2) LAUNCH(2) else if (slots <= 4) LAUNCH(4) else LAUNCH(8)
+#undef LAUNCH
+      launch_sum_partial_rows<A>(grid, sh.C, part, dgp, dbtp, stream);
+      return status_of_launch();
+    }
   }
 
   const uint32_t total = sh.N * sh.C * sh.S;

@@ -526,9 +526,10 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             ((2, 32, 35, 35), 1, 4), ((2, 16, 23, 23), 1, 2), ((1, 32, 63, 63), 1, 4),
             ((2, 8, 4, 257), 1, 2),
             # NHWC samples that fit one workgroup's registers (fused forward: 1, 7-8 and 13
-            # packets per thread; 12 of every 1024 threads idle; more samples than one round)
+            # packets per thread; 12 of every 1024 threads idle; more samples than workgroups,
+            # so that the backward's per-channel shares accumulate over several samples)
             ((2, 14, 14, 64), -1, 4), ((3, 5, 7, 96), -1, 4), ((2, 28, 28, 64), -1, 2),
-            ((300, 4, 4, 32), -1, 2),
+            ((700, 4, 4, 32), -1, 2),
             # the same with groups of 10 and 12 channels: a packet of the fused NHWC forward
             # lies in two groups
             ((2, 7, 7, 320), -1, 32), ((3, 6, 5, 96), -1, 8), ((5, 9, 9, 160), -1, 16)]
