@@ -320,7 +320,18 @@ inline uint32_t launch_reduce2_columns(uint32_t rows, uint32_t cols, const T* in
   if (packets) {
     uint32_t lanes_per_row = 1;
     while (lanes_per_row < kWaveSize && lanes_per_row * kVec < cols) lanes_per_row <<= 1;
-    const uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, lanes_per_row * kVec));
+    uint32_t tiles = static_cast<uint32_t>(ceil_div(cols, lanes_per_row * kVec));
+    // A row of 40, 48 or 80 packets (320, 384, 640 sixteen-bit channels) leaves a
+    // quarter or more of the 64-lane tiles idle: tiles of the largest power of two
+    // that divides the row (128 bytes or more of a row per tile) keep every lane busy.
+    const uint32_t row_packets = cols / kVec;
+    if (static_cast<uint64_t>(row_packets) * 5 < static_cast<uint64_t>(tiles) * lanes_per_row * 4) {
+      const uint32_t pow2 = row_packets & (~row_packets + 1);  // largest power of two dividing it
+      if (pow2 >= 8 && pow2 < lanes_per_row) {
+        lanes_per_row = pow2;
+        tiles = row_packets / pow2;
+      }
+    }
     d.split = pick_split(tiles, static_cast<int64_t>(rows) * kWaveSize * kVec);
     // The pairs are written once and read once, 16 bytes per column and split
     // against rows * sizeof(T) bytes of input per column: where that is more
