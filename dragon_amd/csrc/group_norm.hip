@@ -1474,6 +1474,147 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
   }
 }
 
+// Small groups (up to 256 packets: 14x14 and 7x7 maps with a few channels per
+// group), a wavefront per group and four groups per workgroup: nothing is
+// shared between the wavefronts, so there is no workgroup barrier. x and dy
+// of a group stay in registers; ds / db are wave reductions; a packet holds
+// elements of at most two channels (S >= kVec), whose (dgamma, dbeta) shares go
+// to one LDS entry per packet in the wavefront's own region, and lane d adds
+// the entries of channel d in packet order. partial[(n*C + c)*2 + {0,1}]
+// receives this group's share of dgamma / dbeta, as in the kernels above.
+constexpr int kWaveGroupThreads = 256;
+template <typename T, int kVPT>
+__global__ __launch_bounds__(kWaveGroupThreads) void group_norm_grad_wave_groups(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const T* __restrict__ x, const T* __restrict__ dy,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
+    const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
+    typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
+    typename IO<T>::Acc* __restrict__ partial) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  constexpr int kWaves = kWaveGroupThreads / kWaveSize;
+  __shared__ A entries[kWaves][kWaveSize * kVPT][4];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kWaveSize));
+  const int npackets = L / kVec;
+  const A denom = A(1) / A(L);
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + wave; row < rows;
+       row += static_cast<int64_t>(gridDim.x) * kWaves) {
+    const T* xr = x + row * L;
+    const T* dr = dy + row * L;
+    u32x4 rx[kVPT], rd[kVPT];
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int p = i * kWaveSize + lane;
+      const int64_t off = static_cast<int64_t>(p < npackets ? p : 0) * kVec;
+      rx[i] = load_packet(xr + off);
+      rd[i] = load_packet(dr + off);
+    }
+    const A m = mu[row], r = rsig[row];
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+    // of packet p: the position of its first element in that element's channel,
+    // and gamma of that channel and of the next
+    auto channels_of = [&](int p, uint32_t& rem, A& g0, A& g1) {
+      const uint32_t col = static_cast<uint32_t>(p) * kVec;
+      const uint32_t first = col / S;
+      rem = col - first * S;
+      g0 = gamma[c0 + first];
+      g1 = gamma[c0 + (first + 1 < D ? first + 1 : first)];
+    };
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int p = i * kWaveSize + lane;
+      if (p < npackets) {
+        uint32_t rem;
+        A g0, g1;
+        channels_of(p, rem, g0, g1);
+        A xv[kVec], dv[kVec];
+        IO<T>::unpack(rx[i], xv);
+        IO<T>::unpack(rd[i], dv);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A t = (rem + e >= S ? g1 : g0) * dv[e];
+          s1 += t * xv[e];
+          s2 += t;
+        }
+      }
+    }
+    s1 = wave_allreduce(s1, SumOp());
+    s2 = wave_allreduce(s2, SumOp());
+    if (lane == 0) {
+      ds[row] = s1;
+      db[row] = s2;
+    }
+    const A u0 = (s2 * m - s1) * (r * r * r);
+    const A v0 = s2 * r;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(rx[i]), "+v"(rd[i]));
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      const int p = i * kWaveSize + lane;
+      if (p < npackets) {
+        uint32_t rem;
+        A g0, g1;
+        channels_of(p, rem, g0, g1);
+        A xv[kVec], dv[kVec];
+        IO<T>::unpack(rx[i], xv);
+        IO<T>::unpack(rd[i], dv);
+        A h1 = A(0), h2 = A(0), t1 = A(0), t2 = A(0);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const bool second = rem + e >= S;
+          const A xc = xv[e] - m;
+          const A w = dv[e] * xc * r;
+          h1 += second ? A(0) : w;
+          h2 += second ? A(0) : dv[e];
+          t1 += second ? w : A(0);
+          t2 += second ? dv[e] : A(0);
+          xv[e] = (second ? g1 : g0) * dv[e] * r + (u0 * xc - v0) * denom;
+        }
+        store_packet(dx + row * L + static_cast<int64_t>(p) * kVec, IO<T>::pack(xv));
+        A* entry = entries[wave][p];
+        entry[0] = h1, entry[1] = h2, entry[2] = t1, entry[3] = t2;
+      }
+    }
+    // the wavefront's own entries: its LDS writes are complete before its reads
+    __threadfence_block();
+    // A channel's entries are shared out among `lanes_per_chan` adjacent lanes (a
+    // power of two, so that 64 / lanes_per_chan channels are in work at once), each
+    // of which adds every lanes_per_chan-th packet; xor shuffles combine them.
+    const size_t n = static_cast<size_t>(row / G);
+    uint32_t lanes_per_chan = 1;
+    while (lanes_per_chan * 2 * D <= static_cast<uint32_t>(kWaveSize)) lanes_per_chan <<= 1;
+    const uint32_t chans_at_a_time = kWaveSize / lanes_per_chan;
+    const uint32_t sub = static_cast<uint32_t>(lane) % lanes_per_chan;
+    for (uint32_t cb = 0; cb < D; cb += chans_at_a_time) {
+      const uint32_t c = cb + static_cast<uint32_t>(lane) / lanes_per_chan;
+      A a = A(0), b = A(0);
+      if (c < D) {
+        const uint32_t lo = c * S;
+        const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+#pragma nounroll
+        for (uint32_t p = p0 + sub; p <= p1; p += lanes_per_chan) {
+          const uint32_t part = p * kVec >= lo ? 0u : 2u;
+          a += entries[wave][p][part];
+          b += entries[wave][p][part + 1];
+        }
+      }
+      for (uint32_t o = 1; o < lanes_per_chan; o <<= 1) {
+        a += __shfl_xor(a, static_cast<int>(o), kWaveSize);
+        b += __shfl_xor(b, static_cast<int>(o), kWaveSize);
+      }
+      if (c < D && sub == 0) {
+        A* o = partial + (n * G * D + c0 + c) * 2;
+        o[0] = a;
+        o[1] = b;
+      }
+    }
+    __threadfence_block();  // the entries are rewritten for the wavefront's next group
+  }
+}
+
 // --------------------------------------------------------------------------
 // General NCHW backward, stage one: per (n, c) row of S contiguous elements,
 //   a = sum dy * (x - mu[n, g]),  b = sum dy      -> sums[(n*C + c)*2 + {0,1}]
@@ -3056,6 +3197,25 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          dxp, rows);
     }
     launch_sum_partial_rows<A>(wp.row_chunks, sh.D, rows, dgp, dbtp, stream);
+    return status_of_launch();
+  }
+
+  if (sh.nchw && sh.G * sh.D > 1 && sh.S >= static_cast<uint32_t>(kVec) && (sh.D * sh.S) % kVec == 0 &&
+      sh.D * sh.S / kVec <= 4 * kWaveSize && sizeof(T) <= 4 && aligned16(x) && aligned16(dy) &&
+      aligned16(dx)) {
+    // small groups: a wavefront each
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+    const int L = static_cast<int>(sh.D * sh.S);
+    const int64_t want = ceil_div(rows, kWaveGroupThreads / kWaveSize);
+    const int64_t cap = static_cast<int64_t>(num_cus()) * 32;
+    const dim3 grid(static_cast<unsigned>(want < cap ? want : cap));
+    const int packets = L / kVec;
+#define LAUNCH(VPT)                                                                             \
+  hipLaunchKernelGGL((group_norm_grad_wave_groups<T, VPT>), grid, dim3(kWaveGroupThreads), 0,   \
+                     stream, rows, L, sh.G, sh.D, sh.S, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);
+    if (packets <= kWaveSize) LAUNCH(1) else if (packets <= 2 * kWaveSize) LAUNCH(2) else LAUNCH(4)
+#undef LAUNCH
+    launch_sum_partial_rows<A>(sh.N, sh.C, part, dgp, dbtp, stream);
     return status_of_launch();
   }
 
