@@ -600,6 +600,7 @@ struct CoopForward {
       b += t * t;
     }
   }
+  __device__ __forceinline__ void neutral(A& x, A&) const { x = shift; }
   __device__ __forceinline__ void finish(uint32_t c, bool leader, A a, A b) {
     const A dm = a * inv_n;
     const A mean = shift + dm;
@@ -645,6 +646,7 @@ struct CoopBackward {
       b += dy[e];
     }
   }
+  __device__ __forceinline__ void neutral(A& x, A& dy) const { x = m, dy = A(0); }
   // dx = gamma*rsig*(dy - ((x-mu)*rsig*dgamma + dbeta)/normalizer), with everything that is
   // constant over the channel folded into coefficients: dx = gr*dy + (ca*(x-mu) + cb).
   __device__ __forceinline__ void finish(uint32_t c, bool leader, A a, A b) {

@@ -55,9 +55,10 @@
 // read as the aligned 16-byte packets that cover it, seglen / kVec + 2 packet
 // slots of which the last may lie behind the run and is skipped. A packet
 // wholly inside the run is accumulated, transformed and stored as a packet; of
-// a packet at either end only the run's own elements are accumulated (one call
-// of accumulate<1> each) and stored (one element store each), the neighbouring
-// run's elements in it belonging to another unit and another workgroup. All
+// a packet at either end only the run's own elements count (the others are
+// replaced by the Op's neutral element before they are accumulated) and are
+// stored (one element store each), the neighbouring run's elements in it
+// belonging to another unit and another workgroup. All
 // tensors of a call must then be congruent modulo 16 bytes. An aligned packet
 // that holds a byte of a tensor lies in that byte's page, so a packet that
 // reaches beyond either end of a tensor may be read whole.
@@ -113,9 +114,10 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn, bool windows = false) {
   CoopPlan p = {false, 0, 0, 0};
   if (!windows && u.seglen % kVec != 0) return p;
   // Runs shorter than 256 bytes are left to the split reduction, and so are window
-  // runs under 384 bytes, two of whose packets are taken element by element
-  // (measured on 9x9 fp32 maps: 25.9 us against the split path's 21.3; single-slice
-  // channels of 7x7 maps, which need no exchange: 49.9 us against 32.7).
+  // runs under 384 bytes: two of their packets are stored element by element,
+  // and the gathered 200-byte runs of a channel use their cache lines worse than
+  // the split path's contiguous rows (7x7 fp32 maps, single-slice channels, which
+  // need no exchange: 49 us against 33; 9x9: 15 against 23 the other way).
   if (u.seglen / kVec < (windows ? 24u : 16u)) return p;
   const uint32_t pps = u.seglen / kVec + (windows ? 2 : 0);
   const int64_t P = static_cast<int64_t>(u.nseg) * pps;  // packets per unit
@@ -423,7 +425,8 @@ struct OpBeginReadsInput<Op, std::void_t<decltype(Op::kBeginReadsInput)>>
     : std::bool_constant<Op::kBeginReadsInput> {};
 
 //   kWindows    the Op's accumulate and transform do not depend on the packet
-//               index j and accept V == 1: the window flavour may serve it.
+//               index j, and op.neutral(x, dy) replaces an element by one that
+//               adds nothing to its sums: the window flavour may serve it.
 template <typename Op, typename = void>
 struct OpTakesWindows : std::false_type {};
 template <typename Op>
@@ -509,17 +512,17 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
         static_assert(sizeof(T) == sizeof(A), "rewritten elements must survive the packet");
         op.accumulate_rewrite(xv, a, b);
         s.p0[i] = IO<T>::pack(xv);
-      } else if (!kWin || at.template whole<kVec>()) {
-        op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
       } else {
+        if constexpr (kWin) {
+          // what the packet holds of the neighbouring runs is replaced by values
+          // that add nothing to the Op's sums (no branch: short runs have such a
+          // packet in every wavefront)
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) {
-          if (e >= at.lo && e < at.hi) {
-            const A x1[1] = {xv[e]};
-            const A d1[1] = {Op::kIn == 2 ? dv[e] : A(0)};
-            op.accumulate(it.c, 0u, x1, d1, a, b);
+          for (int e = 0; e < kVec; ++e) {
+            if (e < at.lo || e >= at.hi) op.neutral(xv[e], dv[e]);
           }
         }
+        op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
       }
     }
     if constexpr (kWin) acur.advance(d);
