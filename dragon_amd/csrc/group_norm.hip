@@ -2856,6 +2856,9 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_nhwc_samples(
       gam[e] *= head ? rs0 : rs1;
       mean[e] = head ? mean0 : mean1;
     }
+    // (the offsets are formed again rather than kept from the loads: registers)
+    uint32_t first_out = first;
+    asm volatile("" : "+v"(first_out));
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       const uint32_t row = r + i * rows_at_a_time;
@@ -2864,7 +2867,7 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_nhwc_samples(
         IO<T>::unpack(raw[i], v);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) v[e] = (v[e] - (kTwo ? mean[e] : mean0)) * gam[e] + bet[e];
-        store_packet(ys + (first + i * step), IO<T>::pack(v));
+        store_packet(ys + (first_out + i * step), IO<T>::pack(v));
       }
     }
   }
@@ -2990,6 +2993,9 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
     const A v0 = s2 * rs * denom;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(rx[i]), "+v"(rd[i]));
+    // (the offsets are formed again rather than kept from the loads: registers)
+    uint32_t first_out = first;
+    asm volatile("" : "+v"(first_out));
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (on && r + i * rows_at_a_time < S) {
@@ -2998,7 +3004,7 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
         IO<T>::unpack(rd[i], dv);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
-        store_packet(dx + base + (first + i * step), IO<T>::pack(xv));
+        store_packet(dx + base + (first_out + i * step), IO<T>::pack(xv));
       }
     }
     __syncthreads();  // total is rewritten for the next sample
