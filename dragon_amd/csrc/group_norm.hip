@@ -1067,7 +1067,12 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
   // packets, and how many of their 64 * kVec elements lie in it.
   constexpr uint32_t kSpan = kWaveSize * kVec;
   auto first_channel_elems = [&](int i, uint32_t& chan, uint32_t& in_first) {
-    const uint32_t e0 = static_cast<uint32_t>(i * kTPR + wave * kWaveSize) * kVec;
+    // (16-bit types: found again at every use. Kept per slot across the passes, the
+    // boundaries and both gammas spill 156 bytes at eight packets per thread and
+    // tensor; fp32 has the registers and is 5-9% faster keeping them.)
+    int w = wave;
+    if constexpr (sizeof(T) == 2) asm volatile("" : "+s"(w));
+    const uint32_t e0 = static_cast<uint32_t>(i * kTPR + w * kWaveSize) * kVec;
     chan = e0 / S;
     in_first = (chan + 1) * S - e0;
     if (chan >= D) chan = D - 1, in_first = kSpan;
@@ -2364,12 +2369,8 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
     *mode = per_chan % kWaveSize == 0 ? kChannelWaves : kChannelStraddles;
   } else if (S % kVec == 0 && (per_chan & (per_chan - 1)) == 0) {
     *mode = kChannelLanes;
-  } else if (S >= kWaveSize * kVec && (D * S) % kVec == 0 &&
-             !(kVec == 8 && D * S / kVec > 4096)) {
-    // Channels of 64 packets' worth or more that are not whole packets. Not for
-    // 16-bit groups of more than 4096 packets: eight packets per thread and tensor
-    // plus the per-element boundary code spill 156 bytes at 128 registers, and
-    // the kernel then runs no faster than the general path.
+  } else if (S >= kWaveSize * kVec && (D * S) % kVec == 0) {
+    // channels of 64 packets' worth or more that are not whole packets
     *mode = kChannelStraddlesAny;
   } else if (S >= kVec && (D * S) % kVec == 0 && D * S / kVec <= kMaxEntryPackets) {
     // channels that are not whole packets (or a number of packets the lane
