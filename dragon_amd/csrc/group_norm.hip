@@ -2655,6 +2655,66 @@ inline size_t group_slices_scratch_bytes(int dtype, const GroupShape& sh) {
   }
 }
 
+// Groups of up to 1024 elements (a few channels on 14x14, 8x8 or 7x7 maps) as a
+// policy of the LDS-staged short-row kernel (short_rows.h): several groups per
+// wavefront instead of one group on a fraction of a wavefront's lanes. The
+// channel of each of a lane's elements, relative to the group's first channel,
+// is the same for every group and is found once; gamma / beta are fetched per
+// group.
+template <typename T, int kE>
+struct GroupShortForward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 1;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  A inv_l, eps;
+  const A* gamma;
+  const A* beta;
+  A* mu;
+  A* rsig;
+  uint32_t G, D, S;
+  uint32_t chan[kE];
+  __device__ __forceinline__ void set_packed(bool) {}
+  template <int kL>
+  static constexpr bool packed_ok() { return false; }
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int l, int) {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const uint32_t c = static_cast<uint32_t>(l + j * kL) / S;
+      chan[j] = c < D ? c : D - 1;  // lanes past the group
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A*, int l, int L, A (&v)[kE],
+                                      const A (&)[kE]) const {
+    A s = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) s += v[j];  // lanes past the group hold 0
+    const A mean = group_allreduce<kL>(s, SumOp()) * inv_l;
+    A q = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const A d = v[j] - mean;
+      q += l + j * kL < L ? d * d : A(0);
+    }
+    const A rs = acc_rsqrt_exact(group_allreduce<kL>(q, SumOp()) * inv_l + eps);
+    if (l == 0) {
+      mu[r] = mean;
+      rsig[r] = rs;
+    }
+    const uint32_t c0 = static_cast<uint32_t>(r % G) * D;
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      v[j] = (v[j] - mean) * (gamma[c0 + chan[j]] * rs) + beta[c0 + chan[j]];
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
 // Fused forward: true when the register-resident kernel was launched.
 template <typename T>
 bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x, const void* gamma,
@@ -2666,6 +2726,21 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
   if (!sh.nchw || !pick_row_config(ceil_div(L, kVec), 8, &cfg)) return false;
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+  // Groups of at most 32 packets leave half of a wavefront's lanes or more idle in
+  // the row kernels: several groups per wavefront, staged through LDS (fp16
+  // [4096,96,8,8] 44 -> 31 us, bf16 [4096,64,8,8] 42 -> 21 us; from 49 packets on
+  // the row kernels are ahead).
+  if (ShortPlan sp; sizeof(T) <= 4 && ceil_div(L, kVec) <= 32 && rows >= 4096 && congruent16(x, y) &&
+                    plan_short_rows(L, sizeof(T), 4, aligned16(x), &sp)) {
+    const size_t lds = static_cast<size_t>(sp.stage_packets) * 16;
+    const T* xp = static_cast<const T*>(x);
+    DRAGON_HIP_SHORT_LAUNCH(T, GroupShortForward, sp, lds, short_grid(rows, sp.rows_per_chunk),
+                            stream, rows, static_cast<int>(L), xp, xp, static_cast<T*>(y),
+                            A(1) / A(L), A(eps), static_cast<const A*>(gamma),
+                            static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),
+                            sh.G, sh.D, sh.S, {});
+    return true;
+  }
   if (L % kVec != 0 || !aligned16(x) || !aligned16(y)) {
     if (RowConfig wc; sizeof(T) <= 4 && congruent16(x, y) && pick_row_config(L / kVec + 2, 8, &wc)) {
       // the aligned packets that cover each group

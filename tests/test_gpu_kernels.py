@@ -535,7 +535,10 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             ((2, 7, 7, 320), -1, 32), ((3, 6, 5, 96), -1, 8), ((5, 9, 9, 160), -1, 16),
             # small groups, a wavefront each in the fused backward: more channels per group
             # than lanes, three channels per group, more groups than the grid's wavefronts hold
-            ((2, 160, 3, 3), 1, 2), ((5, 96, 8, 8), 1, 32), ((40, 64, 14, 14), 1, 32)]
+            ((2, 160, 3, 3), 1, 2), ((5, 96, 8, 8), 1, 32), ((40, 64, 14, 14), 1, 32),
+            # thousands of groups of at most 32 packets: several groups per wavefront in the
+            # forward (staged through LDS), channels that are and are not whole packets
+            ((140, 64, 8, 8), 1, 32), ((130, 96, 5, 5), 1, 32)]
 
 
 @pytest.mark.parametrize("fused", [False, True])
