@@ -2715,6 +2715,84 @@ struct GroupShortForward {
   __device__ __forceinline__ void end(A*, int) const {}
 };
 
+// The backward of such groups the same way (x and dy staged). ds / db are
+// reductions over the group's lanes; a channel's dgamma / dbeta share is the
+// sum over the lane's elements of that channel, one pair of reductions per
+// channel of the group (a few channels: D <= 8), written to
+// partial[(n*C + c)*2 + {0,1}] as by the row kernels.
+template <typename T, int kE>
+struct GroupShortBackward {
+  using A = typename IO<T>::Acc;
+  static constexpr int kIn = 2;
+  static constexpr size_t kEndBytes = 0;
+  static constexpr int kSideWords = 0;
+  A denom;
+  const A* gamma;
+  const A* mu;
+  const A* rsig;
+  A* ds;
+  A* db;
+  A* partial;
+  uint32_t G, D, S;
+  uint32_t chan[kE];
+  __device__ __forceinline__ void set_packed(bool) {}
+  template <int kL>
+  static constexpr bool packed_ok() { return false; }
+  __device__ __forceinline__ A fill0() const { return A(0); }
+  __device__ __forceinline__ A fill1() const { return A(0); }
+  template <int kL>
+  __device__ __forceinline__ void begin(int l, int) {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      const uint32_t c = static_cast<uint32_t>(l + j * kL) / S;
+      chan[j] = c < D ? c : D - 1;  // lanes past the group (their dy is 0)
+    }
+  }
+  template <int kL>
+  __device__ __forceinline__ void row(int64_t r, const A*, int l, int, A (&x)[kE],
+                                      const A (&dy)[kE]) const {
+    const A m = mu[r], rs = rsig[r];
+    const uint32_t c0 = static_cast<uint32_t>(r % G) * D;
+    A g[kE];
+    A s1 = A(0), s2 = A(0);
+#pragma unroll
+    for (int j = 0; j < kE; ++j) {
+      g[j] = gamma[c0 + chan[j]];
+      const A t = g[j] * dy[j];
+      s1 += t * x[j];
+      s2 += t;
+    }
+    s1 = group_allreduce<kL>(s1, SumOp());
+    s2 = group_allreduce<kL>(s2, SumOp());
+    if (l == 0) {
+      ds[r] = s1;
+      db[r] = s2;
+    }
+    A* o = partial + (static_cast<size_t>(r / G) * G * D + c0) * 2;
+    for (uint32_t d = 0; d < D; ++d) {
+      A h1 = A(0), h2 = A(0);
+#pragma unroll
+      for (int j = 0; j < kE; ++j) {
+        const bool mine = chan[j] == d;
+        h1 += mine ? dy[j] * (x[j] - m) * rs : A(0);
+        h2 += mine ? dy[j] : A(0);
+      }
+      h1 = group_allreduce<kL>(h1, SumOp());
+      h2 = group_allreduce<kL>(h2, SumOp());
+      if (l == 0) {
+        o[2 * d] = h1;
+        o[2 * d + 1] = h2;
+      }
+    }
+    const A u0 = (s2 * m - s1) * (rs * rs * rs);
+    const A v0 = s2 * rs;
+#pragma unroll
+    for (int j = 0; j < kE; ++j) x[j] = g[j] * dy[j] * rs + (u0 * (x[j] - m) - v0) * denom;
+  }
+  template <int kL>
+  __device__ __forceinline__ void end(A*, int) const {}
+};
+
 // Fused forward: true when the register-resident kernel was launched.
 template <typename T>
 bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x, const void* gamma,
@@ -3279,6 +3357,25 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          dxp, rows);
     }
     launch_sum_partial_rows<A>(wp.row_chunks, sh.D, rows, dgp, dbtp, stream);
+    return status_of_launch();
+  }
+
+  if (ShortPlan gsp; sh.nchw && sh.G * sh.D > 1 && sh.D <= 8 && sizeof(T) <= 4 &&
+                     ceil_div(static_cast<int64_t>(sh.D) * sh.S, kVec) <= 32 &&
+                     static_cast<int64_t>(sh.N) * sh.G >= 4096 && congruent16(x, dy) &&
+                     congruent16(x, dx) &&
+                     plan_short_rows_within(
+                         static_cast<int64_t>(sh.D) * sh.S, sizeof(T), 3, aligned16(x),
+                         [](const ShortPlan& q) { return static_cast<size_t>(q.stage_packets) * 32; },
+                         &gsp)) {
+    // thousands of groups of at most 32 packets: several groups per wavefront, staged through LDS
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+    const int L = static_cast<int>(sh.D * sh.S);
+    const size_t lds = static_cast<size_t>(gsp.stage_packets) * 32;
+    DRAGON_HIP_SHORT_LAUNCH(T, GroupShortBackward, gsp, lds, short_grid(rows, gsp.rows_per_chunk),
+                            stream, rows, L, xp, dyp, dxp, A(1) / A(L), gp, mup, rsp, dsp, dbp, part,
+                            sh.G, sh.D, sh.S, {});
+    launch_sum_partial_rows<A>(sh.N, sh.C, part, dgp, dbtp, stream);
     return status_of_launch();
   }
 
