@@ -914,20 +914,23 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
   }
 }
 
-// The same for any S and any alignment (S not a multiple of a packet, so
-// that a packet may straddle channels and groups start at element-aligned
-// addresses): ragged tiles, the channel of an element found from its column.
-// kWindow: x and y congruent modulo 16 bytes; a group is read and written as the
-// aligned packets that cover it (RowWindow), with regular tiles sized for
-// L / kVec + 2 packets.
-template <typename T, int kTPR, int kVPT, bool kWindow = false>
-__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any(
+// The same for groups that are not whole aligned packets (D * S odd, or a base
+// that is not 16-byte aligned), x and y congruent modulo 16 bytes: a group is
+// read as the aligned packets that cover it (RowWindow; the tile is sized for
+// L / kVec + 2 packets) and kept as raw packets. A packet wholly inside the
+// group that lies in one channel takes the packet code; the packets at the
+// group's ends and those across two channels go element by element; the
+// elements of the neighbouring groups in the two end packets are neither summed
+// nor stored.
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_windows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
     T* __restrict__ y) {
-  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), !kWindow>;
+  using Tile = RowTile<T, kTPR, kVPT>;
+  using Raw = RawRowTile<T, kTPR, kVPT>;
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   __shared__ A slots[2][Tile::kSlots];
@@ -935,15 +938,118 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
   const int lane = Tile::lane();
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
        row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
-    const RowWindow<T> w(x + row * L, L);
-    const int lead = kWindow ? w.lead : 0;          // elements of slot 0, lane 0 before the group
-    const int extent = kWindow ? w.packets : L;     // what Tile::active counts in
-    Tile t;
-    if constexpr (kWindow) {
-      t.load_window(x + row * L, w, A(0));
-    } else {
-      t.load(x + row * L, L, A(0));
+    const T* xr = x + row * L;
+    const RowWindow<T> w(xr, L);
+    const int npackets = w.packets;
+    Raw t;
+    t.load_unmasked(xr - w.lead, npackets);
+    // slot i of this lane: its first element's place in the group (below zero in the
+    // group's first packet), and whether all of its elements belong to the group
+    auto col_of = [&](int i) { return (i * kTPR + lane) * kVec - w.lead; };
+    auto whole = [&](int col) { return col >= 0 && col + kVec <= L; };
+    A s = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        const int col = col_of(i);
+        A v[kVec];
+        t.unpack(i, v);
+        if (whole(col)) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) s += v[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) s += col + e >= 0 && col + e < L ? v[e] : A(0);
+        }
+      }
     }
+    const A mean = Tile::reduce(s, SumOp(), slots[0]) * inv_l;
+    t.refresh();
+    A q = A(0);
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        const int col = col_of(i);
+        A v[kVec];
+        t.unpack(i, v);
+        const bool all = whole(col);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+          const A d = v[e] - mean;
+          q += all || (col + e >= 0 && col + e < L) ? d * d : A(0);
+        }
+      }
+    }
+    const A var = Tile::reduce(q, SumOp(), slots[1]) * inv_l;
+    const A rs = acc_rsqrt_exact(var + eps);
+    if (lane == 0) {
+      mu[row] = mean;
+      rsig[row] = rs;
+    }
+    const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+    T* yr = y + row * L;
+    t.refresh();
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (Tile::active(i, npackets)) {
+        const int col = col_of(i);
+        const uint32_t colp = static_cast<uint32_t>(col < 0 ? 0 : col);
+        const uint32_t first = colp / S;
+        const uint32_t rem = colp - first * S;
+        A v[kVec];
+        t.unpack(i, v);
+        if (col >= 0 && rem + kVec <= S) {  // the packet lies within one channel
+          const A gam = gamma[c0 + first] * rs, bet = beta[c0 + first];
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam + bet;
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            int k = static_cast<int>(rem) + e + (col < 0 ? col : 0);
+            if (k < 0) k = 0;  // before the group: not stored
+            uint32_t c = first;
+            while (static_cast<uint32_t>(k) >= S) k -= static_cast<int>(S), ++c;
+            if (c >= D) c = D - 1;  // beyond the group: not stored
+            v[e] = (v[e] - mean) * (gamma[c0 + c] * rs) + beta[c0 + c];
+          }
+        }
+        if (whole(col)) {
+          store_packet(yr + col, IO<T>::pack(v));
+        } else {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (col + e >= 0 && col + e < L) IO<T>::store1(yr + col + e, v[e]);
+          }
+        }
+      }
+    }
+    if (kTPR != kWaveSize) __syncthreads();
+  }
+}
+
+// The same for any S and any alignment (S not a multiple of a packet, so
+// that a packet may straddle channels and groups start at element-aligned
+// addresses): ragged tiles, the channel of an element found from its column.
+// (x and y not congruent modulo 16 bytes; congruent tensors take the windows above.)
+template <typename T, int kTPR, int kVPT>
+__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any(
+    const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
+    const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y) {
+  using Tile = RowTile<T, kTPR, kVPT, row_threads(kTPR), true>;
+  using A = typename Tile::A;
+  constexpr int kVec = Tile::kVec;
+  __shared__ A slots[2][Tile::kSlots];
+  const A inv_l = A(1) / A(L);
+  const int lane = Tile::lane();
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
+       row < rows; row += static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock) {
+    constexpr int lead = 0;
+    const int extent = L;
+    Tile t;
+    t.load(x + row * L, L, A(0));
     A s = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i)
@@ -990,11 +1096,7 @@ __global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows_any
         }
       }
     }
-    if constexpr (kWindow) {
-      t.store_window(y + row * L, w);
-    } else {
-      t.store(y + row * L, L);
-    }
+    t.store(y + row * L, L);
     if (kTPR != kWaveSize) __syncthreads();
   }
 }
@@ -2825,7 +2927,7 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
-    hipLaunchKernelGGL((group_norm_forward_rows_any<T, TPR, VPT, true>),                        \
+    hipLaunchKernelGGL((group_norm_forward_rows_windows<T, TPR, VPT>),                          \
                        dim3(row_grid(rows, Tile::kRowsPerBlock)), dim3(Tile::kThreads), 0,      \
                        stream, rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),             \
                        static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
