@@ -533,6 +533,8 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # the same with groups of 10 and 12 channels: a packet of the fused NHWC forward
             # lies in two groups
             ((2, 7, 7, 320), -1, 32), ((3, 6, 5, 96), -1, 8), ((5, 9, 9, 160), -1, 16),
+            # groups of half a packet (the column-reduction structure)
+            ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32),
             # small groups, a wavefront each in the fused backward: more channels per group
             # than lanes, three channels per group, more groups than the grid's wavefronts hold
             ((2, 160, 3, 3), 1, 2), ((5, 96, 8, 8), 1, 32), ((40, 64, 14, 14), 1, 32),
