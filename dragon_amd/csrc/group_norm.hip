@@ -1434,7 +1434,13 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
 // its packet's first and second channel in LDS, one entry per packet, and the
 // thread that owns a channel adds the entries of that channel's packets in
 // order. Dynamic LDS: 4 accumulator words per packet of the group.
-template <typename T, int kTPR, int kVPT>
+// kWindow: the groups themselves are not whole aligned packets (D * S odd, or
+// bases that are not 16-byte aligned; x, dy and dx congruent modulo 16 bytes).
+// A group is read as the aligned packets that cover it; what its two end
+// packets hold of the neighbouring groups is replaced by values that add
+// nothing to any sum (dy = 0, x = mean) and is not stored. Dynamic LDS then
+// holds L / kVec + 2 entries.
+template <typename T, int kTPR, int kVPT, bool kWindow = false>
 __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const T* __restrict__ x, const T* __restrict__ dy,
@@ -1449,29 +1455,52 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
   __shared__ A slots[2 * Tile::kSlots];
   extern __shared__ u32x4 dynamic_lds[];
   A* entries = reinterpret_cast<A*>(dynamic_lds);  // [npackets][4]
-  const int npackets = L / kVec;
   const A denom = A(1) / A(L);
   const int lane = threadIdx.x;
+  // a group's window: elements of its first packet before it, and its packets
+  auto lead_of = [&](int64_t row) {
+    return kWindow ? RowWindow<T>(x + row * L, L).lead : 0;
+  };
+  auto packets_of = [&](int lead) { return kWindow ? (lead + L + kVec - 1) / kVec : L / kVec; };
 
   Raw tx, tdy;
   if (blockIdx.x < rows) {
-    tx.load_unmasked(x + static_cast<int64_t>(blockIdx.x) * L, npackets);
-    tdy.load_unmasked(dy + static_cast<int64_t>(blockIdx.x) * L, npackets);
+    const int lead0 = lead_of(blockIdx.x);
+    tx.load_unmasked(x + static_cast<int64_t>(blockIdx.x) * L - lead0, packets_of(lead0));
+    tdy.load_unmasked(dy + static_cast<int64_t>(blockIdx.x) * L - lead0, packets_of(lead0));
   }
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int lead = lead_of(row);
+    const int npackets = packets_of(lead);
     const int64_t next = row + gridDim.x;
     const bool next_valid = next < rows;
-    const T* nx = x + (next_valid ? next : row) * L;
-    const T* ndy = dy + (next_valid ? next : row) * L;
+    const int nlead = lead_of(next_valid ? next : row);
+    const int next_packets = packets_of(nlead);
+    const T* nx = x + (next_valid ? next : row) * L - nlead;
+    const T* ndy = dy + (next_valid ? next : row) * L - nlead;
     const A m = mu[row], r = rsig[row];
     const uint32_t c0 = static_cast<uint32_t>(row % G) * D;
+    // kWindow: the elements of slot i's packet that belong to the group are [lo, hi)
+    auto neutralize = [&](int i, A (&xv)[kVec], A (&dv)[kVec]) {
+      if constexpr (kWindow) {
+        const int col = (i * kTPR + lane) * kVec - lead;
+        if (col < 0 || col + kVec > L) {
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            if (col + e < 0 || col + e >= L) xv[e] = m, dv[e] = A(0);
+          }
+        }
+      }
+    };
 
     // Of slot i's packet: the position of its first element in that element's
     // channel, and gamma of that channel and of the next. Found again in the
     // second pass rather than kept: four more registers per slot cost occupancy.
     auto channels_of = [&](int i, uint32_t& rem, A& g0, A& g1) {
-      const uint32_t col =
-          Tile::active(i, npackets) ? static_cast<uint32_t>(i * kTPR + lane) * kVec : 0u;
+      // (kWindow: the group's first packet starts `lead` elements before it; its
+      // elements count from the group's first, the ones before it as channel 0)
+      const int at = Tile::active(i, npackets) ? (i * kTPR + lane) * kVec - lead : 0;
+      const uint32_t col = static_cast<uint32_t>(at < 0 ? 0 : at);
       const uint32_t first = col / S;
       rem = col - first * S;
       g0 = gamma[c0 + first];
@@ -1487,9 +1516,11 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
+        neutralize(i, xv, dv);
+        const int shift = kWindow && i == 0 && lane == 0 ? lead : 0;  // the first packet's offset
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const A t = (rem + e >= S ? g1 : g0) * dv[e];
+          const A t = (rem + e >= S + shift ? g1 : g0) * dv[e];
           s1 += t * xv[e];
           s2 += t;
         }
@@ -1513,10 +1544,12 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
         tdy.unpack(i, dv);
+        neutralize(i, xv, dv);
+        const int shift = kWindow && i == 0 && lane == 0 ? lead : 0;
         A h1 = A(0), h2 = A(0), t1 = A(0), t2 = A(0);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          const bool second = rem + e >= S;
+          const bool second = rem + e >= S + shift;
           const A xc = xv[e] - m;
           const A w = dv[e] * xc * r;
           h1 += second ? A(0) : w;
@@ -1525,13 +1558,25 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
           t2 += second ? dv[e] : A(0);
           xv[e] = (second ? g1 : g0) * dv[e] * r + (u0 * xc - v0) * denom;
         }
-        tx.store_slot(dx + row * L, i, xv);
+        if constexpr (kWindow) {
+          const int col = (i * kTPR + lane) * kVec - lead;
+          if (col >= 0 && col + kVec <= L) {
+            store_packet(dx + row * L + col, IO<T>::pack(xv));
+          } else {
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              if (col + e >= 0 && col + e < L) IO<T>::store1(dx + row * L + col + e, xv[e]);
+            }
+          }
+        } else {
+          tx.store_slot(dx + row * L, i, xv);
+        }
         A* entry = entries + static_cast<size_t>(i * kTPR + lane) * 4;
         entry[0] = h1, entry[1] = h2, entry[2] = t1, entry[3] = t2;
       }
       if (next_valid) {
-        tx.load_slot_unmasked(nx, i, npackets);
-        tdy.load_slot_unmasked(ndy, i, npackets);
+        tx.load_slot_unmasked(nx, i, next_packets);
+        tdy.load_slot_unmasked(ndy, i, next_packets);
       }
     }
     __syncthreads();
@@ -1542,8 +1587,10 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
     const size_t n = static_cast<size_t>(row / G);
     if (S / kVec <= 32) {
       for (uint32_t c = lane; c < D; c += kTPR) {
-        const uint32_t lo = c * S;
-        const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+        // (kWindow: packet p starts at element p * kVec - lead of the group; the
+        // first packet's elements before the group count as channel 0)
+        const uint32_t lo = c * S + (c == 0 ? 0u : static_cast<uint32_t>(lead));
+        const uint32_t p0 = lo / kVec, p1 = (c * S + lead + S - 1) / kVec;
         A a = A(0), b = A(0);
 #pragma nounroll
         for (uint32_t p = p0; p <= p1; ++p) {
@@ -1560,8 +1607,10 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows_any(
       const uint32_t wave = static_cast<uint32_t>(lane) / kWaveSize;
       const uint32_t wave_lane = static_cast<uint32_t>(lane) & (kWaveSize - 1);
       for (uint32_t c = wave; c < D; c += kWaves) {
-        const uint32_t lo = c * S;
-        const uint32_t p0 = lo / kVec, p1 = (lo + S - 1) / kVec;
+        // (kWindow: packet p starts at element p * kVec - lead of the group; the
+        // first packet's elements before the group count as channel 0)
+        const uint32_t lo = c * S + (c == 0 ? 0u : static_cast<uint32_t>(lead));
+        const uint32_t p0 = lo / kVec, p1 = (c * S + lead + S - 1) / kVec;
         A a = A(0), b = A(0);
         for (uint32_t p = p0 + wave_lane; p <= p1; p += kWaveSize) {
           const uint32_t part = p * kVec >= lo ? 0u : 2u;
@@ -3495,6 +3544,31 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   hipLaunchKernelGGL((group_norm_grad_wave_groups<T, VPT>), grid, dim3(kWaveGroupThreads), 0,   \
                      stream, rows, L, sh.G, sh.D, sh.S, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);
     if (packets <= kWaveSize) LAUNCH(1) else if (packets <= 2 * kWaveSize) LAUNCH(2) else LAUNCH(4)
+#undef LAUNCH
+    launch_sum_partial_rows<A>(sh.N, sh.C, part, dgp, dbtp, stream);
+    return status_of_launch();
+  }
+
+  if (const int64_t wp = static_cast<int64_t>(sh.D) * sh.S / kVec + 2;
+      sh.nchw && sh.G * sh.D > 1 && sizeof(T) <= 4 && sh.S >= static_cast<uint32_t>(kVec) &&
+      ((sh.D * sh.S) % kVec != 0 || !aligned16(x)) && congruent16(x, dy) && congruent16(x, dx) &&
+      wp > 2 * kWaveSize && wp <= kMaxEntryPackets) {
+    // groups that are not whole aligned packets themselves: through their packet windows
+    const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
+    const int L = static_cast<int>(sh.D * sh.S);
+    const unsigned grid = static_cast<unsigned>(rows < (1 << 20) ? rows : (1 << 20));
+    const size_t lds = static_cast<size_t>(wp) * 4 * sizeof(A);
+#define LAUNCH(TPR, VPT)                                                                        \
+  {                                                                                             \
+    auto kernel = group_norm_grad_rows_any<T, TPR, VPT, true>;                                  \
+    if (lds > 32 * 1024) (void)resident_grid(kernel, TPR, lds);                                 \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), lds, stream, rows, L, sh.G, sh.D, sh.S,   \
+                       xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                             \
+  }
+    if (wp <= 256 * 2) LAUNCH(256, 2)
+    else if (wp <= 256 * 4) LAUNCH(256, 4)
+    else if (wp <= 256 * 8) LAUNCH(256, 8)
+    else LAUNCH(1024, 4)
 #undef LAUNCH
     launch_sum_partial_rows<A>(sh.N, sh.C, part, dgp, dbtp, stream);
     return status_of_launch();
