@@ -110,6 +110,8 @@ SIGNATURES = {
     "dragon_hip_exchange_timed_out": (_int, []),
     "dragon_hip_exchange_reset": (None, [ctypes.c_uint]),
     "dragon_hip_exchange_plan": (_int, [_int, _i64, _i64, _i64, _int] + [ctypes.POINTER(_int)] * 4),
+    "dragon_hip_plan_name": (_int, [ctypes.c_char_p, _int, _int, ctypes.POINTER(_i64), _int,
+                                    ctypes.c_char_p, _sz]),
     "dragon_hip_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
 }
 

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include <atomic>
 
@@ -36,6 +37,71 @@ inline int num_cus() {
   cached[device].store(n, std::memory_order_relaxed);
   return n;
 }
+
+// ---------------------------------------------------------------------------
+// Launch trace. Every kernel launch of the library goes through the macro below,
+// which notes the kernel's spelling and workgroup size in a per-thread trace when
+// one is being recorded and, in plan-only mode, launches nothing. The plan query
+// of the C ABI (dragon_hip_plan_name) runs an entry point that way with made-up
+// addresses: it reports which kernel flavours a call would take without touching
+// a device, so that a test can pin the routing of the shapes that matter.
+// ---------------------------------------------------------------------------
+struct LaunchTrace {
+  bool recording = false;
+  bool plan_only = false;  // record only: no kernel is launched
+  char text[1024];
+  size_t used = 0;
+};
+inline LaunchTrace& launch_trace() {
+  static thread_local LaunchTrace trace;
+  return trace;
+}
+inline bool plan_only() { return launch_trace().plan_only; }
+// Appends "name[threads];" with blanks and the outer parentheses of `spelling` removed.
+inline void note_launch(const char* spelling, dim3 block) {
+  LaunchTrace& t = launch_trace();
+  if (!t.recording) return;
+  const size_t cap = sizeof(t.text) - 24;
+  int depth = 0;
+  for (const char* c = spelling; *c && t.used < cap; ++c) {
+    if (*c == ' ' || *c == '\t' || *c == '\n') continue;
+    if (*c == '(' && depth++ == 0 && c == spelling) continue;
+    if (*c == ')' && --depth == 0 && c[1] == 0 && spelling[0] == '(') continue;
+    t.text[t.used++] = *c;
+  }
+  char tail[24];
+  const int n = snprintf(tail, sizeof(tail), "[%u];", block.x * block.y * block.z);
+  for (int i = 0; i < n && t.used + 1 < sizeof(t.text); ++i) t.text[t.used++] = tail[i];
+  t.text[t.used] = 0;
+}
+// A launcher that holds its kernel in a variable names the flavour itself.
+inline void note_flavour(const char* name) {
+  LaunchTrace& t = launch_trace();
+  if (!t.recording) return;
+  for (const char* c = name; *c && t.used + 2 < sizeof(t.text); ++c) t.text[t.used++] = *c;
+  t.text[t.used++] = ':';
+  t.text[t.used] = 0;
+}
+
+// A number that a plan depends on (slices per unit, rows per chunk ...): "key=value:".
+inline void note_number(const char* key, long long value) {
+  LaunchTrace& t = launch_trace();
+  if (!t.recording) return;
+  char item[64];
+  const int n = snprintf(item, sizeof(item), "%s=%lld:", key, value);
+  for (int i = 0; i < n && t.used + 1 < sizeof(t.text); ++i) t.text[t.used++] = item[i];
+  t.text[t.used] = 0;
+}
+
+#undef hipLaunchKernelGGL
+#define hipLaunchKernelGGL(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...)       \
+  do {                                                                                         \
+    ::dragon_hip::note_launch(#kernelName, dim3(numThreads));                                  \
+    if (!::dragon_hip::plan_only()) {                                                          \
+      hipLaunchKernelGGLInternal((kernelName), (numBlocks), (numThreads), (memPerBlock),       \
+                                 (streamId), __VA_ARGS__);                                     \
+    }                                                                                          \
+  } while (0)
 
 // 16-bit storage types: same bit layout as dragon::float16 / dragon::bfloat16
 // (dragon/core/types.h:36-42), a bare unsigned short.
@@ -358,6 +424,10 @@ inline bool congruent16(const void* a, const void* b) {
 }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int status_of_launch() {
+  if (plan_only()) {  // nothing was launched; a host without a device has nothing to report
+    (void)hipGetLastError();
+    return DRAGON_HIP_OK;
+  }
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? DRAGON_HIP_OK : static_cast<int>(e);
 }

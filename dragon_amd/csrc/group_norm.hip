@@ -2374,8 +2374,9 @@ __global__ __launch_bounds__(1024) void sum_partial_rows(const uint32_t P, const
 // A workgroup owns kLanes adjacent packets of every partial row; its
 // 1024 / kLanes lane groups take rows g, g + groups, ..., several loads in
 // flight per lane, and are added up through LDS in a fixed order. kLanes is 32
-// (512 contiguous bytes per row) for wide rows and 8 (one cache line) for
-// narrow ones, which would otherwise leave all but a few compute units idle.
+// (512 contiguous bytes per row) for the widest rows, 16 for rows of up to 4096
+// packets and 8 (one cache line) for narrow ones, which would otherwise leave
+// all but a few compute units idle.
 template <typename A, int kLanes>
 __global__ __launch_bounds__(1024) void sum_partial_rows_packets(const uint32_t P, const uint32_t C,
                                                                  const A* __restrict__ partial,
@@ -2440,9 +2441,15 @@ void launch_sum_partial_rows(uint32_t P, uint32_t C, const A* partial, A* dgamma
   if ((2 * C) % kPer != 0 || !aligned16(partial)) {
     hipLaunchKernelGGL((sum_partial_rows<A>), dim3(static_cast<unsigned>(ceil_div(2 * C, kWaveSize))),
                        dim3(1024), 0, stream, P, C, partial, dgamma, dbeta);
-  } else if (packets >= 32 * 64) {
+  } else if (packets > 4096) {
     hipLaunchKernelGGL((sum_partial_rows_packets<A, 32>),
                        dim3(static_cast<unsigned>(ceil_div(packets, 32))), dim3(1024), 0, stream, P,
+                       C, partial, dgamma, dbeta);
+  } else if (packets > 1024) {
+    // 128 to 256 workgroups: measured on MI355X at C = 4096 (2048 packets), 32 lanes per row
+    // chunk (64 workgroups) take 0.4-1 us longer than 16 or 8
+    hipLaunchKernelGGL((sum_partial_rows_packets<A, 16>),
+                       dim3(static_cast<unsigned>(ceil_div(packets, 16))), dim3(1024), 0, stream, P,
                        C, partial, dgamma, dbeta);
   } else {
     hipLaunchKernelGGL((sum_partial_rows_packets<A, 8>),
@@ -3005,6 +3012,10 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   {                                                                                             \
     using Tile = RowTile<T, TPR, VPT>;                                                          \
     const unsigned one_shot = row_grid(rows, Tile::kRowsPerBlock);                              \
+    note_flavour(sh.S % kVec == 0 ? "group_norm_forward_rows<" #TPR "," #VPT ",0>"           \
+                 : sh.S >= kWaveSize * kVec && !(kVec == 8 && VPT == 8 && TPR == 1024)          \
+                     ? "group_norm_forward_rows<" #TPR "," #VPT ",2>"                          \
+                     : "group_norm_forward_rows<" #TPR "," #VPT ",1>");                        \
     auto kernel = sh.S % kVec == 0 ? group_norm_forward_rows<T, TPR, VPT, 0>                    \
         : sh.S >= kWaveSize * kVec && !(kVec == 8 && VPT == 8 && TPR == 1024) /* spills: 82 us against 66 */ \
             ? group_norm_forward_rows<T, TPR, VPT, 2>                                           \
@@ -3202,6 +3213,7 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
     if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < kSampleThreads * 3) return false;
 #define LAUNCH(VPT)                                                                              \
   {                                                                                              \
+    note_flavour(two ? "group_norm_nhwc_samples<" #VPT ",two>" : "group_norm_nhwc_samples<" #VPT ">"); \
     auto kernel = two ? group_norm_nhwc_samples<T, VPT < 16 ? VPT : 8, true>                     \
                       : group_norm_nhwc_samples<T, VPT, false>;                                  \
     const unsigned resident = resident_grid(kernel, kSampleThreads, 0);                          \
@@ -3446,6 +3458,8 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     const size_t staged_bytes = static_cast<size_t>(ceil_div(sh.D, kVec) * kVec) * sizeof(A);
 #define LAUNCH_T(TPR, VPT, THREADS)                                                           \
   {                                                                                           \
+    note_flavour(ragged ? "layer_norm_grad_rows<" #TPR "," #VPT "," #THREADS ",ragged>"        \
+                        : "layer_norm_grad_rows<" #TPR "," #VPT "," #THREADS ">");             \
     auto kernel = ragged ? layer_norm_grad_rows<T, TPR, VPT, THREADS, true>                   \
                          : layer_norm_grad_rows<T, TPR, VPT, THREADS, false>;                 \
     if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, THREADS, staged_bytes);         \
@@ -3560,6 +3574,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     const size_t lds = static_cast<size_t>(wp) * 4 * sizeof(A);
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
+    note_flavour("group_norm_grad_rows_any<" #TPR "," #VPT ",window>");                         \
     auto kernel = group_norm_grad_rows_any<T, TPR, VPT, true>;                                  \
     if (lds > 32 * 1024) (void)resident_grid(kernel, TPR, lds);                                 \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(TPR), lds, stream, rows, L, sh.G, sh.D, sh.S,   \
@@ -3585,6 +3600,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
   {                                                                                             \
   if (mode == kChannelPackets) {                                                                \
     if constexpr (TPR * VPT <= kMaxEntryPackets) {                                              \
+      note_flavour("group_norm_grad_rows_any<" #TPR "," #VPT ">");                              \
       auto kernel = group_norm_grad_rows_any<T, TPR, VPT>;                                      \
       const size_t lds = static_cast<size_t>(L / kVec) * 4 * sizeof(A);                         \
       if (lds > 32 * 1024) (void)resident_grid(kernel, TPR, lds);                               \
@@ -3592,6 +3608,10 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
                          xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                           \
     }                                                                                           \
   } else {                                                                                      \
+    note_flavour(mode == kChannelStraddles ? "group_norm_grad_rows<" #TPR "," #VPT ",straddles>"  \
+                 : mode == kChannelStraddlesAny ? "group_norm_grad_rows<" #TPR "," #VPT ",straddles_any>" \
+                 : mode == kChannelLanes ? "group_norm_grad_rows<" #TPR "," #VPT ",lanes>"      \
+                                         : "group_norm_grad_rows<" #TPR "," #VPT ",waves>");     \
     auto kernel = mode == kChannelStraddles ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddles> \
         : mode == kChannelStraddlesAny ? group_norm_grad_rows<T, TPR, VPT, kChannelStraddlesAny>   \
         : mode == kChannelLanes             ? group_norm_grad_rows<T, TPR, VPT, kChannelLanes>     \
@@ -3624,6 +3644,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       unsigned grid = 0;
 #define LAUNCH(VPT)                                                                              \
   {                                                                                              \
+    note_flavour("group_norm_grad_nhwc_samples<" #VPT ">");                                      \
     auto kernel = group_norm_grad_nhwc_samples<T, VPT>;                                          \
     const unsigned resident = resident_grid(kernel, kSampleThreads, 0);                          \
     grid = nhwc_sample_rows(sh.N);                                                               \

@@ -376,6 +376,7 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
     }
 #define LAUNCH_T(TPR, VPT, THREADS)                                                          \
   {                                                                                          \
+    note_flavour("layer_norm_wide_rows<" #TPR "," #VPT "," #THREADS ">");                    \
     auto kernel = layer_norm_wide_rows<T, TPR, VPT, THREADS>;                                \
     const int64_t groups = ceil_div(N, static_cast<int64_t>(THREADS / TPR));                 \
     const unsigned resident = resident_grid(kernel, THREADS, staged_bytes);                  \

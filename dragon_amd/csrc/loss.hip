@@ -889,6 +889,7 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
     if (regular && cfg.tpr == 1024) {
 #define LAUNCH_WIDE(VPT)                                                                        \
   {                                                                                             \
+    note_flavour("softmax_ce_wide_rows<" #VPT ">");                                            \
     auto kernel = softmax_ce_wide_rows<T, TargetT, VPT>;                                        \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                   \
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
@@ -902,6 +903,7 @@ int launch_fused_forward(int64_t N, int64_t S, int64_t C, int64_t ignore_index, 
       // rows of 1024-thread size that are not whole aligned packets: through their windows
 #define LAUNCH_WINDOWS(VPT)                                                                     \
   {                                                                                             \
+    note_flavour("softmax_ce_wide_windows<" #VPT ">");                                         \
     auto kernel = softmax_ce_wide_windows<T, TargetT, VPT>;                                     \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                   \
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \

@@ -320,9 +320,9 @@ inline bool plan_short_rows_within(int64_t C, size_t elem_bytes, int packets_per
                                    bool base_aligned, LdsOf lds_of, ShortPlan* p) {
   for (int ppt = packets_per_thread; ppt >= 1; --ppt) {
     if (!plan_short_rows(C, elem_bytes, ppt, base_aligned, p)) return false;
-    if (lds_of(*p) <= 48 * 1024) break;
+    if (lds_of(*p) <= 48 * 1024) return true;
   }
-  return true;
+  return false;  // even one packet per thread needs more: the caller takes its next path
 }
 inline unsigned short_grid(int64_t N, uint32_t rows_per_chunk) {
   const int64_t chunks = ceil_div(N, rows_per_chunk);

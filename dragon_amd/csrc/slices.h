@@ -650,6 +650,7 @@ int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op,
   {                                                                                            \
     const unsigned cap = DRAGON_HIP_COOP_GRID(R);                                              \
     if (p.K > cap) return kNotApplicable;                                                      \
+    note_number("slices", p.K);                                                                \
     if (p.K > 1) fill_unset(scratch, d, stream);                                               \
     hipLaunchKernelGGL((channel_slices<T, R, Op, kWin>), dim3(d.items < cap ? d.items : cap),  \
                        dim3(kCoopThreads), 0, stream, d, in0, in1, out, op, scratch);          \
@@ -673,18 +674,20 @@ template <typename T, typename Op>
 int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T* in1, T* out,
                        typename IO<T>::Acc* scratch, hipStream_t stream) {
   constexpr int kIn = Op::kIn;
-  if (OpBeginReadsInput<Op>::value && static_cast<const void*>(out) == in0) return kNotApplicable;
+  // In place, a repair launch could re-read what another slice of the unit has already
+  // overwritten; a unit of one slice exchanges nothing and is never repaired.
+  const bool in_place_hazard = OpBeginReadsInput<Op>::value && static_cast<const void*>(out) == in0;
   const bool packets = sh.seglen % IO<T>::kVec == 0 && sh.unit_stride % IO<T>::kVec == 0 &&
       sh.seg_stride % IO<T>::kVec == 0 && aligned16(in0) && aligned16(in1) && aligned16(out);
   if (packets) {
     const CoopPlan p = plan_coop<T>(sh, kIn);
-    if (!p.ok) return kNotApplicable;
+    if (!p.ok || (in_place_hazard && p.K > 1)) return kNotApplicable;
     return launch_channel_slices<T, Op, false>(sh, p, op, in0, in1, out, scratch, stream);
   }
   if constexpr (OpTakesWindows<Op>::value) {
     if (sizeof(T) > 4 || !congruent16(in0, in1) || !congruent16(in0, out)) return kNotApplicable;
     const CoopPlan p = plan_coop<T>(sh, kIn, true);
-    if (!p.ok) return kNotApplicable;
+    if (!p.ok || (in_place_hazard && p.K > 1)) return kNotApplicable;
     return launch_channel_slices<T, Op, true>(sh, p, op, in0, in1, out, scratch, stream);
   }
   return kNotApplicable;

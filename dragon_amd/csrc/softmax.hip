@@ -1612,6 +1612,7 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
     if (sizeof(T) == 2 && !regular && congruent16(x, y) && C / kVec + 2 > 4 * 1024 &&
         C / kVec + 2 <= 8 * 1024) {
       if constexpr (sizeof(T) == 2) {
+        note_flavour("softmax_wide_raw_windows");
         auto kernel = softmax_wide_raw_windows<T, kKind>;
         const unsigned resident = resident_grid(kernel, 1024, 0);
         const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident;
@@ -1626,6 +1627,7 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
         !(wcfg.vpt == 8 && sizeof(T) == 2)) {
 #define LAUNCH_WINDOWS(VPT)                                                                  \
   {                                                                                          \
+    note_flavour("softmax_wide_windows<" #VPT ">");                                          \
     auto kernel = softmax_wide_windows<T, kKind, VPT>;                                       \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                \
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
@@ -1641,6 +1643,7 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
       const int64_t rows = regular ? N : N - 1;
 #define LAUNCH_WIDE(VPT)                                                                     \
   {                                                                                          \
+    note_flavour(regular ? "softmax_wide_rows<" #VPT ">" : "softmax_wide_rows<" #VPT ",ragged>"); \
     auto kernel = regular ? softmax_wide_rows<T, kKind, VPT, false>                          \
                           : softmax_wide_rows<T, kKind, VPT, true>;                          \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                \
@@ -1690,6 +1693,7 @@ int launch_softmax(int64_t N, int64_t S, int64_t C, const void* x, void* y, void
 #undef LAUNCH
   } else if (S == 1 && sizeof(T) <= 4 && ceil_div(C, kVec) <= 16 * 1024) {
     const bool regular = C % kVec == 0 && aligned16(x) && aligned16(y);
+    note_flavour(regular ? "softmax_huge_rows" : "softmax_huge_rows<ragged>");
     auto kernel = regular ? softmax_huge_rows<T, kKind, false> : softmax_huge_rows<T, kKind, true>;
     const unsigned resident = resident_grid(kernel, 1024, 0);
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident;
@@ -1773,6 +1777,7 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
   if (S == 1 && regular && pick_row_config(C / kVec, 8, &cfg) && cfg.tpr == 1024) {
 #define LAUNCH_WIDE(VPT, PREFETCH)                                                           \
   {                                                                                          \
+    note_flavour("softmax_grad_wide_rows<" #VPT "," #PREFETCH ">");                            \
     auto kernel = softmax_grad_wide_rows<T, kKind, VPT, PREFETCH>;                           \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                \
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \
@@ -1789,6 +1794,7 @@ int launch_softmax_grad(int64_t N, int64_t S, int64_t C, const void* dy, const v
       pick_row_config(C / kVec + 2, 8, &cfg) && cfg.tpr == 1024) {
 #define LAUNCH_WINDOWS(VPT, PREFETCH)                                                        \
   {                                                                                          \
+    note_flavour("softmax_grad_wide_windows<" #VPT "," #PREFETCH ">");                         \
     auto kernel = softmax_grad_wide_windows<T, kKind, VPT, PREFETCH>;                        \
     const unsigned resident = resident_grid(kernel, 1024, 0);                                \
     const unsigned grid = N < static_cast<int64_t>(resident) ? static_cast<unsigned>(N) : resident; \

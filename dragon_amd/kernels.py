@@ -369,6 +369,19 @@ def exchange_plan(dtype_name, units, nseg, seglen, tensors):
     return tuple(o.value for o in out) if ok else None
 
 
+def plan_name(op, dtype_name, dims, data_format="NCHW"):
+    """The kernels the entry point ``dragon_hip_<op>`` would launch for ``dims`` (its own
+    size arguments, in its order), as text; ValueError when the op or the shape is
+    rejected. Launches nothing and needs no device."""
+    tag = {"float16": 0, "bfloat16": 1, "float32": 2, "float64": 3}[dtype_name]
+    buf = ctypes.create_string_buffer(1024)
+    n = _lib.lib().dragon_hip_plan_name(op.encode(), tag, layout_tag(data_format), _dims(dims),
+                                        len(dims), buf, len(buf))
+    if n < 0:
+        raise ValueError("no plan for %s %s %s (status %d)" % (op, dtype_name, list(dims), n))
+    return buf.value.decode()
+
+
 # ---------------------------------------------------------------- measurement
 
 def stream_probe(mode, src, dst, nbytes):

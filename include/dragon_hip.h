@@ -429,6 +429,29 @@ void dragon_hip_exchange_reset(unsigned patience);
 int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seglen, int tensors,
                              int* slices, int* slice_packets, int* packets_per_thread, int* grid);
 
+/* dragon_hip_plan_name: which kernels an entry point would launch for a shape,
+ * as text "flavour:kernel[threads];kernel[threads];..." in launch order (a
+ * "key=value:" item in front of a kernel is a number its plan depends on). No
+ * counterpart in the reference; it is for tests that pin the routing of a
+ * shape without a GPU: the entry point itself runs in a plan-only mode that
+ * launches nothing and touches no device, with every tensor assumed 16-byte
+ * aligned and not in place, and scratch assumed large enough.
+ * `op` is the entry point's name without the prefix: "layer_norm",
+ * "layer_norm_grad" (group_norm_grad with G = S = 1), "group_norm_forward",
+ * "group_norm_grad", "batch_norm_training_forward", "batch_norm_training_backward",
+ * "softmax", "log_softmax", "softmax_grad", "log_softmax_grad", "l1_norm",
+ * "l2_norm", "l1_norm_grad", "l2_norm_grad", "softmax_cross_entropy_loss_forward",
+ * "softmax_cross_entropy_loss_backward" (int64 targets, VALID reduction).
+ * `dims` holds the entry point's sizes in its own order: (N, C) for the two
+ * LayerNorm ops, (N, G, D, S) for GroupNorm, (N, C, S) for BatchNorm, (N, S, C)
+ * for the rest; `layout` matters where the entry point takes one.
+ * Returns the length of the text written to `buf` (truncated to buf_bytes - 1),
+ * or a negative dragon_hip_status for an unknown op or a shape the entry point
+ * rejects. Counts that depend on the device (the grid of a persistent kernel,
+ * slices per unit) are those of an MI355X when no device is visible. */
+int dragon_hip_plan_name(const char* op, int dtype, int layout, const int64_t* dims, int num_dims,
+                         char* buf, size_t buf_bytes);
+
 /* ------------------------------------------------------------------------ */
 /* Measurement utility (no counterpart in the reference): a streaming read    */
 /* (mode 0: dst receives at most one word), copy (mode 1), fill (mode 2) or    */
