@@ -113,6 +113,7 @@ SIGNATURES = {
     "dragon_hip_plan_name": (_int, [ctypes.c_char_p, _int, _int, ctypes.POINTER(_i64), _int,
                                     ctypes.c_char_p, _sz]),
     "dragon_hip_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
+    "dragon_hip_stream_probe_shape": (_int, [_int, _int, _int, _vp, _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -651,6 +651,7 @@ int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op,
     const unsigned cap = DRAGON_HIP_COOP_GRID(R);                                              \
     if (p.K > cap) return kNotApplicable;                                                      \
     note_number("slices", p.K);                                                                \
+    if (kWin) note_flavour("windows");                                                         \
     if (p.K > 1) fill_unset(scratch, d, stream);                                               \
     hipLaunchKernelGGL((channel_slices<T, R, Op, kWin>), dim3(d.items < cap ? d.items : cap),  \
                        dim3(kCoopThreads), 0, stream, d, in0, in1, out, op, scratch);          \

@@ -20,9 +20,11 @@
 namespace dragon_hip {
 namespace {
 
-constexpr int kProbeThreads = 256;
-constexpr int kInFlight = 4;
-constexpr size_t kChunk = static_cast<size_t>(kProbeThreads) * kInFlight;  // packets
+// The default shape of the probe, and the ones a caller may ask for instead
+// (dragon_hip_stream_probe_shape): which shape streams fastest depends on the
+// size of the tensors, so a benchmark that wants a ceiling takes the best of them.
+constexpr int kDefaultThreads = 256;
+constexpr int kDefaultInFlight = 4;
 
 __device__ __forceinline__ u32x4 load16(const u32x4* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void store16(u32x4* p, const u32x4 v) { __builtin_nontemporal_store(v, p); }
@@ -30,10 +32,11 @@ __device__ __forceinline__ void store16(u32x4* p, const u32x4 v) { __builtin_non
 // kReads source tensors of n packets each (laid out back to back from src),
 // kWrites destination tensors. The chunked body covers whole chunks; the
 // packets past the last whole chunk are walked one by one.
-template <int kReads, int kWrites>
+template <int kReads, int kWrites, int kProbeThreads, int kInFlight>
 __global__ __launch_bounds__(kProbeThreads) void probe_stream(const u32x4* __restrict__ src,
                                                               u32x4* __restrict__ dst, size_t n,
                                                               uint32_t* __restrict__ sink) {
+  constexpr size_t kChunk = static_cast<size_t>(kProbeThreads) * kInFlight;  // packets
   const size_t chunks = n / kChunk;
   u32x4 acc = {0u, 0u, 0u, 0u};
   for (size_t c = blockIdx.x; c < chunks; c += gridDim.x) {
@@ -78,38 +81,55 @@ __global__ __launch_bounds__(kProbeThreads) void probe_stream(const u32x4* __res
   }
 }
 
-} // namespace
-} // namespace dragon_hip
-
-extern "C" int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes,
-                                       void* stream) {
-  using namespace dragon_hip;
-  if (bytes == 0) return DRAGON_HIP_OK;
-  if (bytes % 16 != 0 || !dst || (mode != 2 && !src)) return DRAGON_HIP_EINVAL;
-  if (!aligned16(src) || !aligned16(dst)) return DRAGON_HIP_EINVAL;
+template <int kThreads, int kInFlight>
+int launch_probe(int mode, const void* src, void* dst, size_t bytes, hipStream_t s) {
   const size_t n = bytes / 16;
+  constexpr size_t kChunk = static_cast<size_t>(kThreads) * kInFlight;
   const size_t chunks = n / kChunk;
-  const size_t want = chunks > 0 ? chunks : (n + kProbeThreads - 1) / kProbeThreads;
+  const size_t want = chunks > 0 ? chunks : (n + kThreads - 1) / kThreads;
   const size_t cap = 0x7fffffffu;  // one chunk per workgroup up to the launch limit
   const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const u32x4* sp = static_cast<const u32x4*>(src);
   u32x4* dp = static_cast<u32x4*>(dst);
   uint32_t* sink = static_cast<uint32_t*>(dst);
   switch (mode) {
     case 0:
-      hipLaunchKernelGGL((probe_stream<1, 0>), dim3(grid), dim3(kProbeThreads), 0, s, sp, dp, n, sink);
+      hipLaunchKernelGGL((probe_stream<1, 0, kThreads, kInFlight>), dim3(grid), dim3(kThreads), 0, s, sp, dp, n, sink);
       break;
     case 1:
-      hipLaunchKernelGGL((probe_stream<1, 1>), dim3(grid), dim3(kProbeThreads), 0, s, sp, dp, n, sink);
+      hipLaunchKernelGGL((probe_stream<1, 1, kThreads, kInFlight>), dim3(grid), dim3(kThreads), 0, s, sp, dp, n, sink);
       break;
     case 2:
-      hipLaunchKernelGGL((probe_stream<0, 1>), dim3(grid), dim3(kProbeThreads), 0, s, sp, dp, n, sink);
+      hipLaunchKernelGGL((probe_stream<0, 1, kThreads, kInFlight>), dim3(grid), dim3(kThreads), 0, s, sp, dp, n, sink);
       break;
     case 3:
-      hipLaunchKernelGGL((probe_stream<2, 1>), dim3(grid), dim3(kProbeThreads), 0, s, sp, dp, n, sink);
+      hipLaunchKernelGGL((probe_stream<2, 1, kThreads, kInFlight>), dim3(grid), dim3(kThreads), 0, s, sp, dp, n, sink);
       break;
     default: return DRAGON_HIP_EINVAL;
   }
   return status_of_launch();
+}
+
+} // namespace
+} // namespace dragon_hip
+
+extern "C" int dragon_hip_stream_probe_shape(int mode, int threads, int in_flight, const void* src,
+                                             void* dst, size_t bytes, void* stream) {
+  using namespace dragon_hip;
+  if (bytes == 0) return DRAGON_HIP_OK;
+  if (bytes % 16 != 0 || !dst || (mode != 2 && !src)) return DRAGON_HIP_EINVAL;
+  if (!aligned16(src) || !aligned16(dst)) return DRAGON_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define SHAPE(T, F) \
+  if (threads == T && in_flight == F) return launch_probe<T, F>(mode, src, dst, bytes, s);
+  SHAPE(64, 1) SHAPE(64, 2) SHAPE(64, 4) SHAPE(256, 1) SHAPE(256, 2) SHAPE(256, 4) SHAPE(256, 8)
+  SHAPE(512, 2) SHAPE(1024, 2)
+#undef SHAPE
+  return DRAGON_HIP_EINVAL;
+}
+
+extern "C" int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes,
+                                       void* stream) {
+  return dragon_hip_stream_probe_shape(mode, dragon_hip::kDefaultThreads, dragon_hip::kDefaultInFlight,
+                                       src, dst, bytes, stream);
 }

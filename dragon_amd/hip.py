@@ -73,11 +73,12 @@ def get_device_capability(device_index=None):
 
 
 def memory_allocated(device_index=None, workspace=None):
-    """Bytes of device memory held by the tensors of a workspace (cuda.py:146-169).
-    ``workspace`` is a ``runtime.Workspace``; without one the answer is 0 (this package
-    keeps no process-wide default workspace)."""
+    """Bytes of device memory held by the tensors of the current workspace (cuda.py:146-169):
+    ``runtime.get_workspace()``, i.e. the innermost ``Workspace.as_default()`` or the
+    process-wide default one, unless ``workspace`` names another."""
+    from . import runtime
     if workspace is None:
-        return 0
+        workspace = runtime.get_workspace()
     index = current_device() if device_index is None else int(device_index)
     return workspace.memory_allocated("hip", index)
 

@@ -384,6 +384,11 @@ def plan_name(op, dtype_name, dims, data_format="NCHW"):
 
 # ---------------------------------------------------------------- measurement
 
-def stream_probe(mode, src, dst, nbytes):
-    """Streaming read (0), copy (1) or fill (2) of ``nbytes`` bytes."""
-    _call("dragon_hip_stream_probe", mode, _ptr(src), _ptr(dst), nbytes, _stream())
+def stream_probe(mode, src, dst, nbytes, shape=None):
+    """Streaming read (0), copy (1), fill (2) or two reads and one write (3) of ``nbytes``
+    bytes per tensor; ``shape`` = (threads per workgroup, loads in flight per thread)."""
+    if shape is None:
+        _call("dragon_hip_stream_probe", mode, _ptr(src), _ptr(dst), nbytes, _stream())
+    else:
+        _call("dragon_hip_stream_probe_shape", mode, int(shape[0]), int(shape[1]), _ptr(src), _ptr(dst),
+              nbytes, _stream())

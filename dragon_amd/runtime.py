@@ -11,6 +11,7 @@ computed in Python.
 """
 
 import itertools
+import threading
 
 import numpy as np
 
@@ -50,8 +51,62 @@ def _quote(s):
     return '"' + s.replace("\\", "\\\\").replace('"', '\\"') + '"'
 
 
-def make_def(op_type, inputs, outputs, name="", device_id=0, **args):
-    """OperatorDef in protobuf text format (dragon/proto/dragon.proto:99-116)."""
+# ---------------------------------------------------------------------------
+# Device scope and default workspace: what ``dragon.device(...)`` and
+# ``dragon.get_workspace()`` give the reference's test bodies
+# (dragon/python/core/framework/context.py:24-52,96-103,
+# dragon/python/core/framework/workspace.py). A scope is a per-thread stack of
+# (device_type, device_index); outside any scope the process-wide default of
+# ``hip.set_default_device`` applies.
+# ---------------------------------------------------------------------------
+_tls = threading.local()
+
+
+class _DeviceScope:
+    def __init__(self, device_type, device_index):
+        device_type = device_type.lower()
+        if device_type not in _DEVICE_TO_IDENTIFIER:
+            raise ValueError("Unsupported device type: " + device_type)
+        self.spec = (device_type, int(device_index))
+
+    def __enter__(self):
+        _tls.__dict__.setdefault("devices", []).append(self.spec)
+        return self
+
+    def __exit__(self, *exc):
+        _tls.devices.pop()
+        return False
+
+
+def device(device_type, device_index=0):
+    """Context manager that nests the device, as ``dragon.device`` (context.py:24-52):
+    operator definitions made and tensors fed inside it go to that device."""
+    return _DeviceScope(device_type, device_index)
+
+
+def get_device():
+    """(device_type, device_index) of the innermost scope, else the process default."""
+    stack = getattr(_tls, "devices", None)
+    if stack:
+        return stack[-1]
+    from . import hip
+    d = hip.default_device()
+    return d["device_type"], d["device_index"]
+
+
+def _operator_device_id(device_id):
+    """Operators exist for the HIP device only: an explicit ``device_id`` wins, then the
+    index of a "hip" scope or default; under a CPU scope or default they run on hip:0."""
+    if device_id is not None:
+        return int(device_id)
+    device_type, index = get_device()
+    return index if device_type == "hip" else 0
+
+
+def make_def(op_type, inputs, outputs, name="", device_id=None, **args):
+    """OperatorDef in protobuf text format (dragon/proto/dragon.proto:99-116); its device
+    option is the current device scope unless ``device_id`` names a HIP device."""
+    device_id = _operator_device_id(device_id)
     parts = []
     if name:
         parts.append("name: " + _quote(name))
@@ -90,6 +145,11 @@ class Workspace:
     def close(self):
         self._impl = None
 
+    def as_default(self):
+        """Context manager that makes this the workspace ``get_workspace()`` returns
+        (``dragon.Workspace.as_default``)."""
+        return _WorkspaceScope(self)
+
     def unique_name(self, prefix):
         return "%s_%d" % (prefix, next(Workspace._uid))
 
@@ -100,7 +160,10 @@ class Workspace:
         array = np.asarray(array)
         if dtype == "float16" and array.dtype == np.uint16:
             array, dtype = array.view(np.float16), None
-        device_type, device_id = device if device is not None else ("cpu", 0)
+        if device is None:  # a "hip" scope feeds straight into that device's memory
+            scope = get_device()
+            device = scope if scope[0] == "hip" else ("cpu", 0)
+        device_type, device_id = device
         tensor = self._impl.CreateTensor(name)
         _guard(tensor.FromNumpy, array, dtype or "", device_type, device_id)
         return name
@@ -137,6 +200,36 @@ class Workspace:
         """Gradient OperatorDefs of a forward definition and the names of the input gradients."""
         defs, grad_inputs = _guard(backend.MakeGradientDefs, def_text, list(output_grads))
         return list(defs), list(grad_inputs)
+
+
+class _WorkspaceScope:
+    def __init__(self, ws):
+        self.ws = ws
+
+    def __enter__(self):
+        _tls.__dict__.setdefault("workspaces", []).append(self.ws)
+        return self.ws
+
+    def __exit__(self, *exc):
+        _tls.workspaces.pop()
+        return False
+
+
+_default_workspace = None
+_default_workspace_lock = threading.Lock()
+
+
+def get_workspace():
+    """The innermost ``Workspace.as_default()`` of the thread, else the process-wide
+    default workspace, created on first use (``dragon.get_workspace``)."""
+    global _default_workspace
+    stack = getattr(_tls, "workspaces", None)
+    if stack:
+        return stack[-1]
+    with _default_workspace_lock:
+        if _default_workspace is None:
+            _default_workspace = Workspace("default")
+        return _default_workspace
 
 
 class Tape:

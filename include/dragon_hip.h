@@ -463,6 +463,13 @@ int dragon_hip_plan_name(const char* op, int dtype, int layout, const int64_t* d
 /* profiler byte counters.                                                     */
 /* ------------------------------------------------------------------------ */
 int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes, void* stream);
+/* The same with the probe's shape chosen by the caller: `threads` per workgroup and
+ * 16-byte loads `in_flight` per thread, one of (64, 1|2|4), (256, 1|2|4|8), (512, 2),
+ * (1024, 2); dragon_hip_stream_probe is (256, 4). Which shape streams fastest depends on
+ * the tensor size, so a benchmark that wants a ceiling for a kernel takes the best of them
+ * at that kernel's tensor size. */
+int dragon_hip_stream_probe_shape(int mode, int threads, int in_flight, const void* src, void* dst,
+                                  size_t bytes, void* stream);
 
 #ifdef __cplusplus
 } /* extern "C" */

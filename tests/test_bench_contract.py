@@ -1,7 +1,9 @@
 """bench.py's bookkeeping that needs no GPU: the HBM traffic it reports for the headline kernels
 comes from the counter summaries under profiles/ and stays consistent with the algorithmic
-bytes; every workload of the sweep is named by a parity test at its full size."""
+bytes; every workload of the sweep is named by a parity test at its full size; a bench line
+whose kernel rows beat the streaming probe is reported as broken (the probe is a ceiling)."""
 
+import json
 import os
 import re
 
@@ -40,3 +42,28 @@ def test_every_swept_workload_has_a_full_size_parity_test():
     for workload, shape in shapes.items():
         assert workload in bench.WORKLOADS
         assert shape in text, "no full-size parity test names the shape of %s" % workload
+
+
+def _line():
+    with open(os.path.join(ROOT, "tests", "golden", "bench_line.json")) as f:
+        return json.load(f)
+
+
+def test_a_well_formed_bench_line_has_no_contract_problems():
+    assert bench.contract_problems(_line()) == []
+
+
+def test_a_kernel_row_above_the_probe_is_a_contract_problem():
+    line = _line()
+    line["kernels"][1]["frac_stream_probe"] = 1.02
+    problems = bench.contract_problems(line)
+    assert len(problems) == 1 and "ceiling" in problems[0] and "softmax_grad" in problems[0]
+
+
+def test_other_contract_problems_are_seen():
+    line = _line()
+    del line["cpu_baseline"]
+    line["roofline"]["frac"] = 0.9
+    line["kernels"][0]["frac_hbm_peak"] = 1.2
+    text = " ".join(bench.contract_problems(line))
+    assert "cpu_baseline" in text and "achieved / peak" in text and "above the HBM peak" in text

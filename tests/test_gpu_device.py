@@ -102,3 +102,32 @@ def test_operator_on_a_stream_index(hip):
     stream.synchronize()
     assert stream.query() is True
     assert np.allclose(ws.fetch("y").sum(1), 1.0, atol=1e-5)
+
+
+def test_reference_style_device_wrapper(hip):
+    """The reference re-enters a test body under ``with dragon.device("cuda")``
+    (test/dragon/test_ops.py:4183-4204). The same wrapper with the hip device: the body names
+    no device, tensors fed inside the scope land in device memory, operators run there, and
+    ``hip.memory_allocated()`` reads the current (default) workspace."""
+    from dragon_amd import runtime as rt
+
+    def body():  # a device-agnostic test body: LayerNorm of the reference's literal (test_ops.py:4363-4397)
+        ws = rt.get_workspace()
+        tape = rt.Tape(ws)
+        x = ws.feed("x", np.arange(4, dtype=np.float32).reshape(1, 4) * 0.1)
+        w = ws.feed("w", np.arange(1, 5, dtype=np.float32) * 0.1)
+        b = ws.feed("b", np.arange(4, dtype=np.float32) * 0.1)
+        y = rt.layer_norm(tape, [x, w, b], axis=-1, epsilon=1e-5)
+        dy = ws.feed("dy", np.arange(4, dtype=np.float32).reshape(1, 4) * 10)
+        dx, = tape.gradient(y, [x], output_gradient=dy)
+        assert np.allclose(ws.fetch(dx), [[8.897812, -8.95499, -8.926399, 8.983574]], atol=1e-3)
+        return ws, x
+
+    scoped = rt.Workspace("wrapper")
+    with rt.device("hip", 0), scoped.as_default():
+        before = hip.memory_allocated()
+        ws, x = body()
+        assert ws is scoped and ws.tensor(x).device == ("hip", 0)
+        assert hip.memory_allocated() > before
+        assert hip.memory_allocated() == hip.memory_allocated(workspace=scoped)
+    assert rt.get_workspace() is not scoped

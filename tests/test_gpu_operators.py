@@ -316,8 +316,16 @@ def test_operator_cache_and_error_paths(rt, ws):
 
 # ---------------------------------------------------------------- BASELINE configurations
 
+# Parameter gradients are fp32 quantities: held to the 1e-5 of the parity bar against the
+# fp64 closed form, and to the oracle within the oracle's own distance from fp64 (its column
+# sums are strictly sequential fp32 sums over up to 200704 terms).
+TOL_DGAMMA = 1e-5
+
+
 def _three_way(got, oracle, exact, tol, what):
     ok, e_go, e_ge, e_oe = U.close3(got, oracle, exact, tol)
+    print("three-way %s: gpu-vs-oracle %.3g, gpu-vs-fp64 %.3g, oracle-vs-fp64 %.3g (tol %.0e)"
+          % (what, e_go, e_ge, e_oe, tol))
     assert ok, "%s: gpu-vs-oracle %.3g, gpu-vs-fp64 %.3g, oracle-vs-fp64 %.3g" % (what, e_go, e_ge, e_oe)
 
 
@@ -399,8 +407,8 @@ def test_config3_batch_norm_fp32_64x256x56x56(rt, ws):
     dy64 = dyv.astype(np.float64)
     dg64 = (dy64 * xh64).sum((0, 2, 3))
     db64 = dy64.sum((0, 2, 3))
-    _three_way(ws.fetch(dw), dg_ref, dg64, 2e-5, "dgamma")
-    _three_way(ws.fetch(db), db_ref, db64, 2e-5, "dbeta")
+    _three_way(ws.fetch(dw), dg_ref, dg64, TOL_DGAMMA, "dgamma")
+    _three_way(ws.fetch(db), db_ref, db64, TOL_DGAMMA, "dbeta")
     n = 64 * 56 * 56
     dx64 = (g * rsig64)[None, :, None, None] * (
         dy64 - (xh64 * dg64[None, :, None, None] + db64[None, :, None, None]) / n)
@@ -434,8 +442,13 @@ def test_config4_group_norm_bf16_32x512x64x64(rt, ws):
     dx_ref, dg_ref, db_ref = R.op_group_norm_grad(
         "float32", R.from_bits(xb, "bfloat16"), g, R.from_bits(dyb, "bfloat16"), mu_ref, rsig_ref, 1, G)
     assert U.normwise(U.widen(ws.fetch(dx), "bfloat16"), dx_ref) <= 1e-2
-    assert U.normwise(ws.fetch(dw), dg_ref) <= 1e-4
-    assert U.normwise(ws.fetch(db), db_ref) <= 1e-4
+    # dgamma / dbeta are fp32 sums of 131072 terms per channel: three-way against fp64
+    dy64 = U.widen(dyb, "bfloat16").reshape(32, G, -1)
+    xh64 = (x64 - x64.mean(2, keepdims=True)) / np.sqrt(x64.var(2, keepdims=True) + 1e-5)
+    dg64 = (dy64 * xh64).reshape(32, C, -1).sum((0, 2))
+    db64 = dy64.reshape(32, C, -1).sum((0, 2))
+    _three_way(ws.fetch(dw), dg_ref, dg64, TOL_DGAMMA, "dgamma")
+    _three_way(ws.fetch(db), db_ref, db64, TOL_DGAMMA, "dbeta")
 
 
 @pytest.mark.parametrize("shape", [(8192, 12288), (65536, 1000)])
@@ -468,7 +481,10 @@ def test_config5_layer_norm_bf16(rt, ws, shape):
     assert U.normwise(dxw, dx_ref) <= 1e-2
     # dgamma / dbeta: sequential fp32 column sums over N rows in the oracle
     dy64 = U.widen(dyb, "bfloat16")
-    _three_way(ws.fetch(db), db_ref, dy64.sum(0), 2e-5, "dbeta")
-    assert U.normwise(ws.fetch(dw), dg_ref) <= 1e-4
+    _three_way(ws.fetch(db), db_ref, dy64.sum(0), TOL_DGAMMA, "dbeta")
+    x64 = U.widen(xb, "bfloat16")
+    xh64 = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    _three_way(ws.fetch(dw), dg_ref, (dy64 * xh64).sum(0), TOL_DGAMMA, "dgamma")
+    del x64, xh64
     # property: each row of dx is orthogonal to the all-ones vector (up to bf16 rounding of dx)
     assert np.max(np.abs(dxw.sum(1))) < 0.05 * np.sqrt(C)

@@ -190,3 +190,37 @@ def test_c_runtime_api_still_answers():
     assert api.dragon_c_run_operator(ws, b'type: "Nope" device_option { device_type: 4 }', 0, 1) == -1
     assert b"not registered" in api.dragon_c_last_error()
     assert api.dragon_c_workspace_destroy(ws) == 0
+
+
+def test_device_scope_and_default_workspace():
+    """``runtime.device`` nests like ``dragon.device`` (context.py:24-52) and operator
+    definitions follow it; ``get_workspace`` / ``Workspace.as_default`` give
+    ``hip.memory_allocated()`` the workspace the reference's takes (cuda.py:146-169)."""
+    from dragon_amd import hip
+    assert rt.get_device() == ("cpu", 0)
+    assert "device_id: 0" in rt.make_def("Softmax", ["x"], ["y"])
+    with rt.device("hip", 3):
+        assert rt.get_device() == ("hip", 3)
+        assert "device_type: 4 device_id: 3" in rt.make_def("Softmax", ["x"], ["y"])
+        with rt.device("hip"):
+            assert rt.get_device() == ("hip", 0)
+            assert "device_id: 0" in rt.make_def("Softmax", ["x"], ["y"])
+        with rt.device("cpu"):
+            assert "device_type: 4 device_id: 0" in rt.make_def("Softmax", ["x"], ["y"])
+        assert rt.get_device() == ("hip", 3)
+        assert "device_id: 1" in rt.make_def("Softmax", ["x"], ["y"], device_id=1)  # explicit wins
+    assert rt.get_device() == ("cpu", 0)
+    hip.set_default_device(2)
+    try:
+        assert rt.get_device() == ("hip", 2)
+        assert "device_id: 2" in rt.make_def("Softmax", ["x"], ["y"])
+    finally:
+        hip.set_default_device(-1)
+    with pytest.raises(ValueError):
+        rt.device("tpu")
+    default = rt.get_workspace()
+    assert rt.get_workspace() is default
+    mine = rt.Workspace("scoped")
+    with mine.as_default() as w:
+        assert w is mine and rt.get_workspace() is mine
+    assert rt.get_workspace() is default
