@@ -60,6 +60,13 @@ def parse_args():
     ap.add_argument("--no-sweep", action="store_true", help="measure the headline workload only")
     ap.add_argument("--sweep", default="", help="comma-separated workloads to sweep instead of all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--timeline", default="", metavar="WORKLOAD",
+                    help="print where the time of a LayerNorm workload's backward row kernel goes "
+                         "(per-workgroup phase clock, per XCD) instead of the bench line")
+    ap.add_argument("--structures", type=int, default=0, metavar="MB",
+                    help="print what streaming two reads and one write over tensors of MB megabytes "
+                         "reaches with one chunk per workgroup, as a persistent kernel, and with "
+                         "store wavefronts, instead of the bench line")
     return ap.parse_args()
 
 
@@ -541,6 +548,108 @@ def cpu_baselines(reps=3):
     return out
 
 
+def timeline_report(name, reps=5):
+    """Phase clock of the persistent row kernel behind a LayerNorm workload's backward: one cold
+    call per tensor set with every workgroup recording (start, first row summed, row loop end,
+    end). Prints, per call, the spread over the workgroups and per XCD; times in microseconds
+    since the first workgroup's start."""
+    import torch
+    from dragon_amd import kernels as K
+    import re
+    m = re.match(r"layer_norm_(bf16|f32)_(\d+)x(\d+)", name)
+    if not m:
+        raise SystemExit("--timeline takes a layer_norm_<dtype>_<rows>x<width> workload")
+    dtype = torch.bfloat16 if m.group(1) == "bf16" else torch.float32
+    N, C = int(m.group(2)), int(m.group(3))
+    gen = _gen(4)
+    sets = []
+    nbytes = N * C * (2 if dtype == torch.bfloat16 else 4)
+    for k in range(max(3, int(math.ceil(COLD_BYTES / (3 * nbytes))) + 1)):
+        x, dy = _randn((N, C), dtype, gen), _randn((N, C), dtype, gen)
+        g, b = _affine(C, gen)
+        y, dx = torch.empty_like(x), torch.empty_like(x)
+        mu, rsig = torch.empty(N, device="cuda"), torch.empty(N, device="cuda")
+        K.layer_norm(N, C, 1e-5, x, g, b, mu, rsig, y)
+        sets.append((x, dy, g, mu, rsig, dx, torch.empty(2 * N, device="cuda"),
+                     torch.empty(C, device="cuda"), torch.empty(C, device="cuda")))
+    torch.cuda.synchronize()
+    print("# %s: LayerNorm backward, %d tensor sets of %.0f MB, plan %s" % (
+        name, len(sets), 3 * nbytes / 1e6,
+        K.plan_name("layer_norm_grad", "bfloat16" if dtype == torch.bfloat16 else "float32", (N, C))))
+    import numpy as np
+    calls = []
+    for rep in range(reps + 1):  # the first round warms the code up and is not counted
+        for x, dy, g, mu, rsig, dx, params, dg, db in sets:
+            stamps = K.group_norm_grad_timeline(N, 1, C, 1, "NHWC", x, mu, rsig, g, dy, params, params,
+                                                dg, db, dx)
+            torch.cuda.synchronize()
+            if rep == 0:
+                continue
+            t = stamps.cpu().numpy()
+            t = t[t[:, 0] > 0]
+            if not len(t):
+                raise SystemExit("this workload does not take the persistent row kernel")
+            calls.append((t[:, 4].copy(), (t[:, :4] - t[:, 0].min()) * 0.01, t[:, 5].copy()))
+    us = np.stack([c[1] for c in calls])  # [call, workgroup, phase]
+    print("%d cold calls, %d workgroups, %d rows per row group; microseconds since the first "
+          "workgroup's start, averaged over the calls" % (len(calls), us.shape[1], int(calls[0][2].max())))
+    for c, what in enumerate(("start", "first row summed", "row loop end", "workgroup end")):
+        print("  %-17s first %6.2f   mean %6.2f   last %6.2f" % (
+            what, us[:, :, c].min(1).mean(), us[:, :, c].mean(1).mean(), us[:, :, c].max(1).mean()))
+    span = us[:, :, 3].max(1)
+    busy = (us[:, :, 3] - us[:, :, 0]).mean(1)
+    print("  kernel span (first start to last end) %.2f us; a workgroup is busy %.2f us on average: "
+          "%.2f us (%.1f%%) of the span is waiting for the slowest workgroups"
+          % (span.mean(), busy.mean(), (span - busy).mean(), 100 * ((span - busy) / span).mean()))
+    steps = int(calls[0][2].max())
+    first = (us[:, :, 1] - us[:, :, 0]).mean()
+    steady = ((us[:, :, 2] - us[:, :, 1]).mean()) / max(1, steps - 1)
+    print("  first row %.2f us after the workgroup's start, then %.2f us per row-loop trip; the partial "
+          "row takes %.2f us" % (first, steady, (us[:, :, 3] - us[:, :, 2]).mean()))
+    print("  per XCD (mean over calls and workgroups):")
+    xcd_of = calls[0][0]
+    for xcd in sorted(set(xcd_of)):
+        rows = [c[1][c[0] == xcd] for c in calls]
+        sel = np.concatenate(rows)
+        print("   XCD %d: start %.2f  row loop %.2f  end %.2f (last %.2f)" % (
+            xcd, sel[:, 0].mean(), (sel[:, 2] - sel[:, 0]).mean(), sel[:, 3].mean(),
+            np.mean([r[:, 3].max() for r in rows])))
+
+
+def structures_report(mb, steps=32, reps=3):
+    """What the *structure* of a kernel costs when it streams two reads and one write over three
+    tensors of `mb` megabytes, cold: one chunk per workgroup (the probe's shapes), persistent
+    workgroups with chunks requested ahead, and persistent workgroups whose stores are issued
+    by separate wavefronts."""
+    import torch
+    from dragon_amd import kernels as K
+    nbytes = mb << 20
+    moved = 3 * nbytes
+    count = max(3, int(math.ceil(COLD_BYTES / moved)) + 1)
+    sets = [(torch.randint(1, 255, (2 * nbytes,), dtype=torch.uint8, device="cuda"),
+             torch.empty(nbytes, dtype=torch.uint8, device="cuda")) for _ in range(count)]
+
+    def best(make):
+        fns = [make(a, b) for a, b in sets]
+        return min(time_calls(fns, steps, count)[0] for _ in range(reps)) * 1e3
+
+    print("# two reads and one write, 3 x %d MB, %d buffer sets, best of %d runs of %d calls" % (
+        mb, count, reps, steps))
+    for shape in PROBE_SHAPES + ((1024, 2),):
+        us = best(lambda a, b, shape=shape: (lambda: K.stream_probe(3, a, b, nbytes, shape)))
+        print("one chunk per workgroup   %4d threads x %d in flight                      %7.2f us  %.3f of 8 TB/s"
+              % (shape + (us, moved / us / 8e6)))
+    for threads, flight, per_cu, depth, barrier, split in (
+            (256, 2, 8, 0, 0, 0), (256, 2, 4, 1, 0, 0), (256, 2, 4, 2, 0, 0), (512, 2, 2, 1, 1, 0),
+            (1024, 2, 1, 1, 0, 0), (1024, 2, 1, 1, 1, 0), (1024, 2, 1, 2, 1, 0), (1024, 1, 1, 3, 1, 0),
+            (1024, 2, 1, 1, 1, 1), (1024, 2, 1, 2, 1, 1), (512, 2, 2, 1, 1, 1)):
+        us = best(lambda a, b: (lambda: K.stream_probe_persistent(a, b, nbytes, threads, flight, per_cu, depth,
+                                                                  barrier, split)))
+        print("persistent %-14s %4d threads x %d in flight, %d per CU, %d ahead%s  %7.2f us  %.3f of 8 TB/s"
+              % ("store waves" if split else "", threads, flight, per_cu, depth,
+                 ", barrier" if barrier else "         ", us, moved / us / 8e6))
+
+
 def contract_problems(line):
     """What is wrong with a parsed bench line, as a list of sentences (empty when nothing is):
     the fields the driver reads, the roofline arithmetic, and the probe as a ceiling, i.e. no
@@ -583,6 +692,10 @@ def main():
         sys.exit(1)
     from dragon_amd import _lib
     _lib.lib()  # fail loudly if the HIP library is not built
+    if args.timeline:
+        return timeline_report(args.timeline)
+    if args.structures:
+        return structures_report(args.structures)
 
     head = args.workload
     per_kernel, ms_step, total_bytes = measure_workload(head, args.steps, args.warmup)

@@ -110,9 +110,12 @@ SIGNATURES = {
     "dragon_hip_exchange_timed_out": (_int, []),
     "dragon_hip_exchange_reset": (None, [ctypes.c_uint]),
     "dragon_hip_exchange_plan": (_int, [_int, _i64, _i64, _i64, _int] + [ctypes.POINTER(_int)] * 4),
+    "dragon_hip_group_norm_grad_timeline": (_int, [_int, _i64, _i64, _i64, _i64, _int] + [_vp] * 11 +
+                                            [_sz, _vp, _sz, _vp]),
     "dragon_hip_plan_name": (_int, [ctypes.c_char_p, _int, _int, ctypes.POINTER(_i64), _int,
                                     ctypes.c_char_p, _sz]),
     "dragon_hip_stream_probe": (_int, [_int, _vp, _vp, _sz, _vp]),
+    "dragon_hip_stream_probe_persistent": (_int, [_int, _int, _int, _int, _int, _int, _vp, _vp, _sz, _vp]),
     "dragon_hip_stream_probe_shape": (_int, [_int, _int, _int, _vp, _vp, _sz, _vp]),
 }
 

@@ -93,6 +93,19 @@ inline void note_number(const char* key, long long value) {
   t.text[t.used] = 0;
 }
 
+// Where a kernel that can record its phases leaves them for the calling thread's next launch
+// (null: nothing is recorded). Set only by the *_timeline entry points of the C ABI, which
+// exist for measurement: a handful of device clock reads per workgroup.
+struct TimelineTarget {
+  unsigned long long* stamps = nullptr;  // device memory, kTimelineWords words per workgroup
+  size_t workgroups = 0;                 // how many workgroups it has room for
+};
+constexpr int kTimelineWords = 6;  // start, first data, loop end, end, XCD, rows done
+inline TimelineTarget& timeline_target() {
+  static thread_local TimelineTarget target;
+  return target;
+}
+
 #undef hipLaunchKernelGGL
 #define hipLaunchKernelGGL(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...)       \
   do {                                                                                         \

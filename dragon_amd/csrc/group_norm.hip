@@ -234,9 +234,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
     const typename IO<T>::Acc* __restrict__ rsig, typename IO<T>::Acc* __restrict__ ds,
     typename IO<T>::Acc* __restrict__ db, T* __restrict__ dx,
-    typename IO<T>::Acc* __restrict__ partial) {
+    typename IO<T>::Acc* __restrict__ partial, unsigned long long* __restrict__ stamps) {
   using Tile = RowTile<T, kTPR, kVPT, kGradThreads>;
   using Raw = RawRowTile<T, kTPR, kVPT, kGradThreads>;
+  // Phase clock of this workgroup (100 MHz device clock), only when a timeline is recorded.
+  unsigned long long* const mark =
+      stamps != nullptr && threadIdx.x == 0 ? stamps + static_cast<size_t>(blockIdx.x) * kTimelineWords : nullptr;
+  if (mark) mark[0] = wall_clock64();
   using A = typename Tile::A;
   constexpr int kVec = Tile::kVec;
   constexpr int kGroups = Tile::kRowsPerBlock;
@@ -326,6 +330,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
   }
   __syncthreads();
 
+  unsigned long long rows_done = 0;  // of the marking thread's row group
   // One row: tx / tdy hold it, nx / ndy the row after it.
   auto step = [&](Raw& tx, Raw& tdy, const A m, const A r, Raw& nx, Raw& ndy) {
     const bool valid = row < N;
@@ -350,6 +355,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
       ds[row] = s1;
       db[row] = s2;
     }
+    if (mark && rows_done++ == 0) mark[1] = wall_clock64();  // the first row has arrived and is summed
 
     const A a = (s2 * m - s1) * (r * r * r) * inv_c;
     const A b = -(s2 * r) * inv_c;
@@ -418,6 +424,7 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
     }
   }
 
+  if (mark) mark[2] = wall_clock64();  // the row loop is done; what follows is the partial row
   // Combine the kGroups row groups of this workgroup, kChunk pairs at a time.
   A* out = partial + static_cast<size_t>(blockIdx.x) * C * 2;
 #pragma unroll
@@ -462,6 +469,13 @@ __global__ __launch_bounds__(kGradThreads, kGradThreads == 768 ? 3 : 4) void lay
         }
       }
     }
+  }
+  if (mark) {
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    mark[3] = wall_clock64();
+    mark[4] = xcc & 0xf;
+    mark[5] = rows_done;
   }
 }
 
@@ -3480,6 +3494,8 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     const bool ragged =
         rp.ragged || !(aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma));
     const size_t staged_bytes = static_cast<size_t>(ceil_div(sh.D, kVec) * kVec) * sizeof(A);
+    const TimelineTarget& tl = timeline_target();
+    unsigned long long* marks = tl.stamps != nullptr && tl.workgroups >= rp.grid ? tl.stamps : nullptr;
 #define LAUNCH_T(TPR, VPT, THREADS)                                                           \
   {                                                                                           \
     note_flavour(ragged ? "layer_norm_grad_rows<" #TPR "," #VPT "," #THREADS ",ragged>"        \
@@ -3489,7 +3505,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     if (staged_bytes > 48 * 1024) (void)resident_grid(kernel, THREADS, staged_bytes);         \
     hipLaunchKernelGGL(kernel, dim3(rp.grid), dim3(THREADS), staged_bytes, stream,            \
                        static_cast<int64_t>(sh.N), static_cast<int>(sh.D), xp, dyp, gp, mup,  \
-                       rsp, dsp, dbp, dxp, part);                                             \
+                       rsp, dsp, dbp, dxp, part, marks);                                      \
   }
 #define LAUNCH(TPR, VPT)                                                    \
   {                                                                         \
@@ -3930,6 +3946,23 @@ int dragon_hip_group_norm_grad(int dtype, int64_t N, int64_t G, int64_t D, int64
   void* db_eff = ds == db ? static_cast<char*>(ds) + acc * N * G : db;
   DRAGON_HIP_DISPATCH_DTYPE(dtype, dragon_hip::launch_group_norm_grad, sh, x, mu, rsig, gamma, dy,
                             ds, db_eff, dgamma, dbeta, dx, scratch, scratch_bytes, s);
+}
+
+int dragon_hip_group_norm_grad_timeline(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
+                                        int layout, const void* x, const void* mu, const void* rsig,
+                                        const void* gamma, const void* dy, void* ds, void* db,
+                                        void* dgamma, void* dbeta, void* dx, void* scratch,
+                                        size_t scratch_bytes, void* stamps, size_t workgroups,
+                                        void* stream) {
+  if (!stamps || workgroups == 0) return DRAGON_HIP_EINVAL;
+  dragon_hip::TimelineTarget& target = dragon_hip::timeline_target();
+  target.stamps = static_cast<unsigned long long*>(stamps);
+  target.workgroups = workgroups;
+  const int st = dragon_hip_group_norm_grad(dtype, N, G, D, S, layout, x, mu, rsig, gamma, dy, ds, db,
+                                            dgamma, dbeta, dx, scratch, scratch_bytes, stream);
+  target.stamps = nullptr;
+  target.workgroups = 0;
+  return st;
 }
 
 

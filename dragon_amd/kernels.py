@@ -160,6 +160,21 @@ def group_norm_grad(N, G, D, S, data_format, x, mu, rsig, gamma, dy, ds, db, dga
           _ptr(ws), need, _stream())
 
 
+def group_norm_grad_timeline(N, G, D, S, data_format, x, mu, rsig, gamma, dy, ds, db, dgamma, dbeta,
+                             dx, workgroups=2048):
+    """group_norm_grad with the phase clock of the LayerNorm backward row kernel: returns an
+    int64 tensor [workgroups, 6] (start, first row summed, row loop end, end in 10 ns ticks,
+    XCD, rows of the first row group); workgroups that recorded nothing stay zero."""
+    tag, lay = dtype_tag(x), layout_tag(data_format)
+    need = _lib.lib().dragon_hip_group_norm_grad_scratch_bytes(tag, N, G, D, S, lay)
+    ws = workspace(need, x.device)
+    stamps = torch.zeros((workgroups, 6), dtype=torch.int64, device=x.device)
+    _call("dragon_hip_group_norm_grad_timeline", tag, N, G, D, S, lay, _ptr(x), _ptr(mu), _ptr(rsig),
+          _ptr(gamma), _ptr(dy), _ptr(ds), _ptr(db), _ptr(dgamma), _ptr(dbeta), _ptr(dx),
+          _ptr(ws), need, _ptr(stamps), workgroups, _stream())
+    return stamps
+
+
 def _bn_scratch(tag, N, C, S, lay, device):
     need = _lib.lib().dragon_hip_batch_norm_reduce_scratch_bytes(tag, N, C, S, lay)
     return workspace(need, device), need
@@ -383,6 +398,16 @@ def plan_name(op, dtype_name, dims, data_format="NCHW"):
 
 
 # ---------------------------------------------------------------- measurement
+
+def stream_probe_persistent(src, dst, nbytes, threads, in_flight, per_cu, depth, barrier, store_waves):
+    """Two reads and one write as a *persistent* kernel would stream them: ``per_cu`` workgroups
+    of ``threads`` per compute unit walk the chunks with a grid stride, ``depth`` chunks
+    requested ahead into registers, optionally a workgroup barrier per chunk (as a row
+    reduction has) and optionally with the stores issued by separate wavefronts fed through
+    LDS (``store_waves``: half of the workgroup)."""
+    _call("dragon_hip_stream_probe_persistent", int(threads), int(in_flight), int(per_cu), int(depth),
+          int(bool(barrier)), int(bool(store_waves)), _ptr(src), _ptr(dst), nbytes, _stream())
+
 
 def stream_probe(mode, src, dst, nbytes, shape=None):
     """Streaming read (0), copy (1), fill (2) or two reads and one write (3) of ``nbytes``

@@ -429,6 +429,22 @@ void dragon_hip_exchange_reset(unsigned patience);
 int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seglen, int tensors,
                              int* slices, int* slice_packets, int* packets_per_thread, int* grid);
 
+/* dragon_hip_group_norm_grad with a phase clock: where the call takes the persistent row
+ * kernel of the LayerNorm backward (G = S = 1, rows of up to 16384 elements that are not
+ * short), every workgroup of that kernel leaves six 64-bit words in `stamps` (device memory
+ * with room for `workgroups` workgroups, zero-filled by the caller; workgroup b writes words
+ * 6b .. 6b+5): the device's 100 MHz clock at its start, when its first row had arrived and
+ * been summed, when its row loop ended, and at its end; then the XCD it ran on and the rows
+ * its first row group handled. Other paths, or too few `workgroups`, record nothing.
+ * No counterpart in the reference; it is how the benchmark shows where the microseconds of
+ * this kernel go (first loads, row loop, partial row) and how evenly the dies finish. */
+int dragon_hip_group_norm_grad_timeline(int dtype, int64_t N, int64_t G, int64_t D, int64_t S,
+                                        int layout, const void* x, const void* mu, const void* rsig,
+                                        const void* gamma, const void* dy, void* ds, void* db,
+                                        void* dgamma, void* dbeta, void* dx, void* scratch,
+                                        size_t scratch_bytes, void* stamps, size_t workgroups,
+                                        void* stream);
+
 /* dragon_hip_plan_name: which kernels an entry point would launch for a shape,
  * as text "flavour:kernel[threads];kernel[threads];..." in launch order (a
  * "key=value:" item in front of a kernel is a number its plan depends on). No
@@ -470,6 +486,18 @@ int dragon_hip_stream_probe(int mode, const void* src, void* dst, size_t bytes, 
  * at that kernel's tensor size. */
 int dragon_hip_stream_probe_shape(int mode, int threads, int in_flight, const void* src, void* dst,
                                   size_t bytes, void* stream);
+/* Two reads and one write (mode 3 above) streamed the way a *persistent* kernel does it:
+ * `per_cu` workgroups of `threads` threads per compute unit walk chunks of
+ * threads x in_flight packets with a grid stride, `depth` (0 .. 3) chunks requested ahead
+ * into registers; `barrier` adds a workgroup barrier per chunk, as a row reduction has;
+ * `store_waves` lets the second half of each workgroup do nothing but write out what the
+ * first half leaves in LDS (then threads / 2 load). Shapes: threads 256, 512 or 1024,
+ * in_flight 1 or 2. It measures what the structure of the kernels that must be persistent
+ * (those that carry per-column sums across rows) costs against the one-chunk-per-workgroup
+ * probes. */
+int dragon_hip_stream_probe_persistent(int threads, int in_flight, int per_cu, int depth, int barrier,
+                                       int store_waves, const void* src, void* dst, size_t bytes,
+                                       void* stream);
 
 #ifdef __cplusplus
 } /* extern "C" */
