@@ -789,8 +789,8 @@ __global__ __launch_bounds__(kReduceThreads) void layer_norm_wide_grad(
 // kAnyS: a channel is not whole packets (the group still is), so the elements
 // of a packet may belong to different channels; 2 where a channel is 64 packets'
 // worth or more, 1 for shorter ones.
-template <typename T, int kTPR, int kVPT, int kAnyS = 0, bool kTwoPerCu = false>
-__global__ __launch_bounds__(row_threads(kTPR), kTwoPerCu ? 8 : 1) void group_norm_forward_rows(
+template <typename T, int kTPR, int kVPT, int kAnyS = 0>
+__global__ __launch_bounds__(row_threads(kTPR)) void group_norm_forward_rows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
@@ -807,7 +807,7 @@ __global__ __launch_bounds__(row_threads(kTPR), kTwoPerCu ? 8 : 1) void group_no
 
   // The 1024-thread tile (one or two workgroups per compute unit) requests the
   // next group's packets before it reduces the current group.
-  constexpr bool kPrefetch = kTPR == 1024 && !kTwoPerCu;
+  constexpr bool kPrefetch = kTPR == 1024;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * Tile::kRowsPerBlock;
   int64_t row = static_cast<int64_t>(blockIdx.x) * Tile::kRowsPerBlock + Tile::sub_row();
   // The loaded packets are not masked (a select on them would wait for each
@@ -2986,7 +2986,6 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
   RowConfig cfg;
   const int64_t L = static_cast<int64_t>(sh.D) * sh.S;
   if (!sh.nchw || !pick_row_config(ceil_div(L, kVec), 8, &cfg)) return false;
-  if (getenv("DRAGON_HIP_XP_GN_SLICES")) return false;  // XP
   const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
   // Groups of at most 32 packets leave half of a wavefront's lanes or more idle in
   // the row kernels: several groups per wavefront, staged through LDS (fp16
@@ -3046,25 +3045,13 @@ bool try_group_norm_forward_rows(const GroupShape& sh, float eps, const void* x,
         : sh.S >= kWaveSize * kVec && !(kVec == 8 && VPT == 8 && TPR == 1024) /* spills: 82 us against 66 */ \
             ? group_norm_forward_rows<T, TPR, VPT, 2>                                           \
             : group_norm_forward_rows<T, TPR, VPT, 1>;                                          \
-    unsigned resident = TPR == 1024 ? resident_grid(kernel, TPR, 0) : one_shot;                 \
-    if constexpr (TPR == 1024 && VPT == 8 && sizeof(T) == 2) {                                  \
-      if (getenv("DRAGON_HIP_XP_GN_TWO") && sh.S % kVec == 0) { /* XP */                         \
-        kernel = group_norm_forward_rows<T, TPR, VPT, 0, true>;                                 \
-        resident = atoi(getenv("DRAGON_HIP_XP_GN_TWO")) > 1 ? one_shot : resident_grid(kernel, TPR, 0); \
-      }                                                                                         \
-    }                                                                                           \
+    const unsigned resident = TPR == 1024 ? resident_grid(kernel, TPR, 0) : one_shot;           \
     hipLaunchKernelGGL(kernel,                                                                  \
                        dim3(one_shot < resident ? one_shot : resident), dim3(Tile::kThreads), 0, stream, \
                        rows, static_cast<int>(L), sh.G, sh.D, sh.S, A(eps),                     \
                        static_cast<const T*>(x), static_cast<const A*>(gamma),                  \
                        static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig), \
                        static_cast<T*>(y));                                                     \
-  }
-  if constexpr (sizeof(T) == 2) {
-    if (getenv("DRAGON_HIP_XP_GN_512") && cfg.tpr == 1024 && cfg.vpt == 8 && sh.S % kVec == 0) { /* XP */
-      LAUNCH(512, 16)
-      return true;
-    }
   }
   DRAGON_HIP_ROW_SWITCH(cfg, LAUNCH);
 #undef LAUNCH
@@ -3631,8 +3618,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 
   RowConfig gcfg;
   int mode = kChannelWaves;
-  if (!getenv("DRAGON_HIP_XP_GN_SLICES") /* XP */ &&
-      plan_group_grad_rows<T>(sh.G, sh.D, sh.S, layout, &gcfg, &mode) && aligned16(x) &&
+  if (plan_group_grad_rows<T>(sh.G, sh.D, sh.S, layout, &gcfg, &mode) && aligned16(x) &&
       aligned16(dy) && aligned16(dx)) {
     const int64_t rows = static_cast<int64_t>(sh.N) * sh.G;
     const int L = static_cast<int>(sh.D * sh.S);

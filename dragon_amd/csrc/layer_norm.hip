@@ -380,9 +380,8 @@ int launch_layer_norm(int64_t N, int64_t C, float eps, const void* x, const void
     auto kernel = layer_norm_wide_rows<T, TPR, VPT, THREADS>;                                \
     const int64_t groups = ceil_div(N, static_cast<int64_t>(THREADS / TPR));                 \
     const unsigned resident = resident_grid(kernel, THREADS, staged_bytes);                  \
-    unsigned grid =                                                                          \
+    const unsigned grid =                                                                    \
         groups < static_cast<int64_t>(resident) ? static_cast<unsigned>(groups) : resident;  \
-    if (getenv("DRAGON_HIP_XP_LN_GRID")) grid = atoi(getenv("DRAGON_HIP_XP_LN_GRID")); /* XP */ \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), staged_bytes, stream, N,           \
                        static_cast<int>(C), A(eps), xp, gp, bp, mp, rp, yp);                 \
   }

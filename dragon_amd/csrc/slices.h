@@ -142,10 +142,6 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn, bool windows = false) {
     if (util > best_util + 1e-9) best = k, best_util = util;
     if (util >= 0.96) break;
   }
-  if (const char* xp = getenv("DRAGON_HIP_XP_COOP_K")) {  // XP
-    const int64_t k = atoll(xp);
-    if (k >= kmin && k <= klimit) best = k;
-  }
   p.K = static_cast<uint32_t>(best);
   // whole wavefronts of packets per slice, so that a wavefront never straddles two slices
   p.slice = static_cast<uint32_t>(ceil_div(ceil_div(P, best), kWaveSize) * kWaveSize);
