@@ -40,6 +40,7 @@
 #include "row_loop.h"
 #include "row_tile.h"
 #include "short_rows.h"
+#include "sample_slices.h"
 #include "slices.h"
 
 namespace dragon_hip {
@@ -3872,6 +3873,18 @@ int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShap
   return DRAGON_HIP_OK;
 }
 
+// Exchange bytes of the sliced NHWC forward (0: the shape does not take that path).
+size_t sample_slices_forward_bytes(int dtype, const GroupShape& sh) {
+  SampleSlicePlan p{false, 0u, 0u, 0};
+  switch (dtype) {
+    case DRAGON_HIP_F16: p = plan_sample_slices<f16_t>(sh.S, sh.C, sh.G, sh.D); break;
+    case DRAGON_HIP_BF16: p = plan_sample_slices<bf16_t>(sh.S, sh.C, sh.G, sh.D); break;
+    case DRAGON_HIP_F32: p = plan_sample_slices<float>(sh.S, sh.C, sh.G, sh.D); break;
+    default: break;
+  }
+  return p.ok && !sh.nchw ? sample_slices_exchange_bytes(sh.N, sh.G, p.K, 4) : 0;
+}
+
 template <typename T>
 size_t grad_scratch_t(int64_t N, int64_t G, int64_t D, int64_t S, int layout) {
   return group_norm_grad_scratch<T>(N, G, D, S, layout);
@@ -3984,6 +3997,8 @@ size_t dragon_hip_group_norm_forward_scratch_bytes(int dtype, int64_t N, int64_t
     const size_t nhwc = (dragon_hip::batched_partial_pairs(N, S, G * D) +
                          static_cast<size_t>(N) * G * D) * 2 * (dtype == DRAGON_HIP_F64 ? 8 : 4);
     if (nhwc > bytes) bytes = nhwc;
+    const size_t sliced = dragon_hip::sample_slices_forward_bytes(dtype, sh);
+    if (sliced > bytes) bytes = sliced;
   } else {
     const size_t slices = dragon_hip::group_slices_scratch_bytes(dtype, sh);
     if (slices > bytes) bytes = slices;
@@ -4050,6 +4065,14 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
     if (!scratch || scratch_bytes < dragon_hip_group_norm_forward_scratch_bytes(dtype, N, G, D, S, layout)) {
       return DRAGON_HIP_ESCRATCH;
     }
+    // samples beyond one workgroup's registers: slices that exchange their groups' statistics
+    switch (dtype) {
+      case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::f16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+      case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::bf16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+      case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_nhwc_slices<float>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+      default: st = dragon_hip::kNotApplicable; break;
+    }
+    if (st != dragon_hip::kNotApplicable) return st;
     switch (dtype) {
       case DRAGON_HIP_F16: st = dragon_hip::group_norm_stats_nhwc<dragon_hip::f16_t>(sh, eps, x, mu, rsig, scratch, hs); break;
       case DRAGON_HIP_BF16: st = dragon_hip::group_norm_stats_nhwc<dragon_hip::bf16_t>(sh, eps, x, mu, rsig, scratch, hs); break;

@@ -1,0 +1,590 @@
+// GroupNorm forward over NHWC samples that do not fit one workgroup: x is read once.
+//
+// A sample is S rows of C channels. It is cut into K slices of whole rows; a
+// 256-thread workgroup keeps its slice in registers as raw packets (thread
+// (r, cp) holds packet cp of rows r, r + R, r + 2R, ... of the slice, R =
+// 256 / (C / kVec) rows at a time), so a thread's channels, their group and
+// their parameters are the same for every item it sees. A slice holds a share
+// of every group of the sample, so an item has G partial pairs to exchange, not
+// one. If every slice read every other slice's G pairs, a sample would cost
+// G * K * K uncached reads; instead the groups are dealt out over the sample's
+// slices, and the exchange has two steps:
+//   1. a slice publishes its G partial pairs (before it waits for anything);
+//   2. slice k, the combiner of groups k, k + K, k + 2K, ..., waits for the K
+//      partial pairs of each of them (one wavefront per group, a pair or a
+//      few per lane), forms the group's totals in a fixed order and publishes
+//      them as one pair per group (and writes the group's mean and rsig);
+//   3. every slice waits for the sample's G total pairs and finishes its rows
+//      out of registers.
+// A combiner waits only for partial pairs, which every workgroup publishes
+// before its first wait; totals wait only for combiners. Items are dealt out
+// and walked as in slices.h (item w = n*K + k on workgroup w % grid, ascending;
+// the whole grid resident; K never above the grid), so the same induction
+// shows that every wait is for a workgroup that is running.
+//
+// A pair is two fp32 words, published and read as one 64-bit word with
+// device-scope atomic accesses; a pair is complete when neither half holds the
+// unset pattern (slices.h).
+//
+// The waits are bounded, and an item whose wait runs out is flagged and
+// finished by a second launch behind the first, exactly as in slices.h. By then
+// every partial pair is published, so the repair forms the totals of all G
+// groups itself with the combiner's arithmetic (contraction off: the same bits)
+// and, for the groups its slice combines, writes the mean and rsig the
+// combiner did not. A flagged item wrote no output, so a call may run in place.
+//
+// Partials are (mean, sum of squared deviations) of the slice's share of the
+// group, formed in two passes over the registers; the combiner merges them with
+// the counts the slice geometry gives. Nothing depends on an element outside
+// the slice.
+//
+// Every item pays the two steps of the exchange, about 10 us on MI355X during
+// which its workgroup moves nothing, so the kernel reaches about 4 TB/s where a
+// plain copy reaches 5.5. Measured cold on MI355X against the two-pass path
+// (column statistics, then the map) on tensors of the same size: [32, 64*64,
+// 512] bf16 74 us against 84, fp32 127 against 142; [64, 32*32, 512] bf16 34
+// against 46. A backward built the same way (x and dy in registers, ds / db
+// exchanged) holds half as many rows per item and pays the exchange twice as
+// often: 143 us against 122 for the five-pass path at the first shape, so the
+// backward keeps the five passes.
+#pragma once
+
+#include "slices.h"
+
+namespace dragon_hip {
+
+constexpr int kSliceThreads = 256;
+constexpr uint32_t kMaxSampleSlices = 1024;  // slices per sample (a resident grid holds no more workgroups)
+constexpr uint32_t kMaxSampleGroups = 256;  // groups: one owner thread each
+
+struct SampleSlices {
+  uint32_t N, S, C, G, D;
+  uint32_t K;         // slices per sample
+  uint32_t rows;      // rows per slice (the last slice of a sample may hold fewer)
+  uint32_t items;     // N * K
+  uint32_t patience;  // polls of a slot before a thread gives up
+  uint32_t* flags;    // flags[w] = 1: item w gave up; flags[items] = 1: some item did
+  uint32_t* gave_up_count;
+};
+
+struct SampleSlicePlan {
+  bool ok;
+  uint32_t K, rows;
+  int vpt;  // packets per thread and tensor
+};
+
+// Up to 16 packets per thread, three workgroups per compute unit (four for
+// slices of half that size).
+template <typename T>
+SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
+  constexpr uint32_t kVec = IO<T>::kVec;
+  SampleSlicePlan p{false, 0u, 0u, 0};
+  if (sizeof(T) > 4 || S <= 1 || C % kVec != 0 || D % kVec != 0) return p;
+  const uint32_t cps = C / kVec;
+  if (cps > kSliceThreads || G > kMaxSampleGroups) return p;
+  const uint32_t rows_at_a_time = kSliceThreads / cps;
+  // most of the workgroup's threads must have a row to hold
+  if (cps * rows_at_a_time * 4 < kSliceThreads * 3) return p;
+  const uint32_t vmax = 16u;
+  const uint32_t k0 = static_cast<uint32_t>(ceil_div(S, rows_at_a_time * vmax));
+  // slices of about the same size
+  const uint32_t vpt = static_cast<uint32_t>(ceil_div(ceil_div(S, k0), rows_at_a_time));
+  p.rows = rows_at_a_time * vpt;
+  p.K = static_cast<uint32_t>(ceil_div(S, p.rows));
+  p.vpt = static_cast<int>(vpt);
+  p.ok = p.K <= kMaxSampleSlices;
+  return p;
+}
+
+// Scratch words of a call, in accumulator words: G pairs per item, G pairs per
+// sample, then the flags (a 32-bit word each, one more than there are items).
+inline size_t sample_slices_exchange_words(uint32_t N, uint32_t G, uint32_t K) {
+  return (static_cast<size_t>(N) * K * G + static_cast<size_t>(N) * G) * 2;
+}
+inline size_t sample_slices_exchange_bytes(uint32_t N, uint32_t G, uint32_t K, size_t acc_size) {
+  const size_t bytes = sample_slices_exchange_words(N, G, K) * acc_size +
+      (static_cast<size_t>(N) * K + 1) * sizeof(uint32_t);
+  return (bytes + 255) / 256 * 256;
+}
+
+template <typename T>
+SampleSlices make_sample_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, uint32_t D,
+                                const SampleSlicePlan& p, typename IO<T>::Acc* exchange) {
+  SampleSlices d;
+  d.N = N, d.S = S, d.C = C, d.G = G, d.D = D;
+  d.K = p.K, d.rows = p.rows, d.items = N * p.K;
+  const uint32_t patience = exchange_patience();
+  d.patience = patience ? patience : kCoopPatience;
+  d.flags = reinterpret_cast<uint32_t*>(exchange + sample_slices_exchange_words(N, G, p.K));
+  d.gave_up_count = exchange_gave_up_counter();
+  return d;
+}
+
+// Where a thread sits in its workgroup's slice.
+template <int kVec>
+struct SliceSeat {
+  uint32_t cps, rows_at_a_time, r, cp, g, lanes_per_group;
+  bool on;
+  __device__ explicit SliceSeat(const SampleSlices& d) {
+    cps = d.C / kVec;
+    rows_at_a_time = kSliceThreads / cps;
+    r = threadIdx.x / cps, cp = threadIdx.x - r * cps;
+    on = r < rows_at_a_time;
+    lanes_per_group = d.D / kVec;
+    g = on ? cp / lanes_per_group : 0u;
+  }
+};
+
+struct SliceItem {
+  uint32_t n, k, row0, nrows;
+  __device__ SliceItem(const SampleSlices& d, uint32_t w) {
+    n = w / d.K, k = w - n * d.K;
+    row0 = k * d.rows;
+    nrows = min(d.rows, d.S - row0);
+  }
+};
+
+// Element offset of the thread's first packet of the item, and between its packets.
+template <int kVec>
+__device__ __forceinline__ uint32_t slice_first(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                const SliceItem& it) {
+  return (it.n * d.S + it.row0 + at.r) * d.C + at.cp * kVec;
+}
+
+template <typename T, int kVPT>
+__device__ __forceinline__ void slice_load(const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at,
+                                           const SliceItem& it, const T* in, u32x4 (&raw)[kVPT]) {
+  const uint32_t first = slice_first(d, at, it), step = at.rows_at_a_time * d.C;
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) {
+    const bool has = at.on && at.r + i * at.rows_at_a_time < it.nrows;
+    raw[i] = load_packet(in + (has ? first + i * step : 0u));
+  }
+}
+
+// A pair of fp32 words is published and read as one 64-bit word: one request, and
+// both halves arrive together.
+__device__ __forceinline__ unsigned long long pair_bits(const float a, const float b) {
+  return static_cast<unsigned long long>(publishable_bits(a)) |
+      (static_cast<unsigned long long>(publishable_bits(b)) << 32);
+}
+constexpr unsigned long long kUnsetPair = ~0ull;
+__device__ __forceinline__ void publish_pair(float* slot, const float a, const float b) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(slot), pair_bits(a, b), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long peek_pair(const float* slot) {
+  return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(slot), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool pair_set(unsigned long long u) {
+  return static_cast<uint32_t>(u) != 0xffffffffu && static_cast<uint32_t>(u >> 32) != 0xffffffffu;
+}
+// false: the pair was still unset after `patience` polls (a and b are then meaningless);
+// `u` is what a first look has already seen
+__device__ __forceinline__ bool await_pair(const float* slot, uint32_t patience, unsigned long long u,
+                                           float& a, float& b) {
+  for (;;) {
+    a = __builtin_bit_cast(float, static_cast<uint32_t>(u));
+    b = __builtin_bit_cast(float, static_cast<uint32_t>(u >> 32));
+    if (pair_set(u)) return true;
+    if (--patience == 0) return false;
+    __builtin_amdgcn_s_sleep(8);
+    u = peek_pair(slot);
+  }
+}
+__device__ __forceinline__ bool await_pair(const float* slot, uint32_t patience, float& a, float& b) {
+  return await_pair(slot, patience, peek_pair(slot), a, b);
+}
+
+// The group's totals of kN values per thread, one LDS word per thread and
+// value: the thread that owns group t adds the R * (D / kVec) shares of its
+// group in row order and leaves the sums in total[j][t]. Every thread may read
+// total[j][*] afterwards; the barrier of the next call (or of the exchange)
+// lies between those reads and the next writes.
+template <int kN, int kVec, typename A>
+__device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                 const A (&v)[kN], A (*part)[kSliceThreads],
+                                                 A (*total)[kSliceThreads]) {
+  const uint32_t t = threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < kN; ++j) part[j][t] = at.on ? v[j] : A(0);
+  __syncthreads();
+  if (t < d.G) {
+    A acc[kN];
+#pragma unroll
+    for (int j = 0; j < kN; ++j) acc[j] = A(0);
+    for (uint32_t rr = 0; rr < at.rows_at_a_time; ++rr) {
+      const uint32_t first = rr * at.cps + t * at.lanes_per_group;
+#pragma unroll 8
+      for (uint32_t c = 0; c < at.lanes_per_group; ++c) {
+#pragma unroll
+        for (int j = 0; j < kN; ++j) acc[j] += part[j][first + c];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kN; ++j) total[j][t] = acc[j];
+  }
+  __syncthreads();
+}
+
+constexpr int kSliceWaves = kSliceThreads / kWaveSize;
+
+// How the K partial pairs of a group become its total pair, by one wavefront:
+// lane l folds the pairs of slices l, l + 64, ... into its state one after the
+// other, then the lanes' states are merged pairwise (lane l with lane l ^ 1,
+// l ^ 2, ...). A merge gives the same bits whichever side it is computed from,
+// so every lane ends with the same state. Contraction is off so that the
+// combiner and the repair launch, which reach this code through different
+// callers, round alike.
+struct CombineMoments {  // partials (mean, sum of squared deviations) -> (mean, rsig)
+  template <typename A>
+  struct State {
+    A n, mean, m2;  // elements so far, their mean, their squared deviations from it
+  };
+  template <typename A>
+  static __device__ __forceinline__ State<A> of(const SampleSlices& d, uint32_t q, A a, A b) {
+    return {A(min(d.rows, d.S - q * d.rows) * d.D), a, b};
+  }
+  template <typename A>
+  static __device__ __forceinline__ void merge(State<A>& s, const State<A>& o) {
+#pragma clang fp contract(off)
+    const A n = s.n + o.n;
+    const A ws = s.n * s.mean, wo = o.n * o.mean;
+    const A mean = n > A(0) ? (ws + wo) / n : A(0);
+    const A ds = s.mean - mean, dso = o.mean - mean;
+    const A bs = s.n * ds, bo = o.n * dso;
+    const A between = bs * ds + bo * dso;
+    s.m2 = (s.m2 + o.m2) + between;
+    s.mean = mean;
+    s.n = n;
+  }
+  template <typename A>
+  static __device__ __forceinline__ State<A> shuffled(const State<A>& s, int o) {
+    return {__shfl_xor(s.n, o, kWaveSize), __shfl_xor(s.mean, o, kWaveSize),
+            __shfl_xor(s.m2, o, kWaveSize)};
+  }
+  template <typename A>
+  static __device__ __forceinline__ void finish(const State<A>& s, const A eps, A& o0, A& o1) {
+#pragma clang fp contract(off)
+    o0 = s.mean;
+    o1 = acc_rsqrt_exact(s.m2 / s.n + eps);
+  }
+};
+
+template <typename A>
+struct SliceLds {
+  A part[2][kSliceThreads];
+  A total[2][kSliceThreads];
+};
+
+__device__ __forceinline__ void slice_flag(const SampleSlices& d, uint32_t w) {
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(d.flags + w, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d.flags + d.items, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (d.gave_up_count) {
+      __hip_atomic_fetch_add(d.gave_up_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// One wavefront: the K partial pairs of group g of sample n, then its totals in
+// every lane. false (the same in every lane): a pair was still unset.
+template <typename Combine, typename A>
+__device__ __forceinline__ bool slice_group_totals(const SampleSlices& d, const A* partials,
+                                                   uint32_t n, uint32_t g, uint32_t patience,
+                                                   const A eps, A& o0, A& o1) {
+  const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+  const A* pairs = partials + (static_cast<size_t>(n) * d.K * d.G + g) * 2;
+  typename Combine::template State<A> st{};
+  int gave_up = 0;
+  for (uint32_t q0 = lane; q0 < d.K; q0 += 4 * kWaveSize) {
+    // a first look at up to four pairs at once, then each is waited for in turn
+    unsigned long long u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t q = q0 + j * kWaveSize;
+      u[j] = q < d.K ? peek_pair(pairs + static_cast<size_t>(q) * d.G * 2) : 0ull;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t q = q0 + j * kWaveSize;
+      if (q < d.K) {
+        A a, b;
+        if (!await_pair(pairs + static_cast<size_t>(q) * d.G * 2, patience, u[j], a, b)) gave_up = 1;
+        Combine::merge(st, Combine::of(d, q, a, b));
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 1; o < kWaveSize; o <<= 1) Combine::merge(st, Combine::shuffled(st, o));
+  Combine::finish(st, eps, o0, o1);
+  return !__any(gave_up);
+}
+
+// Step 1 for item w: the owner threads (t < G) publish the item's G partial pairs.
+template <typename A>
+__device__ __forceinline__ void slice_publish(const SampleSlices& d, uint32_t w, const A pa,
+                                              const A pb, A* exchange) {
+  const uint32_t t = threadIdx.x;
+  if (t < d.G) publish_pair(exchange + (static_cast<size_t>(w) * d.G + t) * 2, pa, pb);
+}
+
+// Steps 2 and 3 for item w. Afterwards lds.total[0 / 1][g] hold group g's total
+// pair in every thread's view; out0 / out1 (per (n, g)) have been written for
+// the groups this slice combines. false (for the whole workgroup): a wait ran
+// out and the item has been flagged. kRepair: nothing is published or waited
+// for.
+template <typename Combine, bool kRepair, typename A>
+__device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceItem& it, uint32_t w,
+                                             const A eps, A* exchange, A* out0, A* out1,
+                                             SliceLds<A>& lds) {
+  const uint32_t t = threadIdx.x;
+  const uint32_t wave = t / kWaveSize, lane = t & (kWaveSize - 1);
+  A* partials = exchange;
+  A* totals = exchange + static_cast<size_t>(d.items) * d.G * 2;
+  if constexpr (kRepair) {
+    for (uint32_t g = wave; g < d.G; g += kSliceWaves) {
+      A o0, o1;
+      (void)slice_group_totals<Combine>(d, partials, it.n, g, 1u, eps, o0, o1);
+      if (lane == 0) {
+        lds.total[0][g] = o0, lds.total[1][g] = o1;
+        if (g % d.K == it.k) {
+          out0[static_cast<size_t>(it.n) * d.G + g] = o0;
+          out1[static_cast<size_t>(it.n) * d.G + g] = o1;
+        }
+      }
+    }
+    __syncthreads();
+    return true;
+  } else {
+    // the groups this slice combines: k, k + K, ..., a wavefront each
+    int gave_up = 0;
+    for (uint32_t g = it.k + wave * d.K; g < d.G; g += kSliceWaves * d.K) {
+      A o0, o1;
+      if (!slice_group_totals<Combine>(d, partials, it.n, g, d.patience, eps, o0, o1)) {
+        gave_up = 1;  // the group's totals stay unset: every slice of the sample will be flagged
+      } else if (lane == 0) {
+        publish_pair(totals + (static_cast<size_t>(it.n) * d.G + g) * 2, o0, o1);
+        out0[static_cast<size_t>(it.n) * d.G + g] = o0;
+        out1[static_cast<size_t>(it.n) * d.G + g] = o1;
+      }
+    }
+    if (t < d.G) {
+      A a, b;
+      if (!await_pair(totals + (static_cast<size_t>(it.n) * d.G + t) * 2, d.patience, a, b)) {
+        gave_up = 1;
+      }
+      lds.total[0][t] = a, lds.total[1][t] = b;
+    }
+    if (__syncthreads_or(gave_up)) {
+      slice_flag(d, w);
+      return false;
+    }
+    return true;
+  }
+}
+
+// ---------------------------------------------------------------- forward
+// The slice's share of each group: its mean, then its squared deviations from
+// that mean; the owner threads publish them.
+template <typename T, int kVPT>
+__device__ __forceinline__ void slice_forward_stats(
+    const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w,
+    typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const SliceItem it(d, w);
+  const uint32_t t = threadIdx.x;
+  const A inv_cnt = A(1) / A(it.nrows * d.D);
+  A s[1] = {A(0)};
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) {
+    if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+      A v[kVec];
+      IO<T>::unpack(raw[i], v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) s[0] += v[e];
+    }
+  }
+  slice_group_sums<1, kVec>(d, at, s, lds.part, lds.total);
+  A pa = A(0), pb = A(0);
+  if (t < d.G) pa = lds.total[0][t] * inv_cnt;
+  const A mean_k = lds.total[0][at.g] * inv_cnt;
+  // convert the packets again in each pass instead of keeping every converted element
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
+  s[0] = A(0);
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) {
+    if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+      A v[kVec];
+      IO<T>::unpack(raw[i], v);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        const A dv = v[e] - mean_k;
+        s[0] += dv * dv;
+      }
+    }
+  }
+  slice_group_sums<1, kVec>(d, at, s, lds.part, lds.total);
+  if (t < d.G) pb = lds.total[0][t];
+#pragma unroll
+  for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
+  slice_publish(d, w, pa, pb, exchange);
+}
+
+// Totals of item w, its rows out of `raw`, and item `reload` (if below d.items) into `raw`.
+template <typename T, int kVPT, bool kRepair>
+__device__ __forceinline__ void slice_forward_finish(
+    const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w, uint32_t reload,
+    const typename IO<T>::Acc eps, const T* x, const typename IO<T>::Acc* gamma,
+    const typename IO<T>::Acc* beta, typename IO<T>::Acc* mu, typename IO<T>::Acc* rsig, T* y,
+    typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds) {
+  using A = typename IO<T>::Acc;
+  constexpr int kVec = IO<T>::kVec;
+  const SliceItem it(d, w);
+  const bool complete = slice_totals<CombineMoments, kRepair>(d, it, w, eps, exchange, mu, rsig, lds);
+  const A mean = lds.total[0][at.g], rs = lds.total[1][at.g];
+  const bool more = !kRepair && reload < d.items;  // uniform over the workgroup
+  const SliceItem nit(d, more ? reload : w);
+  const uint32_t first = slice_first(d, at, it), step = at.rows_at_a_time * d.C;
+  const uint32_t nfirst = slice_first(d, at, nit);
+  if (complete) {
+    // The thread's channels are the same for every item, but their parameters are
+    // fetched per item so that they do not occupy registers while the slice is reduced.
+    const A* gp = gamma + (at.on ? at.cp * kVec : 0u);
+    const A* bp = beta + (at.on ? at.cp * kVec : 0u);
+    asm volatile("" : "+v"(gp), "+v"(bp));
+    A gam[kVec], bet[kVec];
+    load_params_ragged<kVec>(gp, kVec, gam);
+    load_params_ragged<kVec>(bp, kVec, bet);
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) gam[e] *= rs;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+      if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+        A v[kVec];
+        IO<T>::unpack(raw[i], v);
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam[e] + bet[e];
+        store_packet(y + (first + i * step), IO<T>::pack(v));
+      }
+      if (more) {
+        const bool has = at.on && at.r + i * at.rows_at_a_time < nit.nrows;
+        raw[i] = load_packet(x + (has ? nfirst + i * step : 0u));
+      }
+    }
+  } else if (more) {
+    slice_load<T, kVPT>(d, at, nit, x, raw);
+  }
+}
+
+// One item at a time per workgroup; the next item's packets are requested while
+// this one's are stored.
+template <typename T, int kVPT, int kWGs>
+__global__ __launch_bounds__(kSliceThreads, kWGs) void group_norm_nhwc_slices(
+    const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y, typename IO<T>::Acc* __restrict__ exchange) {
+  using A = typename IO<T>::Acc;
+  __shared__ SliceLds<A> lds;
+  const SliceSeat<IO<T>::kVec> at(d);
+  const uint32_t step = gridDim.x;
+  uint32_t w = blockIdx.x;
+  u32x4 one[kVPT];
+  if (w < d.items) slice_load<T, kVPT>(d, at, SliceItem(d, w), x, one);
+  for (; w < d.items; w += step) {
+    slice_forward_stats<T, kVPT>(d, at, w, exchange, one, lds);
+    slice_forward_finish<T, kVPT, false>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig, y,
+                                         exchange, one, lds);
+  }
+}
+
+// The launch behind it: nothing to do unless a wait of the first launch ran out.
+template <typename T, int kVPT>
+__global__ __launch_bounds__(kSliceThreads, 4) void group_norm_nhwc_slices_repair(
+    const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
+    const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
+    typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
+    T* __restrict__ y, typename IO<T>::Acc* __restrict__ exchange) {
+  using A = typename IO<T>::Acc;
+  __shared__ SliceLds<A> lds;
+  if (d.flags[d.items] == 0u) return;
+  const SliceSeat<IO<T>::kVec> at(d);
+  for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
+    if (d.flags[w] == 0u) continue;  // the same word in every thread
+    u32x4 raw[kVPT];
+    slice_load<T, kVPT>(d, at, SliceItem(d, w), x, raw);
+    slice_forward_finish<T, kVPT, true>(d, at, w, d.items, eps, x, gamma, beta, mu, rsig, y,
+                                        exchange, raw, lds);
+    __syncthreads();  // the next item rewrites the totals in LDS
+  }
+}
+
+// ---------------------------------------------------------------- host
+constexpr unsigned kSliceRepairGrid = 256;
+
+// The most workgroups the kernel is launched with.
+inline uint32_t sample_slices_max_grid() { return static_cast<uint32_t>(num_cus()) * 4u; }
+
+template <typename A>
+inline void fill_sample_exchange(A* exchange, const SampleSlices& d, hipStream_t stream) {
+  using Bits = typename Unset<A>::Bits;
+  const size_t words = sample_slices_exchange_words(d.N, d.G, d.K);
+  const uint32_t n = static_cast<uint32_t>(words), nflags = d.items + 1;
+  const uint32_t most = n > nflags ? n : nflags;
+  hipLaunchKernelGGL((fill_exchange<Bits>), dim3(static_cast<unsigned>(ceil_div(most, 256))),
+                     dim3(256), 0, stream, reinterpret_cast<Bits*>(exchange), n, Unset<A>::kValue,
+                     d.flags, nflags);
+}
+
+// DRAGON_HIP_OK when the kernels were launched, kNotApplicable when the shape
+// or the addresses leave the call to the other paths. `scratch` holds
+// sample_slices_exchange_bytes(...) bytes.
+template <typename T>
+int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, uint32_t D,
+                                       float eps, const void* x, const void* gamma, const void* beta,
+                                       void* mu, void* rsig, void* y, void* scratch,
+                                       size_t scratch_bytes, hipStream_t stream) {
+  using A = typename IO<T>::Acc;
+  if constexpr (sizeof(T) > 4) {
+    return kNotApplicable;
+  } else {
+    const SampleSlicePlan p = plan_sample_slices<T>(S, C, G, D);
+    if (!p.ok || !aligned16(x) || !aligned16(y)) return kNotApplicable;
+    if (static_cast<uint64_t>(N) * p.K * G * 2 + static_cast<uint64_t>(N) * G * 2 > 0x7fffffffull) {
+      return kNotApplicable;
+    }
+    if (!scratch || scratch_bytes < sample_slices_exchange_bytes(N, G, p.K, sizeof(A))) {
+      return kNotApplicable;
+    }
+    A* exchange = static_cast<A*>(scratch);
+    const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
+#define LAUNCH(VPT, WGS)                                                                          \
+  {                                                                                               \
+    auto kernel = group_norm_nhwc_slices<T, VPT, WGS>;                                                 \
+    unsigned cap = resident_grid(kernel, kSliceThreads, 0);                                       \
+    if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
+    if (p.K > cap) return kNotApplicable;                                                         \
+    note_flavour("group_norm_nhwc_slices<" #VPT "," #WGS ">");                                             \
+    note_number("slices", p.K);                                                                   \
+    fill_sample_exchange(exchange, d, stream);                                                    \
+    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0,       \
+                       stream, d, A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma), \
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),   \
+                       static_cast<T*>(y), exchange);                                             \
+  }
+    if (p.vpt <= 8) LAUNCH(8, 4) else LAUNCH(16, 3)
+#undef LAUNCH
+    hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, 16>),
+                       dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),
+                       dim3(kSliceThreads), 0, stream, d, A(eps), static_cast<const T*>(x),
+                       static_cast<const A*>(gamma), static_cast<const A*>(beta),
+                       static_cast<A*>(mu), static_cast<A*>(rsig), static_cast<T*>(y), exchange);
+    return status_of_launch();
+  }
+}
+
+} // namespace dragon_hip

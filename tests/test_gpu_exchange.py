@@ -74,6 +74,18 @@ def _gn_backward(K, t):
     return [dx, dg, db, params]
 
 
+def _gn_nhwc_forward(K, t, in_place=False):
+    import torch
+    N, S, G, D = 3, 48 * 48, 32, 8  # samples of 1.1 MiB in bf16: 18 slices, fewer than groups
+    x = t.setdefault("x", (torch.randn((N, S, G * D), device="cuda") + 0.3).to(torch.bfloat16))
+    g = t.setdefault("g", torch.rand(G * D, device="cuda") + 0.5)
+    b = t.setdefault("b", torch.randn(G * D, device="cuda") * 0.1)
+    mu, rsig = torch.full((N * G,), -7.0, device="cuda"), torch.full((N * G,), -7.0, device="cuda")
+    y = x.clone() if in_place else torch.full_like(x, -7.0)
+    K.group_norm_forward(N, G, D, S, "NHWC", 1e-5, y if in_place else x, g, b, mu, rsig, y)
+    return [y, mu, rsig]
+
+
 def _softmax_in_place(K, t, log=False, dtype="float32"):
     import torch
     N, C = 6, 131072
@@ -101,6 +113,9 @@ CALLS = {
     "batch_norm_training_backward_57x57": lambda K, t: _bn_backward(K, t, S=57 * 57),
     "group_norm_forward": _gn_forward,
     "group_norm_grad": _gn_backward,
+    # NHWC samples in slices: G pairs per slice, totals formed by one slice per group
+    "group_norm_forward_nhwc": _gn_nhwc_forward,
+    "group_norm_forward_nhwc_in_place": lambda K, t: _gn_nhwc_forward(K, t, in_place=True),
     "softmax_in_place": _softmax_in_place,
     "log_softmax_in_place": lambda K, t: _softmax_in_place(K, t, log=True),
     "softmax_bf16_in_place": lambda K, t: _softmax_in_place(K, t, dtype="bfloat16"),

@@ -533,6 +533,11 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # the same with groups of 10 and 12 channels: a packet of the fused NHWC forward
             # lies in two groups
             ((2, 7, 7, 320), -1, 32), ((3, 6, 5, 96), -1, 8), ((5, 9, 9, 160), -1, 16),
+            # NHWC samples beyond one workgroup's registers: slices of whole rows that exchange
+            # their groups' sums (8 to 32 slices per sample; a ragged last slice and idle
+            # threads; fewer slices than groups and more; more items than workgroups)
+            ((2, 64, 64, 64), -1, 8), ((3, 40, 41, 96), -1, 4), ((1, 48, 48, 256), -1, 32),
+            ((70, 48, 48, 64), -1, 8),
             # groups of half a packet (the column-reduction structure)
             ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32),
             # small groups, a wavefront each in the fused backward: more channels per group
