@@ -417,7 +417,10 @@ int dragon_hip_batch_norm_training_forward_noalloc(int dtype, int64_t N, int64_t
  * interest first.
  * dragon_hip_exchange_reset: clears that count and sets how many polls (of
  * about a microsecond) a wait lasts in later launches from any thread; 0 = the
- * default (about a second).
+ * default (about a second). It is a hook for tests that force the repair
+ * launch: the setting is process-wide, so a process that serves traffic only
+ * ever passes 0 (a small value is still correct, every flagged slice is
+ * repaired, but each repaired slice is read twice).
  * dragon_hip_exchange_plan: how the path would cut `units` reduction units,
  * each `nseg` runs of `seglen` contiguous elements, with `tensors` (1 or 2)
  * tensors held in registers: returns 1 and fills slices (per unit),
