@@ -206,14 +206,14 @@ def wl_layer_norm(N, C, dtype_name, seed, backward=True, outliers=False, k=0):
     return kernels, {"rows": N, "width": C}
 
 
-def wl_group_norm(shape, G, dtype_name, seed=3, k=0):
+def wl_group_norm(shape, G, dtype_name, seed=3, k=0, layout="NCHW"):
     import torch
     from dragon_amd import kernels as K
     dtype = getattr(torch, dtype_name)
     gen = _gen(seed + 1000 * k)
-    N, C = shape[0], shape[1]
+    N, C = shape[0], shape[1] if layout == "NCHW" else shape[-1]
     S = 1
-    for d in shape[2:]:
+    for d in (shape[2:] if layout == "NCHW" else shape[1:-1]):
         S *= d
     D = C // G
     x = _randn(shape, dtype, gen)
@@ -226,13 +226,13 @@ def wl_group_norm(shape, G, dtype_name, seed=3, k=0):
     nbytes = x.numel() * x.element_size()
     kernels = [
         ("group_norm_forward",
-         lambda: K.group_norm_forward(N, G, D, S, "NCHW", 1e-5, x, g, b, mu, rsig, y), 2 * nbytes,
+         lambda: K.group_norm_forward(N, G, D, S, layout, 1e-5, x, g, b, mu, rsig, y), 2 * nbytes,
          "1:1"),
         ("group_norm_grad",
-         lambda: K.group_norm_grad(N, G, D, S, "NCHW", x, mu, rsig, g, dy, params, params, dg, db, dx),
+         lambda: K.group_norm_grad(N, G, D, S, layout, x, mu, rsig, g, dy, params, params, dg, db, dx),
          3 * nbytes, "2:1"),
     ]
-    return kernels, {"shape": list(shape), "groups": G}
+    return kernels, {"shape": list(shape), "groups": G, "layout": layout}
 
 
 def wl_batch_norm(shape, dtype_name, seed=2, k=0):
@@ -295,6 +295,9 @@ WORKLOADS = {
     "batch_norm_f32_64x256x57x57": lambda k: wl_batch_norm((64, 256, 57, 57), "float32", 2, k=k),
     # a vocabulary whose rows are not whole 16-byte packets
     "softmax_bf16_4096x50257": lambda k: wl_softmax((4096, 50257), "bfloat16", 1, k=k),
+    # the BASELINE GroupNorm tensor channels-last: samples of 4 MB cut into slices of rows
+    "group_norm_bf16_32x64x64x512_g32_nhwc": lambda k: wl_group_norm((32, 64, 64, 512), 32, "bfloat16", 3,
+                                                                     k=k, layout="NHWC"),
 }
 
 

@@ -54,6 +54,7 @@
 namespace dragon_hip {
 
 constexpr int kSliceThreads = 256;
+constexpr int kSlicePackets = 16;  // per thread: a slice is up to 64 KB
 constexpr uint32_t kMaxSampleSlices = 1024;  // slices per sample (a resident grid holds no more workgroups)
 constexpr uint32_t kMaxSampleGroups = 256;  // groups: one owner thread each
 
@@ -73,8 +74,7 @@ struct SampleSlicePlan {
   int vpt;  // packets per thread and tensor
 };
 
-// Up to 16 packets per thread, three workgroups per compute unit (four for
-// slices of half that size).
+// Up to 16 packets per thread, three workgroups per compute unit.
 template <typename T>
 SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
   constexpr uint32_t kVec = IO<T>::kVec;
@@ -85,7 +85,7 @@ SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t 
   const uint32_t rows_at_a_time = kSliceThreads / cps;
   // most of the workgroup's threads must have a row to hold
   if (cps * rows_at_a_time * 4 < kSliceThreads * 3) return p;
-  const uint32_t vmax = 16u;
+  const uint32_t vmax = kSlicePackets;
   const uint32_t k0 = static_cast<uint32_t>(ceil_div(S, rows_at_a_time * vmax));
   // slices of about the same size
   const uint32_t vpt = static_cast<uint32_t>(ceil_div(ceil_div(S, k0), rows_at_a_time));
@@ -527,7 +527,7 @@ __global__ __launch_bounds__(kSliceThreads, 4) void group_norm_nhwc_slices_repai
 constexpr unsigned kSliceRepairGrid = 256;
 
 // The most workgroups the kernel is launched with.
-inline uint32_t sample_slices_max_grid() { return static_cast<uint32_t>(num_cus()) * 4u; }
+inline uint32_t sample_slices_max_grid() { return static_cast<uint32_t>(num_cus()) * 3u; }
 
 template <typename A>
 inline void fill_sample_exchange(A* exchange, const SampleSlices& d, hipStream_t stream) {
@@ -562,23 +562,20 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     }
     A* exchange = static_cast<A*>(scratch);
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-#define LAUNCH(VPT, WGS)                                                                          \
-  {                                                                                               \
-    auto kernel = group_norm_nhwc_slices<T, VPT, WGS>;                                                 \
-    unsigned cap = resident_grid(kernel, kSliceThreads, 0);                                       \
-    if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
-    if (p.K > cap) return kNotApplicable;                                                         \
-    note_flavour("group_norm_nhwc_slices<" #VPT "," #WGS ">");                                             \
-    note_number("slices", p.K);                                                                   \
-    fill_sample_exchange(exchange, d, stream);                                                    \
-    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0,       \
-                       stream, d, A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma), \
-                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),   \
-                       static_cast<T*>(y), exchange);                                             \
-  }
-    if (p.vpt <= 8) LAUNCH(8, 4) else LAUNCH(16, 3)
-#undef LAUNCH
-    hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, 16>),
+    // One flavour: a sample of up to eight packets per thread is at most 32 KB, which the
+    // one-workgroup-per-sample kernel takes before this one is asked.
+    auto kernel = group_norm_nhwc_slices<T, kSlicePackets, 3>;
+    unsigned cap = resident_grid(kernel, kSliceThreads, 0);
+    if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();
+    if (p.K > cap) return kNotApplicable;
+    note_flavour("group_norm_nhwc_slices<16,3>");
+    note_number("slices", p.K);
+    fill_sample_exchange(exchange, d, stream);
+    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0, stream, d,
+                       A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma),
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),
+                       static_cast<T*>(y), exchange);
+    hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets>),
                        dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),
                        dim3(kSliceThreads), 0, stream, d, A(eps), static_cast<const T*>(x),
                        static_cast<const A*>(gamma), static_cast<const A*>(beta),

@@ -48,4 +48,5 @@ CASES = {
     "softmax_f32_2048x128256": _rows("softmax", "softmax_grad", 2048, 128256, "float32"),
     "batch_norm_f32_64x256x57x57": _bn(64, 256, 57 * 57, "float32"),
     "softmax_bf16_4096x50257": _rows("softmax", "softmax_grad", 4096, 50257, "bfloat16"),
+    "group_norm_bf16_32x64x64x512_g32_nhwc": _gn(32, 32, 16, 64 * 64, "bfloat16", "NHWC"),
 }

@@ -320,3 +320,44 @@ def test_batch_norm_64x256x57x57_sampled_channels_and_every_channel(K, dtype):
     assert U.normwise(U.widen(dxg, dtype), dx_ref) <= max(tol, 1e-4)
     assert U.normwise(U.to_host(wg[:C][idx]), dg_ref) <= 1e-4
     assert U.normwise(U.to_host(wg[C:][idx]), db_ref) <= 1e-4
+
+
+def test_group_norm_nhwc_32x64x64x512_sampled_samples_and_every_group(K):
+    """The channels-last GroupNorm tensor of the sweep: 32 samples of 4 MB, 64 slices of rows
+    each, more work items than resident workgroups. Two samples against the oracle; every
+    group's statistics against fp64 on the device; every element of y against the defining
+    formula in fp32 on the device."""
+    import torch
+    N, S, G, D = 32, 64 * 64, 32, 16
+    C = G * D
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = (torch.empty((N, S, C), device="cuda").normal_(generator=gen) + 0.3).to(torch.bfloat16)
+    g = torch.empty(C, device="cuda").uniform_(0.5, 1.5, generator=gen)
+    b = torch.empty(C, device="cuda").normal_(generator=gen).mul_(0.1)
+    mu, rsig = torch.empty(N * G, device="cuda"), torch.empty(N * G, device="cuda")
+    y = torch.empty_like(x)
+    K.group_norm_forward(N, G, D, S, "NHWC", 1e-5, x, g, b, mu, rsig, y)
+    torch.cuda.synchronize()
+    assert K.exchange_timed_out() == 0
+    xg = x.double().reshape(N, S, G, D)
+    mean64 = xg.mean((1, 3))
+    rs64 = torch.rsqrt(xg.var((1, 3), unbiased=False) + float(np.float32(1e-5)))
+    assert float((mu.reshape(N, G).double() - mean64).abs().max()) <= 1e-5
+    assert float((rsig.reshape(N, G).double() / rs64 - 1).abs().max()) <= 1e-5
+    want = ((x.float().reshape(N, S, G, D) - mu.reshape(N, 1, G, 1)) * rsig.reshape(N, 1, G, 1)
+            ).reshape(N, S, C) * g + b
+    err = (y.float() - want).abs().max()
+    assert float(err) <= 2 ** -7 * float(want.abs().max())  # one bf16 rounding of the result
+    for n in (0, N - 1):
+        xb = U.to_host(x[n].contiguous())
+        y_ref, mu_ref, rsig_ref = R.op_group_norm("bfloat16", xb.reshape(1, S, C), U.to_host(g),
+                                                  U.to_host(b), -1, G, 1e-5)
+        # the oracle's sequential fp32 sums over 65536 elements are themselves a few 1e-5 off
+        # fp64: three-way, as for the other long reductions
+        rs_n = rs64[n].cpu().numpy()
+        oracle_off = np.max(np.abs(rsig_ref / rs_n - 1))
+        assert U.normwise(U.to_host(mu[n * G:(n + 1) * G]), mu_ref) <= 1e-5 + oracle_off
+        assert np.max(np.abs(U.to_host(rsig[n * G:(n + 1) * G]) / rsig_ref - 1)) <= 1e-5 + oracle_off
+        assert U.normwise(U.widen(U.to_host(y[n].contiguous()), "bfloat16").ravel(),
+                          np.asarray(U.widen(y_ref, "bfloat16")).ravel()) <= U.TIGHT["bfloat16"]
+

@@ -231,6 +231,47 @@ def test_group_norm_shapes(K, N, G, D, S, fmt, dtype, seed):
     assert _untouched(dxbuf, dtype, 0, n)
 
 
+# NHWC samples cut into slices of whole rows: one row at a time per workgroup and many, idle
+# threads (C / packet does not divide 256), a last slice of fewer rows than a workgroup holds at
+# a time, fewer and more slices than groups, more items than resident workgroups, one group,
+# x at an address that is not 16-byte aligned (another path, same answer), in place.
+NHWC_SLICE_CASES = [
+    (1, 1, 8, 70001, "bfloat16", 0), (2, 4, 48, 1537, "float32", 0), (1, 200, 8, 301, "bfloat16", 0),
+    (3, 25, 8, 2049, "float16", 0), (1, 256, 8, 700, "bfloat16", 0), (40, 8, 16, 2304, "float32", 0),
+    (2, 32, 16, 4097, "bfloat16", 0), (2, 32, 16, 4097, "bfloat16", 3), (5, 3, 8, 6000, "float16", 0),
+    (2, 2, 256, 1030, "float32", 0), (1, 64, 4, 3000, "float32", 0), (2, 16, 24, 999, "bfloat16", 0),
+]
+
+
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("N,G,D,S,dtype,shift", NHWC_SLICE_CASES)
+def test_group_norm_forward_nhwc_slice_shapes(K, N, G, D, S, dtype, shift, in_place):
+    import torch
+    rng = np.random.default_rng(7000 + G * D + S)
+    C = G * D
+    n = N * C * S
+    xb, xs = _values(rng, (n,), dtype, 2.0)
+    xs = xs + 0.0
+    x = xs.reshape(N, S, G, D)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    eps = 1e-5
+    mean = x.mean((1, 3))
+    rs = 1 / np.sqrt(((x - mean[:, None, :, None]) ** 2).mean((1, 3)) + np.float64(np.float32(eps)))
+    y_ref = ((x - mean[:, None, :, None]) * rs[:, None, :, None]).reshape(N, S, C) * g + b
+    xbuf, xd = _held(n, dtype, shift, xb)
+    ybuf, yd = (xbuf, xd) if in_place else _held(n, dtype, shift)
+    gd, bd = torch.from_numpy(g).cuda(), torch.from_numpy(b).cuda()
+    mu, rsig = torch.empty(N * G, device="cuda"), torch.empty(N * G, device="cuda")
+    K.group_norm_forward(N, G, D, S, "NHWC", eps, xd, gd, bd, mu, rsig, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, S, C)
+    assert _mean_ok(mu.cpu().numpy(), mean, x)
+    assert np.max(np.abs(rsig.cpu().numpy().astype(np.float64) / rs.ravel() - 1)) <= 5e-5
+    assert U.normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, shift, n)
+    assert K.exchange_timed_out() == 0
+
+
 @pytest.mark.parametrize("N,G,D,S,fmt,dtype,seed", _channel_cases(40, 5))
 def test_batch_norm_training_shapes(K, N, G, D, S, fmt, dtype, seed):
     import torch

@@ -16,9 +16,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 with open(os.path.join(ROOT, "tests", "golden", "plan_names.json")) as f:
     GOLDEN = json.load(f)
 
-# kernels of the multi-pass general paths: none of the pinned shapes may take them
+# kernels of the multi-pass general paths: none of the pinned shapes may take them ...
 FALLBACKS = ("map_flat", "reduce2_", "_looped", "channel_pair_sums", "group_grad_from_channel_sums",
              "layer_norm_wide_row_sums", "softmax_columns", "reduce_gather")
+# ... except where the multi-pass path was measured to be the faster one: the backward of
+# channels-last GroupNorm samples beyond one workgroup (five passes; the sliced form was slower)
+MULTI_PASS_BY_CHOICE = {("group_norm_bf16_32x64x64x512_g32_nhwc", "group_norm_grad")}
 
 
 def _key(op, dt, dims, layout):
@@ -32,6 +35,9 @@ def test_routing_is_the_pinned_one(workload):
         text = K.plan_name(op, dt, dims, layout)
         assert text, (workload, op)
         assert text == GOLDEN[workload][_key(op, dt, dims, layout)], (workload, op, text)
+        if (workload, op) in MULTI_PASS_BY_CHOICE:
+            assert any(name in text for name in FALLBACKS), (workload, op, text)
+            continue
         for name in FALLBACKS:
             assert name not in text, (workload, op, text)
 
