@@ -2,6 +2,7 @@
 // that a host-side HIPContext needs no HIP header. Mirrors what Dragon's device
 // contexts provide (dragon/core/context_cuda.h:156-332).
 #include "common.h"
+#include "dragon_hip_testing.h"
 
 namespace {
 inline int st(hipError_t e) { return e == hipSuccess ? DRAGON_HIP_OK : static_cast<int>(e); }

@@ -415,12 +415,8 @@ int dragon_hip_batch_norm_training_forward_noalloc(int dtype, int64_t N, int64_t
  * be finished that way since the last reset (a diagnostic; copies one word from
  * the device, so it waits for the null stream). Synchronise the streams of
  * interest first.
- * dragon_hip_exchange_reset: clears that count and sets how many polls (of
- * about a microsecond) a wait lasts in later launches from any thread; 0 = the
- * default (about a second). It is a hook for tests that force the repair
- * launch: the setting is process-wide, so a process that serves traffic only
- * ever passes 0 (a small value is still correct, every flagged slice is
- * repaired, but each repaired slice is read twice).
+ * (The count is cleared, and the length of the wait set, by the test hook
+ * dragon_hip_exchange_reset, declared apart in dragon_hip_testing.h.)
  * dragon_hip_exchange_plan: how the path would cut `units` reduction units,
  * each `nseg` runs of `seglen` contiguous elements, with `tensors` (1 or 2)
  * tensors held in registers: returns 1 and fills slices (per unit),
@@ -428,7 +424,6 @@ int dragon_hip_batch_norm_training_forward_noalloc(int dtype, int64_t N, int64_t
  * workgroups it asks for; a unit never has more slices than that), or returns
  * 0 when the shape is left to the split path. */
 int dragon_hip_exchange_timed_out(void);
-void dragon_hip_exchange_reset(unsigned patience);
 int dragon_hip_exchange_plan(int dtype, int64_t units, int64_t nseg, int64_t seglen, int tensors,
                              int* slices, int* slice_packets, int* packets_per_thread, int* grid);
 

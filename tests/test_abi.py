@@ -1,4 +1,5 @@
-"""The C-ABI library builds, loads, and exports exactly what include/dragon_hip.h declares.
+"""The C-ABI library builds, loads, and exports exactly what the headers under include/ declare
+(dragon_hip.h, the boundary, and dragon_hip_testing.h, the hooks that exist for tests).
 
 Runs without a GPU: no compute entry point is called."""
 
@@ -14,9 +15,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "dragon_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(dragon_hip_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in ("dragon_hip.h", "dragon_hip_testing.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(dragon_hip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 @pytest.fixture(scope="module")
