@@ -168,7 +168,6 @@ __device__ __forceinline__ unsigned long long pair_bits(const float a, const flo
   return static_cast<unsigned long long>(publishable_bits(a)) |
       (static_cast<unsigned long long>(publishable_bits(b)) << 32);
 }
-constexpr unsigned long long kUnsetPair = ~0ull;
 __device__ __forceinline__ void publish_pair(float* slot, const float a, const float b) {
   __hip_atomic_store(reinterpret_cast<unsigned long long*>(slot), pair_bits(a, b), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
