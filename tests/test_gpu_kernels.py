@@ -858,7 +858,9 @@ def test_batch_norm_special_values_follow_the_reference(K, shape, axis, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape,axis,group", [((4, 8, 8, 8), 1, 4), ((3, 6, 7, 7), 1, 3),
                                               ((5, 4, 150, 150), 1, 2), ((4, 8, 8, 8), -1, 4),
-                                              ((5, 32, 64, 64), 1, 4), ((5, 6, 14, 14), 1, 0)])
+                                              ((5, 32, 64, 64), 1, 4), ((5, 6, 14, 14), 1, 0),
+                                              # channels-last samples cut into slices of rows
+                                              ((5, 48, 48, 64), -1, 8)])
 def test_group_norm_special_values_follow_the_reference(K, shape, axis, group, dtype):
     """Groups that start with -inf, hold +inf or hold nan (group_norm_op.cc's Moments -> InvStd
     -> GroupNorm sequence on the CPU): mu, rsig and y carry inf / nan in the same places."""
