@@ -151,14 +151,25 @@ __device__ __forceinline__ uint32_t slice_first(const SampleSlices& d, const Sli
   return (it.n * d.S + it.row0 + at.r) * d.C + at.cp * kVec;
 }
 
+// Packet i of a thread exists while i * R < room. The loops over a thread's packets count
+// `room` down and an offset up, one register each: sixteen row numbers and sixteen offsets per
+// thread, which the unrolled loops would otherwise keep across the whole item loop, do not fit.
+template <int kVec>
+__device__ __forceinline__ int slice_room(const SliceSeat<kVec>& at, const SliceItem& it) {
+  return at.on ? static_cast<int>(it.nrows) - static_cast<int>(at.r) : 0;
+}
+
 template <typename T, int kVPT>
 __device__ __forceinline__ void slice_load(const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at,
                                            const SliceItem& it, const T* in, u32x4 (&raw)[kVPT]) {
-  const uint32_t first = slice_first(d, at, it), step = at.rows_at_a_time * d.C;
+  const uint32_t step = at.rows_at_a_time * d.C;
+  int room = slice_room(at, it);
+  uint32_t off = slice_first(d, at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
-    const bool has = at.on && at.r + i * at.rows_at_a_time < it.nrows;
-    raw[i] = load_packet(in + (has ? first + i * step : 0u));
+    raw[i] = load_packet(in + (room > 0 ? off : 0u));
+    room -= static_cast<int>(at.rows_at_a_time), off += step;
+    asm volatile("" : "+v"(room), "+v"(off));
   }
 }
 
@@ -397,9 +408,13 @@ __device__ __forceinline__ void slice_forward_stats(
   const uint32_t t = threadIdx.x;
   const A inv_cnt = A(1) / A(it.nrows * d.D);
   A s[1] = {A(0)};
+  int room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
-    if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+    const bool has = room > 0;
+    room -= static_cast<int>(at.rows_at_a_time);
+    asm volatile("" : "+v"(room));
+    if (has) {
       A v[kVec];
       IO<T>::unpack(raw[i], v);
 #pragma unroll
@@ -414,9 +429,13 @@ __device__ __forceinline__ void slice_forward_stats(
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
   s[0] = A(0);
+  room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
-    if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+    const bool has = room > 0;
+    room -= static_cast<int>(at.rows_at_a_time);
+    asm volatile("" : "+v"(room));
+    if (has) {
       A v[kVec];
       IO<T>::unpack(raw[i], v);
 #pragma unroll
@@ -460,19 +479,21 @@ __device__ __forceinline__ void slice_forward_finish(
     load_params_ragged<kVec>(bp, kVec, bet);
 #pragma unroll
     for (int e = 0; e < kVec; ++e) gam[e] *= rs;
+    int room = slice_room(at, it), nroom = slice_room(at, nit);
+    uint32_t off = first, noff = nfirst;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
-      if (at.on && at.r + i * at.rows_at_a_time < it.nrows) {
+      if (room > 0) {
         A v[kVec];
         IO<T>::unpack(raw[i], v);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam[e] + bet[e];
-        store_packet(y + (first + i * step), IO<T>::pack(v));
+        store_packet(y + off, IO<T>::pack(v));
       }
-      if (more) {
-        const bool has = at.on && at.r + i * at.rows_at_a_time < nit.nrows;
-        raw[i] = load_packet(x + (has ? nfirst + i * step : 0u));
-      }
+      if (more) raw[i] = load_packet(x + (nroom > 0 ? noff : 0u));
+      room -= static_cast<int>(at.rows_at_a_time), nroom -= static_cast<int>(at.rows_at_a_time);
+      off += step, noff += step;
+      asm volatile("" : "+v"(room), "+v"(nroom), "+v"(off), "+v"(noff));
     }
   } else if (more) {
     slice_load<T, kVPT>(d, at, nit, x, raw);
