@@ -538,6 +538,9 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # threads; fewer slices than groups and more; more items than workgroups)
             ((2, 64, 64, 64), -1, 8), ((3, 40, 41, 96), -1, 4), ((1, 48, 48, 256), -1, 32),
             ((70, 48, 48, 64), -1, 8),
+            # rows of 160 / 320 packets leave too many of a slice workgroup's threads without a
+            # row: the column reductions
+            ((2, 40, 41, 1280), -1, 32),
             # groups of half a packet (the column-reduction structure)
             ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32),
             # small groups, a wavefront each in the fused backward: more channels per group
