@@ -715,9 +715,14 @@ def main():
         # tensor size, measured cold like the kernel itself; no kernel can stream faster
         tensors = 2 if k["mix"] == "1:1" else 3
         probe, shape = probe_ceiling(k["algorithmic_bytes"] / tensors, k["mix"])
-        if k["GB/s"] > probe:  # the probe had a slow moment: ask it again, more often
+        # the probe had a slow moment: ask it again, more often and over as many calls per
+        # repetition as the kernel's own figure averages (it is a best-of, so it can only rise)
+        for reps in (8, 16):
+            if k["GB/s"] <= probe:
+                break
             _probe_cache.pop((max(16, (int(k["algorithmic_bytes"] / tensors) + 15) // 16 * 16), k["mix"]), None)
-            again, again_shape = probe_ceiling(k["algorithmic_bytes"] / tensors, k["mix"], reps=8)
+            again, again_shape = probe_ceiling(k["algorithmic_bytes"] / tensors, k["mix"],
+                                               steps=max(16, args.steps), reps=reps)
             if again > probe:
                 probe, shape = again, again_shape
         k["probe_GB/s"] = probe
