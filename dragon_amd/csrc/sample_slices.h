@@ -34,15 +34,15 @@
 // combiner did not. A flagged item wrote no output, so a call may run in place.
 //
 // Partials are (mean, sum of squared deviations) of the slice's share of the
-// group, formed in two passes over the registers; the combiner merges them with
-// the counts the slice geometry gives. Nothing depends on an element outside
+// group, formed in two passes over the registers; the combiner adds them up with
+// the counts the slice geometry gives (slice_group_moments). Nothing depends on an element outside
 // the slice.
 //
 // Every item pays the two steps of the exchange, about 10 us on MI355X during
-// which its workgroup moves nothing, so the kernel reaches about 4 TB/s where a
+// which its workgroup moves nothing, so the kernel reaches 4-4.7 TB/s where a
 // plain copy reaches 5.5. Measured cold on MI355X against the two-pass path
 // (column statistics, then the map) on tensors of the same size: [32, 64*64,
-// 512] bf16 74 us against 84, fp32 127 against 142; [64, 32*32, 512] bf16 34
+// 512] bf16 65 us against 84, fp32 123 against 141; [64, 32*32, 512] bf16 27.5
 // against 46. A backward built the same way (x and dy in registers, ds / db
 // exchanged) holds half as many rows per item and pays the exchange twice as
 // often: 143 us against 122 for the five-pass path at the first shape, so the
@@ -74,7 +74,7 @@ struct SampleSlicePlan {
   int vpt;  // packets per thread and tensor
 };
 
-// Up to 16 packets per thread, three workgroups per compute unit.
+// Up to 16 packets per thread, four workgroups per compute unit (128 registers).
 template <typename T>
 SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
   constexpr uint32_t kVec = IO<T>::kVec;
@@ -240,47 +240,14 @@ __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const Sl
 
 constexpr int kSliceWaves = kSliceThreads / kWaveSize;
 
-// How the K partial pairs of a group become its total pair, by one wavefront:
-// lane l folds the pairs of slices l, l + 64, ... into its state one after the
-// other, then the lanes' states are merged pairwise (lane l with lane l ^ 1,
-// l ^ 2, ...). A merge gives the same bits whichever side it is computed from,
-// so every lane ends with the same state. Contraction is off so that the
-// combiner and the repair launch, which reach this code through different
-// callers, round alike.
-struct CombineMoments {  // partials (mean, sum of squared deviations) -> (mean, rsig)
-  template <typename A>
-  struct State {
-    A n, mean, m2;  // elements so far, their mean, their squared deviations from it
-  };
-  template <typename A>
-  static __device__ __forceinline__ State<A> of(const SampleSlices& d, uint32_t q, A a, A b) {
-    return {A(min(d.rows, d.S - q * d.rows) * d.D), a, b};
-  }
-  template <typename A>
-  static __device__ __forceinline__ void merge(State<A>& s, const State<A>& o) {
-#pragma clang fp contract(off)
-    const A n = s.n + o.n;
-    const A ws = s.n * s.mean, wo = o.n * o.mean;
-    const A mean = n > A(0) ? (ws + wo) / n : A(0);
-    const A ds = s.mean - mean, dso = o.mean - mean;
-    const A bs = s.n * ds, bo = o.n * dso;
-    const A between = bs * ds + bo * dso;
-    s.m2 = (s.m2 + o.m2) + between;
-    s.mean = mean;
-    s.n = n;
-  }
-  template <typename A>
-  static __device__ __forceinline__ State<A> shuffled(const State<A>& s, int o) {
-    return {__shfl_xor(s.n, o, kWaveSize), __shfl_xor(s.mean, o, kWaveSize),
-            __shfl_xor(s.m2, o, kWaveSize)};
-  }
-  template <typename A>
-  static __device__ __forceinline__ void finish(const State<A>& s, const A eps, A& o0, A& o1) {
-#pragma clang fp contract(off)
-    o0 = s.mean;
-    o1 = acc_rsqrt_exact(s.m2 / s.n + eps);
-  }
-};
+// The sum of v over the wavefront, the same bits in every lane (each step adds
+// the two halves of a pair of lanes, which commutes).
+template <typename A>
+__device__ __forceinline__ A wave_total(A v) {
+#pragma unroll
+  for (int o = 1; o < kWaveSize; o <<= 1) v += __shfl_xor(v, o, kWaveSize);
+  return v;
+}
 
 template <typename A>
 struct SliceLds {
@@ -298,37 +265,44 @@ __device__ __forceinline__ void slice_flag(const SampleSlices& d, uint32_t w) {
   }
 }
 
-// One wavefront: the K partial pairs of group g of sample n, then its totals in
-// every lane. false (the same in every lane): a pair was still unset.
-template <typename Combine, typename A>
-__device__ __forceinline__ bool slice_group_totals(const SampleSlices& d, const A* partials,
-                                                   uint32_t n, uint32_t g, uint32_t patience,
-                                                   const A eps, A& o0, A& o1) {
+// One wavefront: the K partial (mean, squared deviations) pairs of group g of
+// sample n become the group's mean and rsig, the same bits in every lane, with
+// two plain sums: the count-weighted mean of the slices' means, then the slices'
+// squared deviations plus what the distances of their means from the total mean
+// add. Lane l takes slices l, l + 64, ...; it keeps its first pair for the
+// second sum and reads any further ones (K > 64) again. Contraction is off so
+// that the combiner and the repair launch, which reach this code through
+// different callers, round alike. false (the same in every lane): a pair was
+// still unset.
+template <typename A>
+__device__ __forceinline__ bool slice_group_moments(const SampleSlices& d, const A* partials,
+                                                    uint32_t n, uint32_t g, uint32_t patience,
+                                                    const A eps, A& o0, A& o1) {
+#pragma clang fp contract(off)
   const uint32_t lane = threadIdx.x & (kWaveSize - 1);
   const A* pairs = partials + (static_cast<size_t>(n) * d.K * d.G + g) * 2;
-  typename Combine::template State<A> st{};
+  const A inv_l = A(1) / A(static_cast<int64_t>(d.D) * d.S);
   int gave_up = 0;
-  for (uint32_t q0 = lane; q0 < d.K; q0 += 4 * kWaveSize) {
-    // a first look at up to four pairs at once, then each is waited for in turn
-    unsigned long long u[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t q = q0 + j * kWaveSize;
-      u[j] = q < d.K ? peek_pair(pairs + static_cast<size_t>(q) * d.G * 2) : 0ull;
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t q = q0 + j * kWaveSize;
-      if (q < d.K) {
-        A a, b;
-        if (!await_pair(pairs + static_cast<size_t>(q) * d.G * 2, patience, u[j], a, b)) gave_up = 1;
-        Combine::merge(st, Combine::of(d, q, a, b));
-      }
-    }
+  A a0 = A(0), b0 = A(0), c0 = A(0), sum = A(0);
+  for (uint32_t q = lane; q < d.K; q += kWaveSize) {
+    A a, b;
+    if (!await_pair(pairs + static_cast<size_t>(q) * d.G * 2, patience, a, b)) gave_up = 1;
+    const A cnt = A(min(d.rows, d.S - q * d.rows) * d.D);
+    sum += cnt * a;
+    if (q == lane) a0 = a, b0 = b, c0 = cnt;
   }
-#pragma unroll
-  for (int o = 1; o < kWaveSize; o <<= 1) Combine::merge(st, Combine::shuffled(st, o));
-  Combine::finish(st, eps, o0, o1);
+  const A mean = wave_total(sum) * inv_l;
+  const A d0 = a0 - mean;
+  A m2 = b0 + (c0 * d0) * d0;
+  for (uint32_t q = lane + kWaveSize; q < d.K; q += kWaveSize) {
+    A a, b;
+    (void)await_pair(pairs + static_cast<size_t>(q) * d.G * 2, 1u, a, b);  // seen set above
+    const A cnt = A(min(d.rows, d.S - q * d.rows) * d.D);
+    const A dq = a - mean;
+    m2 += b + (cnt * dq) * dq;
+  }
+  o0 = mean;
+  o1 = acc_rsqrt_exact(wave_total(m2) * inv_l + eps);
   return !__any(gave_up);
 }
 
@@ -345,7 +319,7 @@ __device__ __forceinline__ void slice_publish(const SampleSlices& d, uint32_t w,
 // the groups this slice combines. false (for the whole workgroup): a wait ran
 // out and the item has been flagged. kRepair: nothing is published or waited
 // for.
-template <typename Combine, bool kRepair, typename A>
+template <bool kRepair, typename A>
 __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceItem& it, uint32_t w,
                                              const A eps, A* exchange, A* out0, A* out1,
                                              SliceLds<A>& lds) {
@@ -356,7 +330,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
   if constexpr (kRepair) {
     for (uint32_t g = wave; g < d.G; g += kSliceWaves) {
       A o0, o1;
-      (void)slice_group_totals<Combine>(d, partials, it.n, g, 1u, eps, o0, o1);
+      (void)slice_group_moments(d, partials, it.n, g, 1u, eps, o0, o1);
       if (lane == 0) {
         lds.total[0][g] = o0, lds.total[1][g] = o1;
         if (g % d.K == it.k) {
@@ -372,7 +346,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
     int gave_up = 0;
     for (uint32_t g = it.k + wave * d.K; g < d.G; g += kSliceWaves * d.K) {
       A o0, o1;
-      if (!slice_group_totals<Combine>(d, partials, it.n, g, d.patience, eps, o0, o1)) {
+      if (!slice_group_moments(d, partials, it.n, g, d.patience, eps, o0, o1)) {
         gave_up = 1;  // the group's totals stay unset: every slice of the sample will be flagged
       } else if (lane == 0) {
         publish_pair(totals + (static_cast<size_t>(it.n) * d.G + g) * 2, o0, o1);
@@ -462,13 +436,16 @@ __device__ __forceinline__ void slice_forward_finish(
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
   const SliceItem it(d, w);
-  const bool complete = slice_totals<CombineMoments, kRepair>(d, it, w, eps, exchange, mu, rsig, lds);
+  const bool complete = slice_totals<kRepair>(d, it, w, eps, exchange, mu, rsig, lds);
   const A mean = lds.total[0][at.g], rs = lds.total[1][at.g];
   const bool more = !kRepair && reload < d.items;  // uniform over the workgroup
   const SliceItem nit(d, more ? reload : w);
   const uint32_t first = slice_first(d, at, it), step = at.rows_at_a_time * d.C;
   const uint32_t nfirst = slice_first(d, at, nit);
-  if (complete) {
+  {
+    // One path whether the item is complete or not (an incomplete item only skips its
+    // stores): with a second path that also loads the next item the register allocator
+    // spilled 120-300 bytes per thread at sixteen packets and 128 registers.
     // The thread's channels are the same for every item, but their parameters are
     // fetched per item so that they do not occupy registers while the slice is reduced.
     const A* gp = gamma + (at.on ? at.cp * kVec : 0u);
@@ -479,7 +456,7 @@ __device__ __forceinline__ void slice_forward_finish(
     load_params_ragged<kVec>(bp, kVec, bet);
 #pragma unroll
     for (int e = 0; e < kVec; ++e) gam[e] *= rs;
-    int room = slice_room(at, it), nroom = slice_room(at, nit);
+    int room = complete ? slice_room(at, it) : 0, nroom = slice_room(at, nit);
     uint32_t off = first, noff = nfirst;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
@@ -495,8 +472,6 @@ __device__ __forceinline__ void slice_forward_finish(
       off += step, noff += step;
       asm volatile("" : "+v"(room), "+v"(nroom), "+v"(off), "+v"(noff));
     }
-  } else if (more) {
-    slice_load<T, kVPT>(d, at, nit, x, raw);
   }
 }
 
@@ -547,7 +522,7 @@ __global__ __launch_bounds__(kSliceThreads, 4) void group_norm_nhwc_slices_repai
 constexpr unsigned kSliceRepairGrid = 256;
 
 // The most workgroups the kernel is launched with.
-inline uint32_t sample_slices_max_grid() { return static_cast<uint32_t>(num_cus()) * 3u; }
+inline uint32_t sample_slices_max_grid() { return static_cast<uint32_t>(num_cus()) * 4u; }
 
 template <typename A>
 inline void fill_sample_exchange(A* exchange, const SampleSlices& d, hipStream_t stream) {
@@ -584,11 +559,11 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
     // One flavour: a sample of up to eight packets per thread is at most 32 KB, which the
     // one-workgroup-per-sample kernel takes before this one is asked.
-    auto kernel = group_norm_nhwc_slices<T, kSlicePackets, 3>;
+    auto kernel = group_norm_nhwc_slices<T, kSlicePackets, 4>;
     unsigned cap = resident_grid(kernel, kSliceThreads, 0);
     if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();
     if (p.K > cap) return kNotApplicable;
-    note_flavour("group_norm_nhwc_slices<16,3>");
+    note_flavour("group_norm_nhwc_slices<16,4>");
     note_number("slices", p.K);
     fill_sample_exchange(exchange, d, stream);
     hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0, stream, d,
