@@ -3120,6 +3120,8 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_nhwc_samples(
     __syncthreads();  // (total is rewritten by the next call)
   };
 
+  // (Requesting the next sample's packets inside the store loop, as the backward does, was
+  // measured slower here: bf16 [1024, 16*16, 256] 63 -> 66 us, [2048, 14*14, 256] 101 -> 106.)
   for (uint32_t n = blockIdx.x; n < N; n += gridDim.x) {
     const T* xs = x + static_cast<size_t>(n) * S * C;
     T* ys = y + static_cast<size_t>(n) * S * C;
@@ -3286,16 +3288,22 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
 #pragma unroll
   for (int e = 0; e < kVec; ++e) t1[e] = t2[e] = A(0);
 
-  for (uint32_t n = blockIdx.x; n < N; n += gridDim.x) {
-    const size_t base = static_cast<size_t>(n) * S * C;
-    const uint32_t first = r * C + cp * kVec, step = rows_at_a_time * C;
-    u32x4 rx[kVPT], rd[kVPT];
+  const uint32_t first = r * C + cp * kVec, step = rows_at_a_time * C;
+  // The next sample's packets are requested while this one's dx is stored.
+  u32x4 rx[kVPT], rd[kVPT];
+  if (blockIdx.x < N) {
+    const size_t base = static_cast<size_t>(blockIdx.x) * S * C;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       const bool has = on && r + i * rows_at_a_time < S;
       rx[i] = load_packet(x + base + (has ? first + i * step : 0u));
       rd[i] = load_packet(dy + base + (has ? first + i * step : 0u));
     }
+  }
+  for (uint32_t n = blockIdx.x; n < N; n += gridDim.x) {
+    const size_t base = static_cast<size_t>(n) * S * C;
+    const bool more = n + gridDim.x < N;  // uniform over the workgroup
+    const size_t nbase = static_cast<size_t>(more ? n + gridDim.x : n) * S * C;
     const A m = mu[static_cast<size_t>(n) * G + g], rs = rsig[static_cast<size_t>(n) * G + g];
     A s1 = A(0), s2 = A(0);
 #pragma unroll
@@ -3348,6 +3356,11 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
 #pragma unroll
         for (int e = 0; e < kVec; ++e) xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
         store_packet(dx + base + (first_out + i * step), IO<T>::pack(xv));
+      }
+      if (more) {
+        const bool has = on && r + i * rows_at_a_time < S;
+        rx[i] = load_packet(x + nbase + (has ? first_out + i * step : 0u));
+        rd[i] = load_packet(dy + nbase + (has ? first_out + i * step : 0u));
       }
     }
     __syncthreads();  // total is rewritten for the next sample
@@ -4036,6 +4049,19 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
       break;
     default:
       return DRAGON_HIP_EDTYPE;
+  }
+  if (!fused && !sh.nchw && S > 1 && scratch) {
+    // Channels-last samples of two slices or more (beyond 64 KB) go to the slice kernel even
+    // where one 1024-thread workgroup could hold them: four 256-thread workgroups per compute
+    // unit overlap their phases, one workgroup of 1024 does not (bf16 [1024, 16*16, 256] 62 ->
+    // 61 us, [2048, 14*14, 256] 100 -> 94 us). Without scratch the one-workgroup kernel stays.
+    switch (dtype) {
+      case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::f16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
+      case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::bf16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
+      case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_nhwc_slices<float>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
+      default: st = dragon_hip::kNotApplicable; break;
+    }
+    if (st != dragon_hip::kNotApplicable) return st;
   }
   if (!fused) {
     switch (dtype) {

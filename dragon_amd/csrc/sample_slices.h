@@ -536,19 +536,20 @@ inline void fill_sample_exchange(A* exchange, const SampleSlices& d, hipStream_t
 }
 
 // DRAGON_HIP_OK when the kernels were launched, kNotApplicable when the shape
-// or the addresses leave the call to the other paths. `scratch` holds
-// sample_slices_exchange_bytes(...) bytes.
+// (or a sample of fewer than `min_slices` slices) or the addresses leave the
+// call to the other paths. `scratch` holds sample_slices_exchange_bytes(...) bytes.
 template <typename T>
 int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, uint32_t D,
                                        float eps, const void* x, const void* gamma, const void* beta,
                                        void* mu, void* rsig, void* y, void* scratch,
-                                       size_t scratch_bytes, hipStream_t stream) {
+                                       size_t scratch_bytes, hipStream_t stream,
+                                       uint32_t min_slices = 1) {
   using A = typename IO<T>::Acc;
   if constexpr (sizeof(T) > 4) {
     return kNotApplicable;
   } else {
     const SampleSlicePlan p = plan_sample_slices<T>(S, C, G, D);
-    if (!p.ok || !aligned16(x) || !aligned16(y)) return kNotApplicable;
+    if (!p.ok || p.K < min_slices || !aligned16(x) || !aligned16(y)) return kNotApplicable;
     if (static_cast<uint64_t>(N) * p.K * G * 2 + static_cast<uint64_t>(N) * G * 2 > 0x7fffffffull) {
       return kNotApplicable;
     }
@@ -557,8 +558,8 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     }
     A* exchange = static_cast<A*>(scratch);
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-    // One flavour: a sample of up to eight packets per thread is at most 32 KB, which the
-    // one-workgroup-per-sample kernel takes before this one is asked.
+    // One flavour, sixteen packets per thread: a slice of fewer packets leaves the others
+    // masked (they read the tensor's first packet again, from the cache).
     auto kernel = group_norm_nhwc_slices<T, kSlicePackets, 4>;
     unsigned cap = resident_grid(kernel, kSliceThreads, 0);
     if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();
