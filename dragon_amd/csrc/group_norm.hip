@@ -2577,7 +2577,7 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
 // The most workgroups the NHWC sample backward (group_norm_grad_nhwc_samples) is
 // launched with: sizes its partial rows.
 inline uint32_t nhwc_sample_rows(int64_t N) {
-  const int64_t cap = static_cast<int64_t>(num_cus()) * 2;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 4;
   return static_cast<uint32_t>(N < cap ? N : cap);
 }
 
@@ -3263,8 +3263,8 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
 // shares stay in registers across samples and leave the workgroup once, as one
 // partial row of 2*C interleaved words per workgroup (summed by
 // sum_partial_rows).
-template <typename T, int kVPT>
-__global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
+template <typename T, int kVPT, int kThreads>
+__global__ __launch_bounds__(kThreads) void group_norm_grad_nhwc_samples(
     const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
     const T* __restrict__ x, const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
     const typename IO<T>::Acc* __restrict__ mu, const typename IO<T>::Acc* __restrict__ rsig,
@@ -3272,10 +3272,10 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
     typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
-  __shared__ A part[2][kSampleThreads];
-  __shared__ A total[2][kSampleThreads];
+  __shared__ A part[2][kThreads];
+  __shared__ A total[2][kThreads];
   const uint32_t cps = C / kVec;
-  const uint32_t rows_at_a_time = kSampleThreads / cps;
+  const uint32_t rows_at_a_time = kThreads / cps;
   const uint32_t t = threadIdx.x;
   const uint32_t r = t / cps, cp = t - r * cps;
   const bool on = r < rows_at_a_time;
@@ -3385,18 +3385,25 @@ __global__ __launch_bounds__(kSampleThreads) void group_norm_grad_nhwc_samples(
   }
 }
 
+// Workgroup size for a sample: the smallest of 256, 512 and 1024 threads (four, two and one
+// workgroup per compute unit; several overlap their phases) whose eight packets per thread and
+// tensor hold it; 0: none.
 template <typename T>
-bool group_norm_grad_nhwc_samples_ok(const GroupShape& sh, int* slots_out) {
+int group_norm_grad_nhwc_samples_threads(const GroupShape& sh, int* slots_out) {
   constexpr int kVec = IO<T>::kVec;
-  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D % kVec != 0) return false;
+  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D % kVec != 0) return 0;
   const uint32_t cps = sh.C / kVec;
-  if (cps > kSampleThreads) return false;
-  const uint32_t rows_at_a_time = kSampleThreads / cps;
-  const int64_t slots = ceil_div(sh.S, rows_at_a_time);
-  if (slots > 8) return false;
-  if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < kSampleThreads * 3) return false;
-  *slots_out = static_cast<int>(slots);
-  return true;
+  for (const uint32_t threads : {256u, 512u, 1024u}) {
+    if (cps > threads) continue;
+    const uint32_t rows_at_a_time = threads / cps;
+    const int64_t slots = ceil_div(sh.S, rows_at_a_time);
+    if (slots > 8) continue;
+    // most of the workgroup's threads must have a row to hold
+    if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < threads * 3) continue;
+    *slots_out = static_cast<int>(slots);
+    return static_cast<int>(threads);
+  }
+  return 0;
 }
 
 template <typename T>
@@ -3679,21 +3686,27 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 
   if constexpr (sizeof(T) <= 4) {
     int slots = 0;
-    if (group_norm_grad_nhwc_samples_ok<T>(sh, &slots) && aligned16(x) && aligned16(dy) &&
-        aligned16(dx)) {
+    const int threads = group_norm_grad_nhwc_samples_threads<T>(sh, &slots);
+    if (threads != 0 && aligned16(x) && aligned16(dy) && aligned16(dx)) {
       // NHWC samples that fit one workgroup's registers: x and dy read once
       unsigned grid = 0;
-#define LAUNCH(VPT)                                                                              \
+#define LAUNCH(VPT, THREADS)                                                                     \
   {                                                                                              \
-    note_flavour("group_norm_grad_nhwc_samples<" #VPT ">");                                      \
-    auto kernel = group_norm_grad_nhwc_samples<T, VPT>;                                          \
-    const unsigned resident = resident_grid(kernel, kSampleThreads, 0);                          \
+    note_flavour("group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");                         \
+    auto kernel = group_norm_grad_nhwc_samples<T, VPT, THREADS>;                                 \
+    const unsigned resident = resident_grid(kernel, THREADS, 0);                                 \
     grid = nhwc_sample_rows(sh.N);                                                               \
     if (grid > resident) grid = resident;                                                        \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kSampleThreads), 0, stream, sh.N, sh.S, sh.C,    \
-                       sh.G, sh.D, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                  \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), 0, stream, sh.N, sh.S, sh.C, sh.G,     \
+                       sh.D, xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                        \
   }
-      if (slots <= 2) LAUNCH(2) else if (slots <= 4) LAUNCH(4) else LAUNCH(8)
+      if (threads == 256) {
+        if (slots <= 2) LAUNCH(2, 256) else if (slots <= 4) LAUNCH(4, 256) else LAUNCH(8, 256)
+      } else if (threads == 512) {
+        LAUNCH(8, 512)  // (a sample of four packets per thread or fewer fits 256 threads)
+      } else {
+        if (slots <= 2) LAUNCH(2, 1024) else if (slots <= 4) LAUNCH(4, 1024) else LAUNCH(8, 1024)
+      }
 #undef LAUNCH
       launch_sum_partial_rows<A>(grid, sh.C, part, dgp, dbtp, stream);
       return status_of_launch();
@@ -4050,15 +4063,15 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
     default:
       return DRAGON_HIP_EDTYPE;
   }
-  if (!fused && !sh.nchw && S > 1 && scratch) {
-    // Channels-last samples of two slices or more (beyond 64 KB) go to the slice kernel even
-    // where one 1024-thread workgroup could hold them: four 256-thread workgroups per compute
-    // unit overlap their phases, one workgroup of 1024 does not (bf16 [1024, 16*16, 256] 62 ->
-    // 61 us, [2048, 14*14, 256] 100 -> 94 us). Without scratch the one-workgroup kernel stays.
+  if (!fused && !sh.nchw && S > 1) {
+    // Channels-last samples go to the slice kernel first, also where one 1024-thread workgroup
+    // could hold them: four 256-thread workgroups per compute unit overlap their phases, one
+    // workgroup of 1024 does not. A sample of several slices needs scratch for the exchange;
+    // without it (and for rows the slice kernel does not take) the one-workgroup kernel stays.
     switch (dtype) {
-      case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::f16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
-      case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::bf16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
-      case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_nhwc_slices<float>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs, 2); break;
+      case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::f16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+      case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_nhwc_slices<dragon_hip::bf16_t>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
+      case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_nhwc_slices<float>(sh.N, sh.S, sh.C, sh.G, sh.D, eps, x, gamma, beta, mu, rsig, y, scratch, scratch_bytes, hs); break;
       default: st = dragon_hip::kNotApplicable; break;
     }
     if (st != dragon_hip::kNotApplicable) return st;

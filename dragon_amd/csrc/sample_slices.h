@@ -115,7 +115,8 @@ SampleSlices make_sample_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, 
   d.K = p.K, d.rows = p.rows, d.items = N * p.K;
   const uint32_t patience = exchange_patience();
   d.patience = patience ? patience : kCoopPatience;
-  d.flags = reinterpret_cast<uint32_t*>(exchange + sample_slices_exchange_words(N, G, p.K));
+  d.flags = exchange ? reinterpret_cast<uint32_t*>(exchange + sample_slices_exchange_words(N, G, p.K))
+                     : nullptr;  // (a sample in one slice: no exchange)
   d.gave_up_count = exchange_gave_up_counter();
   return d;
 }
@@ -325,6 +326,10 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
                                              SliceLds<A>& lds) {
   const uint32_t t = threadIdx.x;
   const uint32_t wave = t / kWaveSize, lane = t & (kWaveSize - 1);
+  if (d.K == 1) {  // the owner threads have left the sample's own statistics in LDS
+    __syncthreads();
+    return true;
+  }
   A* partials = exchange;
   A* totals = exchange + static_cast<size_t>(d.items) * d.G * 2;
   if constexpr (kRepair) {
@@ -375,6 +380,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
 template <typename T, int kVPT>
 __device__ __forceinline__ void slice_forward_stats(
     const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w,
+    const typename IO<T>::Acc eps, typename IO<T>::Acc* mu, typename IO<T>::Acc* rsig,
     typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
@@ -423,7 +429,17 @@ __device__ __forceinline__ void slice_forward_stats(
   if (t < d.G) pb = lds.total[0][t];
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
-  slice_publish(d, w, pa, pb, exchange);
+  if (d.K == 1) {
+    // a sample in one slice: its statistics are this workgroup's own, nothing is exchanged
+    if (t < d.G) {
+      const A rs = acc_rsqrt_exact(pb * inv_cnt + eps);
+      lds.total[0][t] = pa, lds.total[1][t] = rs;
+      mu[static_cast<size_t>(it.n) * d.G + t] = pa;
+      rsig[static_cast<size_t>(it.n) * d.G + t] = rs;
+    }
+  } else {
+    slice_publish(d, w, pa, pb, exchange);
+  }
 }
 
 // Totals of item w, its rows out of `raw`, and item `reload` (if below d.items) into `raw`.
@@ -491,7 +507,7 @@ __global__ __launch_bounds__(kSliceThreads, kWGs) void group_norm_nhwc_slices(
   u32x4 one[kVPT];
   if (w < d.items) slice_load<T, kVPT>(d, at, SliceItem(d, w), x, one);
   for (; w < d.items; w += step) {
-    slice_forward_stats<T, kVPT>(d, at, w, exchange, one, lds);
+    slice_forward_stats<T, kVPT>(d, at, w, eps, mu, rsig, exchange, one, lds);
     slice_forward_finish<T, kVPT, false>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig, y,
                                          exchange, one, lds);
   }
@@ -536,41 +552,46 @@ inline void fill_sample_exchange(A* exchange, const SampleSlices& d, hipStream_t
 }
 
 // DRAGON_HIP_OK when the kernels were launched, kNotApplicable when the shape
-// (or a sample of fewer than `min_slices` slices) or the addresses leave the
-// call to the other paths. `scratch` holds sample_slices_exchange_bytes(...) bytes.
+// or the addresses leave the call to the other paths. `scratch` holds
+// sample_slices_exchange_bytes(...) bytes (none is needed for samples of one slice).
 template <typename T>
 int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, uint32_t D,
                                        float eps, const void* x, const void* gamma, const void* beta,
                                        void* mu, void* rsig, void* y, void* scratch,
-                                       size_t scratch_bytes, hipStream_t stream,
-                                       uint32_t min_slices = 1) {
+                                       size_t scratch_bytes, hipStream_t stream) {
   using A = typename IO<T>::Acc;
   if constexpr (sizeof(T) > 4) {
     return kNotApplicable;
   } else {
     const SampleSlicePlan p = plan_sample_slices<T>(S, C, G, D);
-    if (!p.ok || p.K < min_slices || !aligned16(x) || !aligned16(y)) return kNotApplicable;
+    if (!p.ok || !aligned16(x) || !aligned16(y)) return kNotApplicable;
     if (static_cast<uint64_t>(N) * p.K * G * 2 + static_cast<uint64_t>(N) * G * 2 > 0x7fffffffull) {
       return kNotApplicable;
     }
-    if (!scratch || scratch_bytes < sample_slices_exchange_bytes(N, G, p.K, sizeof(A))) {
+    // a sample in one slice exchanges nothing: no scratch, no fill, no repair launch
+    if (p.K > 1 && (!scratch || scratch_bytes < sample_slices_exchange_bytes(N, G, p.K, sizeof(A)))) {
       return kNotApplicable;
     }
-    A* exchange = static_cast<A*>(scratch);
+    A* exchange = p.K > 1 ? static_cast<A*>(scratch) : nullptr;
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-    // One flavour, sixteen packets per thread: a slice of fewer packets leaves the others
-    // masked (they read the tensor's first packet again, from the cache).
-    auto kernel = group_norm_nhwc_slices<T, kSlicePackets, 4>;
-    unsigned cap = resident_grid(kernel, kSliceThreads, 0);
-    if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();
-    if (p.K > cap) return kNotApplicable;
-    note_flavour("group_norm_nhwc_slices<16,4>");
-    note_number("slices", p.K);
-    fill_sample_exchange(exchange, d, stream);
-    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0, stream, d,
-                       A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma),
-                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),
-                       static_cast<T*>(y), exchange);
+#define LAUNCH(VPT)                                                                               \
+  {                                                                                               \
+    auto kernel = group_norm_nhwc_slices<T, VPT, 4>;                                              \
+    unsigned cap = resident_grid(kernel, kSliceThreads, 0);                                       \
+    if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
+    if (p.K > cap) return kNotApplicable;                                                         \
+    note_flavour("group_norm_nhwc_slices<" #VPT ",4>");                                           \
+    note_number("slices", p.K);                                                                   \
+    if (p.K > 1) fill_sample_exchange(exchange, d, stream);                                       \
+    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0,       \
+                       stream, d, A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma), \
+                       static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),   \
+                       static_cast<T*>(y), exchange);                                             \
+  }
+    if (p.vpt <= 8) LAUNCH(8) else LAUNCH(16)
+#undef LAUNCH
+    if (p.K == 1) return status_of_launch();
+    // (the widest flavour serves every plan: a repair is rare and its speed does not matter)
     hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets>),
                        dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),
                        dim3(kSliceThreads), 0, stream, d, A(eps), static_cast<const T*>(x),
