@@ -1,10 +1,10 @@
 // GroupNorm forward over NHWC samples that do not fit one workgroup: x is read once.
 //
 // A sample is S rows of C channels. It is cut into K slices of whole rows; a
-// 256-thread workgroup keeps its slice in registers as raw packets (thread
-// (r, cp) holds packet cp of rows r, r + R, r + 2R, ... of the slice, R =
-// 256 / (C / kVec) rows at a time), so a thread's channels, their group and
-// their parameters are the same for every item it sees. A slice holds a share
+// workgroup of 256 (or 512) threads keeps its slice in registers as raw packets
+// (thread (r, cp) holds packet cp of rows r, r + R, r + 2R, ... of the slice,
+// R = threads / (C / kVec) rows at a time), so a thread's channels, their group
+// and their parameters are the same for every item it sees. A slice holds a share
 // of every group of the sample, so an item has G partial pairs to exchange, not
 // one. If every slice read every other slice's G pairs, a sample would cost
 // G * K * K uncached reads; instead the groups are dealt out over the sample's
@@ -53,13 +53,16 @@
 
 namespace dragon_hip {
 
-constexpr int kSliceThreads = 256;
+// Workgroup size: 256 threads, four workgroups per compute unit, or 512, two, for rows whose
+// packets would leave too many of 256 threads without a row (C = 1280 in 16-bit types).
+constexpr int kMaxSliceThreads = 512;
 constexpr int kSlicePackets = 16;  // per thread: a slice is up to 64 KB
 constexpr uint32_t kMaxSampleSlices = 1024;  // slices per sample (a resident grid holds no more workgroups)
 constexpr uint32_t kMaxSampleGroups = 256;  // groups: one owner thread each
 
 struct SampleSlices {
   uint32_t N, S, C, G, D;
+  uint32_t threads;   // workgroup size
   uint32_t K;         // slices per sample
   uint32_t rows;      // rows per slice (the last slice of a sample may hold fewer)
   uint32_t items;     // N * K
@@ -70,7 +73,7 @@ struct SampleSlices {
 
 struct SampleSlicePlan {
   bool ok;
-  uint32_t K, rows;
+  uint32_t threads, K, rows;
   int vpt;  // packets per thread and tensor
 };
 
@@ -78,13 +81,19 @@ struct SampleSlicePlan {
 template <typename T>
 SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
   constexpr uint32_t kVec = IO<T>::kVec;
-  SampleSlicePlan p{false, 0u, 0u, 0};
+  SampleSlicePlan p{false, 0u, 0u, 0u, 0};
   if (sizeof(T) > 4 || S <= 1 || C % kVec != 0 || D % kVec != 0) return p;
   const uint32_t cps = C / kVec;
-  if (cps > kSliceThreads || G > kMaxSampleGroups) return p;
-  const uint32_t rows_at_a_time = kSliceThreads / cps;
+  if (G > kMaxSampleGroups) return p;
   // most of the workgroup's threads must have a row to hold
-  if (cps * rows_at_a_time * 4 < kSliceThreads * 3) return p;
+  for (const uint32_t threads : {256u, 512u}) {
+    if (cps <= threads && cps * (threads / cps) * 4 >= threads * 3) {
+      p.threads = threads;
+      break;
+    }
+  }
+  if (p.threads == 0) return p;
+  const uint32_t rows_at_a_time = p.threads / cps;
   const uint32_t vmax = kSlicePackets;
   const uint32_t k0 = static_cast<uint32_t>(ceil_div(S, rows_at_a_time * vmax));
   // slices of about the same size
@@ -112,7 +121,7 @@ SampleSlices make_sample_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, 
                                 const SampleSlicePlan& p, typename IO<T>::Acc* exchange) {
   SampleSlices d;
   d.N = N, d.S = S, d.C = C, d.G = G, d.D = D;
-  d.K = p.K, d.rows = p.rows, d.items = N * p.K;
+  d.threads = p.threads, d.K = p.K, d.rows = p.rows, d.items = N * p.K;
   const uint32_t patience = exchange_patience();
   d.patience = patience ? patience : kCoopPatience;
   d.flags = exchange ? reinterpret_cast<uint32_t*>(exchange + sample_slices_exchange_words(N, G, p.K))
@@ -128,7 +137,7 @@ struct SliceSeat {
   bool on;
   __device__ explicit SliceSeat(const SampleSlices& d) {
     cps = d.C / kVec;
-    rows_at_a_time = kSliceThreads / cps;
+    rows_at_a_time = d.threads / cps;
     r = threadIdx.x / cps, cp = threadIdx.x - r * cps;
     on = r < rows_at_a_time;
     lanes_per_group = d.D / kVec;
@@ -215,8 +224,8 @@ __device__ __forceinline__ bool await_pair(const float* slot, uint32_t patience,
 // lies between those reads and the next writes.
 template <int kN, int kVec, typename A>
 __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
-                                                 const A (&v)[kN], A (*part)[kSliceThreads],
-                                                 A (*total)[kSliceThreads]) {
+                                                 const A (&v)[kN], A (*part)[kMaxSliceThreads],
+                                                 A (*total)[kMaxSliceThreads]) {
   const uint32_t t = threadIdx.x;
 #pragma unroll
   for (int j = 0; j < kN; ++j) part[j][t] = at.on ? v[j] : A(0);
@@ -239,7 +248,6 @@ __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const Sl
   __syncthreads();
 }
 
-constexpr int kSliceWaves = kSliceThreads / kWaveSize;
 
 // The sum of v over the wavefront, the same bits in every lane (each step adds
 // the two halves of a pair of lanes, which commutes).
@@ -252,8 +260,8 @@ __device__ __forceinline__ A wave_total(A v) {
 
 template <typename A>
 struct SliceLds {
-  A part[2][kSliceThreads];
-  A total[2][kSliceThreads];
+  A part[2][kMaxSliceThreads];
+  A total[2][kMaxSliceThreads];
 };
 
 __device__ __forceinline__ void slice_flag(const SampleSlices& d, uint32_t w) {
@@ -325,7 +333,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
                                              const A eps, A* exchange, A* out0, A* out1,
                                              SliceLds<A>& lds) {
   const uint32_t t = threadIdx.x;
-  const uint32_t wave = t / kWaveSize, lane = t & (kWaveSize - 1);
+  const uint32_t wave = t / kWaveSize, lane = t & (kWaveSize - 1), waves = d.threads / kWaveSize;
   if (d.K == 1) {  // the owner threads have left the sample's own statistics in LDS
     __syncthreads();
     return true;
@@ -333,7 +341,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
   A* partials = exchange;
   A* totals = exchange + static_cast<size_t>(d.items) * d.G * 2;
   if constexpr (kRepair) {
-    for (uint32_t g = wave; g < d.G; g += kSliceWaves) {
+    for (uint32_t g = wave; g < d.G; g += waves) {
       A o0, o1;
       (void)slice_group_moments(d, partials, it.n, g, 1u, eps, o0, o1);
       if (lane == 0) {
@@ -349,7 +357,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
   } else {
     // the groups this slice combines: k, k + K, ..., a wavefront each
     int gave_up = 0;
-    for (uint32_t g = it.k + wave * d.K; g < d.G; g += kSliceWaves * d.K) {
+    for (uint32_t g = it.k + wave * d.K; g < d.G; g += waves * d.K) {
       A o0, o1;
       if (!slice_group_moments(d, partials, it.n, g, d.patience, eps, o0, o1)) {
         gave_up = 1;  // the group's totals stay unset: every slice of the sample will be flagged
@@ -493,8 +501,8 @@ __device__ __forceinline__ void slice_forward_finish(
 
 // One item at a time per workgroup; the next item's packets are requested while
 // this one's are stored.
-template <typename T, int kVPT, int kWGs>
-__global__ __launch_bounds__(kSliceThreads, kWGs) void group_norm_nhwc_slices(
+template <typename T, int kVPT, int kThreads>
+__global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_slices(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
@@ -514,8 +522,8 @@ __global__ __launch_bounds__(kSliceThreads, kWGs) void group_norm_nhwc_slices(
 }
 
 // The launch behind it: nothing to do unless a wait of the first launch ran out.
-template <typename T, int kVPT>
-__global__ __launch_bounds__(kSliceThreads, 4) void group_norm_nhwc_slices_repair(
+template <typename T, int kVPT, int kThreads>
+__global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_slices_repair(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
@@ -574,29 +582,35 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     }
     A* exchange = p.K > 1 ? static_cast<A*>(scratch) : nullptr;
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-#define LAUNCH(VPT)                                                                               \
+#define LAUNCH(VPT, THREADS)                                                                      \
   {                                                                                               \
-    auto kernel = group_norm_nhwc_slices<T, VPT, 4>;                                              \
-    unsigned cap = resident_grid(kernel, kSliceThreads, 0);                                       \
+    auto kernel = group_norm_nhwc_slices<T, VPT, THREADS>;                                        \
+    unsigned cap = resident_grid(kernel, THREADS, 0);                                             \
     if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
     if (p.K > cap) return kNotApplicable;                                                         \
-    note_flavour("group_norm_nhwc_slices<" #VPT ",4>");                                           \
+    note_flavour("group_norm_nhwc_slices<" #VPT "," #THREADS ">");                                \
     note_number("slices", p.K);                                                                   \
     if (p.K > 1) fill_sample_exchange(exchange, d, stream);                                       \
-    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(kSliceThreads), 0,       \
-                       stream, d, A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma), \
+    hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(THREADS), 0, stream, d,  \
+                       A(eps), static_cast<const T*>(x), static_cast<const A*>(gamma),            \
                        static_cast<const A*>(beta), static_cast<A*>(mu), static_cast<A*>(rsig),   \
                        static_cast<T*>(y), exchange);                                             \
+    if (p.K > 1) {                                                                                \
+      /* (the widest flavour serves every plan: a repair is rare, its speed does not matter) */   \
+      hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets, THREADS>),              \
+                         dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),           \
+                         dim3(THREADS), 0, stream, d, A(eps), static_cast<const T*>(x),           \
+                         static_cast<const A*>(gamma), static_cast<const A*>(beta),               \
+                         static_cast<A*>(mu), static_cast<A*>(rsig), static_cast<T*>(y),          \
+                         exchange);                                                               \
+    }                                                                                             \
   }
-    if (p.vpt <= 8) LAUNCH(8) else LAUNCH(16)
+    if (p.threads == 256) {
+      if (p.vpt <= 8) LAUNCH(8, 256) else LAUNCH(16, 256)
+    } else {
+      if (p.vpt <= 8) LAUNCH(8, 512) else LAUNCH(16, 512)
+    }
 #undef LAUNCH
-    if (p.K == 1) return status_of_launch();
-    // (the widest flavour serves every plan: a repair is rare and its speed does not matter)
-    hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets>),
-                       dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),
-                       dim3(kSliceThreads), 0, stream, d, A(eps), static_cast<const T*>(x),
-                       static_cast<const A*>(gamma), static_cast<const A*>(beta),
-                       static_cast<A*>(mu), static_cast<A*>(rsig), static_cast<T*>(y), exchange);
     return status_of_launch();
   }
 }
