@@ -86,13 +86,23 @@ SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t 
   const uint32_t cps = C / kVec;
   if (G > kMaxSampleGroups) return p;
   // most of the workgroup's threads must have a row to hold
+  auto fits = [&](uint32_t threads) {
+    return cps <= threads && cps * (threads / cps) * 4 >= threads * 3;
+  };
   for (const uint32_t threads : {256u, 512u}) {
-    if (cps <= threads && cps * (threads / cps) * 4 >= threads * 3) {
+    if (fits(threads)) {
       p.threads = threads;
       break;
     }
   }
   if (p.threads == 0) return p;
+  // A sample that 512 threads hold as one slice and 256 as two takes the one slice: nothing to
+  // exchange (bf16 [1024, 16*16, 256] 61 -> 49 us, [2048, 14*14, 256] 93 -> 79 us). A workgroup of
+  // 1024 (one per compute unit) loses to either: 75 and 125 us on those shapes.
+  if (p.threads == 256 && fits(512u) && S > 256 / cps * kSlicePackets &&
+      S <= 512 / cps * kSlicePackets) {
+    p.threads = 512;
+  }
   const uint32_t rows_at_a_time = p.threads / cps;
   const uint32_t vmax = kSlicePackets;
   const uint32_t k0 = static_cast<uint32_t>(ceil_div(S, rows_at_a_time * vmax));
