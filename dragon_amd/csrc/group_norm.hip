@@ -3264,7 +3264,7 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
 // partial row of 2*C interleaved words per workgroup (summed by
 // sum_partial_rows).
 template <typename T, int kVPT, int kThreads>
-__global__ __launch_bounds__(kThreads) void group_norm_grad_nhwc_samples(
+__global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
     const T* __restrict__ x, const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
     const typename IO<T>::Acc* __restrict__ mu, const typename IO<T>::Acc* __restrict__ rsig,

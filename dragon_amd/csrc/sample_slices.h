@@ -54,7 +54,9 @@
 namespace dragon_hip {
 
 // Workgroup size: 256 threads, four workgroups per compute unit, or 512, two, for rows whose
-// packets would leave too many of 256 threads without a row (C = 1280 in 16-bit types).
+// packets would leave too many of 256 threads without a row (C = 1280 in 16-bit types). Either
+// way four wavefronts per SIMD, i.e. 128 registers (the second launch bound counts wavefronts
+// per SIMD, not workgroups).
 constexpr int kMaxSliceThreads = 512;
 constexpr int kSlicePackets = 16;  // per thread: a slice is up to 64 KB
 constexpr uint32_t kMaxSampleSlices = 1024;  // slices per sample (a resident grid holds no more workgroups)
@@ -73,6 +75,7 @@ struct SampleSlices {
 
 struct SampleSlicePlan {
   bool ok;
+  bool two;  // D is not a multiple of a packet: a packet may lie in two groups
   uint32_t threads, K, rows;
   int vpt;  // packets per thread and tensor
 };
@@ -81,8 +84,10 @@ struct SampleSlicePlan {
 template <typename T>
 SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
   constexpr uint32_t kVec = IO<T>::kVec;
-  SampleSlicePlan p{false, 0u, 0u, 0u, 0};
-  if (sizeof(T) > 4 || S <= 1 || C % kVec != 0 || D % kVec != 0) return p;
+  SampleSlicePlan p{false, false, 0u, 0u, 0u, 0};
+  // (a group of less than a packet would put three groups or more into one packet)
+  if (sizeof(T) > 4 || S <= 1 || C % kVec != 0 || D < kVec) return p;
+  p.two = D % kVec != 0;
   const uint32_t cps = C / kVec;
   if (G > kMaxSampleGroups) return p;
   // most of the workgroup's threads must have a row to hold
@@ -144,6 +149,8 @@ SampleSlices make_sample_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, 
 template <int kVec>
 struct SliceSeat {
   uint32_t cps, rows_at_a_time, r, cp, g, lanes_per_group;
+  uint32_t g1;  // where groups are not whole packets: the group of the packet's last channels,
+  int k0;       // and how many of its channels lie in g (the first group)
   bool on;
   __device__ explicit SliceSeat(const SampleSlices& d) {
     cps = d.C / kVec;
@@ -151,7 +158,9 @@ struct SliceSeat {
     r = threadIdx.x / cps, cp = threadIdx.x - r * cps;
     on = r < rows_at_a_time;
     lanes_per_group = d.D / kVec;
-    g = on ? cp / lanes_per_group : 0u;
+    g = on ? cp * kVec / d.D : 0u;
+    k0 = static_cast<int>(min(static_cast<uint32_t>(kVec), (g + 1) * d.D - (on ? cp : 0u) * kVec));
+    g1 = g + 1 < d.G ? g + 1 : g;
   }
 };
 
@@ -258,6 +267,32 @@ __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const Sl
   __syncthreads();
 }
 
+
+// The same where a packet may lie in two groups: v0 is the thread's share for the group of its
+// packet's first channel, v1 for the next group; the owner of group t adds the shares of the
+// packets that touch it (packet c starts in group t, or, only the first of them, before it).
+template <int kVec, typename A>
+__device__ __forceinline__ void slice_group_sums_two(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                     const A v0, const A v1,
+                                                     A (*part)[kMaxSliceThreads],
+                                                     A (*total)[kMaxSliceThreads]) {
+  const uint32_t t = threadIdx.x;
+  part[0][t] = at.on ? v0 : A(0);
+  part[1][t] = at.on ? v1 : A(0);
+  __syncthreads();
+  if (t < d.G) {
+    const uint32_t lo = t * d.D / kVec, hi = ((t + 1) * d.D - 1) / kVec;
+    A acc = A(0);
+    for (uint32_t rr = 0; rr < at.rows_at_a_time; ++rr) {
+      for (uint32_t c = lo; c <= hi; ++c) {
+        const int share = c * kVec < t * d.D ? 1 : 0;
+        acc += part[share][rr * at.cps + c];
+      }
+    }
+    total[0][t] = acc;
+  }
+  __syncthreads();
+}
 
 // The sum of v over the wavefront, the same bits in every lane (each step adds
 // the two halves of a pair of lanes, which commutes).
@@ -395,7 +430,7 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
 // ---------------------------------------------------------------- forward
 // The slice's share of each group: its mean, then its squared deviations from
 // that mean; the owner threads publish them.
-template <typename T, int kVPT>
+template <typename T, int kVPT, bool kTwo>
 __device__ __forceinline__ void slice_forward_stats(
     const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w,
     const typename IO<T>::Acc eps, typename IO<T>::Acc* mu, typename IO<T>::Acc* rsig,
@@ -405,7 +440,8 @@ __device__ __forceinline__ void slice_forward_stats(
   const SliceItem it(d, w);
   const uint32_t t = threadIdx.x;
   const A inv_cnt = A(1) / A(it.nrows * d.D);
-  A s[1] = {A(0)};
+  // (kTwo: s[0] for the group of the packet's first channel, s[1] for the next one)
+  A s[2] = {A(0), A(0)};
   int room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
@@ -416,17 +452,25 @@ __device__ __forceinline__ void slice_forward_stats(
       A v[kVec];
       IO<T>::unpack(raw[i], v);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) s[0] += v[e];
+      for (int e = 0; e < kVec; ++e) {
+        if (!kTwo || e < at.k0) s[0] += v[e]; else s[1] += v[e];
+      }
     }
   }
-  slice_group_sums<1, kVec>(d, at, s, lds.part, lds.total);
+  if constexpr (kTwo) {
+    slice_group_sums_two<kVec>(d, at, s[0], s[1], lds.part, lds.total);
+  } else {
+    const A one[1] = {s[0]};
+    slice_group_sums<1, kVec>(d, at, one, lds.part, lds.total);
+  }
   A pa = A(0), pb = A(0);
   if (t < d.G) pa = lds.total[0][t] * inv_cnt;
   const A mean_k = lds.total[0][at.g] * inv_cnt;
+  const A mean_k1 = kTwo ? lds.total[0][at.g1] * inv_cnt : A(0);
   // convert the packets again in each pass instead of keeping every converted element
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
-  s[0] = A(0);
+  s[0] = s[1] = A(0);
   room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
@@ -438,12 +482,22 @@ __device__ __forceinline__ void slice_forward_stats(
       IO<T>::unpack(raw[i], v);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        const A dv = v[e] - mean_k;
-        s[0] += dv * dv;
+        if (!kTwo || e < at.k0) {
+          const A dv = v[e] - mean_k;
+          s[0] += dv * dv;
+        } else {
+          const A dv = v[e] - mean_k1;
+          s[1] += dv * dv;
+        }
       }
     }
   }
-  slice_group_sums<1, kVec>(d, at, s, lds.part, lds.total);
+  if constexpr (kTwo) {
+    slice_group_sums_two<kVec>(d, at, s[0], s[1], lds.part, lds.total);
+  } else {
+    const A one[1] = {s[0]};
+    slice_group_sums<1, kVec>(d, at, one, lds.part, lds.total);
+  }
   if (t < d.G) pb = lds.total[0][t];
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
@@ -461,7 +515,7 @@ __device__ __forceinline__ void slice_forward_stats(
 }
 
 // Totals of item w, its rows out of `raw`, and item `reload` (if below d.items) into `raw`.
-template <typename T, int kVPT, bool kRepair>
+template <typename T, int kVPT, bool kRepair, bool kTwo>
 __device__ __forceinline__ void slice_forward_finish(
     const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w, uint32_t reload,
     const typename IO<T>::Acc eps, const T* x, const typename IO<T>::Acc* gamma,
@@ -472,6 +526,7 @@ __device__ __forceinline__ void slice_forward_finish(
   const SliceItem it(d, w);
   const bool complete = slice_totals<kRepair>(d, it, w, eps, exchange, mu, rsig, lds);
   const A mean = lds.total[0][at.g], rs = lds.total[1][at.g];
+  const A mean1 = kTwo ? lds.total[0][at.g1] : A(0), rs1 = kTwo ? lds.total[1][at.g1] : A(0);
   const bool more = !kRepair && reload < d.items;  // uniform over the workgroup
   const SliceItem nit(d, more ? reload : w);
   const uint32_t first = slice_first(d, at, it), step = at.rows_at_a_time * d.C;
@@ -489,7 +544,7 @@ __device__ __forceinline__ void slice_forward_finish(
     load_params_ragged<kVec>(gp, kVec, gam);
     load_params_ragged<kVec>(bp, kVec, bet);
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) gam[e] *= rs;
+    for (int e = 0; e < kVec; ++e) gam[e] *= !kTwo || e < at.k0 ? rs : rs1;
     int room = complete ? slice_room(at, it) : 0, nroom = slice_room(at, nit);
     uint32_t off = first, noff = nfirst;
 #pragma unroll
@@ -498,7 +553,9 @@ __device__ __forceinline__ void slice_forward_finish(
         A v[kVec];
         IO<T>::unpack(raw[i], v);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) v[e] = (v[e] - mean) * gam[e] + bet[e];
+        for (int e = 0; e < kVec; ++e) {
+          v[e] = (v[e] - (!kTwo || e < at.k0 ? mean : mean1)) * gam[e] + bet[e];
+        }
         store_packet(y + off, IO<T>::pack(v));
       }
       if (more) raw[i] = load_packet(x + (nroom > 0 ? noff : 0u));
@@ -511,8 +568,8 @@ __device__ __forceinline__ void slice_forward_finish(
 
 // One item at a time per workgroup; the next item's packets are requested while
 // this one's are stored.
-template <typename T, int kVPT, int kThreads>
-__global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_slices(
+template <typename T, int kVPT, int kThreads, bool kTwo>
+__global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
@@ -525,15 +582,15 @@ __global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_sli
   u32x4 one[kVPT];
   if (w < d.items) slice_load<T, kVPT>(d, at, SliceItem(d, w), x, one);
   for (; w < d.items; w += step) {
-    slice_forward_stats<T, kVPT>(d, at, w, eps, mu, rsig, exchange, one, lds);
-    slice_forward_finish<T, kVPT, false>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig, y,
+    slice_forward_stats<T, kVPT, kTwo>(d, at, w, eps, mu, rsig, exchange, one, lds);
+    slice_forward_finish<T, kVPT, false, kTwo>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig, y,
                                          exchange, one, lds);
   }
 }
 
 // The launch behind it: nothing to do unless a wait of the first launch ran out.
-template <typename T, int kVPT, int kThreads>
-__global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_slices_repair(
+template <typename T, int kVPT, int kThreads, bool kTwo>
+__global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices_repair(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
     typename IO<T>::Acc* __restrict__ mu, typename IO<T>::Acc* __restrict__ rsig,
@@ -546,7 +603,7 @@ __global__ __launch_bounds__(kThreads, 1024 / kThreads) void group_norm_nhwc_sli
     if (d.flags[w] == 0u) continue;  // the same word in every thread
     u32x4 raw[kVPT];
     slice_load<T, kVPT>(d, at, SliceItem(d, w), x, raw);
-    slice_forward_finish<T, kVPT, true>(d, at, w, d.items, eps, x, gamma, beta, mu, rsig, y,
+    slice_forward_finish<T, kVPT, true, kTwo>(d, at, w, d.items, eps, x, gamma, beta, mu, rsig, y,
                                         exchange, raw, lds);
     __syncthreads();  // the next item rewrites the totals in LDS
   }
@@ -592,13 +649,14 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     }
     A* exchange = p.K > 1 ? static_cast<A*>(scratch) : nullptr;
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-#define LAUNCH(VPT, THREADS)                                                                      \
+#define LAUNCH_T(VPT, THREADS, TWO)                                                                   \
   {                                                                                               \
-    auto kernel = group_norm_nhwc_slices<T, VPT, THREADS>;                                        \
+    auto kernel = group_norm_nhwc_slices<T, VPT, THREADS, TWO>;                                   \
     unsigned cap = resident_grid(kernel, THREADS, 0);                                             \
     if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
     if (p.K > cap) return kNotApplicable;                                                         \
-    note_flavour("group_norm_nhwc_slices<" #VPT "," #THREADS ">");                                \
+    note_flavour(TWO ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",two>"                        \
+                     : "group_norm_nhwc_slices<" #VPT "," #THREADS ">");                          \
     note_number("slices", p.K);                                                                   \
     if (p.K > 1) fill_sample_exchange(exchange, d, stream);                                       \
     hipLaunchKernelGGL(kernel, dim3(d.items < cap ? d.items : cap), dim3(THREADS), 0, stream, d,  \
@@ -607,7 +665,7 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
                        static_cast<T*>(y), exchange);                                             \
     if (p.K > 1) {                                                                                \
       /* (the widest flavour serves every plan: a repair is rare, its speed does not matter) */   \
-      hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets, THREADS>),              \
+      hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets, THREADS, TWO>),         \
                          dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),           \
                          dim3(THREADS), 0, stream, d, A(eps), static_cast<const T*>(x),           \
                          static_cast<const A*>(gamma), static_cast<const A*>(beta),               \
@@ -615,12 +673,15 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
                          exchange);                                                               \
     }                                                                                             \
   }
+#define LAUNCH(VPT, THREADS) \
+  { if (p.two) LAUNCH_T(VPT, THREADS, true) else LAUNCH_T(VPT, THREADS, false) }
     if (p.threads == 256) {
       if (p.vpt <= 8) LAUNCH(8, 256) else LAUNCH(16, 256)
     } else {
       if (p.vpt <= 8) LAUNCH(8, 512) else LAUNCH(16, 512)
     }
 #undef LAUNCH
+#undef LAUNCH_T
     return status_of_launch();
   }
 }

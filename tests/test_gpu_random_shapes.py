@@ -240,6 +240,9 @@ NHWC_SLICE_CASES = [
     (3, 25, 8, 2049, "float16", 0), (1, 256, 8, 700, "bfloat16", 0), (40, 8, 16, 2304, "float32", 0),
     (2, 32, 16, 4097, "bfloat16", 0), (2, 32, 16, 4097, "bfloat16", 3), (5, 3, 8, 6000, "float16", 0),
     (2, 2, 256, 1030, "float32", 0), (1, 64, 4, 3000, "float32", 0), (2, 16, 24, 999, "bfloat16", 0),
+    # groups of 10, 12 and 20 channels: a packet may lie in two groups (one slice and several)
+    (2, 32, 10, 1030, "bfloat16", 0), (3, 32, 20, 300, "float16", 0), (2, 16, 10, 2000, "float32", 0),
+    (40, 32, 10, 64, "bfloat16", 0), (3, 8, 12, 5000, "bfloat16", 0),
     # rows of 160, 320 and 384 packets: not sliced (too many idle threads), same answer
     (3, 32, 40, 777, "bfloat16", 0), (2, 32, 40, 600, "float32", 0), (2, 48, 64, 500, "float16", 0),
 ]
