@@ -3257,13 +3257,18 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
 }
 
 // The backward the same way: x and dy of a sample in registers (up to eight
-// packets per thread each, samples of up to 128 KB per tensor), groups of whole
-// packets. ds / db per group go through the group reduction above; a thread's
+// packets per thread each, samples of up to 128 KB per tensor), groups of at
+// least a packet; kTwo: a group need not be whole packets, so a packet may lie
+// in two groups (elements below k0 in group g, the others in g + 1) and a thread
+// carries a share for each. ds / db per group are summed by the group's owner
+// thread out of one LDS word per thread and share; a thread's
 // channels are the same for every sample it sees, so their dgamma / dbeta
 // shares stay in registers across samples and leave the workgroup once, as one
 // partial row of 2*C interleaved words per workgroup (summed by
-// sum_partial_rows).
-template <typename T, int kVPT, int kThreads>
+// sum_partial_rows). (Keeping the shares in LDS between samples instead, one
+// word per thread and share, freed no registers where they are short, in the
+// two-group flavour at eight packets per thread, and was not faster.)
+template <typename T, int kVPT, int kThreads, bool kTwo>
 __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
     const T* __restrict__ x, const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
@@ -3272,15 +3277,24 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
-  __shared__ A part[2][kThreads];
+  __shared__ A part[kTwo ? 4 : 2][kThreads];
   __shared__ A total[2][kThreads];
   const uint32_t cps = C / kVec;
   const uint32_t rows_at_a_time = kThreads / cps;
   const uint32_t t = threadIdx.x;
   const uint32_t r = t / cps, cp = t - r * cps;
   const bool on = r < rows_at_a_time;
-  const uint32_t lanes_per_group = D / kVec;
-  const uint32_t g = on ? cp / lanes_per_group : 0u;
+  const uint32_t lanes_per_group = D / kVec;  // (whole packets only)
+  uint32_t g, g1 = 0;
+  int k0 = kVec;
+  if constexpr (kTwo) {
+    g = on ? cp * kVec / D : 0u;
+    const uint32_t edge = (g + 1) * D - cp * kVec;  // >= 1
+    if (on && edge < static_cast<uint32_t>(kVec)) k0 = static_cast<int>(edge);
+    g1 = k0 < kVec ? g + 1 : g;
+  } else {
+    g = on ? cp / lanes_per_group : 0u;
+  }
   const A denom = A(1) / A(static_cast<int64_t>(D) * S);
   A gam[kVec];
   load_params_ragged<kVec>(gamma + (on ? cp * kVec : 0u), kVec, gam);
@@ -3305,7 +3319,9 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     const bool more = n + gridDim.x < N;  // uniform over the workgroup
     const size_t nbase = static_cast<size_t>(more ? n + gridDim.x : n) * S * C;
     const A m = mu[static_cast<size_t>(n) * G + g], rs = rsig[static_cast<size_t>(n) * G + g];
-    A s1 = A(0), s2 = A(0);
+    const A mb = kTwo ? mu[static_cast<size_t>(n) * G + g1] : A(0);
+    const A rsb = kTwo ? rsig[static_cast<size_t>(n) * G + g1] : A(0);
+    A s1 = A(0), s2 = A(0), s1b = A(0), s2b = A(0);
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       if (on && r + i * rows_at_a_time < S) {
@@ -3315,23 +3331,47 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
           const A gd = gam[e] * dv[e];
-          s1 += gd * xv[e];
-          s2 += gd;
-          t1[e] += dv[e] * (xv[e] - m) * rs;
+          if (!kTwo || e < k0) {
+            s1 += gd * xv[e];
+            s2 += gd;
+            t1[e] += dv[e] * (xv[e] - m) * rs;
+          } else {
+            s1b += gd * xv[e];
+            s2b += gd;
+            t1[e] += dv[e] * (xv[e] - mb) * rsb;
+          }
           t2[e] += dv[e];
         }
       }
     }
-    // the group's ds and db: one LDS word per thread and sum, added by the group's owner thread
+    // the group's ds and db: one LDS word per thread, share and sum, added by the group's owner
+    // thread
     part[0][t] = on ? s1 : A(0);
     part[1][t] = on ? s2 : A(0);
+    if constexpr (kTwo) {
+      part[2][t] = on ? s1b : A(0);
+      part[3][t] = on ? s2b : A(0);
+    }
     __syncthreads();
     if (t < G) {
       A a = A(0), b = A(0);
-      for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
-        for (uint32_t k = 0; k < lanes_per_group; ++k) {
-          a += part[0][rr * cps + t * lanes_per_group + k];
-          b += part[1][rr * cps + t * lanes_per_group + k];
+      if constexpr (kTwo) {
+        // packets lo..hi hold the group's channels; one that begins before the group gives its
+        // second share
+        const uint32_t lo = t * D / kVec, hi = ((t + 1) * D - 1) / kVec;
+        for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+          for (uint32_t c = lo; c <= hi; ++c) {
+            const int share = c * kVec < t * D ? 2 : 0;
+            a += part[share][rr * cps + c];
+            b += part[share + 1][rr * cps + c];
+          }
+        }
+      } else {
+        for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+          for (uint32_t k = 0; k < lanes_per_group; ++k) {
+            a += part[0][rr * cps + t * lanes_per_group + k];
+            b += part[1][rr * cps + t * lanes_per_group + k];
+          }
         }
       }
       total[0][t] = a, total[1][t] = b;
@@ -3342,6 +3382,12 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     s1 = total[0][g], s2 = total[1][g];
     const A u0 = (s2 * m - s1) * (rs * rs * rs) * denom;
     const A v0 = s2 * rs * denom;
+    A u0b = A(0), v0b = A(0);
+    if constexpr (kTwo) {
+      s1b = total[0][g1], s2b = total[1][g1];
+      u0b = (s2b * mb - s1b) * (rsb * rsb * rsb) * denom;
+      v0b = s2b * rsb * denom;
+    }
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(rx[i]), "+v"(rd[i]));
     // (the offsets are formed again rather than kept from the loads: registers)
@@ -3354,7 +3400,13 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
         IO<T>::unpack(rx[i], xv);
         IO<T>::unpack(rd[i], dv);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
+        for (int e = 0; e < kVec; ++e) {
+          if (!kTwo || e < k0) {
+            xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
+          } else {
+            xv[e] = gam[e] * rsb * dv[e] + (u0b * (xv[e] - mb) - v0b);
+          }
+        }
         store_packet(dx + base + (first_out + i * step), IO<T>::pack(xv));
       }
       if (more) {
@@ -3391,7 +3443,7 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
 template <typename T>
 int group_norm_grad_nhwc_samples_threads(const GroupShape& sh, int* slots_out) {
   constexpr int kVec = IO<T>::kVec;
-  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D % kVec != 0) return 0;
+  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D < kVec) return 0;
   const uint32_t cps = sh.C / kVec;
   for (const uint32_t threads : {256u, 512u, 1024u}) {
     if (cps > threads) continue;
@@ -3692,8 +3744,11 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       unsigned grid = 0;
 #define LAUNCH(VPT, THREADS)                                                                     \
   {                                                                                              \
-    note_flavour("group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");                         \
-    auto kernel = group_norm_grad_nhwc_samples<T, VPT, THREADS>;                                 \
+    const bool two = sh.D % kVec != 0; /* a packet may lie in two groups */                      \
+    note_flavour(two ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",two>"                 \
+                     : "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");                   \
+    auto kernel = two ? group_norm_grad_nhwc_samples<T, VPT, THREADS, true>                      \
+                      : group_norm_grad_nhwc_samples<T, VPT, THREADS, false>;                    \
     const unsigned resident = resident_grid(kernel, THREADS, 0);                                 \
     grid = nhwc_sample_rows(sh.N);                                                               \
     if (grid > resident) grid = resident;                                                        \

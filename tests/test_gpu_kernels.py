@@ -531,8 +531,9 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             ((2, 14, 14, 64), -1, 4), ((3, 5, 7, 96), -1, 4), ((2, 28, 28, 64), -1, 2),
             ((700, 4, 4, 32), -1, 2),
             # the same with groups of 10 and 12 channels: a packet of the fused NHWC forward
-            # lies in two groups
+            # and backward lies in two groups (and more samples than workgroups)
             ((2, 7, 7, 320), -1, 32), ((3, 6, 5, 96), -1, 8), ((5, 9, 9, 160), -1, 16),
+            ((1100, 3, 3, 40), -1, 4),
             # NHWC samples beyond one workgroup's registers: slices of whole rows that exchange
             # their groups' sums (8 to 32 slices per sample; a ragged last slice and idle
             # threads; fewer slices than groups and more; more items than workgroups)
