@@ -41,6 +41,7 @@
 #include "row_tile.h"
 #include "short_rows.h"
 #include "sample_slices.h"
+#include "group_items.h"
 #include "slices.h"
 
 namespace dragon_hip {
@@ -4101,6 +4102,18 @@ int dragon_hip_group_norm_forward(int dtype, int64_t N, int64_t G, int64_t D, in
   if (N * S == 0) return DRAGON_HIP_OK;
   if (!x || !gamma || !beta || !mu || !rsig || !y) return DRAGON_HIP_EINVAL;
   hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (sh.nchw) {
+    // Groups of 32 KB and more that 256 or 512 threads hold whole: two or four workgroups per
+    // compute unit, each requesting its next group while it stores, ahead of one 1024-thread
+    // workgroup with two register sets (bf16 groups of 128 KB: 49.9 -> 47.5 us).
+    switch (dtype) {
+      case DRAGON_HIP_F16: st = dragon_hip::try_group_norm_forward_items<dragon_hip::f16_t>(N, G, D, S, eps, x, gamma, beta, mu, rsig, y, hs); break;
+      case DRAGON_HIP_BF16: st = dragon_hip::try_group_norm_forward_items<dragon_hip::bf16_t>(N, G, D, S, eps, x, gamma, beta, mu, rsig, y, hs); break;
+      case DRAGON_HIP_F32: st = dragon_hip::try_group_norm_forward_items<float>(N, G, D, S, eps, x, gamma, beta, mu, rsig, y, hs); break;
+      default: st = dragon_hip::kNotApplicable; break;
+    }
+    if (st != dragon_hip::kNotApplicable) return st;
+  }
   bool fused = false;
   switch (dtype) {
     case DRAGON_HIP_F16:

@@ -277,6 +277,49 @@ def test_group_norm_forward_nhwc_slice_shapes(K, N, G, D, S, dtype, shift, in_pl
     assert K.exchange_timed_out() == 0
 
 
+# NCHW groups that one 256- or 512-thread workgroup holds whole (2048 packets and more, sixteen
+# per thread at most): 9-16 packets per thread, a last slot that few threads fill, channels of
+# fewer packets than the workgroup has threads (several channels per slot, a boundary inside the
+# workgroup) and of more, one channel per group, more groups than resident workgroups, a group
+# count that does not divide the grid, x at an address that is not 16-byte aligned (another
+# path, same answer), in place.
+NCHW_ITEM_CASES = [
+    (2, 3, 6, 3136, "bfloat16", 0), (1, 2, 40, 784, "bfloat16", 0), (2, 2, 20, 784, "float32", 0),
+    (3, 2, 1, 65536, "float16", 0), (1, 5, 16, 4096, "bfloat16", 0), (2, 4, 8, 4096, "float32", 0),
+    (700, 3, 4, 2048, "float32", 0), (2, 2, 256, 128, "bfloat16", 0), (2, 2, 300, 64, "float16", 0),
+    (1, 3, 16, 4096, "bfloat16", 3), (2, 7, 3, 5464, "bfloat16", 0), (1100, 2, 8, 2048, "bfloat16", 0),
+]
+
+
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("N,G,D,S,dtype,shift", NCHW_ITEM_CASES)
+def test_group_norm_forward_nchw_whole_group_shapes(K, N, G, D, S, dtype, shift, in_place):
+    import torch
+    rng = np.random.default_rng(7100 + G * D + S)
+    C = G * D
+    n = N * C * S
+    xb, xs = _values(rng, (n,), dtype, 2.0)
+    xs = xs + 0.0
+    x = xs.reshape(N, G, D, S)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    eps = 1e-5
+    mean = x.mean((2, 3))
+    rs = 1 / np.sqrt(((x - mean[:, :, None, None]) ** 2).mean((2, 3)) + np.float64(np.float32(eps)))
+    y_ref = ((x - mean[:, :, None, None]) * rs[:, :, None, None]).reshape(N, C, S) * g[None, :, None] \
+        + b[None, :, None]
+    xbuf, xd = _held(n, dtype, shift, xb)
+    ybuf, yd = (xbuf, xd) if in_place else _held(n, dtype, shift)
+    gd, bd = torch.from_numpy(g).cuda(), torch.from_numpy(b).cuda()
+    mu, rsig = torch.empty(N * G, device="cuda"), torch.empty(N * G, device="cuda")
+    K.group_norm_forward(N, G, D, S, "NCHW", eps, xd, gd, bd, mu, rsig, yd)
+    y = U.widen(U.to_host(yd.contiguous()), dtype).reshape(N, C, S)
+    assert _mean_ok(mu.cpu().numpy(), mean, x)
+    assert np.max(np.abs(rsig.cpu().numpy().astype(np.float64) / rs.ravel() - 1)) <= 5e-5
+    assert U.normwise(y, y_ref) <= U.TIGHT[dtype]
+    assert _untouched(ybuf, dtype, shift, n)
+
+
 @pytest.mark.parametrize("N,G,D,S,fmt,dtype,seed", _channel_cases(40, 5))
 def test_batch_norm_training_shapes(K, N, G, D, S, fmt, dtype, seed):
     import torch
