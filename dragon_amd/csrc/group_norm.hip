@@ -1160,6 +1160,12 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
   constexpr bool kAnyS = kMode == kChannelStraddlesAny;
   constexpr bool kStraddle = kMode == kChannelStraddles || kAnyS;
   constexpr bool kLanes = kMode == kChannelLanes;
+  // kChannelWaves: the 64 packets of a (slot, wavefront) pair lie in one channel, so their
+  // sums of dy * x and dy, reduced over the wavefront in the first pass, give the group's ds /
+  // db shares (times gamma, a scalar) and the channel's dgamma / dbeta shares
+  // ((sum(dy x) - mu sum(dy)) rsig, as the CPU kernel forms them per (n, c)) at once; the second
+  // pass is then two multiply-adds per element and reduces nothing.
+  constexpr bool kWholeWaves = kMode == kChannelWaves;
   constexpr int kParts = kStraddle ? 4 : 2;  // per entry: (dgamma, dbeta) of one or two channels
   __shared__ A slots[2 * Tile::kSlots];
   __shared__ A chan_part[kVPT][kWaves][kParts];
@@ -1251,6 +1257,29 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
       } else if constexpr (kLanes) {
         const uint32_t chan = static_cast<uint32_t>(i * kTPR + lane) / packets_per_chan;
         gam[i] = gamma[c0 + (chan < D ? chan : D - 1)];
+      } else if constexpr (kWholeWaves) {
+        uint32_t chan, in_first;
+        first_channel(i, chan, in_first);
+        gam[i] = gamma[c0 + chan];
+        A p1 = A(0), p2 = A(0);
+        if (Tile::active(i, npackets)) {
+          A xv[kVec], dv[kVec];
+          tx.unpack(i, xv);
+          tdy.unpack(i, dv);
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            p1 += dv[e] * xv[e];
+            p2 += dv[e];
+          }
+        }
+        p1 = wave_allreduce(p1, SumOp());
+        p2 = wave_allreduce(p2, SumOp());
+        if (wave_lane == 0) {
+          chan_part[i][wave][0] = (p1 - m * p2) * r;
+          chan_part[i][wave][1] = p2;
+        }
+        s1 += gam[i] * p1;  // (the same in every lane: the wavefront's share)
+        s2 += gam[i] * p2;
       } else {
         uint32_t chan, in_first;
         first_channel(i, chan, in_first);
@@ -1260,7 +1289,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           gam[i] = static_cast<uint32_t>(wave_lane) < in_first ? gam[i] : second;
         }
       }
-      if (!kAnyS && Tile::active(i, npackets)) {
+      if (!kAnyS && !kWholeWaves && Tile::active(i, npackets)) {
         // gamma is one value per thread and slot: it multiplies the slot's sums once
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
@@ -1275,7 +1304,18 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
         s2 += gam[i] * p2;
       }
     }
-    Tile::reduce_sum_pair(s1, s2, slots);
+    if constexpr (kWholeWaves) {
+      if (wave_lane == 0) slots[2 * wave] = s1, slots[2 * wave + 1] = s2;
+      __syncthreads();
+      s1 = s2 = A(0);
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        s1 += slots[2 * w];
+        s2 += slots[2 * w + 1];
+      }
+    } else {
+      Tile::reduce_sum_pair(s1, s2, slots);
+    }
     if (lane == 0) {
       ds[row] = s1;
       db[row] = s2;
@@ -1283,13 +1323,24 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     // dx = gamma*rsig * dy + (u*(x - mu) - v) with the row's u, v divided by D*S once
     const A u0 = (s2 * m - s1) * (r * r * r) * denom;
     const A v0 = s2 * r * denom;
+    const A w0 = -(u0 * m + v0);  // kWholeWaves: dx = gamma*rsig * dy + (u x + w)
     tx.refresh();
     tdy.refresh();
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       A t1 = A(0), t2 = A(0);
       A u1 = A(0), u2 = A(0);  // kAnyS: the second channel's share of a packet on the boundary
-      if constexpr (kAnyS) {
+      if constexpr (kWholeWaves) {
+        if (Tile::active(i, npackets)) {
+          A xv[kVec], dv[kVec];
+          tx.unpack(i, xv);
+          tdy.unpack(i, dv);
+          const A gr = gam[i] * r;
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) xv[e] = gr * dv[e] + (u0 * xv[e] + w0);
+          tx.store_slot(dx + row * L, i, xv);
+        }
+      } else if constexpr (kAnyS) {
         uint32_t chan, in_first;
         first_channel_elems(i, chan, in_first);
         const int edge = static_cast<int>(in_first / kVec), km = static_cast<int>(in_first % kVec);
@@ -1390,7 +1441,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           chan_part[i][wave][2] = b1;
           chan_part[i][wave][3] = b2;
         }
-      } else {
+      } else if constexpr (!kWholeWaves) {
         t1 = wave_allreduce(t1, SumOp());
         t2 = wave_allreduce(t2, SumOp());
         if (wave_lane == 0) {
