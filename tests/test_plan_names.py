@@ -55,7 +55,7 @@ def test_single_read_paths_of_the_baseline_configs():
     assert fwd.startswith("slices=16:") and "channel_slices<" in fwd
     assert bwd.startswith("slices=18:") and "channel_slices<" in bwd
     assert K.plan_name("group_norm_forward", "bfloat16", (32, 32, 16, 4096), "NCHW").startswith(
-        "group_norm_forward_rows<1024,8,0>:")
+        "group_norm_forward_items<16,512>:")
     assert K.plan_name("group_norm_grad", "bfloat16", (32, 32, 16, 4096), "NCHW").startswith(
         "group_norm_grad_rows<1024,8,waves>:")
 
