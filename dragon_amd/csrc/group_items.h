@@ -15,6 +15,7 @@
 #pragma once
 
 #include "common.h"
+#include "sample_slices.h"  // wave_total
 
 namespace dragon_hip {
 

@@ -4008,7 +4008,7 @@ int make_shape(int64_t N, int64_t G, int64_t D, int64_t S, int layout, GroupShap
 
 // Exchange bytes of the sliced NHWC forward (0: the shape does not take that path).
 size_t sample_slices_forward_bytes(int dtype, const GroupShape& sh) {
-  SampleSlicePlan p{false, 0u, 0u, 0};
+  SampleSlicePlan p{};
   switch (dtype) {
     case DRAGON_HIP_F16: p = plan_sample_slices<f16_t>(sh.S, sh.C, sh.G, sh.D); break;
     case DRAGON_HIP_BF16: p = plan_sample_slices<bf16_t>(sh.S, sh.C, sh.G, sh.D); break;

@@ -33,6 +33,11 @@
 // and, for the groups its slice combines, writes the mean and rsig the
 // combiner did not. A flagged item wrote no output, so a call may run in place.
 //
+// A group is at least a packet wide. Where it is not whole packets (10, 12, 20
+// channels in 16-bit types) a packet may lie in two groups, never three; the
+// kTwo flavour then keeps two shares per thread (the elements below k0 belong to
+// group g, the others to g + 1) and picks mean and rsig per element.
+//
 // Partials are (mean, sum of squared deviations) of the slice's share of the
 // group, formed in two passes over the registers; the combiner adds them up with
 // the counts the slice geometry gives (slice_group_moments). Nothing depends on an element outside
