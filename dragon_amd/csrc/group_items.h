@@ -1,10 +1,10 @@
 // NCHW GroupNorm forward for groups that one 256- or 512-thread workgroup
-// holds whole (up to sixteen packets per thread: 64 or 128 KB in 16-bit types).
+// holds whole (up to sixteen packets per thread of 512: 128 KB in 16-bit types).
 //
 // A group (n, g) is a contiguous run of D * S elements. Thread t keeps packets
 // t, t + kThreads, ... of the group in registers between the statistics and the
-// normalisation, so x is read once. Four (256 threads) or two (512 threads)
-// workgroups share a compute unit at 128 registers, and a workgroup requests
+// normalisation, so x is read once. Two to seven workgroups share a compute
+// unit, by the packets a thread holds, and a workgroup requests
 // its next group's packets inside the store loop, slot by slot into the
 // registers each store frees, so that the workgroups of a compute unit overlap
 // their loads, reductions and stores. The channel of a packet does not depend on
@@ -22,8 +22,13 @@ namespace dragon_hip {
 constexpr int kItemPackets = 16;      // packets per thread at most
 constexpr uint32_t kMaxItemChannels = 512;  // channels per group whose parameters fit the LDS table
 
+// Wavefronts per SIMD asked of the compiler: four (128 registers) hold sixteen packets per
+// thread; ten packets fit the 80 registers of six, i.e. three 512-thread workgroups per compute
+// unit instead of two (groups of 80 KB in bf16: 58.0 us against 65.2 us).
+constexpr int item_waves_per_simd(int vpt) { return vpt == 10 ? 6 : vpt == 12 ? 5 : 4; }
+
 template <typename T, int kVPT, int kThreads>
-__global__ __launch_bounds__(kThreads, 4) void group_norm_forward_items(
+__global__ __launch_bounds__(kThreads, item_waves_per_simd(kVPT)) void group_norm_forward_items(
     const uint32_t rows, const uint32_t npackets, const uint32_t G, const uint32_t D,
     const uint32_t pps /* packets per channel */, const typename IO<T>::Acc eps,
     const T* __restrict__ x, const typename IO<T>::Acc* __restrict__ gamma,
@@ -148,8 +153,8 @@ struct GroupItemPlan {
   int threads, vpt;
 };
 
-// Groups of whole packets with channels of whole packets that 256 threads (up
-// to 64 KB in 16-bit types) or 512 threads hold at sixteen packets per thread.
+// Groups of whole packets with channels of whole packets that 256 threads hold at
+// ten packets per thread or 512 threads at sixteen.
 template <typename T>
 inline GroupItemPlan plan_group_items(int64_t D, int64_t S) {
   constexpr int kVec = IO<T>::kVec;
@@ -159,11 +164,19 @@ inline GroupItemPlan plan_group_items(int64_t D, int64_t S) {
   // smaller groups stay with the row kernels, which hold several per workgroup
   // (groups of 16 KB in 16-bit types: 45.6 us there against 50.5 us here)
   if (npackets < 256 * 8) return p;
-  for (const int threads : {256, 512}) {
-    if (npackets > static_cast<int64_t>(threads) * kItemPackets || D > threads) continue;
+  // The fewest packets per thread that hold the group, on 256 threads where ten packets do: the
+  // fewer registers, the more workgroups share a compute unit (seven at eight packets and six at
+  // ten on 256 threads; three, three, two and two at eight, ten, twelve and sixteen on 512), and
+  // what counts is the bytes they keep in flight together. Measured cold on MI355X, bf16, groups
+  // of 40 / 64 / 80 / 96 KB, the chosen flavour against sixteen packets on the smallest workgroup
+  // that holds the group: 59.5 / 46.9 / 58.1 / 52.2 us against 61.7 / 50.6 / 63.2 / 53.5 us.
+  struct Choice { int vpt, threads; };
+  constexpr Choice kChoices[] = {{8, 256}, {10, 256}, {8, 512}, {10, 512}, {12, 512}, {16, 512}};
+  for (const Choice& c : kChoices) {
+    if (npackets > static_cast<int64_t>(c.threads) * c.vpt || D > c.threads) continue;
     p.ok = true;
-    p.threads = threads;
-    p.vpt = static_cast<int>(ceil_div(npackets, threads)) <= 8 ? 8 : 16;
+    p.threads = c.threads;
+    p.vpt = c.vpt;
     return p;
   }
   return p;
@@ -195,9 +208,10 @@ int try_group_norm_forward_items(int64_t N, int64_t G, int64_t D, int64_t S, flo
                        static_cast<T*>(y));                                                       \
   }
     if (p.threads == 256) {
-      if (p.vpt == 8) LAUNCH(8, 256) else LAUNCH(16, 256)
+      if (p.vpt == 8) LAUNCH(8, 256) else LAUNCH(10, 256)
     } else {
-      if (p.vpt == 8) LAUNCH(8, 512) else LAUNCH(16, 512)
+      if (p.vpt == 8) LAUNCH(8, 512) else if (p.vpt == 10) LAUNCH(10, 512)
+      else if (p.vpt == 12) LAUNCH(12, 512) else LAUNCH(16, 512)
     }
 #undef LAUNCH
     return status_of_launch();

@@ -288,6 +288,9 @@ NCHW_ITEM_CASES = [
     (3, 2, 1, 65536, "float16", 0), (1, 5, 16, 4096, "bfloat16", 0), (2, 4, 8, 4096, "float32", 0),
     (700, 3, 4, 2048, "float32", 0), (2, 2, 256, 128, "bfloat16", 0), (2, 2, 300, 64, "float16", 0),
     (1, 3, 16, 4096, "bfloat16", 3), (2, 7, 3, 5464, "bfloat16", 0), (1100, 2, 8, 2048, "bfloat16", 0),
+    # every flavour: eight and ten packets on 256 threads, eight to sixteen on 512
+    (2, 2, 20, 1024, "bfloat16", 0), (3, 3, 10, 4096, "bfloat16", 0), (2, 2, 12, 4096, "float16", 0),
+    (2, 5, 10, 1000, "float32", 0), (2, 3, 11, 2048, "float32", 0), (40, 2, 5, 4096, "float32", 0),
 ]
 
 
