@@ -194,12 +194,25 @@ int try_group_norm_forward_items(int64_t N, int64_t G, int64_t D, int64_t S, flo
     const GroupItemPlan p = plan_group_items<T>(D, S);
     const int64_t rows = N * G;
     if (!p.ok || !aligned16(x) || !aligned16(y) || rows > 0x7fffffff) return kNotApplicable;
+    // A workgroup per group, handed out by the hardware as workgroups finish, keeps the memory
+    // system busier than resident workgroups that walk the groups and request one ahead, except
+    // for the 512-thread flavours with nearly every slot filled and fewer than four groups per
+    // resident workgroup (bf16, 2048 groups of 64 KB: 46.9 us walking against 49.2 us; 8192 groups
+    // of 40 KB on 256 threads: 238 us walking against 220 us). Measured cold on MI355X.
+    const int64_t npackets = D * S / kVec;
 #define LAUNCH(VPT, THREADS)                                                                      \
   {                                                                                               \
     auto kernel = group_norm_forward_items<T, VPT, THREADS>;                                      \
     const unsigned resident = resident_grid(kernel, THREADS, 0);                                  \
+    /* (decided on the three or two workgroups per compute unit the flavour is built for, so  */  \
+    /* that the choice does not depend on what the occupancy query answers)                   */  \
+    const int64_t nominal = static_cast<int64_t>(num_cus()) * (VPT <= 10 ? 3 : 2);                \
+    const bool walk = THREADS == 512 && npackets * 4 > static_cast<int64_t>(THREADS) * VPT * 3 && \
+        rows < nominal * 4;                                                                       \
     note_flavour("group_norm_forward_items<" #VPT "," #THREADS ">");                              \
-    hipLaunchKernelGGL(kernel, dim3(rows < resident ? static_cast<unsigned>(rows) : resident),    \
+    note_number("walk", walk ? 1 : 0);                                                            \
+    hipLaunchKernelGGL(kernel,                                                                    \
+                       dim3(walk && rows > resident ? resident : static_cast<unsigned>(rows)),    \
                        dim3(THREADS), 0, stream, static_cast<uint32_t>(rows),                     \
                        static_cast<uint32_t>(D * S / kVec), static_cast<uint32_t>(G),             \
                        static_cast<uint32_t>(D), static_cast<uint32_t>(S / kVec), A(eps),         \
