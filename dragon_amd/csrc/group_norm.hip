@@ -1145,7 +1145,7 @@ enum ChannelMode {
 constexpr int kMaxEntryPackets = 4096;
 
 template <typename T, int kTPR, int kVPT, int kMode>
-__global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
+__global__ __launch_bounds__(kTPR, kTPR == 512 ? 4 : 1) void group_norm_grad_rows(
     const int64_t rows, const int L, const uint32_t G, const uint32_t D, const uint32_t S,
     const T* __restrict__ x, const T* __restrict__ dy,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ mu,
@@ -1222,8 +1222,58 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
 
     A gam[kVPT];
     A s1 = A(0), s2 = A(0);
+    if constexpr (kLanes) {
+      // A channel is packets_per_chan (a power of two below 64) adjacent lanes of a slot. The
+      // slots' sums of dy x and dy are added up over them with xor-shuffles, four slots' worth
+      // in flight together (one slot after the other, between the stores of the second pass,
+      // each shuffle waited for the one before it), and the channel's first lane writes its
+      // (dgamma, dbeta) share, (sum(dy x) - mu sum(dy)) rsig as the CPU kernel forms it per (n, c).
+      constexpr int kBatch = kVPT >= 4 ? 4 : kVPT;
+      const size_t n = static_cast<size_t>(row / G);
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i) {
+      for (int b = 0; b < kVPT; b += kBatch) {
+        A chan1[kBatch], chan2[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          const int i = b + j;
+          const uint32_t chan = static_cast<uint32_t>(i * kTPR + lane) / packets_per_chan;
+          gam[i] = gamma[c0 + (chan < D ? chan : D - 1)];
+          A p1 = A(0), p2 = A(0);
+          if (Tile::active(i, npackets)) {
+            A xv[kVec], dv[kVec];
+            tx.unpack(i, xv);
+            tdy.unpack(i, dv);
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) {
+              p1 += dv[e] * xv[e];
+              p2 += dv[e];
+            }
+          }
+          s1 += gam[i] * p1;
+          s2 += gam[i] * p2;
+          chan1[j] = p1, chan2[j] = p2;
+        }
+        for (uint32_t o = 1; o < packets_per_chan; o <<= 1) {
+#pragma unroll
+          for (int j = 0; j < kBatch; ++j) {
+            chan1[j] += __shfl_xor(chan1[j], static_cast<int>(o), kWaveSize);
+            chan2[j] += __shfl_xor(chan2[j], static_cast<int>(o), kWaveSize);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          const int i = b + j;
+          const uint32_t packet = static_cast<uint32_t>(i * kTPR + lane);
+          if ((packet & (packets_per_chan - 1)) == 0 && Tile::active(i, npackets)) {
+            A* o = partial + (n * G * D + c0 + packet / packets_per_chan) * 2;
+            o[0] = (chan1[j] - m * chan2[j]) * r;
+            o[1] = chan2[j];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < (kLanes ? 0 : kVPT); ++i) {
       if constexpr (kAnyS) {
         uint32_t chan, in_first;
         first_channel_elems(i, chan, in_first);
@@ -1255,8 +1305,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           }
         }
       } else if constexpr (kLanes) {
-        const uint32_t chan = static_cast<uint32_t>(i * kTPR + lane) / packets_per_chan;
-        gam[i] = gamma[c0 + (chan < D ? chan : D - 1)];
+        // (handled above)
       } else if constexpr (kWholeWaves) {
         uint32_t chan, in_first;
         first_channel(i, chan, in_first);
@@ -1289,7 +1338,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           gam[i] = static_cast<uint32_t>(wave_lane) < in_first ? gam[i] : second;
         }
       }
-      if (!kAnyS && !kWholeWaves && Tile::active(i, npackets)) {
+      if (!kAnyS && !kWholeWaves && !kLanes && Tile::active(i, npackets)) {
         // gamma is one value per thread and slot: it multiplies the slot's sums once
         A xv[kVec], dv[kVec];
         tx.unpack(i, xv);
@@ -1323,14 +1372,14 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
     // dx = gamma*rsig * dy + (u*(x - mu) - v) with the row's u, v divided by D*S once
     const A u0 = (s2 * m - s1) * (r * r * r) * denom;
     const A v0 = s2 * r * denom;
-    const A w0 = -(u0 * m + v0);  // kWholeWaves: dx = gamma*rsig * dy + (u x + w)
+    const A w0 = -(u0 * m + v0);  // kWholeWaves, kLanes: dx = gamma*rsig * dy + (u x + w)
     tx.refresh();
     tdy.refresh();
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
       A t1 = A(0), t2 = A(0);
       A u1 = A(0), u2 = A(0);  // kAnyS: the second channel's share of a packet on the boundary
-      if constexpr (kWholeWaves) {
+      if constexpr (kWholeWaves || kLanes) {
         if (Tile::active(i, npackets)) {
           A xv[kVec], dv[kVec];
           tx.unpack(i, xv);
@@ -1412,18 +1461,7 @@ __global__ __launch_bounds__(kTPR) void group_norm_grad_rows(
           chan_part[i][wave][3] = b2;
         }
       } else if constexpr (kLanes) {
-        // packets_per_chan is a power of two below 64: xor-shuffles within the channel's lanes
-        for (uint32_t o = 1; o < packets_per_chan; o <<= 1) {
-          t1 += __shfl_xor(t1, static_cast<int>(o), kWaveSize);
-          t2 += __shfl_xor(t2, static_cast<int>(o), kWaveSize);
-        }
-        const uint32_t packet = static_cast<uint32_t>(i * kTPR + lane);
-        if ((packet & (packets_per_chan - 1)) == 0 && Tile::active(i, npackets)) {
-          const size_t n = static_cast<size_t>(row / G);
-          A* o = partial + (n * G * D + c0 + packet / packets_per_chan) * 2;
-          o[0] = t1;
-          o[1] = t2;
-        }
+        // (its channel sums left the first pass)
       } else if constexpr (kStraddle) {
         uint32_t chan, in_first;
         first_channel(i, chan, in_first);
@@ -2600,6 +2638,9 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
   constexpr int kVec = IO<T>::kVec;
   if (layout != DRAGON_HIP_NCHW || G * D == 1) return false;
   static const RowConfig table[] = {{256, 2}, {256, 4}, {256, 8}, {1024, 4}, {1024, 8}};
+  // (512 threads, two workgroups per compute unit at 128 registers, where 1024 threads with four
+  // packets each leave room for one; not for the entry-per-packet flavour)
+  static const RowConfig table512[] = {{256, 2}, {256, 4}, {256, 8}, {512, 8}, {1024, 8}};
   const int64_t per_chan = S / kVec;
   if (S % kVec == 0 && per_chan >= kWaveSize) {
     *mode = per_chan % kWaveSize == 0 ? kChannelWaves : kChannelStraddles;
@@ -2617,7 +2658,7 @@ bool plan_group_grad_rows(int64_t G, int64_t D, int64_t S, int layout, RowConfig
   }
   const int64_t npackets = D * S / kVec;
   if (npackets <= kWaveSize * 2) return false;  // a wavefront or two: the general path
-  for (const RowConfig& c : table) {
+  for (const RowConfig& c : *mode == kChannelPackets || sizeof(T) > 4 ? table : table512) {
     if (npackets <= static_cast<int64_t>(c.tpr) * c.vpt) {
       *cfg = c;
       return true;
@@ -3751,7 +3792,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
 #define LAUNCH(TPR, VPT)                                                                        \
   {                                                                                             \
   if (mode == kChannelPackets) {                                                                \
-    if constexpr (TPR * VPT <= kMaxEntryPackets) {                                              \
+    if constexpr (TPR * VPT <= kMaxEntryPackets && TPR != 512) {                                \
       note_flavour("group_norm_grad_rows_any<" #TPR "," #VPT ">");                              \
       auto kernel = group_norm_grad_rows_any<T, TPR, VPT>;                                      \
       const size_t lds = static_cast<size_t>(L / kVec) * 4 * sizeof(A);                         \
@@ -3775,6 +3816,7 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     if (gcfg.tpr == 256 && gcfg.vpt == 2) LAUNCH(256, 2)
     else if (gcfg.tpr == 256 && gcfg.vpt == 4) LAUNCH(256, 4)
     else if (gcfg.tpr == 256 && gcfg.vpt == 8) LAUNCH(256, 8)
+    else if (gcfg.tpr == 512 && gcfg.vpt == 8) LAUNCH(512, 8)
     else if (gcfg.tpr == 1024 && gcfg.vpt == 4) LAUNCH(1024, 4)
     else LAUNCH(1024, 8)
 #undef LAUNCH
