@@ -78,9 +78,16 @@ struct SampleSlices {
   uint32_t* gave_up_count;
 };
 
+// How a packet's channels lie in groups.
+enum SliceSplit {
+  kSplitNone = 0,  // groups of whole packets: a packet lies in one group
+  kSplitTwo = 1,   // groups of at least a packet that are not whole packets: in at most two
+  kSplitEach = 2   // groups of less than a packet: every channel of a packet finds its own group
+};
+
 struct SampleSlicePlan {
   bool ok;
-  bool two;  // D is not a multiple of a packet: a packet may lie in two groups
+  int split;  // SliceSplit
   uint32_t threads, K, rows;
   int vpt;  // packets per thread and tensor
 };
@@ -89,10 +96,9 @@ struct SampleSlicePlan {
 template <typename T>
 SampleSlicePlan plan_sample_slices(uint32_t S, uint32_t C, uint32_t G, uint32_t D) {
   constexpr uint32_t kVec = IO<T>::kVec;
-  SampleSlicePlan p{false, false, 0u, 0u, 0u, 0};
-  // (a group of less than a packet would put three groups or more into one packet)
-  if (sizeof(T) > 4 || S <= 1 || C % kVec != 0 || D < kVec) return p;
-  p.two = D % kVec != 0;
+  SampleSlicePlan p{false, kSplitNone, 0u, 0u, 0u, 0};
+  if (sizeof(T) > 4 || S <= 1 || C % kVec != 0) return p;
+  p.split = D % kVec == 0 ? kSplitNone : D > kVec ? kSplitTwo : kSplitEach;
   const uint32_t cps = C / kVec;
   if (G > kMaxSampleGroups) return p;
   // most of the workgroup's threads must have a row to hold
@@ -156,6 +162,7 @@ struct SliceSeat {
   uint32_t cps, rows_at_a_time, r, cp, g, lanes_per_group;
   uint32_t g1;  // where groups are not whole packets: the group of the packet's last channels,
   int k0;       // and how many of its channels lie in g (the first group)
+  uint32_t team;  // adjacent threads that add up one group's shares (a power of two, <= 64)
   bool on;
   __device__ explicit SliceSeat(const SampleSlices& d) {
     cps = d.C / kVec;
@@ -166,6 +173,8 @@ struct SliceSeat {
     g = on ? cp * kVec / d.D : 0u;
     k0 = static_cast<int>(min(static_cast<uint32_t>(kVec), (g + 1) * d.D - (on ? cp : 0u) * kVec));
     g1 = g + 1 < d.G ? g + 1 : g;
+    team = kWaveSize;
+    while (team > 1 && (team * d.G > d.threads || team > rows_at_a_time)) team >>= 1;
   }
 };
 
@@ -241,11 +250,36 @@ __device__ __forceinline__ bool await_pair(const float* slot, uint32_t patience,
   return await_pair(slot, patience, peek_pair(slot), a, b);
 }
 
-// The group's totals of kN values per thread, one LDS word per thread and
-// value: the thread that owns group t adds the R * (D / kVec) shares of its
-// group in row order and leaves the sums in total[j][t]. Every thread may read
-// total[j][*] afterwards; the barrier of the next call (or of the exchange)
-// lies between those reads and the next writes.
+// The group's totals of the threads' shares, one LDS word per thread and share. A team of
+// `at.team` adjacent threads adds up group t: member j takes rows j, j + team, ... of the rows
+// the workgroup holds at a time (`row_sum(g, rr)`: what row rr adds to group g, in a fixed
+// order), the members' sums meet in a butterfly of shuffles, and the team's first thread
+// leaves the total in total[j][t]. The order of the additions depends on the geometry alone.
+// Every thread may read total[j][*] afterwards; the barrier of the next call (or of the
+// exchange) lies between those reads and the next writes.
+template <int kN, int kVec, typename A, typename RowSum>
+__device__ __forceinline__ void slice_team_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                A (*total)[kMaxSliceThreads], RowSum row_sum) {
+  const uint32_t t = threadIdx.x;
+  const uint32_t g = t / at.team, j = t - g * at.team;
+  A acc[kN];
+#pragma unroll
+  for (int k = 0; k < kN; ++k) acc[k] = A(0);
+  if (g < d.G) {
+    for (uint32_t rr = j; rr < at.rows_at_a_time; rr += at.team) row_sum(g, rr, acc);
+  }
+  for (uint32_t o = 1; o < at.team; o <<= 1) {
+#pragma unroll
+    for (int k = 0; k < kN; ++k) acc[k] += __shfl_xor(acc[k], static_cast<int>(o), kWaveSize);
+  }
+  if (g < d.G && j == 0) {
+#pragma unroll
+    for (int k = 0; k < kN; ++k) total[k][g] = acc[k];
+  }
+  __syncthreads();
+}
+
+// Groups of whole packets: kN values per thread, all for the group of its packet.
 template <int kN, int kVec, typename A>
 __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
                                                  const A (&v)[kN], A (*part)[kMaxSliceThreads],
@@ -254,28 +288,18 @@ __device__ __forceinline__ void slice_group_sums(const SampleSlices& d, const Sl
 #pragma unroll
   for (int j = 0; j < kN; ++j) part[j][t] = at.on ? v[j] : A(0);
   __syncthreads();
-  if (t < d.G) {
-    A acc[kN];
+  slice_team_sums<kN, kVec>(d, at, total, [&](uint32_t g, uint32_t rr, A (&acc)[kN]) {
+    const uint32_t first = rr * at.cps + g * at.lanes_per_group;
+    for (uint32_t c = 0; c < at.lanes_per_group; ++c) {
 #pragma unroll
-    for (int j = 0; j < kN; ++j) acc[j] = A(0);
-    for (uint32_t rr = 0; rr < at.rows_at_a_time; ++rr) {
-      const uint32_t first = rr * at.cps + t * at.lanes_per_group;
-#pragma unroll 8
-      for (uint32_t c = 0; c < at.lanes_per_group; ++c) {
-#pragma unroll
-        for (int j = 0; j < kN; ++j) acc[j] += part[j][first + c];
-      }
+      for (int j = 0; j < kN; ++j) acc[j] += part[j][first + c];
     }
-#pragma unroll
-    for (int j = 0; j < kN; ++j) total[j][t] = acc[j];
-  }
-  __syncthreads();
+  });
 }
 
-
 // The same where a packet may lie in two groups: v0 is the thread's share for the group of its
-// packet's first channel, v1 for the next group; the owner of group t adds the shares of the
-// packets that touch it (packet c starts in group t, or, only the first of them, before it).
+// packet's first channel, v1 for the next group; group g takes the shares of the packets that
+// touch it (packet c starts in group g, or, only the first of them, before it).
 template <int kVec, typename A>
 __device__ __forceinline__ void slice_group_sums_two(const SampleSlices& d, const SliceSeat<kVec>& at,
                                                      const A v0, const A v1,
@@ -285,18 +309,44 @@ __device__ __forceinline__ void slice_group_sums_two(const SampleSlices& d, cons
   part[0][t] = at.on ? v0 : A(0);
   part[1][t] = at.on ? v1 : A(0);
   __syncthreads();
-  if (t < d.G) {
-    const uint32_t lo = t * d.D / kVec, hi = ((t + 1) * d.D - 1) / kVec;
-    A acc = A(0);
-    for (uint32_t rr = 0; rr < at.rows_at_a_time; ++rr) {
-      for (uint32_t c = lo; c <= hi; ++c) {
-        const int share = c * kVec < t * d.D ? 1 : 0;
-        acc += part[share][rr * at.cps + c];
-      }
+  slice_team_sums<1, kVec>(d, at, total, [&](uint32_t g, uint32_t rr, A (&acc)[1]) {
+    const uint32_t lo = g * d.D / kVec, hi = ((g + 1) * d.D - 1) / kVec;
+    for (uint32_t c = lo; c <= hi; ++c) {
+      const int share = c * kVec < g * d.D ? 1 : 0;
+      acc[0] += part[share][rr * at.cps + c];
     }
-    total[0][t] = acc;
-  }
+  });
+}
+
+// The same where groups are narrower than a packet: a share per channel of the packet; group g
+// takes the shares of its D channels.
+template <int kVec, typename A>
+__device__ __forceinline__ void slice_group_sums_each(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                      const A (&v)[kVec],
+                                                      A (*each)[kMaxSliceThreads],
+                                                      A (*total)[kMaxSliceThreads]) {
+  const uint32_t t = threadIdx.x;
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) each[e][t] = at.on ? v[e] : A(0);
   __syncthreads();
+  slice_team_sums<1, kVec>(d, at, total, [&](uint32_t g, uint32_t rr, A (&acc)[1]) {
+    for (uint32_t ch = g * d.D; ch < (g + 1) * d.D; ++ch) {
+      acc[0] += each[ch % kVec][rr * at.cps + ch / kVec];
+    }
+  });
+}
+
+// The groups of the kVec channels of the thread's packet (kSplitEach).
+template <int kVec>
+__device__ __forceinline__ void slice_channel_groups(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                     uint32_t (&ge)[kVec]) {
+  uint32_t g = at.g, r = (at.on ? at.cp : 0u) * kVec - at.g * d.D;  // r < D
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) {
+    if (r >= d.D) r -= d.D, ++g;
+    ge[e] = g < d.G ? g : d.G - 1;
+    ++r;
+  }
 }
 
 // The sum of v over the wavefront, the same bits in every lane (each step adds
@@ -435,18 +485,24 @@ __device__ __forceinline__ bool slice_totals(const SampleSlices& d, const SliceI
 // ---------------------------------------------------------------- forward
 // The slice's share of each group: its mean, then its squared deviations from
 // that mean; the owner threads publish them.
-template <typename T, int kVPT, bool kTwo>
+template <typename T, int kVPT, int kSplit>
 __device__ __forceinline__ void slice_forward_stats(
     const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w,
     const typename IO<T>::Acc eps, typename IO<T>::Acc* mu, typename IO<T>::Acc* rsig,
-    typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds) {
+    typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds,
+    typename IO<T>::Acc (*each)[kMaxSliceThreads]) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
+  constexpr bool kTwo = kSplit == kSplitTwo, kEach = kSplit == kSplitEach;
+  constexpr int kShares = kEach ? kVec : 2;
   const SliceItem it(d, w);
   const uint32_t t = threadIdx.x;
   const A inv_cnt = A(1) / A(it.nrows * d.D);
-  // (kTwo: s[0] for the group of the packet's first channel, s[1] for the next one)
-  A s[2] = {A(0), A(0)};
+  // (kTwo: s[0] for the group of the packet's first channel, s[1] for the next one; kEach: a
+  // share per channel)
+  A s[kShares];
+#pragma unroll
+  for (int j = 0; j < kShares; ++j) s[j] = A(0);
   int room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
@@ -458,24 +514,43 @@ __device__ __forceinline__ void slice_forward_stats(
       IO<T>::unpack(raw[i], v);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        if (!kTwo || e < at.k0) s[0] += v[e]; else s[1] += v[e];
+        if constexpr (kEach) {
+          s[e] += v[e];
+        } else {
+          if (!kTwo || e < at.k0) s[0] += v[e]; else s[1] += v[e];
+        }
       }
     }
   }
-  if constexpr (kTwo) {
-    slice_group_sums_two<kVec>(d, at, s[0], s[1], lds.part, lds.total);
-  } else {
-    const A one[1] = {s[0]};
-    slice_group_sums<1, kVec>(d, at, one, lds.part, lds.total);
-  }
+  auto group_sums = [&]() {
+    if constexpr (kEach) {
+      slice_group_sums_each<kVec>(d, at, s, each, lds.total);
+    } else if constexpr (kTwo) {
+      slice_group_sums_two<kVec>(d, at, s[0], s[1], lds.part, lds.total);
+    } else {
+      const A one[1] = {s[0]};
+      slice_group_sums<1, kVec>(d, at, one, lds.part, lds.total);
+    }
+  };
+  group_sums();
   A pa = A(0), pb = A(0);
   if (t < d.G) pa = lds.total[0][t] * inv_cnt;
-  const A mean_k = lds.total[0][at.g] * inv_cnt;
-  const A mean_k1 = kTwo ? lds.total[0][at.g1] * inv_cnt : A(0);
+  // the slice's mean of each share's group
+  A mean_k[kShares];
+  if constexpr (kEach) {
+    uint32_t ge[kVec];
+    slice_channel_groups<kVec>(d, at, ge);
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) mean_k[e] = lds.total[0][ge[e]] * inv_cnt;
+  } else {
+    mean_k[0] = lds.total[0][at.g] * inv_cnt;
+    mean_k[1] = kTwo ? lds.total[0][at.g1] * inv_cnt : A(0);
+  }
   // convert the packets again in each pass instead of keeping every converted element
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
-  s[0] = s[1] = A(0);
+#pragma unroll
+  for (int j = 0; j < kShares; ++j) s[j] = A(0);
   room = slice_room(at, it);
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) {
@@ -487,22 +562,20 @@ __device__ __forceinline__ void slice_forward_stats(
       IO<T>::unpack(raw[i], v);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) {
-        if (!kTwo || e < at.k0) {
-          const A dv = v[e] - mean_k;
+        if constexpr (kEach) {
+          const A dv = v[e] - mean_k[e];
+          s[e] += dv * dv;
+        } else if (!kTwo || e < at.k0) {
+          const A dv = v[e] - mean_k[0];
           s[0] += dv * dv;
         } else {
-          const A dv = v[e] - mean_k1;
+          const A dv = v[e] - mean_k[1];
           s[1] += dv * dv;
         }
       }
     }
   }
-  if constexpr (kTwo) {
-    slice_group_sums_two<kVec>(d, at, s[0], s[1], lds.part, lds.total);
-  } else {
-    const A one[1] = {s[0]};
-    slice_group_sums<1, kVec>(d, at, one, lds.part, lds.total);
-  }
+  group_sums();
   if (t < d.G) pb = lds.total[0][t];
 #pragma unroll
   for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(raw[i]));
@@ -520,7 +593,7 @@ __device__ __forceinline__ void slice_forward_stats(
 }
 
 // Totals of item w, its rows out of `raw`, and item `reload` (if below d.items) into `raw`.
-template <typename T, int kVPT, bool kRepair, bool kTwo>
+template <typename T, int kVPT, bool kRepair, int kSplit>
 __device__ __forceinline__ void slice_forward_finish(
     const SampleSlices& d, const SliceSeat<IO<T>::kVec>& at, uint32_t w, uint32_t reload,
     const typename IO<T>::Acc eps, const T* x, const typename IO<T>::Acc* gamma,
@@ -528,6 +601,7 @@ __device__ __forceinline__ void slice_forward_finish(
     typename IO<T>::Acc* exchange, u32x4 (&raw)[kVPT], SliceLds<typename IO<T>::Acc>& lds) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
+  constexpr bool kTwo = kSplit == kSplitTwo, kEach = kSplit == kSplitEach;
   const SliceItem it(d, w);
   const bool complete = slice_totals<kRepair>(d, it, w, eps, exchange, mu, rsig, lds);
   const A mean = lds.total[0][at.g], rs = lds.total[1][at.g];
@@ -548,8 +622,19 @@ __device__ __forceinline__ void slice_forward_finish(
     A gam[kVec], bet[kVec];
     load_params_ragged<kVec>(gp, kVec, gam);
     load_params_ragged<kVec>(bp, kVec, bet);
+    A mean_e[kEach ? kVec : 1];  // kEach: the mean of each channel's group
+    if constexpr (kEach) {
+      uint32_t ge[kVec];
+      slice_channel_groups<kVec>(d, at, ge);
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) gam[e] *= !kTwo || e < at.k0 ? rs : rs1;
+      for (int e = 0; e < kVec; ++e) {
+        mean_e[e] = lds.total[0][ge[e]];
+        gam[e] *= lds.total[1][ge[e]];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) gam[e] *= !kTwo || e < at.k0 ? rs : rs1;
+    }
     int room = complete ? slice_room(at, it) : 0, nroom = slice_room(at, nit);
     uint32_t off = first, noff = nfirst;
 #pragma unroll
@@ -559,7 +644,11 @@ __device__ __forceinline__ void slice_forward_finish(
         IO<T>::unpack(raw[i], v);
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          v[e] = (v[e] - (!kTwo || e < at.k0 ? mean : mean1)) * gam[e] + bet[e];
+          if constexpr (kEach) {
+            v[e] = (v[e] - mean_e[e]) * gam[e] + bet[e];
+          } else {
+            v[e] = (v[e] - (!kTwo || e < at.k0 ? mean : mean1)) * gam[e] + bet[e];
+          }
         }
         store_packet(y + off, IO<T>::pack(v));
       }
@@ -573,7 +662,7 @@ __device__ __forceinline__ void slice_forward_finish(
 
 // One item at a time per workgroup; the next item's packets are requested while
 // this one's are stored.
-template <typename T, int kVPT, int kThreads, bool kTwo>
+template <typename T, int kVPT, int kThreads, int kSplit>
 __global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
@@ -581,20 +670,22 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices(
     T* __restrict__ y, typename IO<T>::Acc* __restrict__ exchange) {
   using A = typename IO<T>::Acc;
   __shared__ SliceLds<A> lds;
+  // (a word per thread and channel of its packet where groups are narrower than a packet)
+  __shared__ A each[kSplit == kSplitEach ? IO<T>::kVec : 1][kMaxSliceThreads];
   const SliceSeat<IO<T>::kVec> at(d);
   const uint32_t step = gridDim.x;
   uint32_t w = blockIdx.x;
   u32x4 one[kVPT];
   if (w < d.items) slice_load<T, kVPT>(d, at, SliceItem(d, w), x, one);
   for (; w < d.items; w += step) {
-    slice_forward_stats<T, kVPT, kTwo>(d, at, w, eps, mu, rsig, exchange, one, lds);
-    slice_forward_finish<T, kVPT, false, kTwo>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig, y,
-                                         exchange, one, lds);
+    slice_forward_stats<T, kVPT, kSplit>(d, at, w, eps, mu, rsig, exchange, one, lds, each);
+    slice_forward_finish<T, kVPT, false, kSplit>(d, at, w, w + step, eps, x, gamma, beta, mu, rsig,
+                                                 y, exchange, one, lds);
   }
 }
 
 // The launch behind it: nothing to do unless a wait of the first launch ran out.
-template <typename T, int kVPT, int kThreads, bool kTwo>
+template <typename T, int kVPT, int kThreads, int kSplit>
 __global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices_repair(
     const SampleSlices d, const typename IO<T>::Acc eps, const T* __restrict__ x,
     const typename IO<T>::Acc* __restrict__ gamma, const typename IO<T>::Acc* __restrict__ beta,
@@ -608,8 +699,8 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_nhwc_slices_repair(
     if (d.flags[w] == 0u) continue;  // the same word in every thread
     u32x4 raw[kVPT];
     slice_load<T, kVPT>(d, at, SliceItem(d, w), x, raw);
-    slice_forward_finish<T, kVPT, true, kTwo>(d, at, w, d.items, eps, x, gamma, beta, mu, rsig, y,
-                                        exchange, raw, lds);
+    slice_forward_finish<T, kVPT, true, kSplit>(d, at, w, d.items, eps, x, gamma, beta, mu, rsig, y,
+                                                exchange, raw, lds);
     __syncthreads();  // the next item rewrites the totals in LDS
   }
 }
@@ -654,9 +745,9 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     }
     A* exchange = p.K > 1 ? static_cast<A*>(scratch) : nullptr;
     const SampleSlices d = make_sample_slices<T>(N, S, C, G, D, p, exchange);
-#define LAUNCH_T(VPT, THREADS, TWO)                                                                   \
+#define LAUNCH_T(VPT, THREADS, SPLIT)                                                             \
   {                                                                                               \
-    auto kernel = group_norm_nhwc_slices<T, VPT, THREADS, TWO>;                                   \
+    auto kernel = group_norm_nhwc_slices<T, VPT, THREADS, SPLIT>;                                 \
     unsigned cap = resident_grid(kernel, THREADS, 0);                                             \
     if (cap > sample_slices_max_grid()) cap = sample_slices_max_grid();                           \
     if (p.K > cap) return kNotApplicable;                                                         \
@@ -666,8 +757,9 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     /* (bf16 [8192, 7*7, 256] 77.6 -> 71.2 us; with two per workgroup 48.9 against 50.6 us). */ \
     const bool walk = p.K > 1 || d.items < 4u * num_cus() * (THREADS == 256 ? 4u : 2u);          \
     if (!walk) cap = d.items;                                                                     \
-    note_flavour(TWO ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",two>"                        \
-                     : "group_norm_nhwc_slices<" #VPT "," #THREADS ">");                          \
+    note_flavour(SPLIT == kSplitEach ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",each>"       \
+                 : SPLIT == kSplitTwo ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",two>"       \
+                                      : "group_norm_nhwc_slices<" #VPT "," #THREADS ">");         \
     note_number("slices", p.K);                                                                   \
     if (p.K == 1) note_number("walk", walk ? 1 : 0);                                              \
     if (p.K > 1) fill_sample_exchange(exchange, d, stream);                                       \
@@ -677,7 +769,7 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
                        static_cast<T*>(y), exchange);                                             \
     if (p.K > 1) {                                                                                \
       /* (the widest flavour serves every plan: a repair is rare, its speed does not matter) */   \
-      hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets, THREADS, TWO>),         \
+      hipLaunchKernelGGL((group_norm_nhwc_slices_repair<T, kSlicePackets, THREADS, SPLIT>),       \
                          dim3(d.items < kSliceRepairGrid ? d.items : kSliceRepairGrid),           \
                          dim3(THREADS), 0, stream, d, A(eps), static_cast<const T*>(x),           \
                          static_cast<const A*>(gamma), static_cast<const A*>(beta),               \
@@ -685,8 +777,12 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
                          exchange);                                                               \
     }                                                                                             \
   }
-#define LAUNCH(VPT, THREADS) \
-  { if (p.two) LAUNCH_T(VPT, THREADS, true) else LAUNCH_T(VPT, THREADS, false) }
+#define LAUNCH(VPT, THREADS)                                                   \
+  {                                                                            \
+    if (p.split == kSplitEach) LAUNCH_T(VPT, THREADS, kSplitEach)              \
+    else if (p.split == kSplitTwo) LAUNCH_T(VPT, THREADS, kSplitTwo)           \
+    else LAUNCH_T(VPT, THREADS, kSplitNone)                                    \
+  }
     if (p.threads == 256) {
       if (p.vpt <= 8) LAUNCH(8, 256) else LAUNCH(16, 256)
     } else {

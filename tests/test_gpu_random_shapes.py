@@ -243,6 +243,11 @@ NHWC_SLICE_CASES = [
     # groups of 10, 12 and 20 channels: a packet may lie in two groups (one slice and several)
     (2, 32, 10, 1030, "bfloat16", 0), (3, 32, 20, 300, "float16", 0), (2, 16, 10, 2000, "float32", 0),
     (40, 32, 10, 64, "bfloat16", 0), (3, 8, 12, 5000, "bfloat16", 0),
+    # groups of 1-6 channels, narrower than a packet: every channel of a packet finds its own
+    # group (one slice and several, a group count that is not a power of two)
+    (3, 32, 3, 196, "bfloat16", 0), (2, 8, 4, 256, "bfloat16", 0), (2, 32, 6, 64, "float16", 0),
+    (2, 32, 2, 3136, "bfloat16", 0), (2, 16, 2, 1000, "float32", 0), (40, 32, 1, 64, "bfloat16", 0),
+    (2, 24, 3, 3000, "float32", 0), (5000, 8, 4, 16, "bfloat16", 0),
     # rows of 160, 320 and 384 packets: not sliced (too many idle threads), same answer
     (3, 32, 40, 777, "bfloat16", 0), (2, 32, 40, 600, "float32", 0), (2, 48, 64, 500, "float16", 0),
 ]
