@@ -3351,17 +3351,20 @@ bool try_group_norm_forward_nhwc_samples(const GroupShape& sh, float eps, const 
 
 // The backward the same way: x and dy of a sample in registers (up to eight
 // packets per thread each, samples of up to 128 KB per tensor), groups of at
-// least a packet; kTwo: a group need not be whole packets, so a packet may lie
+// least a packet; kSplitTwo: a group need not be whole packets, so a packet may lie
 // in two groups (elements below k0 in group g, the others in g + 1) and a thread
-// carries a share for each. ds / db per group are summed by the group's owner
-// thread out of one LDS word per thread and share; a thread's
+// carries a share for each; kSplitEach: groups narrower than a packet, a share per
+// channel of the packet (up to four packets per thread each). ds / db per group
+// are added up by a team of threads out of one LDS word per thread and share; a thread's
 // channels are the same for every sample it sees, so their dgamma / dbeta
 // shares stay in registers across samples and leave the workgroup once, as one
 // partial row of 2*C interleaved words per workgroup (summed by
 // sum_partial_rows). (Keeping the shares in LDS between samples instead, one
 // word per thread and share, freed no registers where they are short, in the
 // two-group flavour at eight packets per thread, and was not faster.)
-template <typename T, int kVPT, int kThreads, bool kTwo>
+constexpr uint32_t kMaxEachGroups = 256;     // groups narrower than a packet: groups and channels
+constexpr uint32_t kMaxEachChannels = 1024;  // whose statistics and coefficients fit the LDS tables
+template <typename T, int kVPT, int kThreads, int kSplit>
 __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     const uint32_t N, const uint32_t S, const uint32_t C, const uint32_t G, const uint32_t D,
     const T* __restrict__ x, const T* __restrict__ dy, const typename IO<T>::Acc* __restrict__ gamma,
@@ -3370,19 +3373,26 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     typename IO<T>::Acc* __restrict__ partial) {
   using A = typename IO<T>::Acc;
   constexpr int kVec = IO<T>::kVec;
-  __shared__ A part[kTwo ? 4 : 2][kThreads];
+  constexpr bool kTwo = kSplit == kSplitTwo, kEach = kSplit == kSplitEach;
+  __shared__ A part[kEach ? kVec : kTwo ? 4 : 2][kThreads];
   __shared__ A total[2][kThreads];
+  // kEach: the sample's mu / rsig per group, and the three coefficients of dx per channel. They
+  // wait in LDS, not in registers: what does not fit the registers is spilled to memory, and a
+  // reload inside the store loop queues behind the packets requested ahead.
+  __shared__ A stat[2][kEach ? kMaxEachGroups : 1];
+  __shared__ A coef[3][kEach ? kMaxEachChannels : 1];
   const uint32_t cps = C / kVec;
   const uint32_t rows_at_a_time = kThreads / cps;
   const uint32_t t = threadIdx.x;
   const uint32_t r = t / cps, cp = t - r * cps;
   const bool on = r < rows_at_a_time;
   const uint32_t lanes_per_group = D / kVec;  // (whole packets only)
+  const uint32_t team = team_size(G, rows_at_a_time, kThreads);
   uint32_t g, g1 = 0;
   int k0 = kVec;
-  if constexpr (kTwo) {
+  if constexpr (kSplit != kSplitNone) {
     g = on ? cp * kVec / D : 0u;
-    const uint32_t edge = (g + 1) * D - cp * kVec;  // >= 1
+    const uint32_t edge = (g + 1) * D - (on ? cp : 0u) * kVec;  // >= 1
     if (on && edge < static_cast<uint32_t>(kVec)) k0 = static_cast<int>(edge);
     g1 = k0 < kVec ? g + 1 : g;
   } else {
@@ -3411,75 +3421,138 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
     const size_t base = static_cast<size_t>(n) * S * C;
     const bool more = n + gridDim.x < N;  // uniform over the workgroup
     const size_t nbase = static_cast<size_t>(more ? n + gridDim.x : n) * S * C;
-    const A m = mu[static_cast<size_t>(n) * G + g], rs = rsig[static_cast<size_t>(n) * G + g];
-    const A mb = kTwo ? mu[static_cast<size_t>(n) * G + g1] : A(0);
-    const A rsb = kTwo ? rsig[static_cast<size_t>(n) * G + g1] : A(0);
-    A s1 = A(0), s2 = A(0), s1b = A(0), s2b = A(0);
+    A m = A(0), rs = A(0), mb = A(0), rsb = A(0), u0 = A(0), v0 = A(0), u0b = A(0), v0b = A(0);
+    if constexpr (kEach) {
+      if (t < G) {  // requested now, used after the sums
+        stat[0][t] = mu[static_cast<size_t>(n) * G + t];
+        stat[1][t] = rsig[static_cast<size_t>(n) * G + t];
+      }
+      // Groups narrower than a packet: every channel of the packet finds its own group. A
+      // channel's sums of dy x and dy over the thread's rows give its share of the group's ds /
+      // db (times gamma) and of dgamma / dbeta ((sum(dy x) - mu sum(dy)) rsig, as the CPU
+      // kernel forms them per (n, c)).
+      A a[kVec], b[kVec];
 #pragma unroll
-    for (int i = 0; i < kVPT; ++i) {
-      if (on && r + i * rows_at_a_time < S) {
-        A xv[kVec], dv[kVec];
-        IO<T>::unpack(rx[i], xv);
-        IO<T>::unpack(rd[i], dv);
+      for (int e = 0; e < kVec; ++e) a[e] = b[e] = A(0);
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) {
-          const A gd = gam[e] * dv[e];
-          if (!kTwo || e < k0) {
-            s1 += gd * xv[e];
-            s2 += gd;
-            t1[e] += dv[e] * (xv[e] - m) * rs;
-          } else {
-            s1b += gd * xv[e];
-            s2b += gd;
-            t1[e] += dv[e] * (xv[e] - mb) * rsb;
+      for (int i = 0; i < kVPT; ++i) {
+        // (one packet at a time: converted all at once they would not fit the registers)
+        asm volatile("" : "+v"(rx[i]), "+v"(rd[i]), "+v"(a[0]), "+v"(b[0]));
+        if (on && r + i * rows_at_a_time < S) {
+          A xv[kVec], dv[kVec];
+          IO<T>::unpack(rx[i], xv);
+          IO<T>::unpack(rd[i], dv);
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            a[e] += dv[e] * xv[e];
+            b[e] += dv[e];
           }
-          t2[e] += dv[e];
         }
       }
-    }
-    // the group's ds and db: one LDS word per thread, share and sum, added by the group's owner
-    // thread
-    part[0][t] = on ? s1 : A(0);
-    part[1][t] = on ? s2 : A(0);
-    if constexpr (kTwo) {
-      part[2][t] = on ? s1b : A(0);
-      part[3][t] = on ? s2b : A(0);
-    }
-    __syncthreads();
-    if (t < G) {
-      A a = A(0), b = A(0);
+      auto channels_of_group = [&](uint32_t gg, uint32_t rr, A (&acc)[1]) {
+        for (uint32_t ch = gg * D; ch < (gg + 1) * D; ++ch) {
+          acc[0] += part[ch % kVec][rr * cps + ch / kVec];
+        }
+      };
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) part[e][t] = on ? gam[e] * a[e] : A(0);
+      __syncthreads();
+      team_sums<1, A>(G, rows_at_a_time, team, total, channels_of_group);
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) part[e][t] = on ? gam[e] * b[e] : A(0);
+      __syncthreads();
+      team_sums<1, A>(G, rows_at_a_time, team, total + 1, channels_of_group);
+      if (t < G) {
+        ds[static_cast<size_t>(n) * G + t] = total[0][t];
+        db[static_cast<size_t>(n) * G + t] = total[1][t];
+      }
+      // dx = c1 dy + (c2 x + c3) with coefficients per channel: the threads of the first row
+      // leave them in LDS for everybody
+      uint32_t gc = g, rem = (on ? cp : 0u) * kVec - g * D;  // rem < D
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        if (rem >= D) rem -= D, ++gc;
+        const uint32_t ge = gc < G ? gc : G - 1;
+        ++rem;
+        const A me = stat[0][ge], re = stat[1][ge];
+        if (t < cps) {
+          const A q1 = total[0][ge], q2 = total[1][ge];
+          const A u = (q2 * me - q1) * (re * re * re) * denom;
+          coef[0][t * kVec + e] = gam[e] * re;
+          coef[1][t * kVec + e] = u;
+          coef[2][t * kVec + e] = -(u * me + q2 * re * denom);
+        }
+        t1[e] += (a[e] - me * b[e]) * re;
+        t2[e] += b[e];
+      }
+      __syncthreads();
+    } else {
+      m = mu[static_cast<size_t>(n) * G + g], rs = rsig[static_cast<size_t>(n) * G + g];
+      mb = kTwo ? mu[static_cast<size_t>(n) * G + g1] : A(0);
+      rsb = kTwo ? rsig[static_cast<size_t>(n) * G + g1] : A(0);
+      A s1 = A(0), s2 = A(0), s1b = A(0), s2b = A(0);
+#pragma unroll
+      for (int i = 0; i < kVPT; ++i) {
+        if (on && r + i * rows_at_a_time < S) {
+          A xv[kVec], dv[kVec];
+          IO<T>::unpack(rx[i], xv);
+          IO<T>::unpack(rd[i], dv);
+#pragma unroll
+          for (int e = 0; e < kVec; ++e) {
+            const A gd = gam[e] * dv[e];
+            if (!kTwo || e < k0) {
+              s1 += gd * xv[e];
+              s2 += gd;
+              t1[e] += dv[e] * (xv[e] - m) * rs;
+            } else {
+              s1b += gd * xv[e];
+              s2b += gd;
+              t1[e] += dv[e] * (xv[e] - mb) * rsb;
+            }
+            t2[e] += dv[e];
+          }
+        }
+      }
+      // the group's ds and db: one LDS word per thread, share and sum, added up by the group's
+      // team of threads
+      part[0][t] = on ? s1 : A(0);
+      part[1][t] = on ? s2 : A(0);
+      if constexpr (kTwo) {
+        part[2][t] = on ? s1b : A(0);
+        part[3][t] = on ? s2b : A(0);
+      }
+      __syncthreads();
       if constexpr (kTwo) {
         // packets lo..hi hold the group's channels; one that begins before the group gives its
         // second share
-        const uint32_t lo = t * D / kVec, hi = ((t + 1) * D - 1) / kVec;
-        for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+        team_sums<2, A>(G, rows_at_a_time, team, total, [&](uint32_t gg, uint32_t rr, A (&acc)[2]) {
+          const uint32_t lo = gg * D / kVec, hi = ((gg + 1) * D - 1) / kVec;
           for (uint32_t c = lo; c <= hi; ++c) {
-            const int share = c * kVec < t * D ? 2 : 0;
-            a += part[share][rr * cps + c];
-            b += part[share + 1][rr * cps + c];
+            const int share = c * kVec < gg * D ? 2 : 0;
+            acc[0] += part[share][rr * cps + c];
+            acc[1] += part[share + 1][rr * cps + c];
           }
-        }
+        });
       } else {
-        for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
+        team_sums<2, A>(G, rows_at_a_time, team, total, [&](uint32_t gg, uint32_t rr, A (&acc)[2]) {
           for (uint32_t k = 0; k < lanes_per_group; ++k) {
-            a += part[0][rr * cps + t * lanes_per_group + k];
-            b += part[1][rr * cps + t * lanes_per_group + k];
+            acc[0] += part[0][rr * cps + gg * lanes_per_group + k];
+            acc[1] += part[1][rr * cps + gg * lanes_per_group + k];
           }
-        }
+        });
       }
-      total[0][t] = a, total[1][t] = b;
-      ds[static_cast<size_t>(n) * G + t] = a;
-      db[static_cast<size_t>(n) * G + t] = b;
-    }
-    __syncthreads();
-    s1 = total[0][g], s2 = total[1][g];
-    const A u0 = (s2 * m - s1) * (rs * rs * rs) * denom;
-    const A v0 = s2 * rs * denom;
-    A u0b = A(0), v0b = A(0);
-    if constexpr (kTwo) {
-      s1b = total[0][g1], s2b = total[1][g1];
-      u0b = (s2b * mb - s1b) * (rsb * rsb * rsb) * denom;
-      v0b = s2b * rsb * denom;
+      if (t < G) {
+        ds[static_cast<size_t>(n) * G + t] = total[0][t];
+        db[static_cast<size_t>(n) * G + t] = total[1][t];
+      }
+      s1 = total[0][g], s2 = total[1][g];
+      u0 = (s2 * m - s1) * (rs * rs * rs) * denom;
+      v0 = s2 * rs * denom;
+      if constexpr (kTwo) {
+        s1b = total[0][g1], s2b = total[1][g1];
+        u0b = (s2b * mb - s1b) * (rsb * rsb * rsb) * denom;
+        v0b = s2b * rsb * denom;
+      }
     }
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) asm volatile("" : "+v"(rx[i]), "+v"(rd[i]));
@@ -3492,9 +3565,15 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
         A xv[kVec], dv[kVec];
         IO<T>::unpack(rx[i], xv);
         IO<T>::unpack(rd[i], dv);
+        // (read again for every packet: hoisted out of the loop they would be 3 * kVec registers)
+        uint32_t ch0 = cp * kVec;
+        asm volatile("" : "+v"(ch0));
 #pragma unroll
         for (int e = 0; e < kVec; ++e) {
-          if (!kTwo || e < k0) {
+          if constexpr (kEach) {
+            const uint32_t ch = ch0 + e;
+            xv[e] = coef[0][ch] * dv[e] + (coef[1][ch] * xv[e] + coef[2][ch]);
+          } else if (!kTwo || e < k0) {
             xv[e] = gam[e] * rs * dv[e] + (u0 * (xv[e] - m) - v0);
           } else {
             xv[e] = gam[e] * rsb * dv[e] + (u0b * (xv[e] - mb) - v0b);
@@ -3512,16 +3591,17 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
   }
   // this workgroup's partial row: per channel, the shares of its row threads in row order
   A* row = partial + static_cast<size_t>(blockIdx.x) * 2 * C;
+  A (*lds)[kThreads] = part;
 #pragma unroll
   for (int e = 0; e < kVec; ++e) {
-    part[0][t] = on ? t1[e] : A(0);
-    part[1][t] = on ? t2[e] : A(0);
+    lds[0][t] = on ? t1[e] : A(0);
+    lds[1][t] = on ? t2[e] : A(0);
     __syncthreads();
     if (t < cps) {
       A a = A(0), b = A(0);
       for (uint32_t rr = 0; rr < rows_at_a_time; ++rr) {
-        a += part[0][rr * cps + t];
-        b += part[1][rr * cps + t];
+        a += lds[0][rr * cps + t];
+        b += lds[1][rr * cps + t];
       }
       row[2 * (t * kVec + e)] = a;
       row[2 * (t * kVec + e) + 1] = b;
@@ -3536,17 +3616,25 @@ __global__ __launch_bounds__(kThreads, 4) void group_norm_grad_nhwc_samples(
 template <typename T>
 int group_norm_grad_nhwc_samples_threads(const GroupShape& sh, int* slots_out) {
   constexpr int kVec = IO<T>::kVec;
-  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0 || sh.D < kVec) return 0;
+  if (sizeof(T) > 4 || sh.nchw || sh.S <= 1 || sh.C % kVec != 0) return 0;
+  if (sh.G > 256) return 0;  // (a team of threads per group)
+  if (sh.D < kVec && sh.C > kMaxEachChannels) return 0;
   const uint32_t cps = sh.C / kVec;
-  for (const uint32_t threads : {256u, 512u, 1024u}) {
-    if (cps > threads) continue;
-    const uint32_t rows_at_a_time = threads / cps;
-    const int64_t slots = ceil_div(sh.S, rows_at_a_time);
-    if (slots > 8) continue;
-    // most of the workgroup's threads must have a row to hold
-    if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < threads * 3) continue;
-    *slots_out = static_cast<int>(slots);
-    return static_cast<int>(threads);
+  // Groups narrower than a packet keep a sum of dy x and of dy per channel: four packets per
+  // thread and tensor at most (80 bytes per thread are spilled there in 16-bit types, outside
+  // the store loop; the smaller workgroup is still ahead of two packets on twice the threads:
+  // bf16 [8192,16*16,32] 106 against 119 us).
+  for (const int64_t most : {sh.D < kVec ? 4 : 8}) {
+    for (const uint32_t threads : {256u, 512u, 1024u}) {
+      if (cps > threads) continue;
+      const uint32_t rows_at_a_time = threads / cps;
+      const int64_t slots = ceil_div(sh.S, rows_at_a_time);
+      if (slots > most) continue;
+      // most of the workgroup's threads must have a row to hold
+      if (static_cast<int64_t>(cps) * rows_at_a_time * 4 < threads * 3) continue;
+      *slots_out = static_cast<int>(slots);
+      return static_cast<int>(threads);
+    }
   }
   return 0;
 }
@@ -3838,11 +3926,14 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       unsigned grid = 0;
 #define LAUNCH(VPT, THREADS)                                                                     \
   {                                                                                              \
-    const bool two = sh.D % kVec != 0; /* a packet may lie in two groups */                      \
-    note_flavour(two ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",two>"                 \
-                     : "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");                   \
-    auto kernel = two ? group_norm_grad_nhwc_samples<T, VPT, THREADS, true>                      \
-                      : group_norm_grad_nhwc_samples<T, VPT, THREADS, false>;                    \
+    /* how a packet's channels lie in groups */                                                  \
+    const int split = sh.D % kVec == 0 ? kSplitNone : sh.D > kVec ? kSplitTwo : kSplitEach;      \
+    note_flavour(split == kSplitEach ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",each>" \
+                 : split == kSplitTwo ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",two>" \
+                                      : "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");  \
+    auto kernel = split == kSplitEach ? group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitEach> \
+        : split == kSplitTwo ? group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitTwo>          \
+                             : group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitNone>;        \
     const unsigned resident = resident_grid(kernel, THREADS, 0);                                 \
     grid = nhwc_sample_rows(sh.N);                                                               \
     if (grid > resident) grid = resident;                                                        \
@@ -3852,7 +3943,24 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
       if (threads == 256) {
         if (slots <= 2) LAUNCH(2, 256) else if (slots <= 4) LAUNCH(4, 256) else LAUNCH(8, 256)
       } else if (threads == 512) {
-        LAUNCH(8, 512)  // (a sample of four packets per thread or fewer fits 256 threads)
+        // (with groups of a packet or more, a sample of four packets per thread or fewer fits
+        // 256 threads; narrower groups look for two packets per thread first)
+        if (slots <= 4 && sh.D < static_cast<uint32_t>(kVec)) {
+#define LAUNCH_EACH(VPT)                                                                         \
+  {                                                                                              \
+    note_flavour("group_norm_grad_nhwc_samples<" #VPT ",512,each>");                             \
+    auto kernel = group_norm_grad_nhwc_samples<T, VPT, 512, kSplitEach>;                         \
+    const unsigned resident = resident_grid(kernel, 512, 0);                                     \
+    grid = nhwc_sample_rows(sh.N);                                                               \
+    if (grid > resident) grid = resident;                                                        \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), 0, stream, sh.N, sh.S, sh.C, sh.G, sh.D,   \
+                       xp, dyp, gp, mup, rsp, dsp, dbp, dxp, part);                              \
+  }
+          if (slots <= 2) LAUNCH_EACH(2) else LAUNCH_EACH(4)
+#undef LAUNCH_EACH
+        } else {
+          LAUNCH(8, 512)
+        }
       } else {
         if (slots <= 2) LAUNCH(2, 1024) else if (slots <= 4) LAUNCH(4, 1024) else LAUNCH(8, 1024)
       }

@@ -156,6 +156,14 @@ SampleSlices make_sample_slices(uint32_t N, uint32_t S, uint32_t C, uint32_t G, 
   return d;
 }
 
+// Threads that add up one group's shares together (a power of two, adjacent lanes of one
+// wavefront): the team size for G groups, `rows` rows at a time and a workgroup of `threads`.
+__host__ __device__ inline uint32_t team_size(uint32_t G, uint32_t rows, uint32_t threads) {
+  uint32_t team = kWaveSize;
+  while (team > 1 && (team * G > threads || team > rows)) team >>= 1;
+  return team;
+}
+
 // Where a thread sits in its workgroup's slice.
 template <int kVec>
 struct SliceSeat {
@@ -173,8 +181,7 @@ struct SliceSeat {
     g = on ? cp * kVec / d.D : 0u;
     k0 = static_cast<int>(min(static_cast<uint32_t>(kVec), (g + 1) * d.D - (on ? cp : 0u) * kVec));
     g1 = g + 1 < d.G ? g + 1 : g;
-    team = kWaveSize;
-    while (team > 1 && (team * d.G > d.threads || team > rows_at_a_time)) team >>= 1;
+    team = team_size(d.G, rows_at_a_time, d.threads);
   }
 };
 
@@ -257,26 +264,31 @@ __device__ __forceinline__ bool await_pair(const float* slot, uint32_t patience,
 // leaves the total in total[j][t]. The order of the additions depends on the geometry alone.
 // Every thread may read total[j][*] afterwards; the barrier of the next call (or of the
 // exchange) lies between those reads and the next writes.
-template <int kN, int kVec, typename A, typename RowSum>
-__device__ __forceinline__ void slice_team_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
-                                                A (*total)[kMaxSliceThreads], RowSum row_sum) {
+template <int kN, typename A, typename Total, typename RowSum>
+__device__ __forceinline__ void team_sums(uint32_t G, uint32_t rows_at_a_time, uint32_t team,
+                                          Total total, RowSum row_sum) {
   const uint32_t t = threadIdx.x;
-  const uint32_t g = t / at.team, j = t - g * at.team;
+  const uint32_t g = t / team, j = t - g * team;
   A acc[kN];
 #pragma unroll
   for (int k = 0; k < kN; ++k) acc[k] = A(0);
-  if (g < d.G) {
-    for (uint32_t rr = j; rr < at.rows_at_a_time; rr += at.team) row_sum(g, rr, acc);
+  if (g < G) {
+    for (uint32_t rr = j; rr < rows_at_a_time; rr += team) row_sum(g, rr, acc);
   }
-  for (uint32_t o = 1; o < at.team; o <<= 1) {
+  for (uint32_t o = 1; o < team; o <<= 1) {
 #pragma unroll
     for (int k = 0; k < kN; ++k) acc[k] += __shfl_xor(acc[k], static_cast<int>(o), kWaveSize);
   }
-  if (g < d.G && j == 0) {
+  if (g < G && j == 0) {
 #pragma unroll
     for (int k = 0; k < kN; ++k) total[k][g] = acc[k];
   }
   __syncthreads();
+}
+template <int kN, int kVec, typename A, typename RowSum>
+__device__ __forceinline__ void slice_team_sums(const SampleSlices& d, const SliceSeat<kVec>& at,
+                                                A (*total)[kMaxSliceThreads], RowSum row_sum) {
+  team_sums<kN, A>(d.G, at.rows_at_a_time, at.team, total, row_sum);
 }
 
 // Groups of whole packets: kN values per thread, all for the group of its packet.

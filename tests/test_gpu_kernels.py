@@ -542,8 +542,10 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # rows of 160 / 320 packets leave too many of a slice workgroup's threads without a
             # row: the column reductions
             ((2, 40, 41, 1280), -1, 32),
-            # groups of half a packet (the column-reduction structure)
-            ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32),
+            # groups narrower than a packet: a share per channel of the packet (and more samples
+            # than workgroups)
+            ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32), ((600, 4, 4, 96), -1, 32),
+            ((1100, 3, 3, 32), -1, 8),
             # small groups, a wavefront each in the fused backward: more channels per group
             # than lanes, three channels per group, more groups than the grid's wavefronts hold
             ((2, 160, 3, 3), 1, 2), ((5, 96, 8, 8), 1, 32), ((40, 64, 14, 14), 1, 32),
