@@ -3623,8 +3623,13 @@ int group_norm_grad_nhwc_samples_threads(const GroupShape& sh, int* slots_out) {
   // Groups narrower than a packet keep a sum of dy x and of dy per channel: four packets per
   // thread and tensor at most (80 bytes per thread are spilled there in 16-bit types, outside
   // the store loop; the smaller workgroup is still ahead of two packets on twice the threads:
-  // bf16 [8192,16*16,32] 106 against 119 us).
-  for (const int64_t most : {sh.D < kVec ? 4 : 8}) {
+  // bf16 [8192,16*16,32] 106 against 119 us). Groups that are not whole packets look for four
+  // packets first: at eight the two-group flavour spills 110 bytes per thread, and what it
+  // reloads inside the store loop queues behind the packets requested ahead (bf16
+  // [1024,8*8,320] 50 us on 512 threads with eight packets, 39 us on 1024 with four). Groups of
+  // whole packets are better off with eight packets on the smaller workgroup (76-81 us against
+  // 80-90 us on 64 KB samples).
+  for (const int64_t most : {sh.D % kVec != 0 ? 4 : 8, sh.D < kVec ? 4 : 8}) {
     for (const uint32_t threads : {256u, 512u, 1024u}) {
       if (cps > threads) continue;
       const uint32_t rows_at_a_time = threads / cps;
