@@ -133,14 +133,17 @@ CoopPlan plan_coop(const SliceUnits& u, int kIn, bool windows = false) {
   if (kmax < kmin) kmax = kmin;
   if (kmax > klimit) kmax = klimit;
   if (kmax > kmin + 64) kmax = kmin + 64;
-  // The K whose units*K items fill whole rounds of the resident grid best.
-  int64_t best = kmin;
-  double best_util = 0;
+  // The K with the least estimated time: the resident grid works through units*K items in
+  // rounds, and a round costs its slice (packets per workgroup) plus the exchange, which is
+  // worth about 800 packets of streaming (4 us at a workgroup's share of the bandwidth).
+  // More, smaller slices fill the last round better but pay the exchange more often
+  // (GroupNorm bf16 [55,384,56,56] in 16 groups: 8 slices 75 us, 3 slices 60 us).
+  constexpr int64_t kExchangePackets = 800;
+  int64_t best = kmin, best_cost = INT64_MAX;
   for (int64_t k = kmin; k <= kmax; ++k) {
     const int64_t items = static_cast<int64_t>(u.units) * k;
-    const double util = static_cast<double>(items) / (ceil_div(items, grid) * grid);
-    if (util > best_util + 1e-9) best = k, best_util = util;
-    if (util >= 0.96) break;
+    const int64_t cost = ceil_div(items, grid) * (kExchangePackets + ceil_div(P, k));
+    if (cost < best_cost) best = k, best_cost = cost;
   }
   p.K = static_cast<uint32_t>(best);
   // whole wavefronts of packets per slice, so that a wavefront never straddles two slices
