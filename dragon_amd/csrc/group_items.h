@@ -1,5 +1,5 @@
-// NCHW GroupNorm forward for groups that one 256- or 512-thread workgroup
-// holds whole (up to sixteen packets per thread of 512: 128 KB in 16-bit types).
+// NCHW GroupNorm forward for groups that one workgroup of 256, 512 or 1024 threads
+// holds whole (up to sixteen packets per thread of 1024: 256 KB in 16-bit types).
 //
 // A group (n, g) is a contiguous run of D * S elements. Thread t keeps packets
 // t, t + kThreads, ... of the group in registers between the statistics and the
@@ -20,7 +20,7 @@
 namespace dragon_hip {
 
 constexpr int kItemPackets = 16;      // packets per thread at most
-constexpr uint32_t kMaxItemChannels = 512;  // channels per group whose parameters fit the LDS table
+constexpr uint32_t kMaxItemChannels = 1024;  // channels per group whose parameters fit the LDS table
 
 // Wavefronts per SIMD asked of the compiler: four (128 registers) hold sixteen packets per
 // thread; ten packets fit the 80 registers of six, i.e. three 512-thread workgroups per compute
@@ -154,7 +154,7 @@ struct GroupItemPlan {
 };
 
 // Groups of whole packets with channels of whole packets that 256 threads hold at
-// ten packets per thread or 512 threads at sixteen.
+// ten packets per thread, or 512 or 1024 threads at sixteen.
 template <typename T>
 inline GroupItemPlan plan_group_items(int64_t D, int64_t S) {
   constexpr int kVec = IO<T>::kVec;
@@ -171,7 +171,11 @@ inline GroupItemPlan plan_group_items(int64_t D, int64_t S) {
   // of 40 / 64 / 80 / 96 KB, the chosen flavour against sixteen packets on the smallest workgroup
   // that holds the group: 59.5 / 46.9 / 58.1 / 52.2 us against 61.7 / 50.6 / 63.2 / 53.5 us.
   struct Choice { int vpt, threads; };
-  constexpr Choice kChoices[] = {{8, 256}, {10, 256}, {8, 512}, {10, 512}, {12, 512}, {16, 512}};
+  // Beyond 128 KB (in 16-bit types) one 1024-thread workgroup per compute unit: still ahead of
+  // cutting the group into slices that exchange their sums (bf16 groups of 147 / 160 / 196 KB:
+  // 54.9 / 122 / 54.5 us against 65.4 / 145 / 68.8 us; level at 256 KB).
+  constexpr Choice kChoices[] = {{8, 256},  {10, 256}, {8, 512},   {10, 512},  {12, 512},
+                                 {16, 512}, {10, 1024}, {12, 1024}, {16, 1024}};
   for (const Choice& c : kChoices) {
     if (npackets > static_cast<int64_t>(c.threads) * c.vpt || D > c.threads) continue;
     p.ok = true;
@@ -222,9 +226,11 @@ int try_group_norm_forward_items(int64_t N, int64_t G, int64_t D, int64_t S, flo
   }
     if (p.threads == 256) {
       if (p.vpt == 8) LAUNCH(8, 256) else LAUNCH(10, 256)
-    } else {
+    } else if (p.threads == 512) {
       if (p.vpt == 8) LAUNCH(8, 512) else if (p.vpt == 10) LAUNCH(10, 512)
       else if (p.vpt == 12) LAUNCH(12, 512) else LAUNCH(16, 512)
+    } else {
+      if (p.vpt == 10) LAUNCH(10, 1024) else if (p.vpt == 12) LAUNCH(12, 1024) else LAUNCH(16, 1024)
     }
 #undef LAUNCH
     return status_of_launch();

@@ -296,6 +296,11 @@ NCHW_ITEM_CASES = [
     # every flavour: eight and ten packets on 256 threads, eight to sixteen on 512
     (2, 2, 20, 1024, "bfloat16", 0), (3, 3, 10, 4096, "bfloat16", 0), (2, 2, 12, 4096, "float16", 0),
     (2, 5, 10, 1000, "float32", 0), (2, 3, 11, 2048, "float32", 0), (40, 2, 5, 4096, "float32", 0),
+    # groups of 128-256 KB on 1024 threads (ten, twelve and sixteen packets; more channels than
+    # 512 threads; more groups than compute units)
+    (1, 2, 32, 3136, "bfloat16", 0), (1, 3, 24, 3136, "bfloat16", 0), (2, 2, 20, 4096, "float16", 0),
+    (1, 2, 45, 2048, "bfloat16", 0), (1, 2, 12, 4096, "float32", 0), (1, 2, 600, 64, "bfloat16", 0),
+    (6, 16, 16, 4096, "float32", 0),
 ]
 
 
