@@ -215,8 +215,9 @@ int try_group_norm_forward_items(int64_t N, int64_t G, int64_t D, int64_t S, flo
         rows < nominal * 4;                                                                       \
     note_flavour("group_norm_forward_items<" #VPT "," #THREADS ">");                              \
     note_number("walk", walk ? 1 : 0);                                                            \
-    hipLaunchKernelGGL(kernel,                                                                    \
-                       dim3(walk && rows > resident ? resident : static_cast<unsigned>(rows)),    \
+    /* (a launch holds fewer than 2^32 threads: beyond 2^21 workgroups they walk as well) */      \
+    const unsigned most = walk ? resident : 1u << 21;                                             \
+    hipLaunchKernelGGL(kernel, dim3(rows > most ? most : static_cast<unsigned>(rows)),            \
                        dim3(THREADS), 0, stream, static_cast<uint32_t>(rows),                     \
                        static_cast<uint32_t>(D * S / kVec), static_cast<uint32_t>(G),             \
                        static_cast<uint32_t>(D), static_cast<uint32_t>(S / kVec), A(eps),         \

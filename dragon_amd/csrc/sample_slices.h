@@ -768,7 +768,7 @@ int try_group_norm_forward_nhwc_slices(uint32_t N, uint32_t S, uint32_t C, uint3
     /* workgroups finish, is ahead of workgroups that walk the samples and request one ahead */ \
     /* (bf16 [8192, 7*7, 256] 77.6 -> 71.2 us; with two per workgroup 48.9 against 50.6 us). */ \
     const bool walk = p.K > 1 || d.items < 4u * num_cus() * (THREADS == 256 ? 4u : 2u);          \
-    if (!walk) cap = d.items;                                                                     \
+    if (!walk) cap = 1u << 21; /* (a launch holds fewer than 2^32 threads) */                     \
     note_flavour(SPLIT == kSplitEach ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",each>"       \
                  : SPLIT == kSplitTwo ? "group_norm_nhwc_slices<" #VPT "," #THREADS ",two>"       \
                                       : "group_norm_nhwc_slices<" #VPT "," #THREADS ">");         \
