@@ -546,6 +546,8 @@ GN_CASES = [((2, 32, 8, 8), 1, 4), ((3, 12, 5), 1, 3), ((2, 6, 6, 16), -1, 4), (
             # than workgroups)
             ((2, 14, 14, 128), -1, 32), ((3, 6, 6, 64), -1, 32), ((600, 4, 4, 96), -1, 32),
             ((1100, 3, 3, 32), -1, 8),
+            # more narrow groups than the team sums take (512): the column reductions
+            ((2, 4, 4, 1024), -1, 512),
             # small groups, a wavefront each in the fused backward: more channels per group
             # than lanes, three channels per group, more groups than the grid's wavefronts hold
             ((2, 160, 3, 3), 1, 2), ((5, 96, 8, 8), 1, 32), ((40, 64, 14, 14), 1, 32),
