@@ -576,6 +576,7 @@ struct CoopForward {
   static constexpr int kIn = 1;
   static constexpr bool kBeginReadsInput = true;
   static constexpr bool kWindows = true;
+  static constexpr bool kWholeUnits = true;
   using Merge = PairSum;
   A inv_n, momentum, one_minus_momentum, eps;
   const A* gamma;
@@ -628,6 +629,7 @@ struct CoopBackward {
   using A = typename IO<T>::Acc;
   static constexpr int kIn = 2;
   static constexpr bool kWindows = true;
+  static constexpr bool kWholeUnits = true;
   using Merge = PairSum;
   A normalizer;
   const A* mu;

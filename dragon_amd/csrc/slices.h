@@ -185,7 +185,7 @@ struct CoopShape {
   uint32_t seglen;       // elements per run
   uint32_t P;            // packets per unit
   uint32_t seg_stride;   // elements between two runs of a unit
-  uint32_t step_seg, step_p;  // kCoopThreads packets further on = step_seg segments and step_p packets
+  uint32_t step_seg, step_p;  // a workgroup's threads further on = step_seg segments and step_p packets
   uint32_t items;        // units * K
   uint32_t patience;     // polls of a slot before a thread gives up
   uint32_t* flags;       // flags[w] = 1: item w gave up; flags[items] = 1: some item did
@@ -194,7 +194,7 @@ struct CoopShape {
 
 template <typename T>
 CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p, typename IO<T>::Acc* scratch,
-                          bool windows = false) {
+                          bool windows = false, uint32_t threads = kCoopThreads) {
   constexpr int kVec = IO<T>::kVec;
   CoopShape d;
   d.unit_stride = u.unit_stride, d.K = p.K, d.slice = p.slice;
@@ -202,7 +202,7 @@ CoopShape make_coop_shape(const SliceUnits& u, const CoopPlan& p, typename IO<T>
   d.seglen = u.seglen;
   d.P = u.nseg * d.pps;
   d.seg_stride = u.seg_stride;
-  d.step_seg = kCoopThreads / d.pps, d.step_p = kCoopThreads % d.pps;
+  d.step_seg = threads / d.pps, d.step_p = threads % d.pps;
   d.items = u.units * p.K;
   const uint32_t patience = exchange_patience();
   d.patience = patience ? patience : kCoopPatience;
@@ -327,9 +327,9 @@ struct PairSum {
 
 // All-reduce of a pair over the workgroup with Merge; every thread returns the
 // same bits (the per-wavefront results are merged in wavefront order).
-template <typename Merge, typename A>
-__device__ __forceinline__ void block_merge_pair(A& a, A& b, A* lds /*2*kReduceWaves*/) {
-  if constexpr (Merge::kIsSum) {
+template <typename Merge, int kWaves = kReduceWaves, typename A>
+__device__ __forceinline__ void block_merge_pair(A& a, A& b, A* lds /*2*kWaves*/) {
+  if constexpr (Merge::kIsSum && kWaves == kReduceWaves) {
     block_reduce_pair(a, b, lds);
   } else {
 #pragma unroll
@@ -345,7 +345,7 @@ __device__ __forceinline__ void block_merge_pair(A& a, A& b, A* lds /*2*kReduceW
     __syncthreads();
     a = lds[0], b = lds[1];
 #pragma unroll
-    for (int i = 1; i < kReduceWaves; ++i) Merge::merge(a, b, lds[2 * i], lds[2 * i + 1]);
+    for (int i = 1; i < kWaves; ++i) Merge::merge(a, b, lds[2 * i], lds[2 * i + 1]);
   }
 }
 
@@ -451,10 +451,11 @@ struct CoopItem {
     len = j1 > j0 ? j1 - j0 : 0u;
     base = c * d.unit_stride;
   }
-  __device__ __forceinline__ bool has(int i) const { return i * kCoopThreads + threadIdx.x < len; }
+  template <int kThreads = kCoopThreads>
+  __device__ __forceinline__ bool has(int i) const { return i * kThreads + threadIdx.x < len; }
 };
 
-template <typename T, int kR, int kIn, bool kWin>
+template <typename T, int kR, int kIn, bool kWin, int kThreads = kCoopThreads>
 __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const T* in0, const T* in1,
                                           CoopSlice<T, kR, kIn>& s) {
   const CoopItem it(d, w);
@@ -463,7 +464,7 @@ __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const 
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     const CoopSlot at = coop_slot<T, kWin>(d, cur, it.base, in0);
-    const int32_t off = it.has(i) && at.hi > at.lo ? at.off : safe;
+    const int32_t off = it.template has<kThreads>(i) && at.hi > at.lo ? at.off : safe;
     s.p0[i] = load_packet(in0 + off);
     if constexpr (kIn == 2) s.p1[i] = load_packet(in1 + off);
     cur.advance(d);
@@ -474,7 +475,7 @@ __device__ __forceinline__ void coop_load(const CoopShape& d, uint32_t w, const 
 // packets are requested one by one into the registers the second pass has just
 // written out, so they travel while the rest of this item is stored.
 // kRepair: the second launch, which finishes the items whose wait ran out.
-template <typename T, int kR, typename Op, bool kRepair, bool kWin>
+template <typename T, int kR, typename Op, bool kRepair, bool kWin, int kThreads = kCoopThreads>
 __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uint32_t next,
                                              const T* in0, const T* in1, T* out, Op op,
                                              CoopSlice<T, kR, Op::kIn>& s,
@@ -492,7 +493,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
   if constexpr (OpScansFirst<Op>::value) {
 #pragma unroll
     for (int i = 0; i < kR; ++i) {
-      if (it.has(i)) {
+      if (it.template has<kThreads>(i)) {
         A xv[kVec];
         IO<T>::unpack(s.p0[i], xv);
         op.scan(xv);
@@ -507,7 +508,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     const CoopSlot at = coop_slot<T, kWin>(d, acur, it.base, in0);
-    if (it.has(i) && at.hi > at.lo) {
+    if (it.template has<kThreads>(i) && at.hi > at.lo) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
@@ -525,7 +526,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
             if (e < at.lo || e >= at.hi) op.neutral(xv[e], dv[e]);
           }
         }
-        op.accumulate(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv, a, b);
+        op.accumulate(it.c, it.j0 + i * kThreads + threadIdx.x, xv, dv, a, b);
       }
     }
     if constexpr (kWin) acur.advance(d);
@@ -537,8 +538,8 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
     // exchanged (the host launches neither the fill nor the repair). Items take
     // the two LDS buffers by turns: the barrier of one item's reduction lies
     // between another's reads and writes of the same buffer.
-    block_merge_pair<typename Op::Merge>(a, b, ((w / gridDim.x) & 1u) ? lds_b : lds_a);
-  } else {
+    block_merge_pair<typename Op::Merge, kThreads / kWaveSize>(a, b, ((w / gridDim.x) & 1u) ? lds_b : lds_a);
+  } else if constexpr (kThreads == kCoopThreads) {
     complete = coop_channel_totals<typename Op::Merge, kRepair>(d, it.c, w, a, b, partial, lds_a,
                                                                 lds_b);
   }
@@ -557,11 +558,11 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     const CoopSlot at = coop_slot<T, kWin>(d, cur, it.base, in0);
-    if (complete && it.has(i) && at.hi > at.lo) {
+    if (complete && it.template has<kThreads>(i) && at.hi > at.lo) {
       A xv[kVec], dv[kVec];
       IO<T>::unpack(s.p0[i], xv);
       if constexpr (Op::kIn == 2) IO<T>::unpack(s.p1[i], dv);
-      op.transform(it.c, it.j0 + i * kCoopThreads + threadIdx.x, xv, dv);
+      op.transform(it.c, it.j0 + i * kThreads + threadIdx.x, xv, dv);
       if (!kWin || at.template whole<kVec>()) {
         store_packet(out + at.off, IO<T>::pack(xv));
       } else {
@@ -574,7 +575,7 @@ __device__ __forceinline__ void coop_process(const CoopShape& d, uint32_t w, uin
     cur.advance(d);
     if (more) {
       const CoopSlot nat = coop_slot<T, kWin>(d, ncur, nit.base, in0);
-      const int32_t off = nit.has(i) && nat.hi > nat.lo ? nat.off : nsafe;
+      const int32_t off = nit.template has<kThreads>(i) && nat.hi > nat.lo ? nat.off : nsafe;
       s.p0[i] = load_packet(in0 + off);
       if constexpr (Op::kIn == 2) s.p1[i] = load_packet(in1 + off);
       ncur.advance(d);
@@ -623,6 +624,84 @@ __global__ __launch_bounds__(kCoopThreads, kR * Op::kIn > 16 ? 3 : 4) void chann
   }
 }
 
+// What a launcher returns when the shape or the addresses leave the call to another path.
+constexpr int kNotApplicable = 1;
+
+// Units that a workgroup of 512 or 1024 threads holds whole (K = 1: nothing is exchanged, and
+// nothing waits, so the workgroups need not be resident together: one per unit, handed out by
+// the hardware as workgroups finish). Two or one per compute unit at 128 registers.
+template <typename T, int kR, int kThreads, typename Op, bool kWin>
+__global__ __launch_bounds__(kThreads, 4) void channel_whole(
+    const CoopShape d, const T* __restrict__ in0, const T* __restrict__ in1, T* __restrict__ out,
+    const Op op) {
+  using A = typename IO<T>::Acc;
+  __shared__ A lds_a[2 * (kThreads / kWaveSize)];
+  __shared__ A lds_b[2 * (kThreads / kWaveSize)];
+  for (uint32_t w = blockIdx.x; w < d.items; w += gridDim.x) {
+    CoopSlice<T, kR, Op::kIn> s;
+    coop_load<T, kR, Op::kIn, kWin, kThreads>(d, w, in0, in1, s);
+    coop_process<T, kR, Op, false, kWin, kThreads>(d, w, d.items, in0, in1, out, op, s, nullptr,
+                                                   lds_a, lds_b);
+  }
+}
+
+// Whether an Op's units may take channel_whole (BatchNorm's: plain accumulate / transform).
+template <typename Op, typename = void>
+struct OpTakesWholeUnits : std::false_type {};
+template <typename Op>
+struct OpTakesWholeUnits<Op, std::void_t<decltype(Op::kWholeUnits)>>
+    : std::bool_constant<Op::kWholeUnits> {};
+
+// Threads (512 or 1024) and packets per thread and tensor of a unit of P packets that is held
+// whole, 0 where none holds it or 256 threads do: sixteen packets at most for one tensor, eight
+// each for two.
+inline int whole_unit_threads(int64_t P, int kIn, int* r) {
+  const int rmax = kIn == 1 ? 16 : 8;
+  if (P <= static_cast<int64_t>(kCoopThreads) * rmax) return 0;  // a slice of the 256-thread kernel
+  for (const int threads : {512, 1024}) {
+    if (P <= static_cast<int64_t>(threads) * rmax) {
+      const int need = static_cast<int>(ceil_div(P, threads));
+      *r = need <= 8 / kIn ? 8 / kIn : 16 / kIn;
+      return threads;
+    }
+  }
+  return 0;
+}
+
+template <typename T, typename Op, bool kWin>
+int launch_channel_whole(const SliceUnits& sh, const Op& op, const T* in0, const T* in1, T* out,
+                         hipStream_t stream) {
+  constexpr int kIn = Op::kIn;
+  constexpr int kVec = IO<T>::kVec;
+  // (short runs are left to the split reduction, as in plan_coop)
+  if (sh.seglen / kVec < (kWin ? 24u : 16u)) return kNotApplicable;
+  // Fewer units than compute units: slices spread them over more workgroups.
+  if (sh.units < static_cast<uint32_t>(num_cus())) return kNotApplicable;
+  const uint32_t pps = sh.seglen / kVec + (kWin ? 2 : 0);
+  const int64_t P = static_cast<int64_t>(sh.nseg) * pps;
+  int r = 0;
+  const int threads = whole_unit_threads(P, kIn, &r);
+  if (threads == 0) return kNotApplicable;
+  CoopPlan p = {true, 1u, static_cast<uint32_t>(ceil_div(P, kWaveSize) * kWaveSize), r};
+  typename IO<T>::Acc* none = nullptr;  // no pairs, no flags: nothing is exchanged
+  CoopShape d = make_coop_shape<T>(sh, p, none, kWin, static_cast<uint32_t>(threads));
+  d.flags = nullptr;
+  const unsigned grid = d.items < (1u << 21) ? d.items : 1u << 21;
+#define DRAGON_HIP_WHOLE_LAUNCH(R, THREADS)                                                     \
+  {                                                                                            \
+    if (kWin) note_flavour("windows");                                                         \
+    hipLaunchKernelGGL((channel_whole<T, R, THREADS, Op, kWin>), dim3(grid), dim3(THREADS), 0, \
+                       stream, d, in0, in1, out, op);                                          \
+  }
+  if (threads == 512) {
+    if (r * kIn <= 8) DRAGON_HIP_WHOLE_LAUNCH(8 / kIn, 512) else DRAGON_HIP_WHOLE_LAUNCH(16 / kIn, 512)
+  } else {
+    if (r * kIn <= 8) DRAGON_HIP_WHOLE_LAUNCH(8 / kIn, 1024) else DRAGON_HIP_WHOLE_LAUNCH(16 / kIn, 1024)
+  }
+#undef DRAGON_HIP_WHOLE_LAUNCH
+  return status_of_launch();
+}
+
 template <typename A>
 inline void fill_unset(A* pairs, const CoopShape& d, hipStream_t stream) {
   using Bits = typename Unset<A>::Bits;
@@ -635,7 +714,6 @@ inline void fill_unset(A* pairs, const CoopShape& d, hipStream_t stream) {
 // DRAGON_HIP_OK when the single-read kernel was launched, kNotApplicable when
 // the shape or alignment leaves the call to the split path, or an error.
 // `scratch` holds coop_scratch_bytes<T>(sh) bytes.
-constexpr int kNotApplicable = 1;
 constexpr unsigned kCoopRepairGrid = 256;
 template <typename T, typename Op, bool kWin>
 int launch_channel_slices(const SliceUnits& sh, const CoopPlan& p, const Op& op, const T* in0,
@@ -684,12 +762,22 @@ int try_channel_slices(const SliceUnits& sh, const Op& op, const T* in0, const T
   const bool packets = sh.seglen % IO<T>::kVec == 0 && sh.unit_stride % IO<T>::kVec == 0 &&
       sh.seg_stride % IO<T>::kVec == 0 && aligned16(in0) && aligned16(in1) && aligned16(out);
   if (packets) {
+    if constexpr (OpTakesWholeUnits<Op>::value) {
+      // units of 64-256 KB per tensor (64-128 KB each for two): whole, instead of 2-4 slices
+      // that exchange their sums
+      const int st = launch_channel_whole<T, Op, false>(sh, op, in0, in1, out, stream);
+      if (st != kNotApplicable) return st;
+    }
     const CoopPlan p = plan_coop<T>(sh, kIn);
     if (!p.ok || (in_place_hazard && p.K > 1)) return kNotApplicable;
     return launch_channel_slices<T, Op, false>(sh, p, op, in0, in1, out, scratch, stream);
   }
   if constexpr (OpTakesWindows<Op>::value) {
     if (sizeof(T) > 4 || !congruent16(in0, in1) || !congruent16(in0, out)) return kNotApplicable;
+    if constexpr (OpTakesWholeUnits<Op>::value) {
+      const int st = launch_channel_whole<T, Op, true>(sh, op, in0, in1, out, stream);
+      if (st != kNotApplicable) return st;
+    }
     const CoopPlan p = plan_coop<T>(sh, kIn, true);
     if (!p.ok || (in_place_hazard && p.K > 1)) return kNotApplicable;
     return launch_channel_slices<T, Op, true>(sh, p, op, in0, in1, out, scratch, stream);

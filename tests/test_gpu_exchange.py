@@ -22,7 +22,7 @@ def K():
 
 def _bn_forward(K, t, S=56 * 56):
     import torch
-    N, C = 8, 40  # six slices per channel
+    N, C = 24, 40  # 300 KB per channel: several slices (up to 256 KB a workgroup holds it whole)
     x = t["x"] if "x" in t else t.setdefault("x", torch.randn((N, C, S), device="cuda") * 2 + 0.5)
     g = t.setdefault("g", torch.rand(C, device="cuda") + 0.5)
     b = t.setdefault("b", torch.randn(C, device="cuda") * 0.1)
@@ -35,7 +35,7 @@ def _bn_forward(K, t, S=56 * 56):
 
 def _bn_backward(K, t, S=56 * 56):
     import torch
-    N, C = 8, 40
+    N, C = 24, 40
     x = t.setdefault("x", torch.randn((N, C, S), device="cuda") * 2 + 0.5)
     dy = t.setdefault("dy", torch.randn((N, C, S), device="cuda"))
     g = t.setdefault("g", torch.rand(C, device="cuda") + 0.5)
@@ -159,7 +159,7 @@ def test_waits_that_run_out_are_repaired_in_stream_order(K, name):
 
 def test_repaired_batch_norm_matches_the_oracle(K):
     import torch
-    N, C, S = 8, 40, 56 * 56
+    N, C, S = 24, 40, 56 * 56
     rng = U.rng_for(77)
     x = (2 * rng.standard_normal((N, C, S)) + 0.5).astype(np.float32)
     g, b = U.affine_params(rng, C, "float32")
@@ -175,10 +175,14 @@ def test_repaired_batch_norm_matches_the_oracle(K):
     finally:
         K.exchange_reset(0)
     assert U.normwise(U.to_host(y), y_ref) <= 1e-5
-    assert U.normwise(U.to_host(mu), mu_ref) <= 1e-5
-    assert U.normwise(U.to_host(params), params_ref) <= 1e-5
+    # 75264 elements per channel: the oracle's sequential fp32 sum is itself off, so the mean is
+    # judged three-way against the fp64 result
+    mu64 = np.asarray(x, np.float64).mean((0, 2))
+    ok, e_go, e_ge, e_oe = U.close3(U.to_host(mu), mu_ref, mu64, 1e-5)
+    assert ok, (e_go, e_ge, e_oe)
+    assert U.normwise(U.to_host(params), params_ref) <= 2e-5
     # _bn_forward starts the running statistics at 0.25 / 1.5
-    assert U.normwise(U.to_host(rm), 0.9 * np.float32(0.25) + (1 - 0.9) * mu_ref) <= 1e-5
+    assert U.normwise(U.to_host(rm), 0.9 * np.float32(0.25) + (1 - 0.9) * mu64) <= 1e-5
     var_ref = 1.0 / np.asarray(rsig_ref, np.float64) ** 2 - 1e-5
     assert U.normwise(U.to_host(rv), 0.9 * 1.5 + 0.1 * var_ref) <= 1e-4
 
@@ -190,7 +194,7 @@ def test_an_input_holding_the_unset_pattern_does_not_stall_the_exchange(K):
     make it, the others are untouched, and nothing had to be repaired."""
     import torch
     K.exchange_reset(0)
-    N, C, S = 8, 40, 56 * 56
+    N, C, S = 24, 40, 56 * 56
     t = {}
     want = _bn_forward(K, t)
     xp = t["x"].clone()
