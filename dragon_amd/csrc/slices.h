@@ -652,18 +652,14 @@ template <typename Op>
 struct OpTakesWholeUnits<Op, std::void_t<decltype(Op::kWholeUnits)>>
     : std::bool_constant<Op::kWholeUnits> {};
 
-// Threads (512 or 1024) and packets per thread and tensor of a unit of P packets that is held
-// whole, 0 where none holds it or 256 threads do: sixteen packets at most for one tensor, eight
-// each for two.
-inline int whole_unit_threads(int64_t P, int kIn, int* r) {
-  const int rmax = kIn == 1 ? 16 : 8;
+// Threads (512 or 1024) that hold a unit of P packets whole at sixteen packets per thread (one
+// tensor) or eight each (two), 0 where neither does or 256 threads do. (Every such unit needs
+// more than half of those packets, so there is one flavour per workgroup size.)
+inline int whole_unit_threads(int64_t P, int kIn) {
+  const int rmax = 16 / kIn;
   if (P <= static_cast<int64_t>(kCoopThreads) * rmax) return 0;  // a slice of the 256-thread kernel
   for (const int threads : {512, 1024}) {
-    if (P <= static_cast<int64_t>(threads) * rmax) {
-      const int need = static_cast<int>(ceil_div(P, threads));
-      *r = need <= 8 / kIn ? 8 / kIn : 16 / kIn;
-      return threads;
-    }
+    if (P <= static_cast<int64_t>(threads) * rmax) return threads;
   }
   return 0;
 }
@@ -679,26 +675,21 @@ int launch_channel_whole(const SliceUnits& sh, const Op& op, const T* in0, const
   if (sh.units < static_cast<uint32_t>(num_cus())) return kNotApplicable;
   const uint32_t pps = sh.seglen / kVec + (kWin ? 2 : 0);
   const int64_t P = static_cast<int64_t>(sh.nseg) * pps;
-  int r = 0;
-  const int threads = whole_unit_threads(P, kIn, &r);
+  const int threads = whole_unit_threads(P, kIn);
   if (threads == 0) return kNotApplicable;
-  CoopPlan p = {true, 1u, static_cast<uint32_t>(ceil_div(P, kWaveSize) * kWaveSize), r};
+  CoopPlan p = {true, 1u, static_cast<uint32_t>(ceil_div(P, kWaveSize) * kWaveSize), 16 / kIn};
   typename IO<T>::Acc* none = nullptr;  // no pairs, no flags: nothing is exchanged
   CoopShape d = make_coop_shape<T>(sh, p, none, kWin, static_cast<uint32_t>(threads));
   d.flags = nullptr;
   const unsigned grid = d.items < (1u << 21) ? d.items : 1u << 21;
-#define DRAGON_HIP_WHOLE_LAUNCH(R, THREADS)                                                     \
-  {                                                                                            \
-    if (kWin) note_flavour("windows");                                                         \
-    hipLaunchKernelGGL((channel_whole<T, R, THREADS, Op, kWin>), dim3(grid), dim3(THREADS), 0, \
-                       stream, d, in0, in1, out, op);                                          \
-  }
+  if (kWin) note_flavour("windows");
   if (threads == 512) {
-    if (r * kIn <= 8) DRAGON_HIP_WHOLE_LAUNCH(8 / kIn, 512) else DRAGON_HIP_WHOLE_LAUNCH(16 / kIn, 512)
+    hipLaunchKernelGGL((channel_whole<T, 16 / kIn, 512, Op, kWin>), dim3(grid), dim3(512), 0, stream,
+                       d, in0, in1, out, op);
   } else {
-    if (r * kIn <= 8) DRAGON_HIP_WHOLE_LAUNCH(8 / kIn, 1024) else DRAGON_HIP_WHOLE_LAUNCH(16 / kIn, 1024)
+    hipLaunchKernelGGL((channel_whole<T, 16 / kIn, 1024, Op, kWin>), dim3(grid), dim3(1024), 0,
+                       stream, d, in0, in1, out, op);
   }
-#undef DRAGON_HIP_WHOLE_LAUNCH
   return status_of_launch();
 }
 
