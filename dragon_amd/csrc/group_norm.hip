@@ -3936,9 +3936,11 @@ int launch_group_norm_grad(const GroupShape& sh, const void* x, const void* mu, 
     note_flavour(split == kSplitEach ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",each>" \
                  : split == kSplitTwo ? "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ",two>" \
                                       : "group_norm_grad_nhwc_samples<" #VPT "," #THREADS ">");  \
-    auto kernel = split == kSplitEach ? group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitEach> \
-        : split == kSplitTwo ? group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitTwo>          \
-                             : group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitNone>;        \
+    auto kernel = split == kSplitTwo ? group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitTwo>  \
+                                     : group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitNone>; \
+    if constexpr (VPT <= 4) { /* (narrow groups never take eight packets per thread) */          \
+      if (split == kSplitEach) kernel = group_norm_grad_nhwc_samples<T, VPT, THREADS, kSplitEach>; \
+    }                                                                                            \
     const unsigned resident = resident_grid(kernel, THREADS, 0);                                 \
     grid = nhwc_sample_rows(sh.N);                                                               \
     if (grid > resident) grid = resident;                                                        \
